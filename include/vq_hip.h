@@ -1,0 +1,121 @@
+/*
+ * vq_hip.h — C ABI of libvqhip: the codebook hot path of the `vq` crate on MI355X (gfx950).
+ *
+ * The reference is a pure-Rust crate with no FFI layer; the seam this library fills is the
+ * crate-private `utils::lbg_quantize` (src/utils.rs:32-109) and the inline nearest-centroid
+ * loops of the four codebook quantizers.  A Rust `-sys` crate binds exactly these symbols
+ * (plain pointers and sizes, no C++ or torch types).
+ *
+ * Conventions
+ *   - every function returns an int32 status: 0 = VQ_OK, negative = error; the message of
+ *     the last error of a context is returned by vq_last_error().
+ *   - pointers named d_* are DEVICE pointers (from vq_malloc or any HIP allocation on the
+ *     context's device); pointers named h_* are host pointers.
+ *   - matrices are row-major f32, `ld` = row stride in elements; a "column block" s of width
+ *     sub_dim covers columns [s*sub_dim, (s+1)*sub_dim).
+ *   - codes are uint8 (k <= 256), row-major n x m unless stated otherwise.
+ *   - all work is enqueued on the context's stream; functions that return host values
+ *     synchronise that stream before returning, the others are asynchronous.
+ *   - one context = one stream; a context is not re-entrant, distinct contexts are independent.
+ *   - randomness never crosses the boundary as a seed: the host draws the index streams
+ *     (initial rows, re-seed rows) with its own RNG and passes them as arrays.
+ */
+#ifndef VQ_HIP_H
+#define VQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct vq_ctx vq_ctx;
+
+enum vq_status {
+    VQ_OK = 0,
+    VQ_ERR_INVALID_ARG = -1,      /* VqError::InvalidParameter, src/exceptions.rs:19 */
+    VQ_ERR_DIM_MISMATCH = -2,     /* VqError::DimensionMismatch, src/exceptions.rs:11 */
+    VQ_ERR_EMPTY_INPUT = -3,      /* VqError::EmptyInput, src/exceptions.rs:15 */
+    VQ_ERR_UNSUPPORTED = -4,      /* metric or size outside what the kernels cover */
+    VQ_ERR_OOM = -5,
+    VQ_ERR_HIP = -6,
+    VQ_ERR_RESEED_EXHAUSTED = -7  /* more empty clusters met than re-seed indices supplied */
+};
+
+/* Distance variants with a kernel (src/distances.rs:73-88; Chebyshev, Minkowski and Hamming
+ * stay on the host). */
+enum vq_metric {
+    VQ_SQEUCLIDEAN = 0, /* src/distances.rs:130-133 */
+    VQ_EUCLIDEAN = 1,   /* src/distances.rs:134-140 */
+    VQ_COSINE = 2,      /* src/distances.rs:141-151 */
+    VQ_MANHATTAN = 3    /* src/distances.rs:152 */
+};
+
+/* ---- context and device memory ------------------------------------------------------- */
+
+int32_t vq_ctx_create(int32_t device, vq_ctx **out);
+int32_t vq_ctx_destroy(vq_ctx *ctx);
+/* Message of the last failing call on ctx (ctx may be NULL: last failing vq_ctx_create). */
+const char *vq_last_error(const vq_ctx *ctx);
+int32_t vq_ctx_sync(vq_ctx *ctx);
+/* The context's hipStream_t, as an opaque pointer. */
+void *vq_ctx_stream(vq_ctx *ctx);
+
+int32_t vq_malloc(vq_ctx *ctx, size_t bytes, void **d_ptr);
+int32_t vq_free(vq_ctx *ctx, void *d_ptr);
+/* Synchronous copies (they synchronise the context's stream). Replaces the per-vector heap
+ * layout `&[Vector<f32>]` (src/vector.rs:150-152): the host packs rows into one buffer. */
+int32_t vq_h2d(vq_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
+int32_t vq_d2h(vq_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
+
+/* ---- timing (HIP events on the context's stream) --------------------------------------- */
+int32_t vq_timer_start(vq_ctx *ctx);
+/* Records the stop event, synchronises, returns elapsed milliseconds since vq_timer_start. */
+int32_t vq_timer_stop(vq_ctx *ctx, float *h_ms);
+
+/* ---- LBG training: replaces utils::lbg_quantize (src/utils.rs:32-109) ------------------ */
+
+/* m independent LBG problems, one per column block of width sub_dim of d_x (n x ld).
+ * m = 1, sub_dim = dim is the plain lbg_quantize call of src/rvq.rs:107; m > 1 is the batched
+ * form of the per-subspace calls at src/pq.rs:106-121 and src/opq.rs:127-142.
+ *
+ *   h_init_idx       m*k  row indices copied as initial centroids (choose_multiple, utils.rs:54)
+ *   h_reseed_stream  m*n_reseed  successive `choose` draws (utils.rs:100); the i-th empty
+ *                    cluster met by problem s (iteration-major, cluster index ascending) takes
+ *                    h_reseed_stream[s*n_reseed + i].  n_reseed = k*max_iters can never run out.
+ *   d_codebooks      out, m*k*sub_dim
+ *   h_iters_run      out (nullable), m: loop bodies executed per problem (early break, 104-106)
+ *   h_reseeds_used   out (nullable), m
+ * Assignment is squared-L2, sequential f32 accumulation, strict '<' (utils.rs:62-70); the mean
+ * follows mean_vector's order (src/vector.rs:282-318) for clusters of at most 1024 rows and a
+ * fixed midpoint tree above that.
+ * Errors: k == 0 or n < k -> VQ_ERR_INVALID_ARG (utils.rs:39-50); k > 256 -> VQ_ERR_UNSUPPORTED.
+ * Synchronises the stream before returning. */
+int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t m,
+                   int32_t sub_dim, int32_t k, int32_t max_iters, const uint32_t *h_init_idx,
+                   const uint32_t *h_reseed_stream, int32_t n_reseed, float *d_codebooks,
+                   int32_t *h_iters_run, int32_t *h_reseeds_used);
+
+/* ---- nearest-centroid assignment / encode ---------------------------------------------- */
+
+/* d_codes[i*m + s] = first index j minimising metric(x_i[block s], codebook[s][j]), strict '<'.
+ * Replaces the inline loops at src/pq.rs:166-174, src/opq.rs:155-163,250-258,
+ * src/rvq.rs:116-124,189-197 (m = 1 there).  Asynchronous. */
+int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
+                  int32_t sub_dim, int32_t k, const float *d_codebooks, uint8_t *d_codes);
+
+/* d_out[i*(m*sub_dim) + s*sub_dim + t] = f16(codebook[s][code[i][s]][t]) — the value returned by
+ * ProductQuantizer::quantize (src/pq.rs:176-186; f16::from_f32, round to nearest even).
+ * d_out holds IEEE binary16 bit patterns.  Asynchronous. */
+int32_t vq_decode_f16(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sub_dim,
+                      int32_t k, const float *d_codebooks, uint16_t *d_out);
+
+/* Same gather without the f16 conversion (the f32 reconstruction of src/opq.rs:146-168). */
+int32_t vq_decode_f32(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sub_dim,
+                      int32_t k, const float *d_codebooks, float *d_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VQ_HIP_H */

@@ -1,0 +1,161 @@
+"""GPU parity: LBG training and PQ encode through the C ABI against the CPU oracle.
+Integer outputs (codes) and trained centroids are compared bit for bit."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from tests import data
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    import vq_amd
+    c = vq_amd.Context(0)
+    yield c
+    c.close()
+
+
+def gpu_lbg(ctx, x, m, k, iters, init, reseed):
+    n, dim = x.shape
+    sd = dim // m
+    dx = ctx.to_device(x)
+    dcb = ctx.empty((m, k, sd), F)
+    it, used = ctx.lbg_fit(dx, n, dim, m, sd, k, iters, init, reseed, dcb)
+    return dcb.download(), it, used, dx, dcb
+
+
+def gpu_encode(ctx, metric, dx, n, dim, m, k, dcb):
+    dcodes = ctx.empty((n, m), np.uint8)
+    ctx.assign(metric, dx, n, dim, m, dim // m, k, dcb, dcodes)
+    return dcodes.download()
+
+
+LBG_CASES = [
+    # n, dim, m, k, iters, kind
+    (1000, 10, 2, 2, 50, "wide"),      # the reference's own test shape (tests/test_pq.rs)
+    (64, 8, 1, 4, 5, "normal"),
+    (300, 16, 2, 16, 8, "normal"),
+    (257, 8, 1, 256, 3, "normal"),     # k close to n -> empty clusters and re-seeds
+    (5000, 32, 4, 64, 6, "uniform"),
+    (700, 6, 3, 7, 10, "grid"),        # integer grid: exact distance ties, duplicate rows
+    (100, 4, 1, 8, 10, "same"),        # all rows equal: everything in cluster 0, k-1 re-seeds
+    (3000, 2, 1, 2, 6, "normal"),      # clusters above 1024 members -> midpoint tree
+    (9000, 4, 2, 3, 5, "normal"),      # depth-2 trees
+    (400, 7, 1, 5, 6, "normal"),       # sub_dim without a register kernel
+    (400, 40, 2, 9, 4, "normal"),      # sub_dim 20
+    (300, 256, 1, 16, 3, "normal"),    # full-dimension problem (RVQ stage shape)
+    (2049, 3, 3, 1, 4, "normal"),      # k = 1, sub_dim 1
+    (50, 8, 1, 4, 0, "normal"),        # max_iters = 0 -> initial rows
+]
+
+
+@pytest.mark.parametrize("n,dim,m,k,iters,kind", LBG_CASES)
+def test_lbg_fit_matches_oracle_bitwise(ctx, n, dim, m, k, iters, kind):
+    rng = np.random.default_rng(n * 31 + dim)
+    if kind == "normal":
+        x = rng.standard_normal((n, dim)).astype(F)
+    elif kind == "uniform":
+        x = rng.random((n, dim), dtype=F)
+    elif kind == "wide":
+        x = rng.uniform(-1000, 1000, (n, dim)).astype(F)  # tests/utils.rs:9-10
+    elif kind == "grid":
+        x = np.round(rng.standard_normal((n, dim)) * 1.5).astype(F)
+    else:
+        x = np.tile(rng.standard_normal((1, dim)).astype(F), (n, 1))
+    init, reseed = data.index_streams(n, m, k, iters, seed=n)
+    want = O.pq_fit(x, m, k, iters, init, reseed)
+    assert want["rc"] == 0
+    got, it, used, _, _ = gpu_lbg(ctx, x, m, k, iters, init, reseed)
+    assert np.array_equal(it, want["iters"])
+    assert np.array_equal(used, want["reseeds"])
+    assert np.array_equal(got.view(np.uint32), want["codebooks"].view(np.uint32))
+
+
+@pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN, O.COSINE, O.MANHATTAN])
+@pytest.mark.parametrize("n,dim,m,k,kind", [
+    (1000, 128, 16, 256, "uniform"),
+    (777, 10, 2, 2, "wide"),
+    (500, 6, 3, 16, "grid"),
+    (300, 21, 3, 11, "normal"),
+    (200, 256, 1, 37, "normal"),
+    (130, 64, 2, 256, "normal"),
+    (65, 12, 1, 3, "zeros"),
+])
+def test_assign_matches_oracle_bitwise(ctx, metric, n, dim, m, k, kind):
+    rng = np.random.default_rng(n + 7 * metric)
+    if kind == "uniform":
+        x = rng.random((n, dim), dtype=F)
+        cb = rng.random((m, k, dim // m), dtype=F)
+    elif kind == "wide":
+        x = rng.uniform(-1000, 1000, (n, dim)).astype(F)
+        cb = rng.uniform(-1000, 1000, (m, k, dim // m)).astype(F)
+    elif kind == "grid":
+        x = np.round(rng.standard_normal((n, dim)) * 2).astype(F)
+        cb = np.round(rng.standard_normal((m, k, dim // m)) * 2).astype(F)
+    elif kind == "zeros":  # zero-norm rows and centroids (cosine returns 1)
+        x = rng.standard_normal((n, dim)).astype(F)
+        x[::3] = 0
+        cb = rng.standard_normal((m, k, dim // m)).astype(F)
+        cb[:, 1] = 0
+    else:
+        x = rng.standard_normal((n, dim)).astype(F)
+        cb = rng.standard_normal((m, k, dim // m)).astype(F)
+    dx, dcb = ctx.to_device(x), ctx.to_device(cb)
+    got = gpu_encode(ctx, metric, dx, n, dim, m, k, dcb)
+    want = O.pq_encode(metric, x, cb)
+    assert np.array_equal(got, want.astype(np.uint8))
+
+
+def test_euclidean_sqrt_collisions_on_gpu(ctx):
+    # many candidates whose squared distances differ in the last bits: the sqrt of several of
+    # them coincide and the earlier index must win (src/distances.rs:134-140 + strict '<').
+    rng = np.random.default_rng(99)
+    n, k = 4096, 256
+    x = np.zeros((n, 2), F)
+    x[:, 0] = rng.random(n, dtype=F) * F(1e-3)
+    b = (0.5 + rng.random(k) * 2e-5).astype(F)
+    cb = np.stack([np.ones(k, F), b], 1)[None]  # m = 1, k x 2
+    dx, dcb = ctx.to_device(x), ctx.to_device(cb)
+    sq = gpu_encode(ctx, O.SQEUCLIDEAN, dx, n, 2, 1, k, dcb)
+    eu = gpu_encode(ctx, O.EUCLIDEAN, dx, n, 2, 1, k, dcb)
+    want_sq = O.pq_encode(O.SQEUCLIDEAN, x, cb).astype(np.uint8)
+    want_eu = O.pq_encode(O.EUCLIDEAN, x, cb).astype(np.uint8)
+    assert np.array_equal(sq, want_sq) and np.array_equal(eu, want_eu)
+    assert np.count_nonzero(want_sq != want_eu) > 50  # the case is exercised
+
+
+def test_config1_pq_fit_encode_decode(ctx):
+    """PQ on 10,000 x 128 U[0,1) rows, seed 42, m=16, k=256, 10 iterations, Euclidean."""
+    n, dim, m, k, iters = 10000, 128, 16, 256, 10
+    x = data.uniform(n, dim, 42)
+    init, reseed = data.index_streams(n, m, k, iters, seed=42)
+    want = O.pq_fit_encode(O.EUCLIDEAN, x, m, k, iters, init, reseed, threads=8)
+    got_cb, it, used, dx, dcb = gpu_lbg(ctx, x, m, k, iters, init, reseed)
+    assert np.array_equal(got_cb.view(np.uint32), want["codebooks"].view(np.uint32))
+    codes = gpu_encode(ctx, O.EUCLIDEAN, dx, n, dim, m, k, dcb)
+    assert np.array_equal(codes, want["codes"].astype(np.uint8))
+    drec = ctx.empty((n, dim), np.uint16)
+    dcodes = ctx.to_device(codes)
+    ctx.decode_f16(dcodes, n, m, dim // m, k, dcb, drec)
+    rec = drec.download()
+    assert np.array_equal(rec, O.pq_decode_f16(want["codes"], want["codebooks"]))
+    mse = O.mse_f16(x, rec)
+    assert abs(mse - 0.019639) < 4e-4  # notebooks/performance_analysis.ipynb:398,405
+
+
+def test_errors_match_reference_panics(ctx):
+    import vq_amd
+    x = ctx.to_device(np.zeros((4, 8), F))
+    cb = ctx.empty((1, 8, 8), F)
+    with pytest.raises(vq_amd.VqError, match="k must be greater than 0") as e:
+        ctx.lbg_fit(x, 4, 8, 1, 8, 0, 3, np.zeros(1, np.uint32), np.zeros(1, np.uint32), cb)
+    assert e.value.code == -1
+    with pytest.raises(vq_amd.VqError, match="Not enough data points for k clusters"):
+        ctx.lbg_fit(x, 4, 8, 1, 8, 8, 3, np.zeros(8, np.uint32), np.zeros(8, np.uint32), cb)
+    with pytest.raises(vq_amd.VqError, match="Empty input"):
+        ctx.lbg_fit(x, 0, 8, 1, 8, 2, 3, np.zeros(2, np.uint32), np.zeros(2, np.uint32), cb)
+    with pytest.raises(vq_amd.VqError, match="Dimension mismatch"):
+        ctx.assign(0, x, 4, 8, 2, 8, 2, cb, ctx.empty((4, 2), np.uint8))

@@ -1,0 +1,170 @@
+"""ctypes binding of libvqhip.so (the C ABI declared in include/vq_hip.h).
+
+The library is the only compute path: if it is missing or fails to load, importing this
+module raises — there is no CPU fallback.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libvqhip.so")
+
+VQ_OK = 0
+ERR_INVALID_ARG, ERR_DIM_MISMATCH, ERR_EMPTY_INPUT = -1, -2, -3
+ERR_UNSUPPORTED, ERR_OOM, ERR_HIP, ERR_RESEED_EXHAUSTED = -4, -5, -6, -7
+
+SQEUCLIDEAN, EUCLIDEAN, COSINE, MANHATTAN = 0, 1, 2, 3
+
+# every symbol include/vq_hip.h declares: name -> (restype, argtypes)
+_vp, _i32, _i64, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_size_t
+SYMBOLS = {
+    "vq_ctx_create": (_i32, [_i32, C.POINTER(_vp)]),
+    "vq_ctx_destroy": (_i32, [_vp]),
+    "vq_last_error": (C.c_char_p, [_vp]),
+    "vq_ctx_sync": (_i32, [_vp]),
+    "vq_ctx_stream": (_vp, [_vp]),
+    "vq_malloc": (_i32, [_vp, _sz, C.POINTER(_vp)]),
+    "vq_free": (_i32, [_vp, _vp]),
+    "vq_h2d": (_i32, [_vp, _vp, _vp, _sz]),
+    "vq_d2h": (_i32, [_vp, _vp, _vp, _sz]),
+    "vq_timer_start": (_i32, [_vp]),
+    "vq_timer_stop": (_i32, [_vp, C.POINTER(C.c_float)]),
+    "vq_lbg_fit": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp,
+                          _vp]),
+    "vq_assign": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
+    "vq_decode_f16": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
+    "vq_decode_f32": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
+}
+
+
+class VqError(RuntimeError):
+    """Raised for any non-zero status of the C ABI; .code holds the status."""
+
+    def __init__(self, code, message):
+        super().__init__(message)
+        self.code = code
+
+
+def load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(f"{LIB_PATH} is missing: build it with `python -m vq_amd.build` "
+                          "(there is no CPU fallback)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SYMBOLS.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+_lib = load()
+
+
+def lib():
+    return _lib
+
+
+class DeviceArray:
+    """A typed device allocation owned by a Context."""
+
+    def __init__(self, ctx, shape, dtype):
+        self.ctx = ctx
+        self.shape = tuple(int(s) for s in np.atleast_1d(shape))
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape)) * self.dtype.itemsize
+        p = _vp()
+        ctx._check(_lib.vq_malloc(ctx._h, self.nbytes, C.byref(p)))
+        self.ptr = p.value
+
+    def upload(self, host):
+        host = np.ascontiguousarray(host, dtype=self.dtype)
+        assert host.nbytes == self.nbytes, (host.shape, self.shape)
+        self.ctx._check(_lib.vq_h2d(self.ctx._h, self.ptr, host.ctypes.data, self.nbytes))
+        return self
+
+    def download(self):
+        out = np.empty(self.shape, self.dtype)
+        self.ctx._check(_lib.vq_d2h(self.ctx._h, out.ctypes.data, self.ptr, self.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            _lib.vq_free(self.ctx._h, self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Context:
+    def __init__(self, device=0):
+        h = _vp()
+        rc = _lib.vq_ctx_create(device, C.byref(h))
+        if rc != VQ_OK:
+            raise VqError(rc, (_lib.vq_last_error(None) or b"").decode())
+        self._h = h
+
+    def close(self):
+        if self._h:
+            _lib.vq_ctx_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _check(self, rc):
+        if rc != VQ_OK:
+            raise VqError(rc, (_lib.vq_last_error(self._h) or b"").decode())
+
+    # -- memory ------------------------------------------------------------------------------
+    def empty(self, shape, dtype):
+        return DeviceArray(self, shape, dtype)
+
+    def to_device(self, host, dtype=None):
+        host = np.ascontiguousarray(host, dtype=dtype)
+        return DeviceArray(self, host.shape, host.dtype).upload(host)
+
+    def sync(self):
+        self._check(_lib.vq_ctx_sync(self._h))
+
+    def timer_start(self):
+        self._check(_lib.vq_timer_start(self._h))
+
+    def timer_stop(self):
+        ms = C.c_float(0)
+        self._check(_lib.vq_timer_stop(self._h, C.byref(ms)))
+        return ms.value
+
+    # -- compute -----------------------------------------------------------------------------
+    def lbg_fit(self, d_x, n, ld, m, sub_dim, k, max_iters, init_idx, reseed_stream, d_codebooks):
+        init_idx = np.ascontiguousarray(init_idx, np.uint32).reshape(-1)
+        reseed_stream = np.ascontiguousarray(reseed_stream, np.uint32).reshape(m, -1) \
+            if np.size(reseed_stream) else np.zeros((m, 0), np.uint32)
+        n_reseed = reseed_stream.shape[1]
+        iters = np.zeros(m, np.int32)
+        used = np.zeros(m, np.int32)
+        self._check(_lib.vq_lbg_fit(self._h, d_x.ptr, n, ld, m, sub_dim, k, max_iters,
+                                    init_idx.ctypes.data, reseed_stream.ctypes.data if n_reseed
+                                    else None, n_reseed, d_codebooks.ptr, iters.ctypes.data,
+                                    used.ctypes.data))
+        return iters, used
+
+    def assign(self, metric, d_x, n, ld, m, sub_dim, k, d_codebooks, d_codes):
+        self._check(_lib.vq_assign(self._h, metric, d_x.ptr, n, ld, m, sub_dim, k,
+                                   d_codebooks.ptr, d_codes.ptr))
+
+    def decode_f16(self, d_codes, n, m, sub_dim, k, d_codebooks, d_out):
+        self._check(_lib.vq_decode_f16(self._h, d_codes.ptr, n, m, sub_dim, k, d_codebooks.ptr,
+                                       d_out.ptr))
+
+    def decode_f32(self, d_codes, n, m, sub_dim, k, d_codebooks, d_out):
+        self._check(_lib.vq_decode_f32(self._h, d_codes.ptr, n, m, sub_dim, k, d_codebooks.ptr,
+                                       d_out.ptr))

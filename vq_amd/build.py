@@ -1,0 +1,36 @@
+"""Builds libvqhip.so (HIP kernels + C ABI) for gfx950, in-tree."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB = os.path.join(HERE, "libvqhip.so")
+SRC = [os.path.join(HERE, "csrc", "vq_api.hip")]
+
+# -ffp-contract=off: the exact kernels must round multiply and add separately, as the
+#   reference's Rust code does.  Fused operations are written explicitly where wanted.
+# -packed-fp32-ops disabled: no v_pk_*_f32 may be generated.
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+    "-fno-fast-math", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def build_lib(verbose=False, extra=()):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, *FLAGS, *extra, "-o", LIB, *SRC]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    out = "\n".join(l for l in (res.stdout + res.stderr).splitlines()
+                    if "packed-fp32-ops" not in l and "is not a recognized feature" not in l)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out)
+    if verbose and out.strip():
+        print(out)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build_lib(verbose=True, extra=sys.argv[1:]))

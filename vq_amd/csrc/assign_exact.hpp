@@ -1,0 +1,355 @@
+// Exact nearest-centroid assignment on the vector ALU.
+//
+// Every distance is evaluated in the reference's own operation order (sequential f32
+// accumulation from 0.0, separately rounded multiply and add, strict '<' so the lowest index
+// wins: src/utils.rs:62-70, src/vector.rs:197-201,259-264, src/distances.rs:129-152), so the
+// codes are bit-identical to the CPU path by construction.  This translation unit must be
+// compiled with -ffp-contract=off.
+//
+// Mapping: one lane = one row.  The lane keeps its sub-vectors in registers; the centroid
+// operand is identical for all lanes of a wave and is read from LDS as a broadcast.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vq {
+
+enum { M_SQ = 0, M_EUCLID = 1, M_COS = 2, M_L1 = 3 };
+
+struct AssignArgs {
+    const float *x;       // n x ld
+    int64_t n;
+    int64_t ld;
+    int m;                // column blocks
+    int k;                // centroids per block
+    const float *cb;      // m*k*sd
+    const float *cnorm;   // m*k centroid L2 norms (cosine only)
+    uint8_t *codes;       // LBG mode: [m][n] in place (old -> new); encode mode: [n][m]
+    int *changed;         // LBG mode: changed[s] set to 1 when any code of block s differs
+    const int *done;      // LBG mode: blocks with done[s] != 0 are skipped
+};
+
+// sqrt(sum of squares) of every centroid, sequential order (map_sum, src/distances.rs:66-69,144)
+__global__ void k_centroid_norms(const float *__restrict__ cb, int64_t total, int sd,
+                                 float *__restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const float *c = cb + i * sd;
+    float acc = 0.0f;
+    for (int t = 0; t < sd; ++t) {
+        float p = c[t] * c[t];
+        acc = acc + p;
+    }
+    out[i] = sqrtf(acc);
+}
+
+template <int SD>
+__device__ __forceinline__ float d_sq(const float (&x)[SD], const float (&c)[SD]) {
+    float d0 = x[0] - c[0];
+    float acc = d0 * d0;  // 0.0 + p == p for p >= +0
+#pragma unroll
+    for (int t = 1; t < SD; ++t) {
+        float d = x[t] - c[t];
+        float p = d * d;
+        acc = acc + p;
+    }
+    return acc;
+}
+
+template <int SD>
+__device__ __forceinline__ float d_l1(const float (&x)[SD], const float (&c)[SD]) {
+    float acc = fabsf(x[0] - c[0]);
+#pragma unroll
+    for (int t = 1; t < SD; ++t) {
+        float d = x[t] - c[t];
+        acc = acc + fabsf(d);
+    }
+    return acc;
+}
+
+template <int SD>
+__device__ __forceinline__ float d_dot(const float (&x)[SD], const float (&c)[SD]) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int t = 0; t < SD; ++t) {
+        float p = x[t] * c[t];
+        acc = acc + p;
+    }
+    return acc;
+}
+
+template <int SD>
+__device__ __forceinline__ void lds_centroid(const float *lds, int j, float (&c)[SD]) {
+    if constexpr (SD % 4 == 0) {
+        const float4 *p = reinterpret_cast<const float4 *>(lds + j * SD);
+#pragma unroll
+        for (int q = 0; q < SD / 4; ++q) {
+            float4 v = p[q];
+            c[4 * q + 0] = v.x;
+            c[4 * q + 1] = v.y;
+            c[4 * q + 2] = v.z;
+            c[4 * q + 3] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < SD; ++t) c[t] = lds[j * SD + t];
+    }
+}
+
+// Argmin of one row's sub-vector against the k centroids held in LDS.
+template <int SD, int METRIC>
+__device__ __forceinline__ int argmin_lds(const float (&x)[SD], const float *lds, const float *cn,
+                                          int k) {
+    float c[SD];
+    int best = 0;
+    if constexpr (METRIC == M_SQ || METRIC == M_EUCLID) {
+        lds_centroid<SD>(lds, 0, c);
+        float bd = d_sq<SD>(x, c);
+        float pd = __builtin_inff();  // squared distance of the previous running minimum
+#pragma unroll 4
+        for (int j = 1; j < k; ++j) {
+            lds_centroid<SD>(lds, j, c);
+            float d = d_sq<SD>(x, c);
+            bool u = d < bd;
+            if constexpr (METRIC == M_EUCLID) pd = u ? bd : pd;
+            bd = u ? d : bd;
+            best = u ? j : best;
+        }
+        if constexpr (METRIC == M_EUCLID) {
+            // The reference compares sqrt(d2) (src/distances.rs:134-140).  sqrt is monotone, so
+            // its running minimum is the first element of the strictly decreasing chain of d2
+            // minima whose root equals the root of the smallest d2.  Only when the previous
+            // chain element shares that root can the answer be an earlier index: rescan.
+            float s = sqrtf(bd);
+            if (sqrtf(pd) == s) {
+                for (int j = 0; j < best; ++j) {
+                    lds_centroid<SD>(lds, j, c);
+                    if (sqrtf(d_sq<SD>(x, c)) == s) {
+                        best = j;
+                        break;
+                    }
+                }
+            }
+        }
+    } else if constexpr (METRIC == M_L1) {
+        lds_centroid<SD>(lds, 0, c);
+        float bd = d_l1<SD>(x, c);
+#pragma unroll 4
+        for (int j = 1; j < k; ++j) {
+            lds_centroid<SD>(lds, j, c);
+            float d = d_l1<SD>(x, c);
+            bool u = d < bd;
+            bd = u ? d : bd;
+            best = u ? j : best;
+        }
+    } else {  // cosine, src/distances.rs:141-151
+        float sa = 0.0f;
+#pragma unroll
+        for (int t = 0; t < SD; ++t) {
+            float p = x[t] * x[t];
+            sa = sa + p;
+        }
+        float na = sqrtf(sa);
+        float bd = 0.0f;
+        for (int j = 0; j < k; ++j) {
+            lds_centroid<SD>(lds, j, c);
+            float dot = d_dot<SD>(x, c);
+            float nb = cn[j];
+            float den = na * nb;
+            float q = dot / den;
+            float d = 1.0f - q;
+            d = (na == 0.0f || nb == 0.0f) ? 1.0f : d;
+            bool u = (j == 0) || (d < bd);
+            bd = u ? d : bd;
+            best = u ? j : best;
+        }
+    }
+    return best;
+}
+
+// One lane = one row, G consecutive column blocks per lane (G*SD floats in registers, G
+// codebooks in LDS).  blockIdx.x = tile * (m/G) + block group.
+template <int SD, int G, int METRIC, bool LBG>
+__global__ void __launch_bounds__(256) k_assign_static(AssignArgs a) {
+    extern __shared__ float lds[];
+    const int groups = a.m / G;
+    const int sg = blockIdx.x % groups;
+    const int64_t tile = blockIdx.x / groups;
+    const int s0 = sg * G;
+    const int k = a.k;
+    float *lds_cn = lds + (size_t)G * k * SD;
+
+    bool any = true;
+    if constexpr (LBG) {
+        any = false;
+#pragma unroll
+        for (int g = 0; g < G; ++g) any |= (a.done[s0 + g] == 0);
+        if (!any) return;  // uniform over the workgroup
+    }
+    // codebooks of blocks s0..s0+G-1 are contiguous: G*k*SD floats
+    {
+        const float *src = a.cb + (size_t)s0 * k * SD;
+        const int total = G * k * SD;
+        for (int i = threadIdx.x; i < total; i += 256) lds[i] = src[i];
+        if constexpr (METRIC == M_COS) {
+            const float *cn = a.cnorm + (size_t)s0 * k;
+            for (int i = threadIdx.x; i < G * k; i += 256) lds_cn[i] = cn[i];
+        }
+    }
+    __syncthreads();
+
+    const int64_t row = tile * 256 + threadIdx.x;
+    if (row >= a.n) return;
+
+    float x[G][SD];
+    {
+        const float *xr = a.x + row * a.ld + (int64_t)s0 * SD;
+        if constexpr ((G * SD) % 4 == 0) {
+            if ((a.ld % 4 == 0) && ((reinterpret_cast<uintptr_t>(a.x) & 15) == 0)) {
+                const float4 *p = reinterpret_cast<const float4 *>(xr);
+                float *xf = &x[0][0];
+#pragma unroll
+                for (int q = 0; q < G * SD / 4; ++q) {
+                    float4 v = p[q];
+                    xf[4 * q + 0] = v.x;
+                    xf[4 * q + 1] = v.y;
+                    xf[4 * q + 2] = v.z;
+                    xf[4 * q + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < G; ++g)
+#pragma unroll
+                    for (int t = 0; t < SD; ++t) x[g][t] = xr[g * SD + t];
+            }
+        } else {
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+#pragma unroll
+                for (int t = 0; t < SD; ++t) x[g][t] = xr[g * SD + t];
+        }
+    }
+
+    uint32_t packed = 0;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int s = s0 + g;
+        if constexpr (LBG) {
+            if (a.done[s]) continue;  // uniform
+        }
+        int best = argmin_lds<SD, METRIC>(x[g], lds + (size_t)g * k * SD, lds_cn + g * k, k);
+        if constexpr (LBG) {
+            uint8_t *p = a.codes + (size_t)s * a.n + row;
+            if (*p != (uint8_t)best) {
+                *p = (uint8_t)best;
+                a.changed[s] = 1;
+            }
+        } else {
+            if constexpr (G == 4)
+                packed |= (uint32_t)best << (8 * g);
+            else
+                a.codes[row * a.m + s] = (uint8_t)best;
+        }
+    }
+    if constexpr (!LBG && G == 4) {
+        // m % 4 == 0 here, so the 4 codes of this lane are one aligned 32-bit word
+        *reinterpret_cast<uint32_t *>(a.codes + row * a.m + s0) = packed;
+    }
+}
+
+// Fallback for any sub_dim: one lane = one row, one column block per blockIdx.y, sub-vector
+// re-read from memory for every group of 4 centroids; centroids read through wave-uniform
+// addresses.  Same operation order as above.
+template <int METRIC, bool LBG>
+__global__ void __launch_bounds__(256) k_assign_dyn(AssignArgs a, int sd) {
+    const int s = blockIdx.y;
+    if constexpr (LBG) {
+        if (a.done[s]) return;
+    }
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= a.n) return;
+    const int k = a.k;
+    const float *__restrict__ xr = a.x + row * a.ld + (int64_t)s * sd;
+    const float *__restrict__ cb = a.cb + (size_t)s * k * sd;
+    const float *__restrict__ cn = a.cnorm ? a.cnorm + (size_t)s * k : nullptr;
+    int best = 0;
+    float bd = 0.0f, pd = __builtin_inff();
+    float na = 0.0f;
+    if constexpr (METRIC == M_COS) {
+        float sa = 0.0f;
+        for (int t = 0; t < sd; ++t) {
+            float p = xr[t] * xr[t];
+            sa = sa + p;
+        }
+        na = sqrtf(sa);
+    }
+    for (int j0 = 0; j0 < k; j0 += 4) {
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        const int jn = (k - j0 < 4) ? (k - j0) : 4;
+        for (int t = 0; t < sd; ++t) {
+            float xv = xr[t];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (u < jn) {
+                    float cv = cb[(size_t)(j0 + u) * sd + t];
+                    if constexpr (METRIC == M_COS) {
+                        float p = xv * cv;
+                        acc[u] = acc[u] + p;
+                    } else if constexpr (METRIC == M_L1) {
+                        float d = xv - cv;
+                        acc[u] = acc[u] + fabsf(d);
+                    } else {
+                        float d = xv - cv;
+                        float p = d * d;
+                        acc[u] = acc[u] + p;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (u < jn) {
+                float d = acc[u];
+                if constexpr (METRIC == M_COS) {
+                    float nb = cn[j0 + u];
+                    float den = na * nb;
+                    float q = d / den;
+                    d = 1.0f - q;
+                    d = (na == 0.0f || nb == 0.0f) ? 1.0f : d;
+                }
+                bool upd = (j0 + u == 0) || (d < bd);
+                if constexpr (METRIC == M_EUCLID) pd = (upd && (j0 + u) != 0) ? bd : pd;
+                bd = upd ? d : bd;
+                best = upd ? (j0 + u) : best;
+            }
+        }
+    }
+    if constexpr (METRIC == M_EUCLID) {
+        float sr = sqrtf(bd);
+        if (sqrtf(pd) == sr) {
+            for (int j = 0; j < best; ++j) {
+                float acc = 0.0f;
+                for (int t = 0; t < sd; ++t) {
+                    float d = xr[t] - cb[(size_t)j * sd + t];
+                    float p = d * d;
+                    acc = acc + p;
+                }
+                if (sqrtf(acc) == sr) {
+                    best = j;
+                    break;
+                }
+            }
+        }
+    }
+    if constexpr (LBG) {
+        uint8_t *p = a.codes + (size_t)s * a.n + row;
+        if (*p != (uint8_t)best) {
+            *p = (uint8_t)best;
+            a.changed[s] = 1;
+        }
+    } else {
+        a.codes[row * a.m + s] = (uint8_t)best;
+    }
+}
+
+}  // namespace vq

@@ -1,0 +1,444 @@
+// libvqhip — host side of the C ABI declared in include/vq_hip.h.
+// Compile with: hipcc --offload-arch=gfx950 -O3 -ffp-contract=off
+//               -Xclang -target-feature -Xclang -packed-fp32-ops
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../include/vq_hip.h"
+#include "assign_exact.hpp"
+#include "lbg_update.hpp"
+
+namespace {
+
+thread_local std::string g_create_error;
+
+struct DevBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+};
+
+}  // namespace
+
+struct vq_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::string err;
+    // grow-only device workspace
+    DevBuf flags, tables, hist, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;
+};
+
+namespace {
+
+int32_t fail(vq_ctx *ctx, int32_t code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (ctx)
+        ctx->err = buf;
+    else
+        g_create_error = buf;
+    return code;
+}
+
+#define VQ_HIP(ctx, call)                                                                     \
+    do {                                                                                      \
+        hipError_t e__ = (call);                                                              \
+        if (e__ != hipSuccess)                                                                \
+            return fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,            \
+                        "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__, __LINE__); \
+    } while (0)
+
+int32_t ensure(vq_ctx *ctx, DevBuf &b, size_t bytes) {
+    if (bytes <= b.cap) return VQ_OK;
+    if (b.p) {
+        VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        VQ_HIP(ctx, hipFree(b.p));
+        b.p = nullptr;
+        b.cap = 0;
+    }
+    size_t want = bytes + bytes / 8 + 256;
+    VQ_HIP(ctx, hipMalloc(&b.p, want));
+    b.cap = want;
+    return VQ_OK;
+}
+
+#define VQ_TRY(expr)                  \
+    do {                              \
+        int32_t rc__ = (expr);        \
+        if (rc__ != VQ_OK) return rc__; \
+    } while (0)
+
+inline unsigned cdiv(int64_t a, int64_t b) { return (unsigned)((a + b - 1) / b); }
+
+// ---- assignment dispatch -------------------------------------------------------------------
+
+template <int SD, int G, int METRIC, bool LBG>
+int32_t launch_static(vq_ctx *ctx, const vq::AssignArgs &a) {
+    size_t lds = (size_t)G * a.k * SD * sizeof(float);
+    if (METRIC == vq::M_COS) lds += (size_t)G * a.k * sizeof(float);
+    auto kern = vq::k_assign_static<SD, G, METRIC, LBG>;
+    if (lds > 48 * 1024)
+        VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    int64_t tiles = (a.n + 255) / 256;
+    int64_t blocks = tiles * (a.m / G);
+    if (blocks > 0x7fffffffLL) return fail(ctx, VQ_ERR_UNSUPPORTED, "grid too large");
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, ctx->stream, a);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+template <int SD, int METRIC, bool LBG>
+int32_t launch_static_g(vq_ctx *ctx, const vq::AssignArgs &a) {
+    // G column blocks per lane: as many as keep the lane's floats within 32 registers and the
+    // codebooks within 64 KB of LDS.
+    size_t per = (size_t)a.k * SD * sizeof(float) + (METRIC == vq::M_COS ? a.k * sizeof(float) : 0);
+    if constexpr (SD * 4 <= 32) {
+        if (a.m % 4 == 0 && 4 * per <= 64 * 1024) return launch_static<SD, 4, METRIC, LBG>(ctx, a);
+    }
+    if constexpr (SD * 2 <= 32) {
+        if (a.m % 2 == 0 && 2 * per <= 64 * 1024) return launch_static<SD, 2, METRIC, LBG>(ctx, a);
+    }
+    return launch_static<SD, 1, METRIC, LBG>(ctx, a);
+}
+
+template <int METRIC, bool LBG>
+int32_t launch_assign_m(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
+    size_t per = (size_t)a.k * sd * sizeof(float) + a.k * sizeof(float);
+    if (per <= 64 * 1024) {
+        switch (sd) {
+        case 1: return launch_static_g<1, METRIC, LBG>(ctx, a);
+        case 2: return launch_static_g<2, METRIC, LBG>(ctx, a);
+        case 3: return launch_static_g<3, METRIC, LBG>(ctx, a);
+        case 4: return launch_static_g<4, METRIC, LBG>(ctx, a);
+        case 5: return launch_static_g<5, METRIC, LBG>(ctx, a);
+        case 6: return launch_static_g<6, METRIC, LBG>(ctx, a);
+        case 8: return launch_static_g<8, METRIC, LBG>(ctx, a);
+        case 12: return launch_static_g<12, METRIC, LBG>(ctx, a);
+        case 16: return launch_static_g<16, METRIC, LBG>(ctx, a);
+        case 32: return launch_static_g<32, METRIC, LBG>(ctx, a);
+        default: break;
+        }
+    }
+    if (a.m > 65535) return fail(ctx, VQ_ERR_UNSUPPORTED, "m too large for the generic kernel");
+    hipLaunchKernelGGL((vq::k_assign_dyn<METRIC, LBG>), dim3(cdiv(a.n, 256), (unsigned)a.m),
+                       dim3(256), 0, ctx->stream, a, sd);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+template <bool LBG>
+int32_t launch_assign(vq_ctx *ctx, int metric, const vq::AssignArgs &a, int sd) {
+    switch (metric) {
+    case VQ_SQEUCLIDEAN: return launch_assign_m<vq::M_SQ, LBG>(ctx, a, sd);
+    case VQ_EUCLIDEAN: return launch_assign_m<vq::M_EUCLID, LBG>(ctx, a, sd);
+    case VQ_COSINE: return launch_assign_m<vq::M_COS, LBG>(ctx, a, sd);
+    case VQ_MANHATTAN: return launch_assign_m<vq::M_L1, LBG>(ctx, a, sd);
+    default: return fail(ctx, VQ_ERR_UNSUPPORTED, "metric %d has no kernel", metric);
+    }
+}
+
+__global__ void k_decode_f16(const uint8_t *__restrict__ codes, int64_t n, int m, int sd, int k,
+                             const float *__restrict__ cb, uint16_t *__restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t dim = (int64_t)m * sd;
+    if (i >= n * dim) return;
+    int64_t row = i / dim;
+    int c = (int)(i % dim);
+    int s = c / sd, t = c % sd;
+    float v = cb[((size_t)s * k + codes[row * m + s]) * sd + t];
+    out[i] = __half_as_ushort(__float2half_rn(v));
+}
+
+__global__ void k_decode_f32(const uint8_t *__restrict__ codes, int64_t n, int m, int sd, int k,
+                             const float *__restrict__ cb, float *__restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t dim = (int64_t)m * sd;
+    if (i >= n * dim) return;
+    int64_t row = i / dim;
+    int c = (int)(i % dim);
+    int s = c / sd, t = c % sd;
+    out[i] = cb[((size_t)s * k + codes[row * m + s]) * sd + t];
+}
+
+int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t m, int32_t sd,
+                     int32_t k) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return fail(ctx, VQ_ERR_EMPTY_INPUT, "Empty input: at least one vector is required.");
+    if (!x || n < 0 || m <= 0 || sd <= 0)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: null pointer or non-positive size");
+    if (ld < (int64_t)m * sd)
+        return fail(ctx, VQ_ERR_DIM_MISMATCH, "Dimension mismatch: expected %lld, got %lld",
+                    (long long)m * sd, (long long)ld);
+    if (k <= 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: k must be greater than 0");
+    if (k > vq::kMaxK)
+        return fail(ctx, VQ_ERR_UNSUPPORTED, "k = %d: codes are uint8, k must be <= 256", k);
+    if (n >= (1LL << 32)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n must be below 2^32");
+    return VQ_OK;
+}
+
+}  // namespace
+
+// =============================================================================================
+extern "C" {
+
+int32_t vq_ctx_create(int32_t device, vq_ctx **out) {
+    if (!out) return fail(nullptr, VQ_ERR_INVALID_ARG, "out is null");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0)
+        return fail(nullptr, VQ_ERR_HIP, "no HIP device available (%s)",
+                    e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+    if (device < 0 || device >= count)
+        return fail(nullptr, VQ_ERR_INVALID_ARG, "device %d out of range [0,%d)", device, count);
+    vq_ctx *ctx = new vq_ctx;
+    ctx->device = device;
+    if ((e = hipSetDevice(device)) != hipSuccess ||
+        (e = hipStreamCreate(&ctx->stream)) != hipSuccess ||
+        (e = hipEventCreate(&ctx->ev0)) != hipSuccess ||
+        (e = hipEventCreate(&ctx->ev1)) != hipSuccess) {
+        int32_t rc = fail(nullptr, VQ_ERR_HIP, "context set-up failed: %s", hipGetErrorString(e));
+        delete ctx;
+        return rc;
+    }
+    *out = ctx;
+    return VQ_OK;
+}
+
+int32_t vq_ctx_destroy(vq_ctx *ctx) {
+    if (!ctx) return VQ_OK;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
+                      &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm};
+    for (DevBuf *b : bufs)
+        if (b->p) (void)hipFree(b->p);
+    (void)hipEventDestroy(ctx->ev0);
+    (void)hipEventDestroy(ctx->ev1);
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return VQ_OK;
+}
+
+const char *vq_last_error(const vq_ctx *ctx) { return ctx ? ctx->err.c_str() : g_create_error.c_str(); }
+
+int32_t vq_ctx_sync(vq_ctx *ctx) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return VQ_OK;
+}
+
+void *vq_ctx_stream(vq_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+int32_t vq_malloc(vq_ctx *ctx, size_t bytes, void **d_ptr) {
+    if (!ctx || !d_ptr) return VQ_ERR_INVALID_ARG;
+    *d_ptr = nullptr;
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    VQ_HIP(ctx, hipMalloc(d_ptr, bytes ? bytes : 1));
+    return VQ_OK;
+}
+
+int32_t vq_free(vq_ctx *ctx, void *d_ptr) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (!d_ptr) return VQ_OK;
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    VQ_HIP(ctx, hipFree(d_ptr));
+    return VQ_OK;
+}
+
+int32_t vq_h2d(vq_ctx *ctx, void *d_dst, const void *h_src, size_t bytes) {
+    if (!ctx || (bytes && (!d_dst || !h_src))) return VQ_ERR_INVALID_ARG;
+    VQ_HIP(ctx, hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return VQ_OK;
+}
+
+int32_t vq_d2h(vq_ctx *ctx, void *h_dst, const void *d_src, size_t bytes) {
+    if (!ctx || (bytes && (!h_dst || !d_src))) return VQ_ERR_INVALID_ARG;
+    VQ_HIP(ctx, hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return VQ_OK;
+}
+
+int32_t vq_timer_start(vq_ctx *ctx) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    VQ_HIP(ctx, hipEventRecord(ctx->ev0, ctx->stream));
+    return VQ_OK;
+}
+
+int32_t vq_timer_stop(vq_ctx *ctx, float *h_ms) {
+    if (!ctx || !h_ms) return VQ_ERR_INVALID_ARG;
+    VQ_HIP(ctx, hipEventRecord(ctx->ev1, ctx->stream));
+    VQ_HIP(ctx, hipEventSynchronize(ctx->ev1));
+    VQ_HIP(ctx, hipEventElapsedTime(h_ms, ctx->ev0, ctx->ev1));
+    return VQ_OK;
+}
+
+int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t m, int32_t sd,
+                   int32_t k, int32_t max_iters, const uint32_t *h_init_idx,
+                   const uint32_t *h_reseed_stream, int32_t n_reseed, float *d_codebooks,
+                   int32_t *h_iters_run, int32_t *h_reseeds_used) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (k == 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: k must be greater than 0");
+    VQ_TRY(check_common(ctx, d_x, n, ld, m, sd, k));
+    if (n < k)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: Not enough data points for k clusters");
+    if (m > 65535) return fail(ctx, VQ_ERR_UNSUPPORTED, "m must be at most 65535");
+    if (!h_init_idx || !d_codebooks || max_iters < 0 || n_reseed < 0 || (n_reseed && !h_reseed_stream))
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: null pointer or negative size");
+    for (int64_t i = 0; i < (int64_t)m * k; ++i)
+        if (h_init_idx[i] >= (uint64_t)n)
+            return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: init index %u out of range", h_init_idx[i]);
+    for (int64_t i = 0; i < (int64_t)m * n_reseed; ++i)
+        if (h_reseed_stream[i] >= (uint64_t)n)
+            return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: reseed index %u out of range", h_reseed_stream[i]);
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+
+    const int nblk = (int)((n + vq::kRowBlock - 1) / vq::kRowBlock);
+    const int leaf_cap = (int)(k + n / 512 + 1);
+    VQ_TRY(ensure(ctx, ctx->flags, sizeof(int) * (6 * (size_t)m + 1)));
+    VQ_TRY(ensure(ctx, ctx->tables, sizeof(uint32_t) * 5 * (size_t)m * vq::kMaxK));
+    VQ_TRY(ensure(ctx, ctx->hist, sizeof(uint32_t) * (size_t)m * nblk * vq::kMaxK));
+    VQ_TRY(ensure(ctx, ctx->perm, sizeof(uint32_t) * (size_t)m * n));
+    VQ_TRY(ensure(ctx, ctx->leaf_desc, sizeof(uint2) * (size_t)m * leaf_cap));
+    VQ_TRY(ensure(ctx, ctx->leaf_sum, sizeof(float) * (size_t)m * leaf_cap * sd));
+    VQ_TRY(ensure(ctx, ctx->codes, (size_t)m * n));
+    VQ_TRY(ensure(ctx, ctx->idx, sizeof(uint32_t) * (size_t)m * k));
+    VQ_TRY(ensure(ctx, ctx->reseed, sizeof(uint32_t) * ((size_t)m * n_reseed + 1)));
+
+    vq::LbgState S;
+    int *f = (int *)ctx->flags.p;
+    S.changed = f;
+    S.done = f + m;
+    S.iters = f + 2 * m;
+    S.used = f + 3 * m;
+    S.ubase = f + 4 * m;
+    S.nleaves = f + 5 * m;
+    S.err = f + 6 * m;
+    uint32_t *tb = (uint32_t *)ctx->tables.p;
+    const size_t mk = (size_t)m * vq::kMaxK;
+    S.count = tb;
+    S.start = tb + mk;
+    S.leaf_start = tb + 2 * mk;
+    S.depth = tb + 3 * mk;
+    S.empty_rank = tb + 4 * mk;
+    S.hist = (uint32_t *)ctx->hist.p;
+    S.perm = (uint32_t *)ctx->perm.p;
+    S.leaf_desc = (uint2 *)ctx->leaf_desc.p;
+    S.leaf_sum = (float *)ctx->leaf_sum.p;
+    S.codes = (uint8_t *)ctx->codes.p;
+    S.nblk = nblk;
+    S.leaf_cap = leaf_cap;
+
+    VQ_HIP(ctx, hipMemcpyAsync(ctx->idx.p, h_init_idx, sizeof(uint32_t) * (size_t)m * k,
+                               hipMemcpyHostToDevice, st));
+    if (n_reseed)
+        VQ_HIP(ctx, hipMemcpyAsync(ctx->reseed.p, h_reseed_stream,
+                                   sizeof(uint32_t) * (size_t)m * n_reseed, hipMemcpyHostToDevice, st));
+    VQ_HIP(ctx, hipMemsetAsync(S.codes, 0, (size_t)m * n, st));  // assignments = vec![0; n], utils.rs:55
+    hipLaunchKernelGGL(vq::k_lbg_init, dim3(cdiv(m, 64)), dim3(64), 0, st, S, m);
+    hipLaunchKernelGGL(vq::k_gather_rows, dim3(cdiv((int64_t)m * k * sd, 256)), dim3(256), 0, st, d_x,
+                       ld, m, k, sd, (const uint32_t *)ctx->idx.p, d_codebooks);
+    VQ_HIP(ctx, hipGetLastError());
+
+    vq::AssignArgs a;
+    a.x = d_x;
+    a.n = n;
+    a.ld = ld;
+    a.m = m;
+    a.k = k;
+    a.cb = d_codebooks;
+    a.cnorm = nullptr;
+    a.codes = S.codes;
+    a.changed = S.changed;
+    a.done = S.done;
+
+    for (int it = 0; it < max_iters; ++it) {
+        VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd));
+        hipLaunchKernelGGL(vq::k_lbg_hist, dim3(nblk, m), dim3(64), 0, st, S, n);
+        hipLaunchKernelGGL(vq::k_lbg_scan, dim3(m), dim3(256), 0, st, S, k);
+        hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nblk, m), dim3(64), 0, st, S, n);
+        hipLaunchKernelGGL(vq::k_lbg_leafsum, dim3(cdiv((int64_t)leaf_cap * sd, 256), m), dim3(256), 0,
+                           st, S, d_x, n, ld, sd);
+        hipLaunchKernelGGL(vq::k_lbg_finalize, dim3(cdiv((int64_t)k * sd, 256), m), dim3(256), 0, st, S,
+                           d_x, ld, k, sd, (const uint32_t *)ctx->reseed.p, n_reseed, d_codebooks);
+        hipLaunchKernelGGL(vq::k_lbg_advance, dim3(cdiv(m, 64)), dim3(64), 0, st, S, m);
+        VQ_HIP(ctx, hipGetLastError());
+    }
+    std::vector<int> host(6 * (size_t)m + 1);
+    VQ_HIP(ctx, hipMemcpyAsync(host.data(), f, sizeof(int) * host.size(), hipMemcpyDeviceToHost, st));
+    VQ_HIP(ctx, hipStreamSynchronize(st));
+    if (h_iters_run) memcpy(h_iters_run, host.data() + 2 * m, sizeof(int) * m);
+    if (h_reseeds_used) memcpy(h_reseeds_used, host.data() + 3 * m, sizeof(int) * m);
+    if (host[6 * (size_t)m])
+        return fail(ctx, VQ_ERR_RESEED_EXHAUSTED,
+                    "re-seed stream exhausted: pass n_reseed = k*max_iters");
+    return VQ_OK;
+}
+
+int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
+                  int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes) {
+    VQ_TRY(check_common(ctx, d_x, n, ld, m, sd, k));
+    if (!d_codebooks || !d_codes) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: null pointer");
+    if (reinterpret_cast<uintptr_t>(d_codes) & 3)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: d_codes must be 4-byte aligned");
+    if (m > 65535) return fail(ctx, VQ_ERR_UNSUPPORTED, "m must be at most 65535");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    vq::AssignArgs a;
+    a.x = d_x;
+    a.n = n;
+    a.ld = ld;
+    a.m = m;
+    a.k = k;
+    a.cb = d_codebooks;
+    a.cnorm = nullptr;
+    a.codes = d_codes;
+    a.changed = nullptr;
+    a.done = nullptr;
+    if (metric == VQ_COSINE) {
+        VQ_TRY(ensure(ctx, ctx->cnorm, sizeof(float) * (size_t)m * k));
+        hipLaunchKernelGGL(vq::k_centroid_norms, dim3(cdiv((int64_t)m * k, 256)), dim3(256), 0,
+                           ctx->stream, d_codebooks, (int64_t)m * k, sd, (float *)ctx->cnorm.p);
+        a.cnorm = (const float *)ctx->cnorm.p;
+    }
+    return launch_assign<false>(ctx, metric, a, sd);
+}
+
+int32_t vq_decode_f16(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sd, int32_t k,
+                      const float *d_codebooks, uint16_t *d_out) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return VQ_OK;
+    if (!d_codes || !d_codebooks || !d_out || n < 0 || m <= 0 || sd <= 0 || k <= 0 || k > vq::kMaxK)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipLaunchKernelGGL(k_decode_f16, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n,
+                       m, sd, k, d_codebooks, d_out);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+int32_t vq_decode_f32(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sd, int32_t k,
+                      const float *d_codebooks, float *d_out) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return VQ_OK;
+    if (!d_codes || !d_codebooks || !d_out || n < 0 || m <= 0 || sd <= 0 || k <= 0 || k > vq::kMaxK)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipLaunchKernelGGL(k_decode_f32, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n,
+                       m, sd, k, d_codebooks, d_out);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+}  // extern "C"
