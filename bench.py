@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""bench.py — PQ fit + encode throughput on one MI355X, with roofline and CPU baseline.
+
+One step = ProductQuantizer::fit (10 LBG iterations) followed by the encode of every row
+(BASELINE.json configs[1]: 1,000,000 x 128 f32 rows from a mixture of 1,024 isotropic Gaussians,
+m = 16, k = 256, Euclidean encode), with the rows already resident in HBM.
+
+Prints ONE JSON line (see README of the bench contract):
+  value        rows / second over fit + encode (whole job, one GPU)
+  roofline     the dominant kernel (the LBG assignment pass) against the fp32 vector-ALU peak;
+               its time is measured with HIP events recorded on the library's stream around
+               each launch during the timed steps
+  cpu_baseline the C restatement of the reference (oracle/) timed on the host cores on a bounded
+               sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+N_ROWS, DIM, M, K, ITERS = 1_000_000, 128, 16, 256, 10
+PEAK_FP32_VECTOR_TFLOPS = 157.3  # MI355X published fp32 vector peak (packed FMA)
+PEAK_HBM_GBS = 8000.0
+MEASURED_ASSIGN_TRAFFIC_BYTES = int((260168.3 * 2.000 + 11688.5 * 1.000) * 1024)
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--rows", type=int, default=N_ROWS, help="rows of the workload (default 1M)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run the plain copy kernel on the workload's rows (3 launches): the "
+                         "known-size kernel the FETCH_SIZE / WRITE_SIZE counters are scaled by")
+    ap.add_argument("--cpu-sample", type=int, default=100_000,
+                    help="rows of the CPU-baseline sample (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
+            "(the path shards by rows, see DESIGN.md, but no multi-GPU code is built).")
+        sys.exit(2)
+
+    import vq_amd
+    from tests import data
+
+    n = args.rows
+    sd = DIM // M
+    t0 = time.time()
+    x = data.gaussian_mixture(n, DIM, 1024, 0.05, seed=1)
+    init, reseed = data.index_streams(n, M, K, ITERS, seed=1)
+    log(f"[bench] generated {n} x {DIM} mixture rows in {time.time() - t0:.1f}s")
+
+    ctx = vq_amd.Context(0)
+    dx = ctx.to_device(x)
+    dcb = ctx.empty((M, K, sd), np.float32)
+    dcodes = ctx.empty((n, M), np.uint8)
+
+    if args.copy_calibration:
+        dy = ctx.empty((n, DIM), np.float32)
+        for _ in range(3):
+            ctx.copy_f32(dy, dx, n * DIM)
+        ctx.sync()
+        print(json.dumps({"copy_calibration_bytes_read": n * DIM * 4,
+                          "copy_calibration_bytes_written": n * DIM * 4, "launches": 3}))
+        return
+
+    def step():
+        ctx.lbg_fit(dx, n, DIM, M, sd, K, ITERS, init, reseed, dcb)
+        ctx.assign(vq_amd.EUCLIDEAN, dx, n, DIM, M, sd, K, dcb, dcodes)
+
+    for _ in range(args.warmup):
+        step()
+    ctx.sync()
+    ctx.prof_enable(True)
+    ctx.sync()
+    t0 = time.perf_counter()
+    ctx.timer_start()
+    for _ in range(args.steps):
+        step()
+    gpu_ms = ctx.timer_stop()
+    ctx.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    assign_ms, assign_n = ctx.prof_read(vq_amd._ffi.PROF_LBG_ASSIGN)
+    update_ms, update_n = ctx.prof_read(vq_amd._ffi.PROF_LBG_UPDATE)
+    enc_ms, enc_n = ctx.prof_read(vq_amd._ffi.PROF_ENCODE)
+    ctx.prof_enable(False)
+    ms_per_step = wall_ms / args.steps
+    value = n / (ms_per_step * 1e-3)
+
+    # dominant kernel: the LBG assignment pass.  Algorithmic work: k*D element-steps per row,
+    # 3 flop each (subtract, multiply, add) -> 3*k*D*n flop per launch; 4*D + 2*m bytes per row.
+    flop_per_launch = 3.0 * K * DIM * n
+    bytes_per_launch = (4.0 * DIM + 2.0 * M) * n
+    avg_assign_ms = assign_ms / max(assign_n, 1)
+    achieved_tflops = flop_per_launch / (avg_assign_ms * 1e-3) / 1e12
+    roofline = {
+        "bound": "valu",
+        "kernel": "k_assign_static<8,4,SQ,LBG> (LBG assignment pass)",
+        "achieved": round(achieved_tflops, 3),
+        "peak": PEAK_FP32_VECTOR_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved_tflops / PEAK_FP32_VECTOR_TFLOPS, 4),
+        # HBM bytes per launch from rocprofv3 FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000), scaled by
+        # the plain copy kernel; measured at the default workload only
+        # (profiles/pq_fit_encode_1Mx128_exact_valu.md)
+        "traffic": MEASURED_ASSIGN_TRAFFIC_BYTES if n == N_ROWS else None,
+        "avg_launch_ms": round(avg_assign_ms, 4),
+        "launches": assign_n,
+        "hbm_GBs_algorithmic": round(bytes_per_launch / (avg_assign_ms * 1e-3) / 1e9, 1),
+        "hbm_frac": round(bytes_per_launch / (avg_assign_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+    }
+    breakdown = {
+        "lbg_assign_ms_per_step": round(assign_ms / args.steps, 3),
+        "lbg_update_ms_per_step": round(update_ms / args.steps, 3),
+        "encode_ms_per_step": round(enc_ms / args.steps, 3),
+        "gpu_event_ms_per_step": round(gpu_ms / args.steps, 3),
+    }
+
+    # CPU baseline + parity on a bounded sample of the same rows
+    cpu = None
+    parity = None
+    if args.cpu_sample > 0:
+        from oracle import oracle as O
+        ns = min(args.cpu_sample, n)
+        xs = np.ascontiguousarray(x[:ns])
+        init_s, reseed_s = data.index_streams(ns, M, K, ITERS, seed=2)
+        threads = min(os.cpu_count() or 1, 16)
+        t0 = time.perf_counter()
+        ref = O.pq_fit_encode(O.EUCLIDEAN, xs, M, K, ITERS, init_s, reseed_s, threads=threads)
+        cpu_s = time.perf_counter() - t0
+        cpu = {
+            "value": round(ns / cpu_s, 1), "unit": "vectors/s", "cores": ref["threads"],
+            "kind": "port",
+            "sample": f"first {ns} rows of the same workload, full fit (10 LBG iterations) + "
+                      f"encode, C restatement of the reference with OpenMP over rows, {cpu_s:.1f} s",
+            "reference_published": "3,751 vectors/s (266.6 s for 1M x 128 uniform rows, "
+                                   "i7-1355U laptop, reference README.md:79-80)",
+        }
+        dxs = ctx.to_device(xs)
+        dcb_s = ctx.empty((M, K, sd), np.float32)
+        dcodes_s = ctx.empty((ns, M), np.uint8)
+        ctx.lbg_fit(dxs, ns, DIM, M, sd, K, ITERS, init_s, reseed_s, dcb_s)
+        ctx.assign(vq_amd.EUCLIDEAN, dxs, ns, DIM, M, sd, K, dcb_s, dcodes_s)
+        g_cb, g_codes = dcb_s.download(), dcodes_s.download()
+        num = np.sqrt(((g_cb.astype(np.float64) - ref["codebooks"]) ** 2).sum())
+        den = np.sqrt((ref["codebooks"].astype(np.float64) ** 2).sum())
+        parity = {
+            "sample_rows": ns,
+            "code_mismatch_rate": float(np.mean(g_codes != ref["codes"].astype(np.uint8))),
+            "centroid_rel_l2": float(num / den),
+            "centroids_bit_identical": bool(np.array_equal(g_cb.view(np.uint32),
+                                                           ref["codebooks"].view(np.uint32))),
+        }
+
+    out = {
+        "metric": "PQ fit+encode vectors/sec at 1M x 128, m=16, k=256 (10 LBG iterations)",
+        "value": round(value, 1),
+        "unit": "vectors/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"PQ fit (10 LBG iterations) + encode of {n} x {DIM} f32 rows, "
+                               "mixture of 1,024 isotropic Gaussians (sigma 0.05, seed 1), "
+                               "m=16, k=256, Euclidean encode to 16 u8 codes per row",
+                   "rows": n, "dim": DIM, "m": M, "k": K, "lbg_iters": ITERS},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "breakdown": breakdown,
+        "parity": parity,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

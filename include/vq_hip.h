@@ -69,10 +69,29 @@ int32_t vq_free(vq_ctx *ctx, void *d_ptr);
 int32_t vq_h2d(vq_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
 int32_t vq_d2h(vq_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
 
+/* Device-to-device copy of `count` floats by a plain streaming kernel (the initial
+ * `rotated_data = training_data.to_vec()` of src/opq.rs:121 and `residuals = training_data.to_vec()`
+ * of src/rvq.rs:103; also the known-size kernel the HBM counters are calibrated against).
+ * Both pointers 16-byte aligned.  Asynchronous. */
+int32_t vq_copy_f32(vq_ctx *ctx, float *d_dst, const float *d_src, int64_t count);
+
 /* ---- timing (HIP events on the context's stream) --------------------------------------- */
 int32_t vq_timer_start(vq_ctx *ctx);
 /* Records the stop event, synchronises, returns elapsed milliseconds since vq_timer_start. */
 int32_t vq_timer_stop(vq_ctx *ctx, float *h_ms);
+
+/* Per-kernel-class timing with HIP events recorded on the context's stream around the launches
+ * the library makes (no counterpart in the reference; measurement only).  Enabling resets the
+ * accumulators.  vq_prof_read synchronises the stream and returns the summed event time and
+ * the number of timed spans of one class. */
+enum vq_prof_class {
+    VQ_PROF_LBG_ASSIGN = 0, /* the assignment kernel of one LBG iteration (utils.rs:59-73) */
+    VQ_PROF_LBG_UPDATE = 1, /* the update kernels of one LBG iteration (utils.rs:83-102) */
+    VQ_PROF_ENCODE = 2,     /* the kernel of one vq_assign call */
+    VQ_PROF_CLASSES = 3
+};
+int32_t vq_prof_enable(vq_ctx *ctx, int32_t on);
+int32_t vq_prof_read(vq_ctx *ctx, int32_t cls, double *h_total_ms, int64_t *h_spans);
 
 /* ---- LBG training: replaces utils::lbg_quantize (src/utils.rs:32-109) ------------------ */
 

@@ -16,6 +16,7 @@ ERR_INVALID_ARG, ERR_DIM_MISMATCH, ERR_EMPTY_INPUT = -1, -2, -3
 ERR_UNSUPPORTED, ERR_OOM, ERR_HIP, ERR_RESEED_EXHAUSTED = -4, -5, -6, -7
 
 SQEUCLIDEAN, EUCLIDEAN, COSINE, MANHATTAN = 0, 1, 2, 3
+PROF_LBG_ASSIGN, PROF_LBG_UPDATE, PROF_ENCODE = 0, 1, 2
 
 # every symbol include/vq_hip.h declares: name -> (restype, argtypes)
 _vp, _i32, _i64, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_size_t
@@ -29,8 +30,11 @@ SYMBOLS = {
     "vq_free": (_i32, [_vp, _vp]),
     "vq_h2d": (_i32, [_vp, _vp, _vp, _sz]),
     "vq_d2h": (_i32, [_vp, _vp, _vp, _sz]),
+    "vq_copy_f32": (_i32, [_vp, _vp, _vp, _i64]),
     "vq_timer_start": (_i32, [_vp]),
     "vq_timer_stop": (_i32, [_vp, C.POINTER(C.c_float)]),
+    "vq_prof_enable": (_i32, [_vp, _i32]),
+    "vq_prof_read": (_i32, [_vp, _i32, C.POINTER(C.c_double), C.POINTER(_i64)]),
     "vq_lbg_fit": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp,
                           _vp]),
     "vq_assign": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
@@ -132,6 +136,9 @@ class Context:
         host = np.ascontiguousarray(host, dtype=dtype)
         return DeviceArray(self, host.shape, host.dtype).upload(host)
 
+    def copy_f32(self, d_dst, d_src, count):
+        self._check(_lib.vq_copy_f32(self._h, d_dst.ptr, d_src.ptr, count))
+
     def sync(self):
         self._check(_lib.vq_ctx_sync(self._h))
 
@@ -142,6 +149,15 @@ class Context:
         ms = C.c_float(0)
         self._check(_lib.vq_timer_stop(self._h, C.byref(ms)))
         return ms.value
+
+    def prof_enable(self, on=True):
+        self._check(_lib.vq_prof_enable(self._h, 1 if on else 0))
+
+    def prof_read(self, cls):
+        """(total_ms, spans) of PROF_LBG_ASSIGN / PROF_LBG_UPDATE / PROF_ENCODE."""
+        ms, cnt = C.c_double(0), _i64(0)
+        self._check(_lib.vq_prof_read(self._h, cls, C.byref(ms), C.byref(cnt)))
+        return ms.value, cnt.value
 
     # -- compute -----------------------------------------------------------------------------
     def lbg_fit(self, d_x, n, ld, m, sub_dim, k, max_iters, init_idx, reseed_stream, d_codebooks):

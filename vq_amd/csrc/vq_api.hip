@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -32,6 +33,16 @@ struct vq_ctx {
     std::string err;
     // grow-only device workspace
     DevBuf flags, tables, hist, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;
+    // optional per-kernel-class timing (HIP events on the stream)
+    bool prof_on = false;
+    std::vector<hipEvent_t> prof_pool;
+    struct Span {
+        int cls;
+        hipEvent_t a, b;
+    };
+    std::vector<Span> prof_open;
+    double prof_ms[VQ_PROF_CLASSES] = {0};
+    int64_t prof_launches[VQ_PROF_CLASSES] = {0};
 };
 
 namespace {
@@ -78,6 +89,51 @@ int32_t ensure(vq_ctx *ctx, DevBuf &b, size_t bytes) {
     } while (0)
 
 inline unsigned cdiv(int64_t a, int64_t b) { return (unsigned)((a + b - 1) / b); }
+
+// ---- per-kernel-class timing -----------------------------------------------------------------
+hipEvent_t prof_event(vq_ctx *ctx) {
+    if (!ctx->prof_pool.empty()) {
+        hipEvent_t e = ctx->prof_pool.back();
+        ctx->prof_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    (void)hipEventCreate(&e);
+    return e;
+}
+
+struct ProfSpan {
+    vq_ctx *ctx;
+    int cls;
+    hipEvent_t a = nullptr;
+    ProfSpan(vq_ctx *c, int k) : ctx(c), cls(k) {
+        if (ctx->prof_on) {
+            a = prof_event(ctx);
+            (void)hipEventRecord(a, ctx->stream);
+        }
+    }
+    ~ProfSpan() {
+        if (a) {
+            hipEvent_t b = prof_event(ctx);
+            (void)hipEventRecord(b, ctx->stream);
+            ctx->prof_open.push_back({cls, a, b});
+        }
+    }
+};
+
+// Resolves the recorded spans; the stream must have been synchronised.
+void prof_collect(vq_ctx *ctx) {
+    for (auto &sp : ctx->prof_open) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, sp.a, sp.b) == hipSuccess) {
+            ctx->prof_ms[sp.cls] += ms;
+            ctx->prof_launches[sp.cls] += 1;
+        }
+        ctx->prof_pool.push_back(sp.a);
+        ctx->prof_pool.push_back(sp.b);
+    }
+    ctx->prof_open.clear();
+}
 
 // ---- assignment dispatch -------------------------------------------------------------------
 
@@ -170,6 +226,16 @@ __global__ void k_decode_f32(const uint8_t *__restrict__ codes, int64_t n, int m
     out[i] = cb[((size_t)s * k + codes[row * m + s]) * sd + t];
 }
 
+__global__ void __launch_bounds__(256) k_copy_f32(const float4 *__restrict__ src,
+                                                  float4 *__restrict__ dst, int64_t n4,
+                                                  const float *__restrict__ src_tail,
+                                                  float *__restrict__ dst_tail, int tail) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    int64_t stride = (int64_t)gridDim.x * 256;
+    for (; i < n4; i += stride) dst[i] = src[i];
+    if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
+}
+
 int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t m, int32_t sd,
                      int32_t k) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
@@ -223,6 +289,8 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
+    prof_collect(ctx);
+    for (hipEvent_t e : ctx->prof_pool) (void)hipEventDestroy(e);
     (void)hipEventDestroy(ctx->ev0);
     (void)hipEventDestroy(ctx->ev1);
     (void)hipStreamDestroy(ctx->stream);
@@ -281,6 +349,43 @@ int32_t vq_timer_stop(vq_ctx *ctx, float *h_ms) {
     VQ_HIP(ctx, hipEventRecord(ctx->ev1, ctx->stream));
     VQ_HIP(ctx, hipEventSynchronize(ctx->ev1));
     VQ_HIP(ctx, hipEventElapsedTime(h_ms, ctx->ev0, ctx->ev1));
+    return VQ_OK;
+}
+
+int32_t vq_prof_enable(vq_ctx *ctx, int32_t on) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    prof_collect(ctx);
+    ctx->prof_on = on != 0;
+    for (int i = 0; i < VQ_PROF_CLASSES; ++i) {
+        ctx->prof_ms[i] = 0;
+        ctx->prof_launches[i] = 0;
+    }
+    return VQ_OK;
+}
+
+int32_t vq_prof_read(vq_ctx *ctx, int32_t cls, double *h_total_ms, int64_t *h_spans) {
+    if (!ctx || cls < 0 || cls >= VQ_PROF_CLASSES || !h_total_ms || !h_spans)
+        return VQ_ERR_INVALID_ARG;
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    prof_collect(ctx);
+    *h_total_ms = ctx->prof_ms[cls];
+    *h_spans = ctx->prof_launches[cls];
+    return VQ_OK;
+}
+
+int32_t vq_copy_f32(vq_ctx *ctx, float *d_dst, const float *d_src, int64_t count) {
+    if (!ctx || count < 0 || (count && (!d_dst || !d_src))) return VQ_ERR_INVALID_ARG;
+    if ((reinterpret_cast<uintptr_t>(d_dst) | reinterpret_cast<uintptr_t>(d_src)) & 15)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: buffers must be 16-byte aligned");
+    if (count == 0) return VQ_OK;
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    int64_t n4 = count / 4;
+    int tail = (int)(count % 4);
+    unsigned blocks = (unsigned)std::min<int64_t>(std::max<int64_t>((n4 + 255) / 256, 1), 256 * 32);
+    hipLaunchKernelGGL(k_copy_f32, dim3(blocks), dim3(256), 0, ctx->stream, (const float4 *)d_src,
+                       (float4 *)d_dst, n4, d_src + n4 * 4, d_dst + n4 * 4, tail);
+    VQ_HIP(ctx, hipGetLastError());
     return VQ_OK;
 }
 
@@ -365,7 +470,11 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
     a.done = S.done;
 
     for (int it = 0; it < max_iters; ++it) {
-        VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd));
+        {
+            ProfSpan sp(ctx, VQ_PROF_LBG_ASSIGN);
+            VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd));
+        }
+        ProfSpan sp(ctx, VQ_PROF_LBG_UPDATE);
         hipLaunchKernelGGL(vq::k_lbg_hist, dim3(nblk, m), dim3(64), 0, st, S, n);
         hipLaunchKernelGGL(vq::k_lbg_scan, dim3(m), dim3(256), 0, st, S, k);
         hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nblk, m), dim3(64), 0, st, S, n);
@@ -379,6 +488,7 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
     std::vector<int> host(6 * (size_t)m + 1);
     VQ_HIP(ctx, hipMemcpyAsync(host.data(), f, sizeof(int) * host.size(), hipMemcpyDeviceToHost, st));
     VQ_HIP(ctx, hipStreamSynchronize(st));
+    prof_collect(ctx);
     if (h_iters_run) memcpy(h_iters_run, host.data() + 2 * m, sizeof(int) * m);
     if (h_reseeds_used) memcpy(h_reseeds_used, host.data() + 3 * m, sizeof(int) * m);
     if (host[6 * (size_t)m])
@@ -412,6 +522,7 @@ int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int6
                            ctx->stream, d_codebooks, (int64_t)m * k, sd, (float *)ctx->cnorm.p);
         a.cnorm = (const float *)ctx->cnorm.p;
     }
+    ProfSpan sp(ctx, VQ_PROF_ENCODE);
     return launch_assign<false>(ctx, metric, a, sd);
 }
 
