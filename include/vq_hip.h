@@ -134,6 +134,69 @@ int32_t vq_decode_f16(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m,
 int32_t vq_decode_f32(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sub_dim,
                       int32_t k, const float *d_codebooks, float *d_out);
 
+/* ---- residual quantizer (src/rvq.rs) -------------------------------------------------------- */
+
+/* d_res[i] -= d_codebook[d_codes[i]] for every row (the residual update of src/rvq.rs:127).
+ * d_codes: n uint8 (the output of vq_assign with m = 1).  Asynchronous. */
+int32_t vq_residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
+                        const float *d_codebook, const uint8_t *d_codes);
+
+/* *h_out = (sum_i sqrt(sum_t x[i][t]^2)) / n — the early-stop statistic of src/rvq.rs:131-138.
+ * Row norms follow the reference's sequential f32 order; the sum over rows (a Rayon sum of
+ * unspecified order in the reference) is a fixed-shape f64 tree.  Synchronises. */
+int32_t vq_mean_l2norm(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, float *h_out);
+
+/* ResidualQuantizer::quantize for every row (src/rvq.rs:171-215): stage by stage argmin under
+ * `metric` (index 0 when k < 2), sum += c, residual -= c, the row stops when
+ * ||residual|| < epsilon.
+ *   d_codebooks    stages*k*dim
+ *   d_codes        out, n*stages uint8 (0 for stages a row did not reach)
+ *   d_stages_used  out (nullable), n uint8: stages applied to the row
+ *   d_recon_f16    out (nullable), n*dim binary16 bit patterns of the f32 sum (rvq.rs:209-214)
+ * Asynchronous. */
+int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t dim,
+                      int32_t stages, int32_t k, const float *d_codebooks, float epsilon,
+                      uint8_t *d_codes, uint8_t *d_stages_used, uint16_t *d_recon_f16);
+
+/* ---- optimized product quantizer (src/opq.rs) ---------------------------------------------- */
+
+/* d_y[i] = R * d_x[i] for every row, R row-major dim x dim (src/opq.rs:186-194, 232-234).
+ * d_y is n x dim, compact.  f32 fused multiply-add accumulation (the reference's nalgebra
+ * rounding is implementation-defined).  Asynchronous. */
+int32_t vq_rotate(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, const float *d_R,
+                  float *d_y);
+
+/* h_A[a*dim + b] = sum_i d_y[i][a] * d_x[i][b], both n x dim compact — the matrix A = Y X^T of
+ * src/opq.rs:172-179, accumulated in f64 in a fixed order.  dim <= 128.  Synchronises. */
+int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n, int32_t dim, double *h_A);
+
+/* ---- tree-structured VQ (src/tsvq.rs) ------------------------------------------------------ */
+
+typedef struct vq_tree vq_tree;
+
+/* TSVQ::new / TSVQNode::fit (src/tsvq.rs:71-148, 209-215): node mean, leaf test, per-dimension
+ * sum of squared deviations in row order, last-maximum split dimension, exact median, stable
+ * partition by `<= median`, children only when non-empty and strictly smaller.  Nodes are
+ * numbered breadth-first (root 0, left before right).  Synchronises. */
+int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim,
+                      int32_t max_depth, vq_tree **out);
+/* A tree from host arrays (children must have larger indices than their parent; -1 = none). */
+int32_t vq_tree_create(vq_ctx *ctx, int32_t n_nodes, int32_t dim, const float *h_centroids,
+                       const int32_t *h_left, const int32_t *h_right, vq_tree **out);
+int32_t vq_tree_free(vq_ctx *ctx, vq_tree *tree);
+int32_t vq_tree_info(const vq_tree *tree, int32_t *n_nodes, int32_t *dim);
+/* Any output may be NULL.  h_split_dim is -1 and h_count 0 where unknown. */
+int32_t vq_tree_download(const vq_tree *tree, float *h_centroids, int32_t *h_left, int32_t *h_right,
+                         int32_t *h_split_dim, float *h_split_val, int64_t *h_count);
+
+/* TSVQNode::quantize_with_distance for every row (src/tsvq.rs:162-181): d_leaf[i] = index of the
+ * leaf reached; `<=` goes left, single children are followed.  Asynchronous. */
+int32_t vq_tsvq_descend(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld,
+                        const vq_tree *tree, int32_t *d_leaf);
+/* d_out[i] = f16(centroid of leaf d_leaf[i]) (src/tsvq.rs:241-248), n x dim.  Asynchronous. */
+int32_t vq_tsvq_decode_f16(vq_ctx *ctx, const vq_tree *tree, const int32_t *d_leaf, int64_t n,
+                           uint16_t *d_out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,179 @@
+"""GPU parity for the residual quantizer and the optimized product quantizer pieces."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from tests import data
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    import vq_amd
+    c = vq_amd.Context(0)
+    yield c
+    c.close()
+
+
+def gpu_rvq_fit(ctx, metric, x, stages, k, iters, eps, init, reseed):
+    """ResidualQuantizer::fit (src/rvq.rs:87-154) composed from the C-ABI calls."""
+    n, dim = x.shape
+    dx = ctx.to_device(x)
+    dres = ctx.empty((n, dim), F)
+    ctx.copy_f32(dres, dx, n * dim)
+    dcb = ctx.empty((stages, k, dim), F)
+    dcodes = ctx.empty(n, np.uint8)
+    norms = []
+    produced = 0
+    for st in range(stages):
+        cb_ptr = dcb.ptr + st * k * dim * 4
+        ctx.lbg_fit(dres, n, dim, 1, dim, k, iters, init[st], reseed[st], cb_ptr)
+        produced += 1
+        if k < 2:
+            dcodes.upload(np.zeros(n, np.uint8))
+        else:
+            ctx.assign(metric, dres, n, dim, 1, dim, k, cb_ptr, dcodes)
+        ctx.residual_sub(dres, n, dim, dim, k, cb_ptr, dcodes)
+        norms.append(ctx.mean_l2norm(dres, n, dim, dim))
+        if norms[-1] < eps:
+            break
+    return dcb.download()[:produced], dres.download(), np.array(norms, F), dcb
+
+
+@pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN, O.COSINE, O.MANHATTAN])
+@pytest.mark.parametrize("n,dim,stages,k,iters", [(1000, 10, 2, 2, 50), (600, 32, 3, 16, 5),
+                                                    (400, 256, 2, 8, 3), (3000, 6, 2, 2, 4)])
+def test_rvq_fit_and_quantize_match_oracle(ctx, metric, n, dim, stages, k, iters):
+    rng = np.random.default_rng(n + dim)
+    x = rng.standard_normal((n, dim)).astype(F)
+    init, reseed = data.index_streams(n, stages, k, iters, seed=3)
+    want = O.rvq_fit(metric, x, stages, k, iters, 0.0, init, reseed)
+    cb, res, norms, dcb = gpu_rvq_fit(ctx, metric, x, stages, k, iters, 0.0, init, reseed)
+    assert want["stages"] == len(cb)
+    assert np.array_equal(cb.view(np.uint32), want["codebooks"].view(np.uint32))
+    assert np.array_equal(res.view(np.uint32), want["residuals"].view(np.uint32))
+    # sum of row norms: Rayon order in the reference, so a tolerance (1e-5 relative)
+    assert np.allclose(norms, want["avg_norms"], rtol=1e-5, atol=0)
+    # quantize
+    wcodes, wrec = O.rvq_quantize(metric, x, want["codebooks"], 0.0)
+    dx = ctx.to_device(x)
+    dcodes = ctx.empty((n, stages), np.uint8)
+    dused = ctx.empty(n, np.uint8)
+    drec = ctx.empty((n, dim), np.uint16)
+    ctx.rvq_encode(metric, dx, n, dim, dim, stages, k, dcb, 0.0, dcodes, dused, drec)
+    assert np.array_equal(dcodes.download(), wcodes.astype(np.uint8))
+    assert np.all(dused.download() == stages)
+    assert np.array_equal(drec.download(), wrec)
+
+
+def test_rvq_quantize_epsilon_stops_rows_individually(ctx):
+    rng = np.random.default_rng(8)
+    n, dim, stages, k = 500, 8, 3, 4
+    cb = rng.standard_normal((stages, k, dim)).astype(F)
+    x = rng.standard_normal((n, dim)).astype(F)
+    x[::5] = cb[0, 2]          # these rows hit a codeword exactly -> residual 0 after stage 1
+    x[1::5] = cb[0, 1] + cb[1, 3]  # and these after stage 2 (if stage 1 picks codeword 1)
+    eps = 1e-3
+    wcodes, wrec = O.rvq_quantize(O.EUCLIDEAN, x, cb, eps)
+    dx, dcb = ctx.to_device(x), ctx.to_device(cb)
+    dcodes = ctx.empty((n, stages), np.uint8)
+    dused = ctx.empty(n, np.uint8)
+    drec = ctx.empty((n, dim), np.uint16)
+    ctx.rvq_encode(O.EUCLIDEAN, dx, n, dim, dim, stages, k, dcb, eps, dcodes, dused, drec)
+    used = dused.download()
+    reached = wcodes != 0xFFFFFFFF
+    assert np.array_equal(used, reached.sum(1))
+    assert used.min() == 1 and used.max() == stages
+    got = dcodes.download()
+    assert np.array_equal(got[reached], wcodes[reached].astype(np.uint8))
+    assert np.all(got[~reached] == 0)
+    assert np.array_equal(drec.download(), wrec)
+
+
+def test_rvq_k1_and_early_training_stop(ctx):
+    x = np.tile(np.array([[1, 2, 3, 4]], F), (20, 1))
+    init = np.array([[0, 1], [0, 1], [0, 1]], np.uint32)
+    reseed = np.zeros((3, 30), np.uint32)
+    want = O.rvq_fit(O.SQEUCLIDEAN, x, 3, 2, 5, 0.01, init, reseed)
+    cb, res, norms, _ = gpu_rvq_fit(ctx, O.SQEUCLIDEAN, x, 3, 2, 5, 0.01, init, reseed)
+    assert len(cb) == want["stages"] == 1 and norms[0] == 0.0
+    assert np.array_equal(cb, want["codebooks"])
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((30, 3)).astype(F)
+    init1, reseed1 = np.array([[4], [5]], np.uint32), np.zeros((2, 3), np.uint32)
+    want = O.rvq_fit(O.COSINE, x, 2, 1, 3, 0.0, init1, reseed1)
+    cb, res, _, _ = gpu_rvq_fit(ctx, O.COSINE, x, 2, 1, 3, 0.0, init1, reseed1)
+    assert np.array_equal(cb, want["codebooks"]) and np.array_equal(res, want["residuals"])
+
+
+# ---- OPQ pieces -------------------------------------------------------------------------------
+@pytest.mark.parametrize("n,dim", [(1000, 10), (4097, 128), (300, 64), (70, 33)])
+def test_rotate_matches_matrix_product(ctx, n, dim):
+    rng = np.random.default_rng(dim)
+    x = rng.standard_normal((n, dim)).astype(F)
+    Q, _ = np.linalg.qr(rng.standard_normal((dim, dim)))
+    R = Q.astype(F)
+    dx, dR, dy = ctx.to_device(x), ctx.to_device(R), ctx.empty((n, dim), F)
+    ctx.rotate(dx, n, dim, dim, dR, dy)
+    y = dy.download()
+    exact = x.astype(np.float64) @ R.astype(np.float64).T
+    # f32 accumulation of dim products: tolerance 1e-5 relative to the row norm
+    assert np.abs(y - exact).max() <= 1e-5 * np.abs(exact).max()
+    assert np.abs(y - O.rotate(x, R)).max() <= 1e-5 * np.abs(exact).max()
+    ctx.rotate(dx, n, dim, dim, ctx.to_device(np.eye(dim, dtype=F)), dy)
+    assert np.array_equal(dy.download(), x)  # identity is exact (opq.rs:119-121)
+
+
+@pytest.mark.parametrize("n,dim", [(1000, 10), (5000, 128), (2049, 32)])
+def test_cross_cov_matches_f64_product(ctx, n, dim):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal((n, dim)).astype(F)
+    y = rng.standard_normal((n, dim)).astype(F)
+    A = ctx.cross_cov(ctx.to_device(y), ctx.to_device(x), n, dim)
+    exact = y.astype(np.float64).T @ x.astype(np.float64)
+    assert np.allclose(A, exact, rtol=1e-12, atol=1e-10)
+    # deterministic: the same call gives the same bits
+    assert np.array_equal(A, ctx.cross_cov(ctx.to_device(y), ctx.to_device(x), n, dim))
+
+
+def test_opq_outer_iteration_stepwise(ctx):
+    """One OPQ outer iteration (src/opq.rs:124-195) on the GPU, every step checked against the
+    oracle on identical inputs; the rotation's rounding is the only tolerance."""
+    rng = np.random.default_rng(43)
+    n, dim, m, k, iters = 3000, 16, 4, 16, 6
+    sd = dim // m
+    x = (rng.standard_normal((n, dim)) @ rng.standard_normal((dim, dim))).astype(F)
+    init, reseed = data.index_streams(n, m, k, iters, seed=5)
+    dx = ctx.to_device(x)
+    drot = ctx.empty((n, dim), F)
+    ctx.copy_f32(drot, dx, n * dim)
+    dcb = ctx.empty((m, k, sd), F)
+    dcodes = ctx.empty((n, m), np.uint8)
+    drec = ctx.empty((n, dim), F)
+    R = np.eye(dim, dtype=F)
+    for outer in range(2):
+        rot = drot.download()
+        ctx.lbg_fit(drot, n, dim, m, sd, k, iters, init, reseed, dcb)
+        want_cb = O.pq_fit(rot, m, k, iters, init, reseed)["codebooks"]
+        assert np.array_equal(dcb.download(), want_cb)
+        ctx.assign(O.EUCLIDEAN, drot, n, dim, m, sd, k, dcb, dcodes)
+        want_codes = O.pq_encode(O.EUCLIDEAN, rot, want_cb)
+        assert np.array_equal(dcodes.download(), want_codes.astype(np.uint8))
+        ctx.decode_f32(dcodes, n, m, sd, k, dcb, drec)
+        rec = np.concatenate([want_cb[s][want_codes[:, s]] for s in range(m)], 1)
+        assert np.array_equal(drec.download(), rec)
+        A = ctx.cross_cov(drec, drot, n, dim)
+        assert np.allclose(A, rec.astype(np.float64).T @ rot.astype(np.float64), rtol=1e-12, atol=1e-9)
+        Rd = O.procrustes(A.astype(F).astype(np.float64))
+        assert np.allclose(Rd.T @ Rd, np.eye(dim), atol=1e-10)
+        R = Rd.astype(F)
+        ctx.rotate(dx, n, dim, dim, ctx.to_device(R), drot)
+        assert np.abs(drot.download() - O.rotate(x, R)).max() <= 1e-5 * np.abs(x).max() * np.sqrt(dim)
+    # the quantizer that fit returns: codebooks of the last iteration, rotation R_T; encode
+    dy = ctx.empty((n, dim), F)
+    ctx.rotate(dx, n, dim, dim, ctx.to_device(R), dy)
+    ctx.assign(O.EUCLIDEAN, dy, n, dim, m, sd, k, dcb, dcodes)
+    want = O.pq_encode(O.EUCLIDEAN, dy.download(), dcb.download())
+    assert np.array_equal(dcodes.download(), want.astype(np.uint8))

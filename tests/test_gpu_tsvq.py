@@ -1,0 +1,131 @@
+"""GPU parity for the tree-structured VQ: build (node statistics) and descent encode."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from tests import data
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    import vq_amd
+    c = vq_amd.Context(0)
+    yield c
+    c.close()
+
+
+def bfs_order(tree):
+    """Renumber an oracle tree (pre-order ids) breadth-first, left before right."""
+    order, frontier = [], [0]
+    while frontier:
+        nxt = []
+        for v in frontier:
+            order.append(v)
+            for c in (tree["left"][v], tree["right"][v]):
+                if c >= 0:
+                    nxt.append(c)
+        frontier = nxt
+    new_id = {old: i for i, old in enumerate(order)}
+    remap = lambda a: np.array([new_id[c] if c >= 0 else -1 for c in a[order]], np.int32)
+    return dict(n_nodes=len(order), centroids=tree["centroids"][order], left=remap(tree["left"]),
+                right=remap(tree["right"]), split_dim=tree["split_dim"][order],
+                split_val=tree["split_val"][order], count=tree["count"][order]), new_id
+
+
+def assert_same_tree(got, want):
+    assert got["n_nodes"] == want["n_nodes"]
+    assert np.array_equal(got["left"], want["left"]) and np.array_equal(got["right"], want["right"])
+    assert np.array_equal(got["count"], want["count"])
+    assert np.array_equal(got["split_dim"], want["split_dim"])
+    internal = want["split_dim"] >= 0
+    assert np.array_equal(got["split_val"][internal], want["split_val"][internal])
+    assert np.array_equal(got["centroids"].view(np.uint32), want["centroids"].view(np.uint32))
+
+
+@pytest.mark.parametrize("n,dim,depth,kind", [
+    (1000, 10, 3, "wide"),     # tests/test_tsvq.rs:25-41
+    (10, 5, 3, "same"),        # tests/test_tsvq.rs:11-22
+    (5000, 16, 6, "normal"),
+    (3001, 7, 10, "normal"),   # odd counts, deep
+    (600, 4, 12, "grid"),      # duplicates: ties at the median, children that do not shrink
+    (40, 3, 20, "normal"),     # deeper than log2(n): single-row leaves
+    (20000, 8, 2, "normal"),   # nodes above 1024 rows -> midpoint-tree means
+    (1, 4, 3, "normal"),
+    (700, 6, 0, "normal"),     # max_depth 0: the root is a leaf
+])
+def test_build_matches_oracle(ctx, n, dim, depth, kind):
+    rng = np.random.default_rng(n + depth)
+    if kind == "normal":
+        x = rng.standard_normal((n, dim)).astype(F)
+    elif kind == "wide":
+        x = rng.uniform(-1000, 1000, (n, dim)).astype(F)
+    elif kind == "grid":
+        x = np.round(rng.standard_normal((n, dim))).astype(F)
+    else:
+        x = np.tile(np.array([[1, 2, 3, 4, 5]], F)[:, :dim], (n, 1))
+    want, _ = bfs_order(O.tsvq_fit(x, depth))
+    tree = ctx.tsvq_build(ctx.to_device(x), n, dim, dim, depth)
+    assert_same_tree(tree.download(), want)
+    tree.free()
+
+
+def test_equal_variances_take_the_last_dimension(ctx):
+    x = np.array([[0, 0, 0], [2, 2, 2], [0, 2, 0], [2, 0, 2]], F)
+    tree = ctx.tsvq_build(ctx.to_device(x), 4, 3, 3, 1)
+    assert tree.download()["split_dim"][0] == 2
+
+
+@pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN, O.COSINE, O.MANHATTAN])
+@pytest.mark.parametrize("n,dim,depth", [(4000, 16, 6), (1000, 10, 3), (777, 128, 8)])
+def test_descent_matches_oracle(ctx, metric, n, dim, depth):
+    rng = np.random.default_rng(n + metric)
+    x = data.unit_rows(n, dim, seed=3) if dim == 128 else rng.standard_normal((n, dim)).astype(F)
+    otree = O.tsvq_fit(x, depth)
+    want_tree, new_id = bfs_order(otree)
+    dx = ctx.to_device(x)
+    tree = ctx.tsvq_build(dx, n, dim, dim, depth)
+    q = np.concatenate([x, rng.standard_normal((500, dim)).astype(F), np.zeros((3, dim), F)])
+    want = np.array([new_id[v] for v in O.tsvq_descend(metric, q, otree)], np.int32)
+    dq = ctx.to_device(q)
+    dleaf = ctx.empty(len(q), np.int32)
+    ctx.tsvq_descend(metric, dq, len(q), dim, tree, dleaf)
+    leaf = dleaf.download()
+    assert np.array_equal(leaf, want)
+    dout = ctx.empty((len(q), dim), np.uint16)
+    ctx.tsvq_decode_f16(tree, dleaf, len(q), dout)
+    assert np.array_equal(dout.download(),
+                          want_tree["centroids"][want].astype(np.float16).view(np.uint16))
+
+
+def test_descent_on_a_hand_made_tree_with_single_children_and_ties(ctx):
+    # node 0 -> (1, 2); node 1 -> left only (3); node 2 -> right only (4); 3, 4 leaves
+    cen = np.array([[0, 0], [-1, 0], [1, 0], [-1, 5], [1, 5]], F)
+    left = np.array([1, 3, -1, -1, -1], np.int32)
+    right = np.array([2, -1, 4, -1, -1], np.int32)
+    tree = ctx.tree_create(cen, left, right)
+    q = np.array([[-3, 0], [3, 0], [0, 7]], F)  # the last one is equidistant -> left (`<=`)
+    dleaf = ctx.empty(3, np.int32)
+    ctx.tsvq_descend(O.SQEUCLIDEAN, ctx.to_device(q), 3, 2, tree, dleaf)
+    assert np.array_equal(dleaf.download(), [3, 4, 3])
+    want = O.tsvq_descend(O.SQEUCLIDEAN, q, dict(centroids=cen, left=left, right=right))
+    assert np.array_equal(dleaf.download(), want)
+
+
+def test_config5_shape_unit_rows_cosine_then_manhattan(ctx):
+    """Depth-8 tree on unit-normalised N(0,1) rows (seed 3), cosine descent, then Manhattan on the
+    same tree; 20,000 rows here, the oracle needs seconds."""
+    n, dim, depth = 20000, 128, 8
+    x = data.unit_rows(n, dim, seed=3)
+    otree = O.tsvq_fit(x, depth)
+    want_tree, new_id = bfs_order(otree)
+    dx = ctx.to_device(x)
+    tree = ctx.tsvq_build(dx, n, dim, dim, depth)
+    assert_same_tree(tree.download(), want_tree)
+    dleaf = ctx.empty(n, np.int32)
+    for metric in (O.COSINE, O.MANHATTAN):
+        ctx.tsvq_descend(metric, dx, n, dim, tree, dleaf)
+        want = np.array([new_id[v] for v in O.tsvq_descend(metric, x, otree)], np.int32)
+        assert np.array_equal(dleaf.download(), want)

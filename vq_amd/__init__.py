@@ -3,5 +3,5 @@
 Importing the package loads libvqhip.so; a missing library is an ImportError.
 """
 from . import _ffi
-from ._ffi import (COSINE, EUCLIDEAN, MANHATTAN, SQEUCLIDEAN, Context, DeviceArray,  # noqa: F401
+from ._ffi import (COSINE, EUCLIDEAN, MANHATTAN, SQEUCLIDEAN, Context, DeviceArray, Tree,  # noqa: F401
                    VqError)

@@ -40,6 +40,19 @@ SYMBOLS = {
     "vq_assign": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_decode_f16": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_decode_f32": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
+    "vq_residual_sub": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp]),
+    "vq_mean_l2norm": (_i32, [_vp, _vp, _i64, _i64, _i32, C.POINTER(C.c_float)]),
+    "vq_rvq_encode": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, C.c_float, _vp, _vp,
+                             _vp]),
+    "vq_rotate": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp]),
+    "vq_cross_cov": (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
+    "vq_tsvq_build": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, C.POINTER(_vp)]),
+    "vq_tree_create": (_i32, [_vp, _i32, _i32, _vp, _vp, _vp, C.POINTER(_vp)]),
+    "vq_tree_free": (_i32, [_vp, _vp]),
+    "vq_tree_info": (_i32, [_vp, C.POINTER(_i32), C.POINTER(_i32)]),
+    "vq_tree_download": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "vq_tsvq_descend": (_i32, [_vp, _i32, _vp, _i64, _i64, _vp, _vp]),
+    "vq_tsvq_decode_f16": (_i32, [_vp, _vp, _vp, _i64, _vp]),
 }
 
 
@@ -97,6 +110,39 @@ class DeviceArray:
         if self.ptr:
             _lib.vq_free(self.ctx._h, self.ptr)
             self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Tree:
+    """A TSVQ node table held by the library (breadth-first node numbering)."""
+
+    def __init__(self, ctx, handle):
+        self.ctx, self._h = ctx, handle
+        nn, dim = _i32(0), _i32(0)
+        ctx._check(_lib.vq_tree_info(handle, C.byref(nn), C.byref(dim)))
+        self.n_nodes, self.dim = nn.value, dim.value
+
+    def download(self):
+        nn, dim = self.n_nodes, self.dim
+        cen = np.empty((nn, dim), np.float32)
+        left, right, sdim = (np.empty(nn, np.int32) for _ in range(3))
+        sval = np.empty(nn, np.float32)
+        cnt = np.empty(nn, np.int64)
+        self.ctx._check(_lib.vq_tree_download(self._h, cen.ctypes.data, left.ctypes.data,
+                                              right.ctypes.data, sdim.ctypes.data, sval.ctypes.data,
+                                              cnt.ctypes.data))
+        return dict(n_nodes=nn, centroids=cen, left=left, right=right, split_dim=sdim,
+                    split_val=sval, count=cnt)
+
+    def free(self):
+        if self._h:
+            _lib.vq_tree_free(self.ctx._h, self._h)
+            self._h = None
 
     def __del__(self):
         try:
@@ -167,15 +213,15 @@ class Context:
         n_reseed = reseed_stream.shape[1]
         iters = np.zeros(m, np.int32)
         used = np.zeros(m, np.int32)
-        self._check(_lib.vq_lbg_fit(self._h, d_x.ptr, n, ld, m, sub_dim, k, max_iters,
+        self._check(_lib.vq_lbg_fit(self._h, _ptr(d_x), n, ld, m, sub_dim, k, max_iters,
                                     init_idx.ctypes.data, reseed_stream.ctypes.data if n_reseed
-                                    else None, n_reseed, d_codebooks.ptr, iters.ctypes.data,
+                                    else None, n_reseed, _ptr(d_codebooks), iters.ctypes.data,
                                     used.ctypes.data))
         return iters, used
 
     def assign(self, metric, d_x, n, ld, m, sub_dim, k, d_codebooks, d_codes):
-        self._check(_lib.vq_assign(self._h, metric, d_x.ptr, n, ld, m, sub_dim, k,
-                                   d_codebooks.ptr, d_codes.ptr))
+        self._check(_lib.vq_assign(self._h, metric, _ptr(d_x), n, ld, m, sub_dim, k,
+                                   _ptr(d_codebooks), _ptr(d_codes)))
 
     def decode_f16(self, d_codes, n, m, sub_dim, k, d_codebooks, d_out):
         self._check(_lib.vq_decode_f16(self._h, d_codes.ptr, n, m, sub_dim, k, d_codebooks.ptr,
@@ -184,3 +230,55 @@ class Context:
     def decode_f32(self, d_codes, n, m, sub_dim, k, d_codebooks, d_out):
         self._check(_lib.vq_decode_f32(self._h, d_codes.ptr, n, m, sub_dim, k, d_codebooks.ptr,
                                        d_out.ptr))
+
+    # -- residual quantizer --------------------------------------------------------------------
+    def residual_sub(self, d_res, n, ld, dim, k, d_codebook, d_codes):
+        self._check(_lib.vq_residual_sub(self._h, d_res.ptr, n, ld, dim, k, _ptr(d_codebook),
+                                         d_codes.ptr))
+
+    def mean_l2norm(self, d_x, n, ld, dim):
+        out = C.c_float(0)
+        self._check(_lib.vq_mean_l2norm(self._h, d_x.ptr, n, ld, dim, C.byref(out)))
+        return out.value
+
+    def rvq_encode(self, metric, d_x, n, ld, dim, stages, k, d_codebooks, epsilon, d_codes,
+                   d_used=None, d_recon=None):
+        self._check(_lib.vq_rvq_encode(self._h, metric, d_x.ptr, n, ld, dim, stages, k,
+                                       d_codebooks.ptr, epsilon, d_codes.ptr,
+                                       d_used.ptr if d_used else None,
+                                       d_recon.ptr if d_recon else None))
+
+    # -- optimized product quantizer -----------------------------------------------------------
+    def rotate(self, d_x, n, ld, dim, d_R, d_y):
+        self._check(_lib.vq_rotate(self._h, d_x.ptr, n, ld, dim, d_R.ptr, d_y.ptr))
+
+    def cross_cov(self, d_y, d_x, n, dim):
+        A = np.empty((dim, dim), np.float64)
+        self._check(_lib.vq_cross_cov(self._h, d_y.ptr, d_x.ptr, n, dim, A.ctypes.data))
+        return A
+
+    # -- tree-structured VQ --------------------------------------------------------------------
+    def tsvq_build(self, d_x, n, ld, dim, max_depth):
+        h = _vp()
+        self._check(_lib.vq_tsvq_build(self._h, d_x.ptr, n, ld, dim, max_depth, C.byref(h)))
+        return Tree(self, h)
+
+    def tree_create(self, centroids, left, right):
+        cen = np.ascontiguousarray(centroids, np.float32)
+        left = np.ascontiguousarray(left, np.int32)
+        right = np.ascontiguousarray(right, np.int32)
+        h = _vp()
+        self._check(_lib.vq_tree_create(self._h, cen.shape[0], cen.shape[1], cen.ctypes.data,
+                                        left.ctypes.data, right.ctypes.data, C.byref(h)))
+        return Tree(self, h)
+
+    def tsvq_descend(self, metric, d_x, n, ld, tree, d_leaf):
+        self._check(_lib.vq_tsvq_descend(self._h, metric, d_x.ptr, n, ld, tree._h, d_leaf.ptr))
+
+    def tsvq_decode_f16(self, tree, d_leaf, n, d_out):
+        self._check(_lib.vq_tsvq_decode_f16(self._h, tree._h, d_leaf.ptr, n, d_out.ptr))
+
+
+def _ptr(a):
+    """Device address of a DeviceArray or a raw integer address."""
+    return a.ptr if isinstance(a, DeviceArray) else a

@@ -5,21 +5,20 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libvqhip.so")
-SRC = [os.path.join(HERE, "csrc", "vq_api.hip")]
+SRC = [os.path.join(HERE, "csrc", f) for f in
+       ("vq_api.hip", "vq_api_rvq_opq.hip", "vq_api_tsvq.hip")]
 
 # -ffp-contract=off: the exact kernels must round multiply and add separately, as the
 #   reference's Rust code does.  Fused operations are written explicitly where wanted.
 # -packed-fp32-ops disabled: no v_pk_*_f32 may be generated.
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-fno-fast-math", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
 
 
-def build_lib(verbose=False, extra=()):
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *FLAGS, *extra, "-o", LIB, *SRC]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -29,6 +28,19 @@ def build_lib(verbose=False, extra=()):
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
+
+
+def build_lib(verbose=False, extra=()):
+    """Compiles every translation unit (in parallel) and links libvqhip.so."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = [os.path.join(objdir, os.path.basename(s)[:-4] + ".o") for s in SRC]
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        list(ex.map(lambda so: _run([hipcc, *FLAGS, *extra, "-c", so[0], "-o", so[1]], verbose),
+                    zip(SRC, objs)))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs], verbose)
     return LIB
 
 

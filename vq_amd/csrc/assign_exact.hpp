@@ -30,7 +30,7 @@ struct AssignArgs {
 };
 
 // sqrt(sum of squares) of every centroid, sequential order (map_sum, src/distances.rs:66-69,144)
-__global__ void k_centroid_norms(const float *__restrict__ cb, int64_t total, int sd,
+static __global__ void k_centroid_norms(const float *__restrict__ cb, int64_t total, int sd,
                                  float *__restrict__ out) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;

@@ -1,0 +1,137 @@
+// Shared host-side state of libvqhip: the context, error reporting, the grow-only device
+// workspace and the per-kernel-class event timing.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "../../include/vq_hip.h"
+
+struct DevBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+};
+
+struct vq_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::string err;
+    // grow-only device workspace
+    DevBuf flags, tables, hist, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;
+    DevBuf tmp_a, tmp_b, tmp_c, tmp_d, tmp_e, tmp_f;  // scratch of the RVQ / OPQ / TSVQ entry points
+    // optional per-kernel-class timing (HIP events on the stream)
+    bool prof_on = false;
+    std::vector<hipEvent_t> prof_pool;
+    struct Span {
+        int cls;
+        hipEvent_t a, b;
+    };
+    std::vector<Span> prof_open;
+    double prof_ms[VQ_PROF_CLASSES] = {0};
+    int64_t prof_launches[VQ_PROF_CLASSES] = {0};
+};
+
+namespace vqh {
+
+std::string &create_error();
+
+inline int32_t fail(vq_ctx *ctx, int32_t code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (ctx)
+        ctx->err = buf;
+    else
+        create_error() = buf;
+    return code;
+}
+
+#define VQ_HIP(ctx, call)                                                                          \
+    do {                                                                                           \
+        hipError_t e__ = (call);                                                                   \
+        if (e__ != hipSuccess)                                                                     \
+            return vqh::fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,            \
+                             "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__, __LINE__); \
+    } while (0)
+
+#define VQ_TRY(expr)                    \
+    do {                                \
+        int32_t rc__ = (expr);          \
+        if (rc__ != VQ_OK) return rc__; \
+    } while (0)
+
+inline int32_t ensure(vq_ctx *ctx, DevBuf &b, size_t bytes) {
+    if (bytes <= b.cap) return VQ_OK;
+    if (b.p) {
+        VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        VQ_HIP(ctx, hipFree(b.p));
+        b.p = nullptr;
+        b.cap = 0;
+    }
+    size_t want = bytes + bytes / 8 + 256;
+    VQ_HIP(ctx, hipMalloc(&b.p, want));
+    b.cap = want;
+    return VQ_OK;
+}
+
+inline unsigned cdiv(int64_t a, int64_t b) { return (unsigned)((a + b - 1) / b); }
+
+inline hipEvent_t prof_event(vq_ctx *ctx) {
+    if (!ctx->prof_pool.empty()) {
+        hipEvent_t e = ctx->prof_pool.back();
+        ctx->prof_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    (void)hipEventCreate(&e);
+    return e;
+}
+
+struct ProfSpan {
+    vq_ctx *ctx;
+    int cls;
+    hipEvent_t a = nullptr;
+    ProfSpan(vq_ctx *c, int k) : ctx(c), cls(k) {
+        if (ctx->prof_on) {
+            a = prof_event(ctx);
+            (void)hipEventRecord(a, ctx->stream);
+        }
+    }
+    ~ProfSpan() {
+        if (a) {
+            hipEvent_t b = prof_event(ctx);
+            (void)hipEventRecord(b, ctx->stream);
+            ctx->prof_open.push_back({cls, a, b});
+        }
+    }
+};
+
+// Resolves the recorded spans; the stream must have been synchronised.
+inline void prof_collect(vq_ctx *ctx) {
+    for (auto &sp : ctx->prof_open) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, sp.a, sp.b) == hipSuccess) {
+            ctx->prof_ms[sp.cls] += ms;
+            ctx->prof_launches[sp.cls] += 1;
+        }
+        ctx->prof_pool.push_back(sp.a);
+        ctx->prof_pool.push_back(sp.b);
+    }
+    ctx->prof_open.clear();
+}
+
+// Argument checks shared by the entry points that take a row matrix and codebooks.
+int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t m, int32_t sd, int32_t k);
+
+// Launchers defined in vq_api.hip, used by the RVQ / OPQ entry points.
+int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
+                     int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes);
+
+}  // namespace vqh

@@ -43,7 +43,7 @@ struct LbgState {
     int leaf_cap;
 };
 
-__global__ void k_lbg_init(LbgState st, int m) {
+static __global__ void k_lbg_init(LbgState st, int m) {
     int s = blockIdx.x * blockDim.x + threadIdx.x;
     if (s < m) {
         st.changed[s] = 0;
@@ -57,7 +57,7 @@ __global__ void k_lbg_init(LbgState st, int m) {
 }
 
 // codebook[s][j][t] = x[idx[s][j]][s*sd + t]     (src/utils.rs:54)
-__global__ void k_gather_rows(const float *__restrict__ x, int64_t ld, int m, int k, int sd,
+static __global__ void k_gather_rows(const float *__restrict__ x, int64_t ld, int m, int k, int sd,
                               const uint32_t *__restrict__ idx, float *__restrict__ cb) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     int64_t total = (int64_t)m * k * sd;
@@ -69,7 +69,7 @@ __global__ void k_gather_rows(const float *__restrict__ x, int64_t ld, int m, in
 }
 
 // One wave per (row block, column block): histogram of the codes of kRowBlock rows.
-__global__ void __launch_bounds__(64) k_lbg_hist(LbgState st, int64_t n) {
+static __global__ void __launch_bounds__(64) k_lbg_hist(LbgState st, int64_t n) {
     const int s = blockIdx.y, b = blockIdx.x;
     if (st.done[s]) return;
     __shared__ uint32_t cnt[kMaxK];
@@ -94,7 +94,7 @@ __device__ __forceinline__ uint32_t tree_depth(uint32_t count) {
 // Turns the histograms into exclusive prefixes over row blocks, derives cluster offsets,
 // tree depths, leaf descriptors, the rank of every empty cluster, and advances the re-seed
 // cursor by the number of empty clusters.
-__global__ void __launch_bounds__(256) k_lbg_scan(LbgState st, int k) {
+static __global__ void __launch_bounds__(256) k_lbg_scan(LbgState st, int k) {
     const int s = blockIdx.x, j = threadIdx.x;
     if (st.done[s]) return;
     __shared__ uint32_t sh_cnt[kMaxK], sh_leaf[kMaxK], sh_empty[kMaxK];
@@ -149,7 +149,7 @@ __global__ void __launch_bounds__(256) k_lbg_scan(LbgState st, int k) {
 }
 
 // One wave per (row block, column block): stable ranked scatter of row ids into perm[s].
-__global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t n) {
+static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t n) {
     const int s = blockIdx.y, b = blockIdx.x;
     if (st.done[s]) return;
     __shared__ uint32_t base[kMaxK];
@@ -187,7 +187,7 @@ __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t n) {
 }
 
 // One lane per (leaf, component): sequential sum of the leaf's members in list order.
-__global__ void __launch_bounds__(256) k_lbg_leafsum(LbgState st, const float *__restrict__ x,
+static __global__ void __launch_bounds__(256) k_lbg_leafsum(LbgState st, const float *__restrict__ x,
                                                      int64_t n, int64_t ld, int sd) {
     const int s = blockIdx.y;
     if (st.done[s]) return;
@@ -213,7 +213,7 @@ __global__ void __launch_bounds__(256) k_lbg_leafsum(LbgState st, const float *_
 
 // One lane per (cluster, component): combine leaves left + right, divide by the count
 // (src/vector.rs:315-316), or copy the re-seed row for an empty cluster (src/utils.rs:98-101).
-__global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const float *__restrict__ x,
+static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const float *__restrict__ x,
                                                       int64_t ld, int k, int sd,
                                                       const uint32_t *__restrict__ reseed,
                                                       int n_reseed, float *__restrict__ cb) {
@@ -245,7 +245,7 @@ __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const float *
 }
 
 // Loop control of src/utils.rs:57,104-106, one thread per column block.
-__global__ void k_lbg_advance(LbgState st, int m) {
+static __global__ void k_lbg_advance(LbgState st, int m) {
     int s = blockIdx.x * blockDim.x + threadIdx.x;
     if (s >= m || st.done[s]) return;
     st.iters[s] += 1;

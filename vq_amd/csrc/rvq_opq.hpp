@@ -1,0 +1,182 @@
+// Kernels around the assignment for the residual and the optimized product quantizer:
+// residual update and norms (src/rvq.rs:111-141,200-207), rotation y = R x
+// (src/opq.rs:186-194,232-234) and the cross-covariance A = Y X^T (src/opq.rs:172-179).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vq {
+
+// res[i] -= codebook[code[i]]   (src/rvq.rs:127).  One lane per element.
+static __global__ void __launch_bounds__(256) k_residual_sub(float *__restrict__ res, int64_t n, int64_t ld,
+                                                      int dim, const float *__restrict__ cb,
+                                                      const uint8_t *__restrict__ codes,
+                                                      int code_stride) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n * dim) return;
+    int64_t row = i / dim;
+    int t = (int)(i % dim);
+    float *p = res + row * ld + t;
+    *p = *p - cb[(size_t)codes[row * code_stride] * dim + t];
+}
+
+// norms[i] = sqrt(sum_t x[i][t]^2), sequential f32 order (src/rvq.rs:134-135).
+static __global__ void __launch_bounds__(256) k_row_norms(const float *__restrict__ x, int64_t n, int64_t ld,
+                                                   int dim, float *__restrict__ norms) {
+    int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= n) return;
+    const float *p = x + row * ld;
+    float acc = 0.0f;
+    for (int t = 0; t < dim; ++t) {
+        float q = p[t] * p[t];
+        acc = acc + q;
+    }
+    norms[row] = sqrtf(acc);
+}
+
+// Fixed-shape two-level sum of n floats in f64: every workgroup sums a contiguous slice with a
+// fixed intra-group tree; a second launch of one workgroup sums the partials the same way.
+static __global__ void __launch_bounds__(256) k_sum_f64(const float *__restrict__ in_f32,
+                                                 const double *__restrict__ in_f64, int64_t n,
+                                                 int64_t per_block, double *__restrict__ out) {
+    __shared__ double sh[256];
+    int64_t lo = (int64_t)blockIdx.x * per_block;
+    int64_t hi = lo + per_block < n ? lo + per_block : n;
+    double acc = 0.0;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += 256) acc += in_f32 ? (double)in_f32[i] : in_f64[i];
+    sh[threadIdx.x] = acc;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) sh[threadIdx.x] += sh[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = sh[0];
+}
+
+// One stage of ResidualQuantizer::quantize for every row still active (src/rvq.rs:200-207):
+// sum += c; residual -= c; stop the row when ||residual|| < epsilon.
+static __global__ void __launch_bounds__(256) k_rvq_stage_apply(float *__restrict__ res, float *__restrict__ sum,
+                                                         int64_t n, int dim, const float *__restrict__ cb,
+                                                         const uint8_t *__restrict__ stage_codes,
+                                                         uint8_t *__restrict__ codes_out, int stages,
+                                                         int stage, uint8_t *__restrict__ active,
+                                                         uint8_t *__restrict__ used, float epsilon) {
+    int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= n) return;
+    if (!active[row]) {
+        codes_out[row * stages + stage] = 0;
+        return;
+    }
+    int code = stage_codes[row];
+    codes_out[row * stages + stage] = (uint8_t)code;
+    const float *c = cb + (size_t)code * dim;
+    float *r = res + row * dim;
+    float *s = sum + row * dim;
+    float acc = 0.0f;
+    for (int t = 0; t < dim; ++t) {
+        s[t] = s[t] + c[t];
+        float v = r[t] - c[t];
+        r[t] = v;
+        float q = v * v;
+        acc = acc + q;
+    }
+    used[row] = (uint8_t)(stage + 1);
+    if (sqrtf(acc) < epsilon) active[row] = 0;
+}
+
+static __global__ void __launch_bounds__(256) k_f32_to_f16(const float *__restrict__ in, int64_t count,
+                                                    uint16_t *__restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) out[i] = __half_as_ushort(__float2half_rn(in[i]));
+}
+
+static __global__ void __launch_bounds__(256) k_fill_u8(uint8_t *__restrict__ p, int64_t count, uint8_t v) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) p[i] = v;
+}
+
+static __global__ void __launch_bounds__(256) k_fill_f32(float *__restrict__ p, int64_t count, float v) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) p[i] = v;
+}
+
+// ---- rotation ------------------------------------------------------------------------------
+// y[i][a] = sum_b R[a][b] * x[i][b].  Generic dimension: one workgroup = 64 rows, x tile and
+// (a slab of) R staged in LDS, fused multiply-add accumulation in ascending b.
+static __global__ void __launch_bounds__(256) k_rotate_generic(const float *__restrict__ x, int64_t n,
+                                                        int64_t ld, int dim,
+                                                        const float *__restrict__ R,
+                                                        float *__restrict__ y) {
+    extern __shared__ float lds[];  // 64 * (dim + 1) floats of x
+    const int stride = dim + 1;
+    const int64_t row0 = (int64_t)blockIdx.x * 64;
+    for (int i = threadIdx.x; i < 64 * dim; i += 256) {
+        int r = i / dim, t = i % dim;
+        int64_t row = row0 + r;
+        lds[r * stride + t] = row < n ? x[row * ld + t] : 0.0f;
+    }
+    __syncthreads();
+    // thread -> (row r = tid % 64, outputs a = tid / 64, +4, +8, ...)
+    const int r = threadIdx.x % 64;
+    const int64_t row = row0 + r;
+    for (int a = threadIdx.x / 64; a < dim; a += 4) {
+        const float *Ra = R + (size_t)a * dim;  // wave-uniform
+        float acc = 0.0f;
+        for (int b = 0; b < dim; ++b) acc = __builtin_fmaf(Ra[b], lds[r * stride + b], acc);
+        if (row < n) y[row * dim + a] = acc;
+    }
+}
+
+// ---- cross-covariance ----------------------------------------------------------------------
+// part[c][a][b] = sum over the rows of chunk c of yr[i][a] * x[i][b], accumulated in f64 in row
+// order; chunks are combined in chunk order by k_crosscov_reduce.  Generic dimension.
+static __global__ void __launch_bounds__(256) k_crosscov_partial(const float *__restrict__ yr,
+                                                          const float *__restrict__ x, int64_t n,
+                                                          int dim, int64_t rows_per_chunk,
+                                                          double *__restrict__ part) {
+    extern __shared__ float lds[];  // 2 * 32 * dim floats
+    float *ly = lds, *lx = lds + 32 * dim;
+    const int64_t lo = (int64_t)blockIdx.x * rows_per_chunk;
+    const int64_t hi = lo + rows_per_chunk < n ? lo + rows_per_chunk : n;
+    const int total = dim * dim;
+    // each thread owns outputs e = tid, tid+256, ... (at most 64 per thread: dim <= 128)
+    double acc[64];
+#pragma unroll
+    for (int u = 0; u < 64; ++u) acc[u] = 0.0;
+    for (int64_t r0 = lo; r0 < hi; r0 += 32) {
+        int rows = (int)((hi - r0) < 32 ? (hi - r0) : 32);
+        __syncthreads();
+        for (int i = threadIdx.x; i < rows * dim; i += 256) {
+            ly[i] = yr[r0 * dim + i];
+            lx[i] = x[r0 * dim + i];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 64; ++u) {
+            int e = threadIdx.x + u * 256;
+            if (e < total) {
+                int a = e / dim, b = e % dim;
+                double s = acc[u];
+                for (int r = 0; r < rows; ++r) s += (double)ly[r * dim + a] * (double)lx[r * dim + b];
+                acc[u] = s;
+            }
+        }
+    }
+    double *out = part + (size_t)blockIdx.x * total;
+#pragma unroll
+    for (int u = 0; u < 64; ++u) {
+        int e = threadIdx.x + u * 256;
+        if (e < total) out[e] = acc[u];
+    }
+}
+
+static __global__ void __launch_bounds__(256) k_crosscov_reduce(const double *__restrict__ part, int chunks,
+                                                         int total, double *__restrict__ out) {
+    int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= total) return;
+    double s = 0.0;
+    for (int c = 0; c < chunks; ++c) s += part[(size_t)c * total + e];
+    out[e] = s;
+}
+
+}  // namespace vq

@@ -1,0 +1,288 @@
+// Tree-structured VQ: node statistics for the build (src/tsvq.rs:71-148) and the descent
+// encode (src/tsvq.rs:162-181).
+//
+// Build, one tree level at a time.  `perm` lists row ids so that the rows of every node of the
+// level are contiguous and in original row order (the reference's partition is stable).
+//   mean      mean_vector over the node's rows: sequential up to 1024 rows, the fixed midpoint
+//             tree above (same order as the LBG update)
+//   variance  per dimension, sum over the node's rows IN ROW ORDER of (x - mean)^2, f32
+//             (Iterator::sum is sequential, src/tsvq.rs:88-99) — one lane per (node, dimension)
+//   median    of the split column by a segmented sort (host picks the middle values)
+//   partition stable, by `x[split] <= median`
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vq {
+
+// One lane per (leaf, component): sequential sum over perm[lo, hi).
+static __global__ void __launch_bounds__(256) k_seg_leafsum(const uint32_t *__restrict__ perm,
+                                                     const uint2 *__restrict__ desc, int64_t nleaves,
+                                                     const float *__restrict__ x, int64_t ld, int sd,
+                                                     float *__restrict__ leaf_sum) {
+    int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    int64_t leaf = gid / sd;
+    int t = (int)(gid % sd);
+    if (leaf >= nleaves) return;
+    uint2 d = desc[leaf];
+    const float *__restrict__ xc = x + t;
+    float acc = 0.0f;
+    uint32_t p = d.x;
+    for (; p + 8 <= d.y; p += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = xc[(int64_t)perm[p + u] * ld];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc = acc + v[u];
+    }
+    for (; p < d.y; ++p) acc = acc + xc[(int64_t)perm[p] * ld];
+    leaf_sum[leaf * sd + t] = acc;
+}
+
+// One lane per (segment, component): combine 2^depth leaves left + right, divide by the count.
+// seg_info[g] = {first leaf, depth, count, unused}
+static __global__ void __launch_bounds__(256) k_seg_mean(float *__restrict__ leaf_sum,
+                                                  const uint4 *__restrict__ seg_info, int nseg, int sd,
+                                                  float *__restrict__ out, int64_t out_first) {
+    int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    int g = (int)(gid / sd);
+    int t = (int)(gid % sd);
+    if (g >= nseg) return;
+    uint4 info = seg_info[g];
+    uint32_t nl = 1u << info.y;
+    float *ls = leaf_sum + (size_t)info.x * sd + t;
+    for (uint32_t h = 1; h < nl; h <<= 1)
+        for (uint32_t i = 0; i < nl; i += 2 * h)
+            ls[(size_t)i * sd] = ls[(size_t)i * sd] + ls[(size_t)(i + h) * sd];
+    out[(out_first + g) * sd + t] = ls[0] / __uint2float_rn(info.z);
+}
+
+// One lane per (segment, dimension): sequential sum of squared deviations in row order.
+// seg_range[g] = {lo, hi} positions in perm; mean of segment g at means[(first + g) * dim].
+static __global__ void __launch_bounds__(64) k_seg_variance(const uint32_t *__restrict__ perm,
+                                                     const uint2 *__restrict__ seg_range, int nseg,
+                                                     const float *__restrict__ means, int64_t first,
+                                                     const float *__restrict__ x, int64_t ld, int dim,
+                                                     float *__restrict__ var) {
+    int64_t gid = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    int g = (int)(gid / dim);
+    int t = (int)(gid % dim);
+    if (g >= nseg) return;
+    uint2 r = seg_range[g];
+    const float mu = means[(first + g) * dim + t];
+    const float *__restrict__ xc = x + t;
+    float acc = 0.0f;
+    uint32_t p = r.x;
+    for (; p + 16 <= r.y; p += 16) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = xc[(int64_t)perm[p + u] * ld];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            float d = v[u] - mu;
+            float q = d * d;
+            acc = acc + q;
+        }
+    }
+    for (; p < r.y; ++p) {
+        float d = xc[(int64_t)perm[p] * ld] - mu;
+        float q = d * d;
+        acc = acc + q;
+    }
+    var[(size_t)g * dim + t] = acc;
+}
+
+__device__ __forceinline__ int find_segment(const uint2 *__restrict__ seg_range, int nseg, uint32_t p) {
+    // segments are sorted by position and disjoint; returns -1 when p lies in none
+    int lo = 0, hi = nseg - 1;
+    while (lo <= hi) {
+        int mid = (lo + hi) >> 1;
+        uint2 r = seg_range[mid];
+        if (p < r.x)
+            hi = mid - 1;
+        else if (p >= r.y)
+            lo = mid + 1;
+        else
+            return mid;
+    }
+    return -1;
+}
+
+// vals[p] = x[perm[p]][split_dim[segment of p]]; positions outside every segment get +inf
+static __global__ void __launch_bounds__(256) k_seg_gather_col(const uint32_t *__restrict__ perm, int64_t n,
+                                                        const uint2 *__restrict__ seg_range, int nseg,
+                                                        const int *__restrict__ split_dim,
+                                                        const float *__restrict__ x, int64_t ld,
+                                                        float *__restrict__ vals) {
+    int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (p >= n) return;
+    int g = find_segment(seg_range, nseg, (uint32_t)p);
+    vals[p] = g < 0 ? __builtin_inff() : x[(int64_t)perm[p] * ld + split_dim[g]];
+}
+
+// flags[p] = 1 when the row at position p goes left (value <= median of its segment)
+static __global__ void __launch_bounds__(256) k_seg_flags(const float *__restrict__ vals, int64_t n,
+                                                   const uint2 *__restrict__ seg_range, int nseg,
+                                                   const float *__restrict__ median,
+                                                   uint32_t *__restrict__ flags) {
+    int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (p >= n) return;
+    int g = find_segment(seg_range, nseg, (uint32_t)p);
+    flags[p] = (g >= 0 && vals[p] <= median[g]) ? 1u : 0u;
+}
+
+// Stable partition inside every segment using the exclusive scan of flags.
+// nleft[g] = number of rows going left.
+static __global__ void __launch_bounds__(256) k_seg_partition(const uint32_t *__restrict__ perm_in, int64_t n,
+                                                       const uint2 *__restrict__ seg_range, int nseg,
+                                                       const uint32_t *__restrict__ flags,
+                                                       const uint32_t *__restrict__ scan,
+                                                       uint32_t *__restrict__ perm_out,
+                                                       uint32_t *__restrict__ nleft) {
+    int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (p >= n) return;
+    int g = find_segment(seg_range, nseg, (uint32_t)p);
+    if (g < 0) {
+        perm_out[p] = perm_in[p];
+        return;
+    }
+    uint2 r = seg_range[g];
+    uint32_t before = scan[p] - scan[r.x];                       // left rows before p in the segment
+    uint32_t total_left = scan[r.y - 1] + flags[r.y - 1] - scan[r.x];
+    uint32_t dst = flags[p] ? r.x + before : r.x + total_left + ((uint32_t)p - r.x - before);
+    perm_out[dst] = perm_in[p];
+    if ((uint32_t)p == r.x) nleft[g] = total_left;
+}
+
+static __global__ void __launch_bounds__(256) k_iota_u32(uint32_t *__restrict__ p, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = (uint32_t)i;
+}
+
+// mids[2g], mids[2g+1] = the two middle values of the sorted segment g (equal for odd counts)
+static __global__ void k_seg_middles(const float *__restrict__ sorted, const uint2 *__restrict__ seg_range,
+                              int nseg, float *__restrict__ mids) {
+    int g = blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= nseg) return;
+    uint2 r = seg_range[g];
+    uint32_t c = r.y - r.x;
+    if (c % 2 == 0) {
+        mids[2 * g] = sorted[r.x + c / 2 - 1];
+        mids[2 * g + 1] = sorted[r.x + c / 2];
+    } else {
+        mids[2 * g] = mids[2 * g + 1] = sorted[r.x + c / 2];
+    }
+}
+
+// ---- descent -------------------------------------------------------------------------------
+template <int METRIC>
+__device__ __forceinline__ float tsvq_dist(const float *__restrict__ xr, const float *__restrict__ c,
+                                           int dim, float na, float nb) {
+    float acc = 0.0f;
+    if constexpr (METRIC == M_COS) {
+        for (int t = 0; t < dim; ++t) {
+            float p = xr[t] * c[t];
+            acc = acc + p;
+        }
+        float den = na * nb;
+        float q = acc / den;
+        float d = 1.0f - q;
+        return (na == 0.0f || nb == 0.0f) ? 1.0f : d;
+    } else if constexpr (METRIC == M_L1) {
+        for (int t = 0; t < dim; ++t) {
+            float d = xr[t] - c[t];
+            acc = acc + fabsf(d);
+        }
+        return acc;
+    } else {
+        for (int t = 0; t < dim; ++t) {
+            float d = xr[t] - c[t];
+            float p = d * d;
+            acc = acc + p;
+        }
+        return METRIC == M_EUCLID ? sqrtf(acc) : acc;
+    }
+}
+
+// One lane = one row; walks from the root, `<=` goes left (src/tsvq.rs:171), single children are
+// followed unconditionally (177-178).  Both distances of a level are accumulated together.
+template <int METRIC>
+__global__ void __launch_bounds__(256) k_tsvq_descend(const float *__restrict__ x, int64_t n, int64_t ld,
+                                                      int dim, const float *__restrict__ cen,
+                                                      const float *__restrict__ cnorm,
+                                                      const int *__restrict__ left,
+                                                      const int *__restrict__ right,
+                                                      int *__restrict__ leaf) {
+    int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= n) return;
+    const float *__restrict__ xr = x + row * ld;
+    float na = 0.0f;
+    if constexpr (METRIC == M_COS) {
+        float sa = 0.0f;
+        for (int t = 0; t < dim; ++t) {
+            float p = xr[t] * xr[t];
+            sa = sa + p;
+        }
+        na = sqrtf(sa);
+    }
+    int node = 0;
+    for (;;) {
+        int l = left[node], r = right[node];
+        if (l >= 0 && r >= 0) {
+            const float *__restrict__ cl = cen + (size_t)l * dim;
+            const float *__restrict__ cr = cen + (size_t)r * dim;
+            float al = 0.0f, ar = 0.0f;
+            for (int t = 0; t < dim; ++t) {
+                float xv = xr[t];
+                if constexpr (METRIC == M_COS) {
+                    float pl = xv * cl[t], pr = xv * cr[t];
+                    al = al + pl;
+                    ar = ar + pr;
+                } else if constexpr (METRIC == M_L1) {
+                    float dl = xv - cl[t], dr = xv - cr[t];
+                    al = al + fabsf(dl);
+                    ar = ar + fabsf(dr);
+                } else {
+                    float dl = xv - cl[t], dr = xv - cr[t];
+                    float pl = dl * dl, pr = dr * dr;
+                    al = al + pl;
+                    ar = ar + pr;
+                }
+            }
+            float dl, dr;
+            if constexpr (METRIC == M_COS) {
+                float nl = cnorm[l], nr = cnorm[r];
+                float ql = al / (na * nl), qr = ar / (na * nr);
+                dl = (na == 0.0f || nl == 0.0f) ? 1.0f : 1.0f - ql;
+                dr = (na == 0.0f || nr == 0.0f) ? 1.0f : 1.0f - qr;
+            } else if constexpr (METRIC == M_EUCLID) {
+                dl = sqrtf(al);
+                dr = sqrtf(ar);
+            } else {
+                dl = al;
+                dr = ar;
+            }
+            node = (dl <= dr) ? l : r;
+        } else if (l >= 0) {
+            node = l;
+        } else if (r >= 0) {
+            node = r;
+        } else {
+            break;
+        }
+    }
+    leaf[row] = node;
+}
+
+// out[i][t] = f16(centroid[leaf[i]][t])   (src/tsvq.rs:242-248)
+static __global__ void __launch_bounds__(256) k_tsvq_decode_f16(const int *__restrict__ leaf, int64_t n, int dim,
+                                                         const float *__restrict__ cen,
+                                                         uint16_t *__restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n * dim) return;
+    int64_t row = i / dim;
+    int t = (int)(i % dim);
+    out[i] = __half_as_ushort(__float2half_rn(cen[(size_t)leaf[row] * dim + t]));
+}
+
+}  // namespace vq

@@ -11,129 +11,20 @@
 #include <string>
 #include <vector>
 
-#include "../../include/vq_hip.h"
+#include "ctx.hpp"
 #include "assign_exact.hpp"
 #include "lbg_update.hpp"
 
-namespace {
-
-thread_local std::string g_create_error;
-
-struct DevBuf {
-    void *p = nullptr;
-    size_t cap = 0;
-};
-
-}  // namespace
-
-struct vq_ctx {
-    int device = 0;
-    hipStream_t stream = nullptr;
-    hipEvent_t ev0 = nullptr, ev1 = nullptr;
-    std::string err;
-    // grow-only device workspace
-    DevBuf flags, tables, hist, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;
-    // optional per-kernel-class timing (HIP events on the stream)
-    bool prof_on = false;
-    std::vector<hipEvent_t> prof_pool;
-    struct Span {
-        int cls;
-        hipEvent_t a, b;
-    };
-    std::vector<Span> prof_open;
-    double prof_ms[VQ_PROF_CLASSES] = {0};
-    int64_t prof_launches[VQ_PROF_CLASSES] = {0};
-};
-
-namespace {
-
-int32_t fail(vq_ctx *ctx, int32_t code, const char *fmt, ...) {
-    char buf[512];
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(buf, sizeof buf, fmt, ap);
-    va_end(ap);
-    if (ctx)
-        ctx->err = buf;
-    else
-        g_create_error = buf;
-    return code;
-}
-
-#define VQ_HIP(ctx, call)                                                                     \
-    do {                                                                                      \
-        hipError_t e__ = (call);                                                              \
-        if (e__ != hipSuccess)                                                                \
-            return fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,            \
-                        "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__, __LINE__); \
-    } while (0)
-
-int32_t ensure(vq_ctx *ctx, DevBuf &b, size_t bytes) {
-    if (bytes <= b.cap) return VQ_OK;
-    if (b.p) {
-        VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
-        VQ_HIP(ctx, hipFree(b.p));
-        b.p = nullptr;
-        b.cap = 0;
-    }
-    size_t want = bytes + bytes / 8 + 256;
-    VQ_HIP(ctx, hipMalloc(&b.p, want));
-    b.cap = want;
-    return VQ_OK;
-}
-
-#define VQ_TRY(expr)                  \
-    do {                              \
-        int32_t rc__ = (expr);        \
-        if (rc__ != VQ_OK) return rc__; \
-    } while (0)
-
-inline unsigned cdiv(int64_t a, int64_t b) { return (unsigned)((a + b - 1) / b); }
-
-// ---- per-kernel-class timing -----------------------------------------------------------------
-hipEvent_t prof_event(vq_ctx *ctx) {
-    if (!ctx->prof_pool.empty()) {
-        hipEvent_t e = ctx->prof_pool.back();
-        ctx->prof_pool.pop_back();
-        return e;
-    }
-    hipEvent_t e = nullptr;
-    (void)hipEventCreate(&e);
+namespace vqh {
+std::string &create_error() {
+    thread_local std::string e;
     return e;
 }
+}  // namespace vqh
 
-struct ProfSpan {
-    vq_ctx *ctx;
-    int cls;
-    hipEvent_t a = nullptr;
-    ProfSpan(vq_ctx *c, int k) : ctx(c), cls(k) {
-        if (ctx->prof_on) {
-            a = prof_event(ctx);
-            (void)hipEventRecord(a, ctx->stream);
-        }
-    }
-    ~ProfSpan() {
-        if (a) {
-            hipEvent_t b = prof_event(ctx);
-            (void)hipEventRecord(b, ctx->stream);
-            ctx->prof_open.push_back({cls, a, b});
-        }
-    }
-};
+using namespace vqh;
 
-// Resolves the recorded spans; the stream must have been synchronised.
-void prof_collect(vq_ctx *ctx) {
-    for (auto &sp : ctx->prof_open) {
-        float ms = 0.f;
-        if (hipEventElapsedTime(&ms, sp.a, sp.b) == hipSuccess) {
-            ctx->prof_ms[sp.cls] += ms;
-            ctx->prof_launches[sp.cls] += 1;
-        }
-        ctx->prof_pool.push_back(sp.a);
-        ctx->prof_pool.push_back(sp.b);
-    }
-    ctx->prof_open.clear();
-}
+namespace {
 
 // ---- assignment dispatch -------------------------------------------------------------------
 
@@ -236,6 +127,9 @@ __global__ void __launch_bounds__(256) k_copy_f32(const float4 *__restrict__ src
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
 }
 
+}  // namespace
+
+namespace vqh {
 int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t m, int32_t sd,
                      int32_t k) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
@@ -252,7 +146,37 @@ int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t 
     return VQ_OK;
 }
 
-}  // namespace
+
+int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
+                  int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes) {
+    VQ_TRY(check_common(ctx, d_x, n, ld, m, sd, k));
+    if (!d_codebooks || !d_codes) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: null pointer");
+    if (reinterpret_cast<uintptr_t>(d_codes) & 3)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: d_codes must be 4-byte aligned");
+    if (m > 65535) return fail(ctx, VQ_ERR_UNSUPPORTED, "m must be at most 65535");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    vq::AssignArgs a;
+    a.x = d_x;
+    a.n = n;
+    a.ld = ld;
+    a.m = m;
+    a.k = k;
+    a.cb = d_codebooks;
+    a.cnorm = nullptr;
+    a.codes = d_codes;
+    a.changed = nullptr;
+    a.done = nullptr;
+    if (metric == VQ_COSINE) {
+        VQ_TRY(ensure(ctx, ctx->cnorm, sizeof(float) * (size_t)m * k));
+        hipLaunchKernelGGL(vq::k_centroid_norms, dim3(cdiv((int64_t)m * k, 256)), dim3(256), 0,
+                           ctx->stream, d_codebooks, (int64_t)m * k, sd, (float *)ctx->cnorm.p);
+        a.cnorm = (const float *)ctx->cnorm.p;
+    }
+    ProfSpan sp(ctx, VQ_PROF_ENCODE);
+    return launch_assign<false>(ctx, metric, a, sd);
+}
+
+}  // namespace vqh
 
 // =============================================================================================
 extern "C" {
@@ -286,7 +210,8 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
-                      &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm};
+                      &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
+                      &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     prof_collect(ctx);
@@ -298,7 +223,7 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     return VQ_OK;
 }
 
-const char *vq_last_error(const vq_ctx *ctx) { return ctx ? ctx->err.c_str() : g_create_error.c_str(); }
+const char *vq_last_error(const vq_ctx *ctx) { return ctx ? ctx->err.c_str() : vqh::create_error().c_str(); }
 
 int32_t vq_ctx_sync(vq_ctx *ctx) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
@@ -499,31 +424,7 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
 
 int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                   int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes) {
-    VQ_TRY(check_common(ctx, d_x, n, ld, m, sd, k));
-    if (!d_codebooks || !d_codes) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: null pointer");
-    if (reinterpret_cast<uintptr_t>(d_codes) & 3)
-        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: d_codes must be 4-byte aligned");
-    if (m > 65535) return fail(ctx, VQ_ERR_UNSUPPORTED, "m must be at most 65535");
-    VQ_HIP(ctx, hipSetDevice(ctx->device));
-    vq::AssignArgs a;
-    a.x = d_x;
-    a.n = n;
-    a.ld = ld;
-    a.m = m;
-    a.k = k;
-    a.cb = d_codebooks;
-    a.cnorm = nullptr;
-    a.codes = d_codes;
-    a.changed = nullptr;
-    a.done = nullptr;
-    if (metric == VQ_COSINE) {
-        VQ_TRY(ensure(ctx, ctx->cnorm, sizeof(float) * (size_t)m * k));
-        hipLaunchKernelGGL(vq::k_centroid_norms, dim3(cdiv((int64_t)m * k, 256)), dim3(256), 0,
-                           ctx->stream, d_codebooks, (int64_t)m * k, sd, (float *)ctx->cnorm.p);
-        a.cnorm = (const float *)ctx->cnorm.p;
-    }
-    ProfSpan sp(ctx, VQ_PROF_ENCODE);
-    return launch_assign<false>(ctx, metric, a, sd);
+    return vqh::assign_codes(ctx, metric, d_x, n, ld, m, sd, k, d_codebooks, d_codes);
 }
 
 int32_t vq_decode_f16(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sd, int32_t k,

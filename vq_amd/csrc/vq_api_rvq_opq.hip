@@ -1,0 +1,132 @@
+// libvqhip — entry points around the assignment for ResidualQuantizer and
+// OptimizedProductQuantizer (declared in include/vq_hip.h).
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <algorithm>
+#include <vector>
+
+#include "ctx.hpp"
+#include "rvq_opq.hpp"
+
+using namespace vqh;
+
+extern "C" {
+
+int32_t vq_residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
+                        const float *d_codebook, const uint8_t *d_codes) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return VQ_OK;
+    if (!d_res || !d_codebook || !d_codes || n < 0 || dim <= 0 || ld < dim || k <= 0 || k > 256)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipLaunchKernelGGL(vq::k_residual_sub, dim3(cdiv(n * dim, 256)), dim3(256), 0, ctx->stream, d_res, n,
+                       ld, dim, d_codebook, d_codes, 1);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+int32_t vq_mean_l2norm(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, float *h_out) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return fail(ctx, VQ_ERR_EMPTY_INPUT, "Empty input: at least one vector is required.");
+    if (!d_x || !h_out || n < 0 || dim <= 0 || ld < dim) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    const int64_t per_block = 4096;
+    const int blocks = (int)cdiv(n, per_block);
+    VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(float) * (size_t)n));
+    VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * ((size_t)blocks + 1)));
+    float *norms = (float *)ctx->tmp_a.p;
+    double *part = (double *)ctx->tmp_b.p;
+    hipLaunchKernelGGL(vq::k_row_norms, dim3(cdiv(n, 256)), dim3(256), 0, ctx->stream, d_x, n, ld, dim, norms);
+    hipLaunchKernelGGL(vq::k_sum_f64, dim3(blocks), dim3(256), 0, ctx->stream, norms,
+                       (const double *)nullptr, n, per_block, part);
+    hipLaunchKernelGGL(vq::k_sum_f64, dim3(1), dim3(256), 0, ctx->stream, (const float *)nullptr, part,
+                       (int64_t)blocks, (int64_t)blocks, part + blocks);
+    VQ_HIP(ctx, hipGetLastError());
+    double total = 0.0;
+    VQ_HIP(ctx, hipMemcpyAsync(&total, part + blocks, sizeof(double), hipMemcpyDeviceToHost, ctx->stream));
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    *h_out = (float)total / (float)n;  // src/rvq.rs:137-138
+    return VQ_OK;
+}
+
+int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t dim,
+                      int32_t stages, int32_t k, const float *d_codebooks, float epsilon, uint8_t *d_codes,
+                      uint8_t *d_stages_used, uint16_t *d_recon_f16) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return VQ_OK;
+    if (!d_x || !d_codebooks || !d_codes || n < 0 || dim <= 0 || ld < dim || stages < 0 || k <= 0 || k > 256)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(float) * (size_t)n * dim));   // residual
+    VQ_TRY(ensure(ctx, ctx->tmp_d, sizeof(float) * (size_t)n * dim));   // running sum
+    VQ_TRY(ensure(ctx, ctx->tmp_e, (size_t)n * 3 + 16));                // stage codes, active, used
+    float *res = (float *)ctx->tmp_c.p;
+    float *sum = (float *)ctx->tmp_d.p;
+    uint8_t *stage_codes = (uint8_t *)ctx->tmp_e.p;
+    uint8_t *active = stage_codes + ((n + 3) & ~(int64_t)3);
+    uint8_t *used = active + n;
+    VQ_HIP(ctx, hipMemcpy2DAsync(res, sizeof(float) * dim, d_x, sizeof(float) * ld, sizeof(float) * dim,
+                                 (size_t)n, hipMemcpyDeviceToDevice, st));
+    hipLaunchKernelGGL(vq::k_fill_f32, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, sum, n * dim, 0.0f);
+    hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, active, n, (uint8_t)1);
+    hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, used, n, (uint8_t)0);
+    for (int s = 0; s < stages; ++s) {
+        const float *cb = d_codebooks + (size_t)s * k * dim;
+        if (k < 2)  // src/rvq.rs:186-187
+            hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, stage_codes, n, (uint8_t)0);
+        else
+            VQ_TRY(assign_codes(ctx, metric, res, n, dim, 1, dim, k, cb, stage_codes));
+        hipLaunchKernelGGL(vq::k_rvq_stage_apply, dim3(cdiv(n, 256)), dim3(256), 0, st, res, sum, n, dim, cb,
+                           stage_codes, d_codes, stages, s, active, used, epsilon);
+    }
+    if (d_stages_used)
+        VQ_HIP(ctx, hipMemcpyAsync(d_stages_used, used, (size_t)n, hipMemcpyDeviceToDevice, st));
+    if (d_recon_f16)
+        hipLaunchKernelGGL(vq::k_f32_to_f16, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, sum, n * dim,
+                           d_recon_f16);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+int32_t vq_rotate(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, const float *d_R,
+                  float *d_y) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return VQ_OK;
+    if (!d_x || !d_R || !d_y || n < 0 || dim <= 0 || ld < dim) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    size_t lds = sizeof(float) * 64 * ((size_t)dim + 1);
+    if (lds > 160 * 1024) return fail(ctx, VQ_ERR_UNSUPPORTED, "rotation: dim %d too large", dim);
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    if (lds > 48 * 1024)
+        VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(vq::k_rotate_generic),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(vq::k_rotate_generic, dim3(cdiv(n, 64)), dim3(256), lds, ctx->stream, d_x, n, ld,
+                       dim, d_R, d_y);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n, int32_t dim, double *h_A) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return fail(ctx, VQ_ERR_EMPTY_INPUT, "Empty input: at least one vector is required.");
+    if (!d_y || !d_x || !h_A || n < 0 || dim <= 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    if (dim > 128) return fail(ctx, VQ_ERR_UNSUPPORTED, "cross-covariance: dim %d > 128", dim);
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    const int64_t rows_per_chunk = 2048;
+    const int chunks = (int)cdiv(n, rows_per_chunk);
+    const int total = dim * dim;
+    VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(double) * (size_t)chunks * total));
+    VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * (size_t)total));
+    size_t lds = sizeof(float) * 2 * 32 * (size_t)dim;
+    hipLaunchKernelGGL(vq::k_crosscov_partial, dim3(chunks), dim3(256), lds, ctx->stream, d_y, d_x, n, dim,
+                       rows_per_chunk, (double *)ctx->tmp_a.p);
+    hipLaunchKernelGGL(vq::k_crosscov_reduce, dim3(cdiv(total, 256)), dim3(256), 0, ctx->stream,
+                       (const double *)ctx->tmp_a.p, chunks, total, (double *)ctx->tmp_b.p);
+    VQ_HIP(ctx, hipGetLastError());
+    VQ_HIP(ctx, hipMemcpyAsync(h_A, ctx->tmp_b.p, sizeof(double) * total, hipMemcpyDeviceToHost, ctx->stream));
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return VQ_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,433 @@
+// libvqhip — tree-structured VQ entry points: build (TSVQNode::fit, src/tsvq.rs:71-148) and
+// descent encode (src/tsvq.rs:162-181,231-249).
+#include <cstring>
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <rocprim/rocprim.hpp>
+
+#include <algorithm>
+#include <vector>
+
+#include "ctx.hpp"
+#include "assign_exact.hpp"
+#include "tsvq.hpp"
+
+using namespace vqh;
+
+// Nodes are numbered breadth-first: the root is 0; children are appended level by level, left
+// before right.  left/right hold -1 for "no child".
+struct vq_tree {
+    int device = 0;
+    int32_t n_nodes = 0;
+    int32_t dim = 0;
+    std::vector<float> h_centroids;
+    std::vector<int32_t> h_left, h_right, h_split_dim;
+    std::vector<float> h_split_val;
+    std::vector<int64_t> h_count;
+    float *d_centroids = nullptr, *d_cnorm = nullptr;
+    int32_t *d_left = nullptr, *d_right = nullptr;
+};
+
+namespace {
+
+constexpr int kLeafMaxRows = 1024;  // PARALLEL_THRESHOLD, src/vector.rs:16
+
+int tree_depth(uint64_t count) {
+    int d = 0;
+    while (count > ((uint64_t)kLeafMaxRows << d)) ++d;
+    return d;
+}
+
+struct Seg {
+    int32_t node;
+    uint32_t lo, hi;
+};
+
+int32_t tree_to_device(vq_ctx *ctx, vq_tree *t) {
+    size_t nn = (size_t)t->n_nodes, dim = (size_t)t->dim;
+    VQ_HIP(ctx, hipMalloc(&t->d_centroids, sizeof(float) * nn * dim));
+    VQ_HIP(ctx, hipMalloc(&t->d_cnorm, sizeof(float) * nn));
+    VQ_HIP(ctx, hipMalloc(&t->d_left, sizeof(int32_t) * nn));
+    VQ_HIP(ctx, hipMalloc(&t->d_right, sizeof(int32_t) * nn));
+    hipStream_t st = ctx->stream;
+    VQ_HIP(ctx, hipMemcpyAsync(t->d_centroids, t->h_centroids.data(), sizeof(float) * nn * dim,
+                               hipMemcpyHostToDevice, st));
+    VQ_HIP(ctx, hipMemcpyAsync(t->d_left, t->h_left.data(), sizeof(int32_t) * nn, hipMemcpyHostToDevice, st));
+    VQ_HIP(ctx, hipMemcpyAsync(t->d_right, t->h_right.data(), sizeof(int32_t) * nn, hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL(vq::k_centroid_norms, dim3(cdiv((int64_t)nn, 256)), dim3(256), 0, st, t->d_centroids,
+                       (int64_t)nn, (int)dim, t->d_cnorm);
+    VQ_HIP(ctx, hipGetLastError());
+    VQ_HIP(ctx, hipStreamSynchronize(st));
+    return VQ_OK;
+}
+
+void tree_release(vq_tree *t) {
+    if (!t) return;
+    (void)hipFree(t->d_centroids);
+    (void)hipFree(t->d_cnorm);
+    (void)hipFree(t->d_left);
+    (void)hipFree(t->d_right);
+    delete t;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, int32_t max_depth,
+                      vq_tree **out) {
+    if (!ctx || !out) return VQ_ERR_INVALID_ARG;
+    *out = nullptr;
+    if (n == 0) return fail(ctx, VQ_ERR_EMPTY_INPUT, "Empty input: at least one vector is required.");
+    if (!d_x || n < 0 || dim <= 0 || ld < dim || max_depth < 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    if (n >= (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n must be below 2^31");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+
+    // workspace: two row-id lists, column values (+sorted), flags, scan
+    VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(uint32_t) * (size_t)n));
+    VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(uint32_t) * (size_t)n));
+    VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(float) * (size_t)n));
+    VQ_TRY(ensure(ctx, ctx->tmp_d, sizeof(float) * (size_t)n));
+    VQ_TRY(ensure(ctx, ctx->tmp_e, sizeof(uint32_t) * (size_t)n));
+    VQ_TRY(ensure(ctx, ctx->tmp_f, sizeof(uint32_t) * (size_t)n));
+    uint32_t *perm = (uint32_t *)ctx->tmp_a.p, *perm2 = (uint32_t *)ctx->tmp_b.p;
+    float *vals = (float *)ctx->tmp_c.p, *sorted = (float *)ctx->tmp_d.p;
+    uint32_t *flags = (uint32_t *)ctx->tmp_e.p, *scan = (uint32_t *)ctx->tmp_f.p;
+    hipLaunchKernelGGL(vq::k_iota_u32, dim3(cdiv(n, 256)), dim3(256), 0, st, perm, n);
+
+    vq_tree *T = new vq_tree;
+    T->device = ctx->device;
+    T->dim = dim;
+    std::vector<Seg> level{{0, 0u, (uint32_t)n}};
+    T->h_left.push_back(-1);
+    T->h_right.push_back(-1);
+    T->h_split_dim.push_back(-1);
+    T->h_split_val.push_back(0.f);
+    T->h_count.push_back(n);
+    int depth_left = max_depth;
+
+    // small per-level device tables, re-allocated per level (a level has at most 2^level nodes)
+    auto cleanup_fail = [&](int32_t rc) {
+        tree_release(T);
+        return rc;
+    };
+    void *rp_tmp = nullptr;
+    size_t rp_cap = 0;
+    int32_t rc = VQ_OK;
+
+    while (!level.empty()) {
+        const int nseg = (int)level.size();
+        // ---- means of every node of the level ------------------------------------------------
+        std::vector<uint2> desc;
+        std::vector<uint4> info(nseg);
+        for (int g = 0; g < nseg; ++g) {
+            uint32_t cnt = level[g].hi - level[g].lo;
+            int dep = tree_depth(cnt);
+            info[g] = make_uint4((uint32_t)desc.size(), (uint32_t)dep, cnt, 0u);
+            for (uint32_t l = 0; l < (1u << dep); ++l) {
+                uint32_t lo = 0, hi = cnt;
+                for (int bit = dep - 1; bit >= 0; --bit) {
+                    uint32_t mid = lo + (hi - lo) / 2;
+                    if ((l >> bit) & 1u)
+                        lo = mid;
+                    else
+                        hi = mid;
+                }
+                desc.push_back(make_uint2(level[g].lo + lo, level[g].lo + hi));
+            }
+        }
+        const size_t nleaves = desc.size();
+        void *d_desc = nullptr, *d_info = nullptr, *d_lsum = nullptr, *d_means = nullptr;
+        auto free_level = [&]() {
+            (void)hipFree(d_desc);
+            (void)hipFree(d_info);
+            (void)hipFree(d_lsum);
+            (void)hipFree(d_means);
+        };
+#define LV_HIP(call)                                                                              \
+    do {                                                                                          \
+        hipError_t e__ = (call);                                                                  \
+        if (e__ != hipSuccess) {                                                                  \
+            free_level();                                                                         \
+            (void)hipFree(rp_tmp);                                                                \
+            return cleanup_fail(fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,   \
+                                     "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__,   \
+                                     __LINE__));                                                  \
+        }                                                                                         \
+    } while (0)
+        LV_HIP(hipMalloc(&d_desc, sizeof(uint2) * nleaves));
+        LV_HIP(hipMalloc(&d_info, sizeof(uint4) * nseg));
+        LV_HIP(hipMalloc(&d_lsum, sizeof(float) * nleaves * dim));
+        LV_HIP(hipMalloc(&d_means, sizeof(float) * (size_t)nseg * dim));
+        LV_HIP(hipMemcpyAsync(d_desc, desc.data(), sizeof(uint2) * nleaves, hipMemcpyHostToDevice, st));
+        LV_HIP(hipMemcpyAsync(d_info, info.data(), sizeof(uint4) * nseg, hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(vq::k_seg_leafsum, dim3(cdiv((int64_t)nleaves * dim, 256)), dim3(256), 0, st, perm,
+                           (const uint2 *)d_desc, (int64_t)nleaves, d_x, ld, dim, (float *)d_lsum);
+        hipLaunchKernelGGL(vq::k_seg_mean, dim3(cdiv((int64_t)nseg * dim, 256)), dim3(256), 0, st,
+                           (float *)d_lsum, (const uint4 *)d_info, nseg, dim, (float *)d_means, (int64_t)0);
+        LV_HIP(hipGetLastError());
+        const int32_t first_node = level[0].node;
+        T->h_centroids.resize((size_t)(first_node + nseg) * dim);
+        LV_HIP(hipMemcpyAsync(T->h_centroids.data() + (size_t)first_node * dim, d_means,
+                              sizeof(float) * (size_t)nseg * dim, hipMemcpyDeviceToHost, st));
+        LV_HIP(hipStreamSynchronize(st));
+
+        // ---- which nodes split (src/tsvq.rs:78) ---------------------------------------------
+        std::vector<int> split;  // indices into level
+        if (depth_left > 0)
+            for (int g = 0; g < nseg; ++g)
+                if (level[g].hi - level[g].lo > 1) split.push_back(g);
+        if (split.empty()) {
+            free_level();
+            break;
+        }
+        const int ns = (int)split.size();
+        std::vector<uint2> range(ns);
+        for (int i = 0; i < ns; ++i) range[i] = make_uint2(level[split[i]].lo, level[split[i]].hi);
+        // means of the splitting nodes, compacted
+        std::vector<float> smeans((size_t)ns * dim);
+        for (int i = 0; i < ns; ++i)
+            std::copy_n(T->h_centroids.data() + (size_t)level[split[i]].node * dim, dim,
+                        smeans.data() + (size_t)i * dim);
+        void *d_range = nullptr, *d_smeans = nullptr, *d_var = nullptr, *d_sdim = nullptr, *d_mids = nullptr,
+             *d_median = nullptr, *d_nleft = nullptr, *d_begin = nullptr, *d_end = nullptr;
+        auto free_split = [&]() {
+            (void)hipFree(d_range);
+            (void)hipFree(d_smeans);
+            (void)hipFree(d_var);
+            (void)hipFree(d_sdim);
+            (void)hipFree(d_mids);
+            (void)hipFree(d_median);
+            (void)hipFree(d_nleft);
+            (void)hipFree(d_begin);
+            (void)hipFree(d_end);
+        };
+#define SP_HIP(call)                                                                              \
+    do {                                                                                          \
+        hipError_t e__ = (call);                                                                  \
+        if (e__ != hipSuccess) {                                                                  \
+            free_split();                                                                         \
+            free_level();                                                                         \
+            (void)hipFree(rp_tmp);                                                                \
+            return cleanup_fail(fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,   \
+                                     "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__,   \
+                                     __LINE__));                                                  \
+        }                                                                                         \
+    } while (0)
+        SP_HIP(hipMalloc(&d_range, sizeof(uint2) * ns));
+        SP_HIP(hipMalloc(&d_smeans, sizeof(float) * (size_t)ns * dim));
+        SP_HIP(hipMalloc(&d_var, sizeof(float) * (size_t)ns * dim));
+        SP_HIP(hipMalloc(&d_sdim, sizeof(int) * ns));
+        SP_HIP(hipMalloc(&d_mids, sizeof(float) * 2 * ns));
+        SP_HIP(hipMalloc(&d_median, sizeof(float) * ns));
+        SP_HIP(hipMalloc(&d_nleft, sizeof(uint32_t) * ns));
+        SP_HIP(hipMalloc(&d_begin, sizeof(uint32_t) * ns));
+        SP_HIP(hipMalloc(&d_end, sizeof(uint32_t) * ns));
+        SP_HIP(hipMemcpyAsync(d_range, range.data(), sizeof(uint2) * ns, hipMemcpyHostToDevice, st));
+        SP_HIP(hipMemcpyAsync(d_smeans, smeans.data(), sizeof(float) * (size_t)ns * dim, hipMemcpyHostToDevice, st));
+        // per-dimension sums of squared deviations (src/tsvq.rs:88-99)
+        hipLaunchKernelGGL(vq::k_seg_variance, dim3(cdiv((int64_t)ns * dim, 64)), dim3(64), 0, st, perm,
+                           (const uint2 *)d_range, ns, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
+                           (float *)d_var);
+        SP_HIP(hipGetLastError());
+        std::vector<float> var((size_t)ns * dim);
+        SP_HIP(hipMemcpyAsync(var.data(), d_var, sizeof(float) * (size_t)ns * dim, hipMemcpyDeviceToHost, st));
+        SP_HIP(hipStreamSynchronize(st));
+        // argmax with the LAST maximal element winning (Iterator::max_by, src/tsvq.rs:102-106)
+        std::vector<int> sdim(ns);
+        for (int i = 0; i < ns; ++i) {
+            const float *v = var.data() + (size_t)i * dim;
+            int best = 0;
+            for (int t = 1; t < dim; ++t)
+                if (!(v[t] < v[best])) best = t;
+            sdim[i] = best;
+        }
+        SP_HIP(hipMemcpyAsync(d_sdim, sdim.data(), sizeof(int) * ns, hipMemcpyHostToDevice, st));
+        // split column, segmented sort, middle values (src/tsvq.rs:109-117)
+        hipLaunchKernelGGL(vq::k_seg_gather_col, dim3(cdiv(n, 256)), dim3(256), 0, st, perm, n,
+                           (const uint2 *)d_range, ns, (const int *)d_sdim, d_x, ld, vals);
+        std::vector<uint32_t> begin(ns), end(ns);
+        for (int i = 0; i < ns; ++i) {
+            begin[i] = range[i].x;
+            end[i] = range[i].y;
+        }
+        SP_HIP(hipMemcpyAsync(d_begin, begin.data(), sizeof(uint32_t) * ns, hipMemcpyHostToDevice, st));
+        SP_HIP(hipMemcpyAsync(d_end, end.data(), sizeof(uint32_t) * ns, hipMemcpyHostToDevice, st));
+        size_t need = 0;
+        SP_HIP(rocprim::segmented_radix_sort_keys(nullptr, need, vals, sorted, (unsigned)n, (unsigned)ns,
+                                                  (const uint32_t *)d_begin, (const uint32_t *)d_end, 0, 32, st));
+        if (need > rp_cap) {
+            (void)hipFree(rp_tmp);
+            rp_tmp = nullptr;
+            SP_HIP(hipMalloc(&rp_tmp, need));
+            rp_cap = need;
+        }
+        SP_HIP(rocprim::segmented_radix_sort_keys(rp_tmp, need, vals, sorted, (unsigned)n, (unsigned)ns,
+                                                  (const uint32_t *)d_begin, (const uint32_t *)d_end, 0, 32, st));
+        hipLaunchKernelGGL(vq::k_seg_middles, dim3(cdiv(ns, 64)), dim3(64), 0, st, sorted,
+                           (const uint2 *)d_range, ns, (float *)d_mids);
+        SP_HIP(hipGetLastError());
+        std::vector<float> mids(2 * (size_t)ns), median(ns);
+        SP_HIP(hipMemcpyAsync(mids.data(), d_mids, sizeof(float) * 2 * ns, hipMemcpyDeviceToHost, st));
+        SP_HIP(hipStreamSynchronize(st));
+        for (int i = 0; i < ns; ++i) {
+            uint32_t cnt = range[i].y - range[i].x;
+            if (cnt % 2 == 0) {
+                volatile float s = mids[2 * i] + mids[2 * i + 1];  // f32 add, then f32 divide
+                median[i] = s / 2.0f;
+            } else {
+                median[i] = mids[2 * i];
+            }
+        }
+        SP_HIP(hipMemcpyAsync(d_median, median.data(), sizeof(float) * ns, hipMemcpyHostToDevice, st));
+        // stable partition by `<= median` (src/tsvq.rs:120-123)
+        hipLaunchKernelGGL(vq::k_seg_flags, dim3(cdiv(n, 256)), dim3(256), 0, st, vals, n, (const uint2 *)d_range,
+                           ns, (const float *)d_median, flags);
+        need = 0;
+        SP_HIP(rocprim::exclusive_scan(nullptr, need, flags, scan, 0u, (size_t)n, rocprim::plus<uint32_t>(), st));
+        if (need > rp_cap) {
+            (void)hipFree(rp_tmp);
+            rp_tmp = nullptr;
+            SP_HIP(hipMalloc(&rp_tmp, need));
+            rp_cap = need;
+        }
+        SP_HIP(rocprim::exclusive_scan(rp_tmp, need, flags, scan, 0u, (size_t)n, rocprim::plus<uint32_t>(), st));
+        hipLaunchKernelGGL(vq::k_seg_partition, dim3(cdiv(n, 256)), dim3(256), 0, st, perm, n,
+                           (const uint2 *)d_range, ns, flags, scan, perm2, (uint32_t *)d_nleft);
+        SP_HIP(hipGetLastError());
+        std::vector<uint32_t> nleft(ns);
+        SP_HIP(hipMemcpyAsync(nleft.data(), d_nleft, sizeof(uint32_t) * ns, hipMemcpyDeviceToHost, st));
+        SP_HIP(hipStreamSynchronize(st));
+        free_split();
+        free_level();
+        std::swap(perm, perm2);
+
+        // ---- children (src/tsvq.rs:126-141) ---------------------------------------------------
+        std::vector<Seg> next;
+        for (int i = 0; i < ns; ++i) {
+            const Seg &sg = level[split[i]];
+            uint32_t cnt = sg.hi - sg.lo, nl = nleft[i], nr = cnt - nl;
+            T->h_split_dim[sg.node] = sdim[i];
+            T->h_split_val[sg.node] = median[i];
+            auto add_child = [&](uint32_t lo, uint32_t hi) {
+                int32_t id = (int32_t)T->h_left.size();
+                T->h_left.push_back(-1);
+                T->h_right.push_back(-1);
+                T->h_split_dim.push_back(-1);
+                T->h_split_val.push_back(0.f);
+                T->h_count.push_back((int64_t)hi - lo);
+                next.push_back({id, lo, hi});
+                return id;
+            };
+            if (nl > 0 && nl < cnt) T->h_left[sg.node] = add_child(sg.lo, sg.lo + nl);
+            if (nr > 0 && nr < cnt) T->h_right[sg.node] = add_child(sg.lo + nl, sg.hi);
+        }
+        level.swap(next);
+        --depth_left;
+    }
+#undef LV_HIP
+#undef SP_HIP
+    (void)hipFree(rp_tmp);
+    T->n_nodes = (int32_t)T->h_left.size();
+    rc = tree_to_device(ctx, T);
+    if (rc != VQ_OK) return cleanup_fail(rc);
+    *out = T;
+    return VQ_OK;
+}
+
+int32_t vq_tree_create(vq_ctx *ctx, int32_t n_nodes, int32_t dim, const float *h_centroids,
+                       const int32_t *h_left, const int32_t *h_right, vq_tree **out) {
+    if (!ctx || !out) return VQ_ERR_INVALID_ARG;
+    *out = nullptr;
+    if (n_nodes <= 0 || dim <= 0 || !h_centroids || !h_left || !h_right)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    for (int i = 0; i < n_nodes; ++i)
+        if (h_left[i] < -1 || h_left[i] >= n_nodes || h_right[i] < -1 || h_right[i] >= n_nodes ||
+            (h_left[i] >= 0 && h_left[i] <= i) || (h_right[i] >= 0 && h_right[i] <= i))
+            return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: child index of node %d (children must have larger indices)", i);
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    vq_tree *T = new vq_tree;
+    T->device = ctx->device;
+    T->n_nodes = n_nodes;
+    T->dim = dim;
+    T->h_centroids.assign(h_centroids, h_centroids + (size_t)n_nodes * dim);
+    T->h_left.assign(h_left, h_left + n_nodes);
+    T->h_right.assign(h_right, h_right + n_nodes);
+    T->h_split_dim.assign(n_nodes, -1);
+    T->h_split_val.assign(n_nodes, 0.f);
+    T->h_count.assign(n_nodes, 0);
+    int32_t rc = tree_to_device(ctx, T);
+    if (rc != VQ_OK) {
+        tree_release(T);
+        return rc;
+    }
+    *out = T;
+    return VQ_OK;
+}
+
+int32_t vq_tree_free(vq_ctx *ctx, vq_tree *tree) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (!tree) return VQ_OK;
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    tree_release(tree);
+    return VQ_OK;
+}
+
+int32_t vq_tree_info(const vq_tree *tree, int32_t *n_nodes, int32_t *dim) {
+    if (!tree) return VQ_ERR_INVALID_ARG;
+    if (n_nodes) *n_nodes = tree->n_nodes;
+    if (dim) *dim = tree->dim;
+    return VQ_OK;
+}
+
+int32_t vq_tree_download(const vq_tree *tree, float *h_centroids, int32_t *h_left, int32_t *h_right,
+                         int32_t *h_split_dim, float *h_split_val, int64_t *h_count) {
+    if (!tree) return VQ_ERR_INVALID_ARG;
+    size_t nn = (size_t)tree->n_nodes;
+    if (h_centroids) std::copy(tree->h_centroids.begin(), tree->h_centroids.end(), h_centroids);
+    if (h_left) std::copy_n(tree->h_left.begin(), nn, h_left);
+    if (h_right) std::copy_n(tree->h_right.begin(), nn, h_right);
+    if (h_split_dim) std::copy_n(tree->h_split_dim.begin(), nn, h_split_dim);
+    if (h_split_val) std::copy_n(tree->h_split_val.begin(), nn, h_split_val);
+    if (h_count) std::copy_n(tree->h_count.begin(), nn, h_count);
+    return VQ_OK;
+}
+
+int32_t vq_tsvq_descend(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld,
+                        const vq_tree *tree, int32_t *d_leaf) {
+    if (!ctx || !tree) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return VQ_OK;
+    if (!d_x || !d_leaf || n < 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    if (ld < tree->dim)
+        return fail(ctx, VQ_ERR_DIM_MISMATCH, "Dimension mismatch: expected %d, got %lld", tree->dim, (long long)ld);
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    dim3 grid(cdiv(n, 256)), block(256);
+#define DESC(M)                                                                                       \
+    hipLaunchKernelGGL((vq::k_tsvq_descend<M>), grid, block, 0, ctx->stream, d_x, n, ld, tree->dim,   \
+                       tree->d_centroids, tree->d_cnorm, tree->d_left, tree->d_right, d_leaf)
+    switch (metric) {
+    case VQ_SQEUCLIDEAN: DESC(vq::M_SQ); break;
+    case VQ_EUCLIDEAN: DESC(vq::M_EUCLID); break;
+    case VQ_COSINE: DESC(vq::M_COS); break;
+    case VQ_MANHATTAN: DESC(vq::M_L1); break;
+    default: return fail(ctx, VQ_ERR_UNSUPPORTED, "metric %d has no kernel", metric);
+    }
+#undef DESC
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+int32_t vq_tsvq_decode_f16(vq_ctx *ctx, const vq_tree *tree, const int32_t *d_leaf, int64_t n, uint16_t *d_out) {
+    if (!ctx || !tree) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return VQ_OK;
+    if (!d_leaf || !d_out || n < 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipLaunchKernelGGL(vq::k_tsvq_decode_f16, dim3(cdiv(n * tree->dim, 256)), dim3(256), 0, ctx->stream, d_leaf,
+                       n, tree->dim, tree->d_centroids, d_out);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+}  // extern "C"
