@@ -1,0 +1,175 @@
+"""The reference's own tests, restated against the host classes that mirror its API
+(tests/test_pq.rs, test_opq.rs, test_rvq.rs, test_tsvq.rs, src/utils.rs:111-161), plus parity
+of the same calls with the CPU oracle when the index streams are passed explicitly."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from tests import data
+from tests.test_gpu_tsvq import bfs_order
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+@pytest.fixture(scope="module")
+def vq():
+    from vq_amd import api
+    return api
+
+
+def generate_test_data(n, dim):  # tests/utils.rs:16-25 (own generator: rand is not available)
+    return np.random.default_rng(42).uniform(-1000.0, 1000.0, (n, dim)).astype(F)
+
+
+# ---- src/utils.rs tests ------------------------------------------------------------------------
+def test_lbg_quantize_basic_functionality(vq):
+    d = np.array([[1, 2], [2, 3], [3, 4], [4, 5]], F)
+    assert vq.lbg_quantize(d, 2, 10, 42).shape == (2, 2)
+    assert vq.lbg_quantize(d, 2, 100, 42).shape == (2, 2)
+
+
+def test_lbg_quantize_k_zero(vq):
+    with pytest.raises(vq.VqError, match="k must be greater than 0"):
+        vq.lbg_quantize(np.array([[1, 2], [2, 3]], F), 0, 10, 42)
+
+
+def test_lbg_quantize_not_enough_data_points(vq):
+    with pytest.raises(vq.VqError, match="Not enough data points for k clusters"):
+        vq.lbg_quantize(np.array([[1, 2]], F), 2, 10, 42)
+
+
+def test_lbg_quantize_single_data_point(vq):
+    c = vq.lbg_quantize(np.array([[1, 2]], F), 1, 10, 42)
+    assert np.array_equal(c, np.array([[1, 2]], F))
+
+
+# ---- tests/test_pq.rs ----------------------------------------------------------------------------
+def test_pq_on_random_vectors(vq):
+    training = generate_test_data(1000, 10)
+    pq = vq.ProductQuantizer.fit(training, 2, 2, 50, vq.Distance.SquaredEuclidean, 42)
+    for v in training[:50]:
+        q = pq.quantize(v)
+        assert len(q) == len(v)
+        assert np.isfinite(np.abs(v - q.astype(F)).sum())
+    qb = pq.quantize_batch(training)
+    assert qb.shape == training.shape and np.isfinite(np.abs(training - qb.astype(F)).sum())
+    assert np.array_equal(qb[:50], np.stack([pq.quantize(v) for v in training[:50]]))
+
+
+def test_pq_panics(vq):
+    x = generate_test_data(20, 10)
+    with pytest.raises(vq.VqError, match="Empty input"):
+        vq.ProductQuantizer.fit(np.zeros((0, 10), F), 2, 2, 5, vq.Distance.Euclidean, 1)
+    with pytest.raises(vq.VqError, match="Data dimension must be at least m"):
+        vq.ProductQuantizer.fit(x, 11, 2, 5, vq.Distance.Euclidean, 1)
+    with pytest.raises(vq.VqError, match="Data dimension must be divisible by m"):
+        vq.ProductQuantizer.fit(x, 3, 2, 5, vq.Distance.Euclidean, 1)
+    pq = vq.ProductQuantizer.fit(x, 2, 2, 5, vq.Distance.Euclidean, 1)
+    with pytest.raises(vq.VqError, match="Dimension mismatch: expected 10, got 9"):
+        pq.quantize(x[0, :9])
+    with pytest.raises(vq.VqError, match="Invalid metric parameter for Chebyshev"):
+        vq.ProductQuantizer.fit(x, 2, 2, 5, vq.Distance.Chebyshev, 1).quantize(x[0])
+
+
+def test_pq_matches_oracle_with_explicit_streams(vq):
+    x = data.uniform(3000, 32, 7)
+    m, k, iters = 4, 64, 8
+    streams = data.index_streams(3000, m, k, iters, seed=9)
+    pq = vq.ProductQuantizer.fit(x, m, k, iters, vq.Distance.Euclidean, 42, streams=streams)
+    want = O.pq_fit_encode(O.EUCLIDEAN, x, m, k, iters, *streams)
+    assert np.array_equal(pq.codebooks(), want["codebooks"])
+    assert np.array_equal(pq.encode(x), want["codes"].astype(np.uint8))
+    assert np.array_equal(pq.quantize_batch(x).view(np.uint16),
+                          O.pq_decode_f16(want["codes"], want["codebooks"]))
+    # seeded fit without streams: deterministic in the seed, different seeds differ
+    a = vq.ProductQuantizer.fit(x, m, k, iters, vq.Distance.Euclidean, 42).codebooks()
+    b = vq.ProductQuantizer.fit(x, m, k, iters, vq.Distance.Euclidean, 42).codebooks()
+    c = vq.ProductQuantizer.fit(x, m, k, iters, vq.Distance.Euclidean, 43).codebooks()
+    assert np.array_equal(a, b) and not np.array_equal(a, c)
+
+
+# ---- tests/test_opq.rs ---------------------------------------------------------------------------
+def test_opq_on_random_vectors(vq):
+    training = generate_test_data(1000, 10)
+    opq = vq.OptimizedProductQuantizer.fit(training, 2, 2, 50, 5, vq.Distance.SquaredEuclidean, 42)
+    qb = opq.quantize_batch(training)
+    assert qb.shape == training.shape and np.isfinite(np.abs(training - qb.astype(F)).sum())
+    q = opq.quantize(training[3])
+    assert len(q) == 10 and np.array_equal(q, qb[3])
+    R = opq.rotation().astype(np.float64)
+    assert np.allclose(R.T @ R, np.eye(10), atol=1e-5)
+    with pytest.raises(vq.VqError, match="Dimension must be divisible by m"):
+        vq.OptimizedProductQuantizer.fit(training, 3, 2, 5, 2, vq.Distance.Euclidean, 1)
+
+
+def test_opq_first_outer_iteration_matches_oracle(vq):
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((2000, 16)) @ rng.standard_normal((16, 16))).astype(F)
+    m, k, iters = 4, 16, 6
+    streams = data.index_streams(2000, m, k, iters, seed=4)
+    got = vq.OptimizedProductQuantizer.fit(x, m, k, iters, 1, vq.Distance.Euclidean, 0, streams=streams)
+    want = O.opq_fit(O.EUCLIDEAN, x, m, k, iters, 1, *streams)
+    # codebooks of the first outer iteration are trained on un-rotated data: bit-exact
+    assert np.array_equal(got.codebooks(), want["codebooks"])
+    # the rotation goes through a host SVD in both: equal to f32 rounding
+    assert np.allclose(got.rotation(), want["rotation"], atol=2e-6)
+    # three outer iterations: same reconstruction quality as the oracle's run (1e-3 relative)
+    got3 = vq.OptimizedProductQuantizer.fit(x, m, k, iters, 3, vq.Distance.Euclidean, 0, streams=streams)
+    want3 = O.opq_fit(O.EUCLIDEAN, x, m, k, iters, 3, *streams)
+
+    def mse(R, cb, codes):
+        y = x.astype(np.float64) @ R.astype(np.float64).T
+        rec = np.concatenate([cb[s][codes[:, s]] for s in range(m)], 1)
+        return ((y - rec) ** 2).mean()
+    e_got = mse(got3.rotation(), got3.codebooks(), got3.encode(x))
+    e_want = mse(want3["rotation"], want3["codebooks"],
+                 O.opq_encode(O.EUCLIDEAN, x, want3["rotation"], want3["codebooks"]))
+    assert abs(e_got - e_want) <= 0.02 * e_want
+
+
+# ---- tests/test_rvq.rs ---------------------------------------------------------------------------
+def test_rvq_on_random_vectors(vq):
+    training = generate_test_data(1000, 10)
+    rvq = vq.ResidualQuantizer.fit(training, 2, 2, 50, 1e-6, vq.Distance.SquaredEuclidean, 42)
+    qb = rvq.quantize_batch(training)
+    assert qb.shape == training.shape and np.isfinite(np.abs(training - qb.astype(F)).sum())
+    assert np.array_equal(rvq.quantize(training[0]), qb[0])
+
+
+def test_rvq_matches_oracle_with_explicit_streams(vq):
+    x = np.random.default_rng(3).standard_normal((1500, 24)).astype(F)
+    stages, k, iters = 3, 16, 5
+    streams = data.index_streams(1500, stages, k, iters, seed=6)
+    rvq = vq.ResidualQuantizer.fit(x, stages, k, iters, 0.0, vq.Distance.Euclidean, 1, streams=streams)
+    want = O.rvq_fit(O.EUCLIDEAN, x, stages, k, iters, 0.0, *streams)
+    assert rvq.stages == want["stages"] == stages
+    assert np.array_equal(rvq.codebooks(), want["codebooks"])
+    wcodes, wrec = O.rvq_quantize(O.EUCLIDEAN, x, want["codebooks"], 0.0)
+    assert np.array_equal(rvq.encode(x), wcodes.astype(np.uint8))
+    assert np.array_equal(rvq.quantize_batch(x).view(np.uint16), wrec)
+
+
+# ---- tests/test_tsvq.rs --------------------------------------------------------------------------
+def test_tsvq_on_identical_vectors(vq):
+    v = np.array([1.0, 2.0, 3.0, 4.0, 5.0], F)
+    tsvq = vq.TSVQ.new(np.tile(v, (10, 1)), 3, vq.Distance.SquaredEuclidean)
+    q = tsvq.quantize(v)
+    assert len(q) == len(v) and np.all(np.abs(v - q.astype(F)) < 1e-6)
+
+
+def test_tsvq_on_random_vectors(vq):
+    training = generate_test_data(1000, 10)
+    tsvq = vq.TSVQ.new(training, 3, vq.Distance.SquaredEuclidean)
+    qb = tsvq.quantize_batch(training)
+    assert qb.shape == training.shape and np.isfinite(np.abs(training - qb.astype(F)).sum())
+    otree = O.tsvq_fit(training, 3)
+    want_tree, new_id = bfs_order(otree)
+    want = np.array([new_id[v] for v in O.tsvq_descend(O.SQEUCLIDEAN, training, otree)])
+    assert np.array_equal(tsvq.leaves(training), want)
+    assert np.array_equal(qb.view(np.uint16),
+                          want_tree["centroids"][want].astype(np.float16).view(np.uint16))
+    with pytest.raises(vq.VqError, match="Dimension mismatch: expected 10, got 4"):
+        tsvq.quantize(training[0, :4])
+    with pytest.raises(vq.VqError, match="Empty input"):
+        vq.TSVQ.new(np.zeros((0, 10), F), 3, vq.Distance.Euclidean)

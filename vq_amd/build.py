@@ -44,5 +44,22 @@ def build_lib(verbose=False, extra=()):
     return LIB
 
 
+HOST_LIB = os.path.join(HERE, "libvqhost.so")
+
+
+def build_host(verbose=False):
+    """Compiles the C++ host mirror (plain g++: it only needs the C ABI) and links it to libvqhip."""
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-Wall",
+           os.path.join(HERE, "host", "vq_host_c.cpp"), "-o", HOST_LIB,
+           "-L" + HERE, "-lvqhip", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("g++ failed:\n" + res.stdout + res.stderr)
+    return HOST_LIB
+
+
 if __name__ == "__main__":
     print(build_lib(verbose=True, extra=sys.argv[1:]))
+    print(build_host(verbose=True))

@@ -1,0 +1,655 @@
+// vq.hpp — host-side mirror of the `vq` crate's public API for the codebook quantizers, written
+// in C++ above the C ABI of libvqhip (include/vq_hip.h).  The reference is Rust; this image has
+// no Rust toolchain, so this header plays the role the Rust host crate would: same type names,
+// same argument order and meaning, same validation, and the reference's panic messages as
+// exception texts.
+//
+//   Vector<T>                      src/vector.rs:149-173
+//   Distance                       src/distances.rs:73-88 (kernels: the first four variants)
+//   VqError                        src/exceptions.rs:9-25   (panics become C++ exceptions)
+//   lbg_quantize                   src/utils.rs:32-109
+//   ProductQuantizer               src/pq.rs:52-188
+//   OptimizedProductQuantizer      src/opq.rs:57-265
+//   ResidualQuantizer              src/rvq.rs:57-216
+//   TSVQ                           src/tsvq.rs:189-250
+//
+// Beyond the reference API every quantizer offers batch calls (quantize_batch, encode): one
+// vector at a time cannot feed a GPU.
+//
+// Randomness.  The reference seeds rand 0.9's StdRng (`seed + i` per sub-problem) and draws
+// `choose_multiple` / `choose`.  That crate is not available here, so IndexStreams::from_seed
+// is this host's OWN documented sampler (SplitMix64 + Floyd's algorithm): same contract
+// (k distinct rows, uniform re-seed rows, deterministic in the seed), different numbers.
+// A host that owns the real generator passes explicit IndexStreams instead.
+#pragma once
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <unordered_set>
+#include <vector>
+
+#include "../../include/vq_hip.h"
+
+namespace vq {
+
+// ---- errors (src/exceptions.rs) ----------------------------------------------------------------
+struct VqError : std::runtime_error {
+    int code;
+    VqError(int c, const std::string &m) : std::runtime_error(m), code(c) {}
+    static VqError DimensionMismatch(size_t expected, size_t found) {
+        return VqError(VQ_ERR_DIM_MISMATCH, "Dimension mismatch: expected " + std::to_string(expected) +
+                                                ", got " + std::to_string(found));
+    }
+    static VqError EmptyInput() {
+        return VqError(VQ_ERR_EMPTY_INPUT, "Empty input: at least one vector is required.");
+    }
+    static VqError InvalidParameter(const std::string &s) {
+        return VqError(VQ_ERR_INVALID_ARG, "Invalid parameter: " + s);
+    }
+    static VqError InvalidMetricParameter(const std::string &metric, const std::string &details) {
+        return VqError(VQ_ERR_UNSUPPORTED, "Invalid metric parameter for " + metric + ": " + details);
+    }
+};
+
+// ---- f16 and Vector (src/vector.rs) ------------------------------------------------------------
+struct f16 {
+    uint16_t bits = 0;
+    float to_f32() const {
+        uint32_t sign = ((uint32_t)bits & 0x8000u) << 16, exp = (bits >> 10) & 0x1fu, man = bits & 0x3ffu, x;
+        if (exp == 0) {
+            if (man == 0) {
+                x = sign;
+            } else {
+                int e = -1;
+                do {
+                    man <<= 1;
+                    ++e;
+                } while (!(man & 0x400u));
+                x = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3ffu) << 13);
+            }
+        } else if (exp == 0x1f) {
+            x = sign | 0x7f800000u | (man << 13);
+        } else {
+            x = sign | ((exp - 15 + 127) << 23) | (man << 13);
+        }
+        float f;
+        std::memcpy(&f, &x, 4);
+        return f;
+    }
+    bool operator==(const f16 &o) const { return bits == o.bits; }
+};
+
+template <class T>
+struct Vector {
+    std::vector<T> data;
+    Vector() = default;
+    explicit Vector(std::vector<T> d) : data(std::move(d)) {}
+    size_t len() const { return data.size(); }
+    bool is_empty() const { return data.empty(); }
+    bool operator==(const Vector &o) const { return data == o.data; }
+};
+
+// ---- Distance (src/distances.rs:73-88) ------------------------------------------------------------
+struct Distance {
+    enum Kind { SquaredEuclidean, Euclidean, CosineDistance, Manhattan, Chebyshev, Minkowski, Hamming };
+    Kind kind = SquaredEuclidean;
+    double p = 0.0;
+    Distance() = default;
+    Distance(Kind k, double p_ = 0.0) : kind(k), p(p_) {}
+    // The metric id of the C ABI; the three variants without a kernel are rejected.
+    int32_t abi_metric() const {
+        switch (kind) {
+        case SquaredEuclidean: return VQ_SQEUCLIDEAN;
+        case Euclidean: return VQ_EUCLIDEAN;
+        case CosineDistance: return VQ_COSINE;
+        case Manhattan: return VQ_MANHATTAN;
+        case Chebyshev: throw VqError::InvalidMetricParameter("Chebyshev", "no device kernel");
+        case Minkowski: throw VqError::InvalidMetricParameter("Minkowski", "no device kernel");
+        default: throw VqError::InvalidMetricParameter("Hamming", "no device kernel");
+        }
+    }
+};
+
+// ---- index streams -----------------------------------------------------------------------------
+struct IndexStreams {
+    std::vector<uint32_t> init;    // problems * k
+    std::vector<uint32_t> reseed;  // problems * n_reseed
+    int32_t n_reseed = 0;
+
+    static uint64_t splitmix(uint64_t &s) {
+        uint64_t z = (s += 0x9e3779b97f4a7c15ull);
+        z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+        z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+        return z ^ (z >> 31);
+    }
+    static uint64_t below(uint64_t &s, uint64_t bound) {  // unbiased, by rejection
+        uint64_t lim = UINT64_MAX - UINT64_MAX % bound;
+        uint64_t r;
+        do r = splitmix(s);
+        while (r >= lim);
+        return r % bound;
+    }
+    // Problem i is seeded with seed + i (src/pq.rs:119, src/opq.rs:140, src/rvq.rs:107): first k
+    // distinct rows (Floyd's algorithm, insertion order), then k*max_iters re-seed draws.
+    static IndexStreams from_seed(uint64_t seed, size_t problems, size_t n, size_t k, size_t max_iters) {
+        IndexStreams st;
+        st.n_reseed = (int32_t)(k * max_iters);
+        st.init.resize(problems * k);
+        st.reseed.resize(problems * (size_t)st.n_reseed);
+        for (size_t i = 0; i < problems; ++i) {
+            uint64_t s = seed + i;
+            std::unordered_set<uint32_t> seen;
+            size_t w = 0;
+            for (size_t j = n - k; j < n; ++j) {
+                uint32_t t = (uint32_t)below(s, j + 1);
+                uint32_t pick = seen.insert(t).second ? t : (uint32_t)j;
+                if (pick == (uint32_t)j) seen.insert(pick);
+                st.init[i * k + w++] = pick;
+            }
+            for (int32_t r = 0; r < st.n_reseed; ++r)
+                st.reseed[i * (size_t)st.n_reseed + r] = (uint32_t)below(s, n);
+        }
+        return st;
+    }
+};
+
+// ---- device plumbing ---------------------------------------------------------------------------
+class Device {
+public:
+    explicit Device(int index = 0) {
+        if (vq_ctx_create(index, &ctx_) != VQ_OK) throw VqError(VQ_ERR_HIP, vq_last_error(nullptr));
+    }
+    ~Device() { vq_ctx_destroy(ctx_); }
+    Device(const Device &) = delete;
+    Device &operator=(const Device &) = delete;
+    vq_ctx *ctx() const { return ctx_; }
+    void check(int32_t rc) const {
+        if (rc != VQ_OK) throw VqError(rc, vq_last_error(ctx_));
+    }
+    static std::shared_ptr<Device> shared() {
+        static std::shared_ptr<Device> d = std::make_shared<Device>(0);
+        return d;
+    }
+
+private:
+    vq_ctx *ctx_ = nullptr;
+};
+
+template <class T>
+class DeviceBuffer {
+public:
+    DeviceBuffer() = default;
+    DeviceBuffer(std::shared_ptr<Device> d, size_t count) : dev_(std::move(d)), count_(count) {
+        void *p = nullptr;
+        dev_->check(vq_malloc(dev_->ctx(), count * sizeof(T), &p));
+        ptr_ = static_cast<T *>(p);
+    }
+    DeviceBuffer(DeviceBuffer &&o) noexcept { *this = std::move(o); }
+    DeviceBuffer &operator=(DeviceBuffer &&o) noexcept {
+        release();
+        dev_ = std::move(o.dev_);
+        ptr_ = o.ptr_;
+        count_ = o.count_;
+        o.ptr_ = nullptr;
+        o.count_ = 0;
+        return *this;
+    }
+    ~DeviceBuffer() { release(); }
+    T *get() const { return ptr_; }
+    size_t size() const { return count_; }
+    void upload(const T *src, size_t count) { dev_->check(vq_h2d(dev_->ctx(), ptr_, src, count * sizeof(T))); }
+    void download(T *dst, size_t count) const { dev_->check(vq_d2h(dev_->ctx(), dst, ptr_, count * sizeof(T))); }
+    std::vector<T> to_host() const {
+        std::vector<T> v(count_);
+        if (count_) download(v.data(), count_);
+        return v;
+    }
+
+private:
+    void release() {
+        if (ptr_ && dev_) vq_free(dev_->ctx(), ptr_);
+        ptr_ = nullptr;
+    }
+    std::shared_ptr<Device> dev_;
+    T *ptr_ = nullptr;
+    size_t count_ = 0;
+};
+
+// Packs `&[Vector<f32>]` (one heap allocation per vector, src/vector.rs:150-152) into one
+// row-major buffer and checks that all rows have the same length.
+inline std::vector<float> pack_rows(const std::vector<Vector<float>> &rows, size_t dim) {
+    std::vector<float> flat(rows.size() * dim);
+    for (size_t i = 0; i < rows.size(); ++i) {
+        if (rows[i].len() != dim) throw VqError::DimensionMismatch(dim, rows[i].len());
+        std::memcpy(flat.data() + i * dim, rows[i].data.data(), dim * sizeof(float));
+    }
+    return flat;
+}
+
+inline std::vector<Vector<f16>> unpack_f16(const std::vector<uint16_t> &flat, size_t n, size_t dim) {
+    std::vector<Vector<f16>> out(n);
+    for (size_t i = 0; i < n; ++i) {
+        out[i].data.resize(dim);
+        for (size_t t = 0; t < dim; ++t) out[i].data[t].bits = flat[i * dim + t];
+    }
+    return out;
+}
+
+// ---- lbg_quantize (src/utils.rs:32-109) --------------------------------------------------------
+inline std::vector<Vector<float>> lbg_quantize(const std::vector<Vector<float>> &data, size_t k,
+                                               size_t max_iters, uint64_t seed,
+                                               const IndexStreams *streams = nullptr,
+                                               std::shared_ptr<Device> dev = Device::shared()) {
+    size_t n = data.size();
+    if (k == 0) throw VqError::InvalidParameter("k must be greater than 0");
+    if (n < k) throw VqError::InvalidParameter("Not enough data points for k clusters");
+    size_t dim = data[0].len();
+    std::vector<float> flat = pack_rows(data, dim);
+    IndexStreams own;
+    if (!streams) {
+        own = IndexStreams::from_seed(seed, 1, n, k, max_iters);
+        streams = &own;
+    }
+    DeviceBuffer<float> dx(dev, n * dim), dcb(dev, k * dim);
+    dx.upload(flat.data(), flat.size());
+    dev->check(vq_lbg_fit(dev->ctx(), dx.get(), (int64_t)n, (int64_t)dim, 1, (int32_t)dim, (int32_t)k,
+                          (int32_t)max_iters, streams->init.data(), streams->reseed.data(),
+                          streams->n_reseed, dcb.get(), nullptr, nullptr));
+    std::vector<float> cb = dcb.to_host();
+    std::vector<Vector<float>> out(k);
+    for (size_t j = 0; j < k; ++j) out[j].data.assign(cb.begin() + j * dim, cb.begin() + (j + 1) * dim);
+    return out;
+}
+
+// ---- ProductQuantizer (src/pq.rs) ----------------------------------------------------------------
+class ProductQuantizer {
+public:
+    // src/pq.rs:79-129
+    static ProductQuantizer fit(const std::vector<Vector<float>> &training_data, size_t m, size_t k,
+                                size_t max_iters, Distance distance, uint64_t seed,
+                                const IndexStreams *streams = nullptr,
+                                std::shared_ptr<Device> dev = Device::shared()) {
+        if (training_data.empty()) throw VqError::EmptyInput();
+        size_t n = training_data[0].len();
+        if (n < m) throw VqError::InvalidParameter("Data dimension must be at least m");
+        if (n % m != 0) throw VqError::InvalidParameter("Data dimension must be divisible by m");
+        size_t rows = training_data.size();
+        if (k == 0) throw VqError::InvalidParameter("k must be greater than 0");
+        if (rows < k) throw VqError::InvalidParameter("Not enough data points for k clusters");
+        ProductQuantizer pq;
+        pq.dev_ = dev;
+        pq.m_ = m;
+        pq.k_ = k;
+        pq.sub_dim_ = n / m;
+        pq.distance_ = distance;
+        std::vector<float> flat = pack_rows(training_data, n);
+        IndexStreams own;
+        if (!streams) {
+            own = IndexStreams::from_seed(seed, m, rows, k, max_iters);
+            streams = &own;
+        }
+        DeviceBuffer<float> dx(dev, rows * n);
+        dx.upload(flat.data(), flat.size());
+        pq.codebooks_ = DeviceBuffer<float>(dev, m * k * pq.sub_dim_);
+        dev->check(vq_lbg_fit(dev->ctx(), dx.get(), (int64_t)rows, (int64_t)n, (int32_t)m, (int32_t)pq.sub_dim_,
+                              (int32_t)k, (int32_t)max_iters, streams->init.data(), streams->reseed.data(),
+                              streams->n_reseed, pq.codebooks_.get(), nullptr, nullptr));
+        return pq;
+    }
+
+    // src/pq.rs:146-187
+    Vector<f16> quantize(const Vector<float> &vector) const {
+        if (vector.len() != sub_dim_ * m_) throw VqError::DimensionMismatch(sub_dim_ * m_, vector.len());
+        return quantize_batch({vector})[0];
+    }
+
+    std::vector<Vector<f16>> quantize_batch(const std::vector<Vector<float>> &vectors) const {
+        size_t dim = sub_dim_ * m_, n = vectors.size();
+        if (n == 0) return {};
+        std::vector<float> flat = pack_rows(vectors, dim);
+        DeviceBuffer<float> dx(dev_, n * dim);
+        dx.upload(flat.data(), flat.size());
+        DeviceBuffer<uint8_t> dcodes(dev_, n * m_);
+        DeviceBuffer<uint16_t> dout(dev_, n * dim);
+        dev_->check(vq_assign(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim, (int32_t)m_,
+                              (int32_t)sub_dim_, (int32_t)k_, codebooks_.get(), dcodes.get()));
+        dev_->check(vq_decode_f16(dev_->ctx(), dcodes.get(), (int64_t)n, (int32_t)m_, (int32_t)sub_dim_,
+                                  (int32_t)k_, codebooks_.get(), dout.get()));
+        return unpack_f16(dout.to_host(), n, dim);
+    }
+
+    // The integer codes the reference keeps only as `best_index` (src/pq.rs:166-174): n x m bytes.
+    std::vector<uint8_t> encode(const std::vector<Vector<float>> &vectors) const {
+        size_t dim = sub_dim_ * m_, n = vectors.size();
+        if (n == 0) return {};
+        std::vector<float> flat = pack_rows(vectors, dim);
+        DeviceBuffer<float> dx(dev_, n * dim);
+        dx.upload(flat.data(), flat.size());
+        DeviceBuffer<uint8_t> dcodes(dev_, n * m_);
+        dev_->check(vq_assign(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim, (int32_t)m_,
+                              (int32_t)sub_dim_, (int32_t)k_, codebooks_.get(), dcodes.get()));
+        return dcodes.to_host();
+    }
+
+    std::vector<float> codebooks() const { return codebooks_.to_host(); }  // m*k*sub_dim
+    size_t m() const { return m_; }
+    size_t k() const { return k_; }
+    size_t sub_dim() const { return sub_dim_; }
+
+private:
+    std::shared_ptr<Device> dev_;
+    DeviceBuffer<float> codebooks_;
+    size_t sub_dim_ = 0, m_ = 0, k_ = 0;
+    Distance distance_;
+};
+
+// ---- orthogonal Procrustes on the host (src/opq.rs:180-183) -------------------------------------
+// R = V U^T for A = U S V^T, by a cyclic one-sided Jacobi SVD in f64; row-major dim x dim.
+inline void procrustes_rotation(const std::vector<double> &A, size_t dim, std::vector<double> &R) {
+    const size_t n = dim;
+    std::vector<double> U(A), V(n * n, 0.0);
+    for (size_t i = 0; i < n; ++i) V[i * n + i] = 1.0;
+    for (int sweep = 0; sweep < 60; ++sweep) {
+        double off = 0.0;
+        for (size_t p = 0; p + 1 < n; ++p)
+            for (size_t q = p + 1; q < n; ++q) {
+                double alpha = 0, beta = 0, gamma = 0;
+                for (size_t i = 0; i < n; ++i) {
+                    alpha += U[i * n + p] * U[i * n + p];
+                    beta += U[i * n + q] * U[i * n + q];
+                    gamma += U[i * n + p] * U[i * n + q];
+                }
+                if (gamma == 0.0) continue;
+                off = std::max(off, std::fabs(gamma) / std::sqrt(alpha * beta + 1e-300));
+                double zeta = (beta - alpha) / (2.0 * gamma);
+                double t = (zeta >= 0 ? 1.0 : -1.0) / (std::fabs(zeta) + std::sqrt(1.0 + zeta * zeta));
+                double c = 1.0 / std::sqrt(1.0 + t * t), s = c * t;
+                for (size_t i = 0; i < n; ++i) {
+                    double up = U[i * n + p], uq = U[i * n + q];
+                    U[i * n + p] = c * up - s * uq;
+                    U[i * n + q] = s * up + c * uq;
+                    double vp = V[i * n + p], vq = V[i * n + q];
+                    V[i * n + p] = c * vp - s * vq;
+                    V[i * n + q] = s * vp + c * vq;
+                }
+            }
+        if (off < 1e-15) break;
+    }
+    for (size_t j = 0; j < n; ++j) {
+        double s = 0;
+        for (size_t i = 0; i < n; ++i) s += U[i * n + j] * U[i * n + j];
+        s = std::sqrt(s);
+        if (s > 0)
+            for (size_t i = 0; i < n; ++i) U[i * n + j] /= s;
+    }
+    R.assign(n * n, 0.0);
+    for (size_t i = 0; i < n; ++i)
+        for (size_t j = 0; j < n; ++j) {
+            double acc = 0;
+            for (size_t l = 0; l < n; ++l) acc += V[i * n + l] * U[j * n + l];
+            R[i * n + j] = acc;
+        }
+}
+
+// ---- OptimizedProductQuantizer (src/opq.rs) -----------------------------------------------------
+class OptimizedProductQuantizer {
+public:
+    // src/opq.rs:90-205
+    static OptimizedProductQuantizer fit(const std::vector<Vector<float>> &training_data, size_t m, size_t k,
+                                         size_t max_iters, size_t opq_iters, Distance distance, uint64_t seed,
+                                         const IndexStreams *streams = nullptr,
+                                         std::shared_ptr<Device> dev = Device::shared()) {
+        if (training_data.empty()) throw VqError::EmptyInput();
+        size_t dim = training_data[0].len();
+        if (dim < m) throw VqError::InvalidParameter("Dimension must be at least m");
+        if (dim % m != 0) throw VqError::InvalidParameter("Dimension must be divisible by m");
+        size_t n = training_data.size(), sd = dim / m;
+        if (k == 0) throw VqError::InvalidParameter("k must be greater than 0");
+        if (n < k) throw VqError::InvalidParameter("Not enough data points for k clusters");
+        OptimizedProductQuantizer q;
+        q.dev_ = dev;
+        q.m_ = m;
+        q.k_ = k;
+        q.sub_dim_ = sd;
+        q.dim_ = dim;
+        q.distance_ = distance;
+        const int32_t metric = distance.abi_metric();
+        std::vector<float> flat = pack_rows(training_data, dim);
+        IndexStreams own;
+        if (!streams) {  // the same streams in every outer iteration (opq.rs:140 re-seeds seed + i)
+            own = IndexStreams::from_seed(seed, m, n, k, max_iters);
+            streams = &own;
+        }
+        vq_ctx *c = dev->ctx();
+        DeviceBuffer<float> dx(dev, n * dim), drot(dev, n * dim), drec(dev, n * dim);
+        DeviceBuffer<uint8_t> dcodes(dev, n * m);
+        dx.upload(flat.data(), flat.size());
+        dev->check(vq_copy_f32(c, drot.get(), dx.get(), (int64_t)(n * dim)));  // opq.rs:121
+        q.codebooks_ = DeviceBuffer<float>(dev, m * k * sd);
+        q.rotation_.assign(dim * dim, 0.f);
+        for (size_t i = 0; i < dim; ++i) q.rotation_[i * dim + i] = 1.f;  // opq.rs:119
+        q.d_rotation_ = DeviceBuffer<float>(dev, dim * dim);
+        std::vector<double> A(dim * dim), Rd;
+        for (size_t it = 0; it < opq_iters; ++it) {
+            dev->check(vq_lbg_fit(c, drot.get(), (int64_t)n, (int64_t)dim, (int32_t)m, (int32_t)sd, (int32_t)k,
+                                  (int32_t)max_iters, streams->init.data(), streams->reseed.data(),
+                                  streams->n_reseed, q.codebooks_.get(), nullptr, nullptr));  // 127-142
+            dev->check(vq_assign(c, metric, drot.get(), (int64_t)n, (int64_t)dim, (int32_t)m, (int32_t)sd,
+                                 (int32_t)k, q.codebooks_.get(), dcodes.get()));                // 146-163
+            dev->check(vq_decode_f32(c, dcodes.get(), (int64_t)n, (int32_t)m, (int32_t)sd, (int32_t)k,
+                                     q.codebooks_.get(), drec.get()));                            // 164-167
+            dev->check(vq_cross_cov(c, drec.get(), drot.get(), (int64_t)n, (int32_t)dim, A.data())); // 172-179
+            for (double &v : A) v = (double)(float)v;  // the reference's A is a DMatrix<f32>
+            procrustes_rotation(A, dim, Rd);           // 180-183, on the host
+            for (size_t i = 0; i < dim * dim; ++i) q.rotation_[i] = (float)Rd[i];
+            q.d_rotation_.upload(q.rotation_.data(), dim * dim);
+            dev->check(vq_rotate(c, dx.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, q.d_rotation_.get(),
+                                 drot.get()));                                                    // 186-194
+        }
+        if (opq_iters == 0) q.d_rotation_.upload(q.rotation_.data(), dim * dim);
+        return q;
+    }
+
+    // src/opq.rs:222-264
+    Vector<f16> quantize(const Vector<float> &vector) const {
+        if (vector.len() != dim_) throw VqError::DimensionMismatch(dim_, vector.len());
+        return quantize_batch({vector})[0];
+    }
+
+    std::vector<Vector<f16>> quantize_batch(const std::vector<Vector<float>> &vectors) const {
+        size_t n = vectors.size();
+        if (n == 0) return {};
+        DeviceBuffer<uint8_t> dcodes = encode_device(vectors);
+        DeviceBuffer<uint16_t> dout(dev_, n * dim_);
+        dev_->check(vq_decode_f16(dev_->ctx(), dcodes.get(), (int64_t)n, (int32_t)m_, (int32_t)sub_dim_,
+                                  (int32_t)k_, codebooks_.get(), dout.get()));
+        return unpack_f16(dout.to_host(), n, dim_);
+    }
+
+    std::vector<uint8_t> encode(const std::vector<Vector<float>> &vectors) const {
+        if (vectors.empty()) return {};
+        return encode_device(vectors).to_host();
+    }
+
+    std::vector<float> codebooks() const { return codebooks_.to_host(); }
+    const std::vector<float> &rotation() const { return rotation_; }  // row-major dim x dim
+
+private:
+    DeviceBuffer<uint8_t> encode_device(const std::vector<Vector<float>> &vectors) const {
+        size_t n = vectors.size();
+        std::vector<float> flat = pack_rows(vectors, dim_);
+        DeviceBuffer<float> dx(dev_, n * dim_), dy(dev_, n * dim_);
+        dx.upload(flat.data(), flat.size());
+        DeviceBuffer<uint8_t> dcodes(dev_, n * m_);
+        vq_ctx *c = dev_->ctx();
+        dev_->check(vq_rotate(c, dx.get(), (int64_t)n, (int64_t)dim_, (int32_t)dim_, d_rotation_.get(), dy.get()));
+        dev_->check(vq_assign(c, distance_.abi_metric(), dy.get(), (int64_t)n, (int64_t)dim_, (int32_t)m_,
+                              (int32_t)sub_dim_, (int32_t)k_, codebooks_.get(), dcodes.get()));
+        dev_->check(vq_ctx_sync(c));
+        return dcodes;
+    }
+    std::shared_ptr<Device> dev_;
+    DeviceBuffer<float> codebooks_, d_rotation_;
+    std::vector<float> rotation_;
+    size_t sub_dim_ = 0, m_ = 0, k_ = 0, dim_ = 0;
+    Distance distance_;
+};
+
+// ---- ResidualQuantizer (src/rvq.rs) --------------------------------------------------------------
+class ResidualQuantizer {
+public:
+    // src/rvq.rs:87-154
+    static ResidualQuantizer fit(const std::vector<Vector<float>> &training_data, size_t stages, size_t k,
+                                 size_t max_iters, float epsilon, Distance distance, uint64_t seed,
+                                 const IndexStreams *streams = nullptr,
+                                 std::shared_ptr<Device> dev = Device::shared()) {
+        if (training_data.empty()) throw VqError::EmptyInput();
+        size_t dim = training_data[0].len(), n = training_data.size();
+        if (stages > 0) {
+            if (k == 0) throw VqError::InvalidParameter("k must be greater than 0");
+            if (n < k) throw VqError::InvalidParameter("Not enough data points for k clusters");
+        }
+        ResidualQuantizer q;
+        q.dev_ = dev;
+        q.dim_ = dim;
+        q.k_ = k;
+        q.epsilon_ = epsilon;
+        q.distance_ = distance;
+        const int32_t metric = distance.abi_metric();
+        std::vector<float> flat = pack_rows(training_data, dim);
+        IndexStreams own;
+        if (!streams) {
+            own = IndexStreams::from_seed(seed, stages, n, k, max_iters);
+            streams = &own;
+        }
+        vq_ctx *c = dev->ctx();
+        DeviceBuffer<float> dx(dev, n * dim), dres(dev, n * dim);
+        DeviceBuffer<uint8_t> dcodes(dev, n + 16);
+        dx.upload(flat.data(), flat.size());
+        dev->check(vq_copy_f32(c, dres.get(), dx.get(), (int64_t)(n * dim)));  // rvq.rs:103
+        q.codebooks_ = DeviceBuffer<float>(dev, std::max<size_t>(stages * k * dim, 1));
+        std::vector<uint8_t> zeros(n, 0);
+        size_t produced = 0;
+        for (size_t st = 0; st < stages; ++st) {
+            float *cb = q.codebooks_.get() + st * k * dim;
+            dev->check(vq_lbg_fit(c, dres.get(), (int64_t)n, (int64_t)dim, 1, (int32_t)dim, (int32_t)k,
+                                  (int32_t)max_iters, streams->init.data() + st * k,
+                                  streams->reseed.data() + st * (size_t)streams->n_reseed, streams->n_reseed, cb,
+                                  nullptr, nullptr));  // rvq.rs:107
+            ++produced;
+            if (k < 2)  // rvq.rs:113-115
+                dcodes.upload(zeros.data(), n);
+            else
+                dev->check(vq_assign(c, metric, dres.get(), (int64_t)n, (int64_t)dim, 1, (int32_t)dim, (int32_t)k,
+                                     cb, dcodes.get()));  // rvq.rs:116-125
+            dev->check(vq_residual_sub(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)k, cb,
+                                       dcodes.get()));  // rvq.rs:127
+            float avg = 0.f;
+            dev->check(vq_mean_l2norm(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, &avg));  // 131-138
+            if (avg < epsilon) break;  // rvq.rs:139-141
+        }
+        q.stages_ = produced;  // rvq.rs:145
+        return q;
+    }
+
+    // src/rvq.rs:171-215
+    Vector<f16> quantize(const Vector<float> &vector) const {
+        if (vector.len() != dim_) throw VqError::DimensionMismatch(dim_, vector.len());
+        return quantize_batch({vector})[0];
+    }
+
+    std::vector<Vector<f16>> quantize_batch(const std::vector<Vector<float>> &vectors,
+                                            std::vector<uint8_t> *codes = nullptr) const {
+        size_t n = vectors.size();
+        if (n == 0) return {};
+        std::vector<float> flat = pack_rows(vectors, dim_);
+        DeviceBuffer<float> dx(dev_, n * dim_);
+        dx.upload(flat.data(), flat.size());
+        DeviceBuffer<uint8_t> dcodes(dev_, std::max<size_t>(n * stages_, 1));
+        DeviceBuffer<uint16_t> dout(dev_, n * dim_);
+        dev_->check(vq_rvq_encode(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim_,
+                                  (int32_t)dim_, (int32_t)stages_, (int32_t)std::max<size_t>(k_, 1),
+                                  codebooks_.get(), epsilon_, dcodes.get(), nullptr, dout.get()));
+        if (codes) *codes = dcodes.to_host();
+        return unpack_f16(dout.to_host(), n, dim_);
+    }
+
+    size_t stages() const { return stages_; }
+    std::vector<float> codebooks() const {  // stages*k*dim
+        std::vector<float> all = codebooks_.to_host();
+        all.resize(stages_ * k_ * dim_);
+        return all;
+    }
+
+private:
+    std::shared_ptr<Device> dev_;
+    DeviceBuffer<float> codebooks_;
+    size_t stages_ = 0, dim_ = 0, k_ = 0;
+    float epsilon_ = 0.f;
+    Distance distance_;
+};
+
+// ---- TSVQ (src/tsvq.rs) --------------------------------------------------------------------------
+class TSVQ {
+public:
+    Distance distance;  // `pub distance`, src/tsvq.rs:193
+
+    // TSVQ::new, src/tsvq.rs:209-215
+    static TSVQ create(const std::vector<Vector<float>> &training_data, size_t max_depth, Distance distance,
+                       std::shared_ptr<Device> dev = Device::shared()) {
+        if (training_data.empty()) throw VqError::EmptyInput();
+        size_t dim = training_data[0].len(), n = training_data.size();
+        std::vector<float> flat = pack_rows(training_data, dim);
+        TSVQ t;
+        t.dev_ = dev;
+        t.distance = distance;
+        t.dim_ = dim;
+        DeviceBuffer<float> dx(dev, n * dim);
+        dx.upload(flat.data(), flat.size());
+        vq_tree *tree = nullptr;
+        dev->check(vq_tsvq_build(dev->ctx(), dx.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)max_depth,
+                                 &tree));
+        std::shared_ptr<Device> keep = dev;
+        t.tree_ = std::shared_ptr<vq_tree>(tree, [keep](vq_tree *p) { vq_tree_free(keep->ctx(), p); });
+        return t;
+    }
+
+    // src/tsvq.rs:231-249
+    Vector<f16> quantize(const Vector<float> &vector) const {
+        if (vector.len() != dim_) throw VqError::DimensionMismatch(dim_, vector.len());
+        return quantize_batch({vector})[0];
+    }
+
+    std::vector<Vector<f16>> quantize_batch(const std::vector<Vector<float>> &vectors,
+                                            std::vector<int32_t> *leaves = nullptr) const {
+        size_t n = vectors.size();
+        if (n == 0) return {};
+        std::vector<float> flat = pack_rows(vectors, dim_);
+        DeviceBuffer<float> dx(dev_, n * dim_);
+        dx.upload(flat.data(), flat.size());
+        DeviceBuffer<int32_t> dleaf(dev_, n);
+        DeviceBuffer<uint16_t> dout(dev_, n * dim_);
+        dev_->check(vq_tsvq_descend(dev_->ctx(), distance.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim_,
+                                    tree_.get(), dleaf.get()));
+        dev_->check(vq_tsvq_decode_f16(dev_->ctx(), tree_.get(), dleaf.get(), (int64_t)n, dout.get()));
+        if (leaves) *leaves = dleaf.to_host();
+        return unpack_f16(dout.to_host(), n, dim_);
+    }
+
+    int32_t n_nodes() const {
+        int32_t nn = 0;
+        vq_tree_info(tree_.get(), &nn, nullptr);
+        return nn;
+    }
+    const vq_tree *tree() const { return tree_.get(); }
+
+private:
+    std::shared_ptr<Device> dev_;
+    std::shared_ptr<vq_tree> tree_;
+    size_t dim_ = 0;
+};
+
+}  // namespace vq
