@@ -95,6 +95,7 @@ def main():
     update_ms, update_n = ctx.prof_read(vq_amd._ffi.PROF_LBG_UPDATE)
     enc_ms, enc_n = ctx.prof_read(vq_amd._ffi.PROF_ENCODE)
     ctx.prof_enable(False)
+    recheck_pairs = ctx.last_recheck_count()
     ms_per_step = wall_ms / args.steps
     value = n / (ms_per_step * 1e-3)
 
@@ -125,6 +126,7 @@ def main():
         "lbg_update_ms_per_step": round(update_ms / args.steps, 3),
         "encode_ms_per_step": round(enc_ms / args.steps, 3),
         "gpu_event_ms_per_step": round(gpu_ms / args.steps, 3),
+        "encode_recheck_fraction": round(recheck_pairs / float(n * M), 6),
     }
 
     # CPU baseline + parity on a bounded sample of the same rows

@@ -62,6 +62,16 @@ int32_t vq_ctx_sync(vq_ctx *ctx);
 /* The context's hipStream_t, as an opaque pointer. */
 void *vq_ctx_stream(vq_ctx *ctx);
 
+/* Which kernels decide the squared-L2 / Euclidean assignment where both exist:
+ *   0 (default)  matrix-core pass with an exact re-check of every undecided (row, block) pair
+ *   1            the all-vector-ALU kernel in the reference's operation order
+ * Both give bit-identical codes; the switch exists for measurement and tests. */
+int32_t vq_ctx_set_assign_path(vq_ctx *ctx, int32_t path);
+
+/* Number of (row, block) pairs the most recent matrix-core assignment pass left to the exact
+ * re-check (0 if that path has not run).  Synchronises.  Measurement only. */
+int32_t vq_ctx_last_recheck_count(vq_ctx *ctx, uint32_t *h_count);
+
 int32_t vq_malloc(vq_ctx *ctx, size_t bytes, void **d_ptr);
 int32_t vq_free(vq_ctx *ctx, void *d_ptr);
 /* Synchronous copies (they synchronise the context's stream). Replaces the per-vector heap

@@ -159,3 +159,66 @@ def test_errors_match_reference_panics(ctx):
         ctx.lbg_fit(x, 0, 8, 1, 8, 2, 3, np.zeros(2, np.uint32), np.zeros(2, np.uint32), cb)
     with pytest.raises(vq_amd.VqError, match="Dimension mismatch"):
         ctx.assign(0, x, 4, 8, 2, 8, 2, cb, ctx.empty((4, 2), np.uint8))
+
+
+# ---- matrix-core assignment path vs vector-ALU path ---------------------------------------------
+@pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN])
+@pytest.mark.parametrize("n,m,k,kind", [
+    (5000, 16, 256, "uniform"), (1000, 16, 256, "mixture"), (700, 4, 100, "normal"),
+    (513, 1, 1, "normal"), (64, 2, 33, "grid"), (2000, 16, 256, "offset"), (300, 3, 7, "same"),
+    (900, 16, 256, "nonfinite"),
+])
+def test_mfma_path_equals_oracle_and_valu_path(ctx, metric, n, m, k, kind):
+    """sub_dim 8: the default path is the matrix-core pass + exact re-check.  It must give the
+    oracle's codes bit for bit on ties, near ties, offsets that blow up the error bound,
+    padding (k not a multiple of 32) and non-finite values."""
+    rng = np.random.default_rng(n + k)
+    dim = 8 * m
+    if kind == "uniform":
+        x, cb = rng.random((n, dim), dtype=F), rng.random((m, k, 8), dtype=F)
+    elif kind == "mixture":
+        x = data.gaussian_mixture(n, dim, 64, 0.05, seed=1)
+        cb = x[rng.choice(n, k, replace=False)].reshape(k, m, 8).transpose(1, 0, 2).copy()
+    elif kind == "grid":
+        x = np.round(rng.standard_normal((n, dim))).astype(F)
+        cb = np.round(rng.standard_normal((m, k, 8))).astype(F)
+    elif kind == "offset":  # far from the origin: the error bound is large, most pairs re-checked
+        x = (1000 + rng.random((n, dim))).astype(F)
+        cb = (1000 + rng.random((m, k, 8))).astype(F)
+    elif kind == "same":
+        x = np.tile(rng.standard_normal((1, dim)).astype(F), (n, 1))
+        cb = np.tile(x[:1].reshape(m, 1, 8), (1, k, 1)).copy()
+    elif kind == "nonfinite":
+        x, cb = rng.random((n, dim), dtype=F), rng.random((m, k, 8), dtype=F)
+        x[::7, 3] = np.inf
+        x[1::11, 9] = np.nan
+        x[2::13, 20] = 1e30
+        cb[1, 5, 2] = np.nan
+        cb[2, 0, :] = np.nan  # NaN at index 0 can never be displaced (strict '<')
+        cb[3, 9, 1] = -np.inf
+    else:
+        x, cb = rng.standard_normal((n, dim)).astype(F), rng.standard_normal((m, k, 8)).astype(F)
+    dx, dcb = ctx.to_device(x), ctx.to_device(cb)
+    with np.errstate(all="ignore"):
+        want = O.pq_encode(metric, x, cb).astype(np.uint8)
+    ctx.set_assign_path(0)
+    got = gpu_encode(ctx, metric, dx, n, dim, m, k, dcb)
+    ctx.set_assign_path(1)
+    valu = gpu_encode(ctx, metric, dx, n, dim, m, k, dcb)
+    ctx.set_assign_path(0)
+    assert np.array_equal(valu, want)
+    assert np.array_equal(got, want)
+
+
+def test_lbg_fit_same_result_on_both_assignment_paths(ctx):
+    n, dim, m, k, iters = 20000, 128, 16, 256, 5
+    x = data.gaussian_mixture(n, dim, 256, 0.05, seed=1)
+    init, reseed = data.index_streams(n, m, k, iters, seed=11)
+    ctx.set_assign_path(1)
+    a, it_a, used_a, _, _ = gpu_lbg(ctx, x, m, k, iters, init, reseed)
+    ctx.set_assign_path(0)
+    b, it_b, used_b, _, _ = gpu_lbg(ctx, x, m, k, iters, init, reseed)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    assert np.array_equal(it_a, it_b) and np.array_equal(used_a, used_b)
+    want = O.pq_fit(x, m, k, iters, init, reseed)
+    assert np.array_equal(b.view(np.uint32), want["codebooks"].view(np.uint32))

@@ -26,6 +26,8 @@ SYMBOLS = {
     "vq_last_error": (C.c_char_p, [_vp]),
     "vq_ctx_sync": (_i32, [_vp]),
     "vq_ctx_stream": (_vp, [_vp]),
+    "vq_ctx_set_assign_path": (_i32, [_vp, _i32]),
+    "vq_ctx_last_recheck_count": (_i32, [_vp, C.POINTER(C.c_uint32)]),
     "vq_malloc": (_i32, [_vp, _sz, C.POINTER(_vp)]),
     "vq_free": (_i32, [_vp, _vp]),
     "vq_h2d": (_i32, [_vp, _vp, _vp, _sz]),
@@ -184,6 +186,15 @@ class Context:
 
     def copy_f32(self, d_dst, d_src, count):
         self._check(_lib.vq_copy_f32(self._h, d_dst.ptr, d_src.ptr, count))
+
+    def set_assign_path(self, path):
+        """0 = matrix cores + exact re-check (default), 1 = vector ALU only."""
+        self._check(_lib.vq_ctx_set_assign_path(self._h, path))
+
+    def last_recheck_count(self):
+        c = C.c_uint32(0)
+        self._check(_lib.vq_ctx_last_recheck_count(self._h, C.byref(c)))
+        return c.value
 
     def sync(self):
         self._check(_lib.vq_ctx_sync(self._h))

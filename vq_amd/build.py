@@ -15,6 +15,8 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-fno-fast-math", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
+    # matrix-core accumulators stay in architectural VGPRs (no copies through the AGPR half)
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
 
 

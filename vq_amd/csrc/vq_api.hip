@@ -13,6 +13,11 @@
 
 #include "ctx.hpp"
 #include "assign_exact.hpp"
+#include "assign_mfma.hpp"
+
+#ifndef VQ_MFMA_TILES
+#define VQ_MFMA_TILES 4  // tiles of 32 rows per wave in the matrix-core assignment
+#endif
 #include "lbg_update.hpp"
 
 namespace vqh {
@@ -83,8 +88,49 @@ int32_t launch_assign_m(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     return VQ_OK;
 }
 
+// Matrix-core pass + exact re-check of the undecided pairs (assign_mfma.hpp).
+template <int SD, int METRIC, bool LBG>
+int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
+    const int nb = (a.k + 31) / 32;
+    const size_t n_atab = (size_t)a.m * nb * 64 * (SD / 2), n_c2 = (size_t)a.m * nb * 32;
+    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + a.m) + 64));
+    VQ_TRY(ensure(ctx, ctx->mfma_list, sizeof(uint32_t) * ((size_t)a.n * a.m + 4)));
+    float *atab = (float *)ctx->mfma_tab.p;
+    float *c2perm = atab + n_atab;
+    float *maxc2 = c2perm + n_c2;
+    uint32_t *count = (uint32_t *)ctx->mfma_list.p;
+    uint32_t *list = count + 4;
+    hipLaunchKernelGGL((vq::k_mfma_prep<SD>), dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, atab,
+                       c2perm, maxc2, count);
+    vq::MfmaTables tb{atab, c2perm, maxc2, list, count, nb};
+    const size_t lds = sizeof(float) * n_c2;
+    constexpr int TILES = VQ_MFMA_TILES;
+    auto kern = vq::k_assign_mfma<SD, LBG, TILES>;
+    if (lds > 48 * 1024)
+        VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3(cdiv(a.n, 4 * 32 * TILES)), dim3(256), lds, ctx->stream, a, tb);
+    hipLaunchKernelGGL((vq::k_assign_recheck<SD, METRIC, LBG>), dim3(1024), dim3(256), 0, ctx->stream, a,
+                       (const uint32_t *)list, (const uint32_t *)count);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+template <int METRIC, bool LBG>
+bool mfma_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
+    if (ctx->assign_path != 0) return false;
+    if (METRIC != vq::M_SQ && METRIC != vq::M_EUCLID) return false;
+    if (sd != 8) return false;
+    // tables must fit LDS; tiny inputs gain nothing
+    return (size_t)a.m * ((a.k + 31) / 32) * 32 * sizeof(float) <= 64 * 1024 && (int64_t)a.n * a.m < (1LL << 32);
+}
+
 template <bool LBG>
 int32_t launch_assign(vq_ctx *ctx, int metric, const vq::AssignArgs &a, int sd) {
+    if (metric == VQ_SQEUCLIDEAN && mfma_applicable<vq::M_SQ, LBG>(ctx, a, sd))
+        return launch_mfma<8, vq::M_SQ, LBG>(ctx, a);
+    if (metric == VQ_EUCLIDEAN && mfma_applicable<vq::M_EUCLID, LBG>(ctx, a, sd))
+        return launch_mfma<8, vq::M_EUCLID, LBG>(ctx, a);
     switch (metric) {
     case VQ_SQEUCLIDEAN: return launch_assign_m<vq::M_SQ, LBG>(ctx, a, sd);
     case VQ_EUCLIDEAN: return launch_assign_m<vq::M_EUCLID, LBG>(ctx, a, sd);
@@ -211,7 +257,7 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
-                      &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
+                      &ctx->mfma_tab, &ctx->mfma_list, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     prof_collect(ctx);
@@ -274,6 +320,21 @@ int32_t vq_timer_stop(vq_ctx *ctx, float *h_ms) {
     VQ_HIP(ctx, hipEventRecord(ctx->ev1, ctx->stream));
     VQ_HIP(ctx, hipEventSynchronize(ctx->ev1));
     VQ_HIP(ctx, hipEventElapsedTime(h_ms, ctx->ev0, ctx->ev1));
+    return VQ_OK;
+}
+
+int32_t vq_ctx_set_assign_path(vq_ctx *ctx, int32_t path) {
+    if (!ctx || (path != 0 && path != 1)) return VQ_ERR_INVALID_ARG;
+    ctx->assign_path = path;
+    return VQ_OK;
+}
+
+int32_t vq_ctx_last_recheck_count(vq_ctx *ctx, uint32_t *h_count) {
+    if (!ctx || !h_count) return VQ_ERR_INVALID_ARG;
+    *h_count = 0;
+    if (!ctx->mfma_list.p) return VQ_OK;
+    VQ_HIP(ctx, hipMemcpyAsync(h_count, ctx->mfma_list.p, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return VQ_OK;
 }
 
