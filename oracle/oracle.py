@@ -52,6 +52,8 @@ def lib():
         L.vqo_tree_depth.argtypes = [_i64]
         L.vqo_mean_rows.restype = None
         L.vqo_mean_rows.argtypes = [_f32p, _i64, _i64, _i64, _u32p, _i64, _f32p]
+        L.vqo_mean_rows_parts.restype = None
+        L.vqo_mean_rows_parts.argtypes = [_f32p, _i64, _i64, _i64, _u32p, _i64, _i64, _f32p]
         L.vqo_lbg.restype = C.c_int
         L.vqo_lbg.argtypes = [_f32p, _i64, _i64, _i64, _i64, _i64, _i64, _u32p, _u32p, _i64,
                               _f32p, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -131,6 +133,17 @@ def mean_rows(x, rows, off=0, d=None):
     rows = _u32(rows)
     out = np.empty(d, np.float32)
     lib().vqo_mean_rows(x, ld, off, d, rows, rows.size, out)
+    return out
+
+
+def mean_rows_parts(x, rows, off=0, d=None):
+    """mean_vector in the order lbg_quantize uses (parts of 4096 rows above 1024 members)."""
+    x = _f32(x)
+    ld = x.shape[1]
+    d = ld - off if d is None else d
+    rows = _u32(rows)
+    out = np.empty(d, np.float32)
+    lib().vqo_mean_rows_parts(x, ld, off, d, rows, rows.size, x.shape[0], out)
     return out
 
 

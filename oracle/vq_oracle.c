@@ -25,14 +25,17 @@
  *                    deterministic order;
  *   >  1024 members: the reference uses a Rayon reduce whose tree depends on
  *                    work stealing (not reproducible even by the reference).
- *                    The oracle fixes ONE member of that family: split the
- *                    member list at its midpoint, recursively, to the uniform
- *                    depth d = min{d : count <= 1024 * 2^d}; every leaf is
- *                    summed sequentially from 0.0, siblings are added
- *                    left + right.  (Rayon splits slices at len/2 and folds
- *                    each leaf from the identity, so this tree is one the
- *                    reference can produce.)
- * PARITY UNPINNED (by construction of the reference): the >1024 tree shape.
+ *                    The oracle fixes ONE order per call site:
+ *      - inside lbg_quantize (vqo_mean_rows_parts): the rows are cut into parts
+ *        of 4096 consecutive row indices; the cluster's members inside a part are
+ *        added in row order from 0.0, and the per-part sums are added in part
+ *        order from 0.0.  (Chosen because it is a single streaming pass on the
+ *        GPU; it is a fixed order, not a tree Rayon would build.)
+ *      - for a TSVQ node (vqo_mean_rows): the member list is split at its
+ *        midpoint, recursively, to the uniform depth
+ *        d = min{d : count <= 1024 * 2^d}; leaves are summed sequentially from
+ *        0.0, siblings are added left + right (a tree Rayon can produce).
+ * PARITY UNPINNED (by construction of the reference): the order above 1024.
  *
  * Other places where the reference's own order is not fixed and the oracle
  * picks the sequential order: Rayon `sum` of residual norms (src/rvq.rs:131-138),
@@ -226,6 +229,31 @@ void vqo_mean_rows(const float *x, int64_t ld, int64_t off, int64_t d, const uin
     for (int64_t t = 0; t < d; ++t) out[t] = out[t] / n;
 }
 
+#define VQO_PART_ROWS 4096
+
+/* mean_vector as used inside lbg_quantize: rows[] ascending row indices of the
+ * cluster's members.  See the file header for the order above 1024 members. */
+void vqo_mean_rows_parts(const float *x, int64_t ld, int64_t off, int64_t d, const uint32_t *rows,
+                         int64_t count, int64_t n_rows, float *out) {
+    if (count <= VQO_PARALLEL_THRESHOLD) {
+        sum_seq(x, ld, off, d, rows, 0, count, out);
+    } else {
+        float *part = (float *)malloc(sizeof(float) * (size_t)d);
+        for (int64_t t = 0; t < d; ++t) out[t] = 0.0f;
+        int64_t p = 0;
+        int64_t nparts = (n_rows + VQO_PART_ROWS - 1) / VQO_PART_ROWS;
+        for (int64_t q = 0; q < nparts; ++q) {
+            int64_t lo = p;
+            while (p < count && (int64_t)rows[p] < (q + 1) * VQO_PART_ROWS) ++p;
+            sum_seq(x, ld, off, d, rows, lo, p, part); /* 0.0 for a part without members */
+            for (int64_t t = 0; t < d; ++t) out[t] = out[t] + part[t];
+        }
+        free(part);
+    }
+    float n = (float)(double)count;
+    for (int64_t t = 0; t < d; ++t) out[t] = out[t] / n;
+}
+
 /* ------------------------------------------------------------ L2: the LBG  */
 
 /* Nearest centroid under squared L2 with strict '<' (src/utils.rs:62-71). */
@@ -302,7 +330,7 @@ int vqo_lbg(const float *x, int64_t n, int64_t ld, int64_t off, int64_t d, int64
         for (int64_t j = 0; j < k; ++j) {
             int64_t cnt = start[j + 1] - start[j];
             if (cnt > 0) {
-                vqo_mean_rows(x, ld, off, d, members + start[j], cnt, centroids + j * d);
+                vqo_mean_rows_parts(x, ld, off, d, members + start[j], cnt, n, centroids + j * d);
             } else {
                 if (used >= n_reseed) {
                     rc = -3;

@@ -85,6 +85,24 @@ def mean_tree(rows, leaf=1024):
     return rec(0, c, depth) / F(np.float64(c))
 
 
+def mean_parts(X, rows, part=4096, seq_max=1024):
+    """The order used inside lbg_quantize: sequential up to 1024 members; above, per part of
+    4096 consecutive row indices a sequential sum from 0, parts added in order from 0."""
+    X = np.asarray(X, F)
+    rows = np.asarray(rows, np.int64)
+    c = len(rows)
+    if c <= seq_max:
+        return mean_seq(X[rows])
+    acc = np.zeros(X.shape[1], F)
+    for q in range((X.shape[0] + part - 1) // part):
+        sel = rows[(rows >= q * part) & (rows < (q + 1) * part)]
+        sub = np.zeros(X.shape[1], F)
+        for r in sel:
+            sub = sub + X[r]
+        acc = acc + sub
+    return acc / F(np.float64(c))
+
+
 def lbg(X, k, max_iters, init_idx, reseed_stream):
     X = np.asarray(X, F)
     n = X.shape[0]
@@ -97,9 +115,9 @@ def lbg(X, k, max_iters, init_idx, reseed_stream):
         changed = bool(np.any(new != assign))
         assign = new
         for j in range(k):
-            mem = X[assign == j]
+            mem = np.flatnonzero(assign == j)
             if len(mem):
-                cen[j] = mean_tree(mem)
+                cen[j] = mean_parts(X, mem)
             else:
                 cen[j] = X[int(reseed_stream[used])]
                 used += 1

@@ -49,6 +49,11 @@ LBG_CASES = [
     (300, 256, 1, 16, 3, "normal"),    # full-dimension problem (RVQ stage shape)
     (2049, 3, 3, 1, 4, "normal"),      # k = 1, sub_dim 1
     (50, 8, 1, 4, 0, "normal"),        # max_iters = 0 -> initial rows
+    (50000, 32, 4, 8, 4, "normal"),    # sub_dim 8: every cluster large -> streaming part sums
+    (30000, 32, 4, 24, 4, "skewed"),   # sub_dim 8: small and large clusters side by side
+    (70000, 16, 2, 3, 3, "same"),      # sub_dim 8: one huge cluster, empties re-seeded
+    (13000, 24, 3, 5, 3, "normal"),    # sub_dim 8 but m % 4 != 0 -> per-part leaves, gather path
+    (13000, 6, 1, 4, 3, "normal"),     # sub_dim 6, clusters above 1024 -> per-part leaves
 ]
 
 
@@ -63,6 +68,11 @@ def test_lbg_fit_matches_oracle_bitwise(ctx, n, dim, m, k, iters, kind):
         x = rng.uniform(-1000, 1000, (n, dim)).astype(F)  # tests/utils.rs:9-10
     elif kind == "grid":
         x = np.round(rng.standard_normal((n, dim)) * 1.5).astype(F)
+    elif kind == "skewed":  # a few tight far-away blobs with few rows + one broad mass
+        x = rng.standard_normal((n, dim)).astype(F)
+        for b in range(6):
+            x[b * 150:(b + 1) * 150] = (20.0 * (b + 1) + 0.01 * rng.standard_normal((150, dim))).astype(F)
+        x = x[rng.permutation(n)]
     else:
         x = np.tile(rng.standard_normal((1, dim)).astype(F), (n, 1))
     init, reseed = data.index_streams(n, m, k, iters, seed=n)

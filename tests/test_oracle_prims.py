@@ -150,6 +150,20 @@ def test_mean_tree_branch(c):
     assert np.allclose(got, exact, rtol=1e-4, atol=1e-3)
 
 
+@pytest.mark.parametrize("n,c", [(5000, 1025), (9000, 3000), (20000, 1500), (4096 * 3 + 5, 9000)])
+def test_mean_parts_order_used_by_lbg(n, c):
+    rng = np.random.default_rng(n + c)
+    x = (rng.standard_normal((n, 3)) * 100).astype(F)
+    rows = np.sort(rng.choice(n, c, replace=False))
+    got = O.mean_rows_parts(x, rows)
+    assert np.array_equal(got, np_ref.mean_parts(x, rows))
+    if n > 4096:  # more than one part: differs from the plain sequential sum
+        assert not np.array_equal(got, np_ref.mean_seq(x[rows]))
+    assert np.allclose(got, x[rows].astype(np.float64).mean(0), rtol=1e-4, atol=1e-3)
+    small = rows[:1024]  # at most 1024 members: the reference's sequential order
+    assert np.array_equal(O.mean_rows_parts(x, small), np_ref.mean_seq(x[small]))
+
+
 def test_tree_depth_rule():
     L = O.lib()
     assert L.vqo_tree_depth(1) == 0 and L.vqo_tree_depth(1024) == 0

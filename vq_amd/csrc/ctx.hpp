@@ -22,7 +22,7 @@ struct vq_ctx {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::string err;
     // grow-only device workspace
-    DevBuf flags, tables, hist, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;
+    DevBuf flags, tables, hist, seg, part_sum, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;
     DevBuf mfma_tab, mfma_list;  // tables and re-check list of the matrix-core assignment
     int assign_path = 0;         // 0 = matrix cores where a kernel exists, 1 = vector ALU only
     DevBuf tmp_a, tmp_b, tmp_c, tmp_d, tmp_e, tmp_f;  // scratch of the RVQ / OPQ / TSVQ entry points

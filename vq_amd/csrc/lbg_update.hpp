@@ -1,12 +1,18 @@
-// Centroid update of the LBG loop (src/utils.rs:83-102) as a deterministic segmented sum.
+// Centroid update of the LBG loop (src/utils.rs:83-102) as a deterministic ordered sum.
 //
 // The reference gathers the members of every cluster in row order and calls mean_vector
-// (src/vector.rs:282-318): a sequential f32 sum in row order for at most 1024 members.  To
-// reproduce that order bit for bit the rows are first grouped by code with a STABLE counting
-// sort (per-row-block histograms -> exclusive scan -> ranked scatter), then every cluster is
-// summed by walking its member list in order, one lane per (leaf, component).  Clusters above
-// 1024 members are split at the midpoint of the member list to the uniform depth
-// d = min{d : count <= 1024 << d}; leaves are summed sequentially and combined left + right.
+// (src/vector.rs:282-318).  Order of the f32 additions, per cluster:
+//   1..1024 members ("small"): one sequential sum in row order from 0.0 — the reference's own,
+//       deterministic order.  The rows of the small clusters are grouped by code with a STABLE
+//       counting sort (per-part histograms -> exclusive scans -> ballot-ranked scatter of row
+//       ids) and every cluster's list is walked by one lane per component.
+//   more than 1024 ("large"): the reference switches to a Rayon reduce whose tree depends on
+//       work stealing and cannot be reproduced even by itself.  Here the order is fixed as:
+//       the rows are cut into parts of 4096 consecutive rows; inside a part the cluster's
+//       members are added in row order from 0.0; the per-part sums are added in part order
+//       from 0.0.  For 32-byte sub-vectors this is one streaming pass over the rows
+//       (k_lbg_stream8) with the accumulators in LDS; other shapes take per-part leaves
+//       through the gather path.
 // No floating-point atomics anywhere; integer LDS atomics only for the histograms.
 #pragma once
 #include <hip/hip_runtime.h>
@@ -14,9 +20,10 @@
 
 namespace vq {
 
-constexpr int kRowBlock = 2048;      // rows per histogram block
+constexpr int kPartRows = 4096;      // rows per part (histogram block and summation part)
+constexpr int kScanSeg = 32;         // parts per scan segment
 constexpr int kMaxK = 256;           // codes are uint8
-constexpr int kLeafMax = 1024;       // PARALLEL_THRESHOLD, src/vector.rs:16
+constexpr int kSeqMax = 1024;        // PARALLEL_THRESHOLD, src/vector.rs:16
 
 struct LbgState {
     // per column block s
@@ -26,21 +33,25 @@ struct LbgState {
     int *used;             // m   re-seed entries consumed so far
     int *ubase;            // m   value of used[s] at the start of the current update
     int *nleaves;          // m
+    int *nsmall;           // m   clusters with 1..1024 members
     int *err;              // 1   set to 1 when a re-seed stream runs out
     // per (s, j)
     uint32_t *count;       // m*256
     uint32_t *start;       // m*256 first position of cluster j in perm[s]
     uint32_t *leaf_start;  // m*256
-    uint32_t *depth;       // m*256
     uint32_t *empty_rank;  // m*256 rank of an empty cluster among the empty clusters of s
     // bulk
-    uint32_t *hist;        // m*nblk*256 (histogram, then exclusive prefix over blocks)
+    uint32_t *hist;        // m*nparts*256 (histogram, then exclusive prefix over parts)
+    uint32_t *seg;         // m*nseg*256 (per-segment sums, then exclusive prefix over segments)
     uint32_t *perm;        // m*n  row ids grouped by code, row order inside a group
     uint2 *leaf_desc;      // m*leaf_cap  [lo, hi) positions in perm[s]
     float *leaf_sum;       // m*leaf_cap*sd
+    float *part_sum;       // m*nparts*256*8 per-part sums of the streaming kernel, or null
     uint8_t *codes;        // m*n  (column-block major)
-    int nblk;
+    int nparts;
+    int nseg;
     int leaf_cap;
+    int stream;            // 1: the large clusters are summed by k_lbg_stream8 / k_lbg_combine8
 };
 
 static __global__ void k_lbg_init(LbgState st, int m) {
@@ -52,6 +63,7 @@ static __global__ void k_lbg_init(LbgState st, int m) {
         st.used[s] = 0;
         st.ubase[s] = 0;
         st.nleaves[s] = 0;
+        st.nsmall[s] = 0;
     }
     if (s == 0) st.err[0] = 0;
 }
@@ -68,7 +80,7 @@ static __global__ void k_gather_rows(const float *__restrict__ x, int64_t ld, in
     cb[i] = x[(int64_t)idx[sj] * ld + (int64_t)s * sd + t];
 }
 
-// One wave per (row block, column block): histogram of the codes of kRowBlock rows.
+// One wave per (part, column block): histogram of the codes of kPartRows rows.
 static __global__ void __launch_bounds__(64) k_lbg_hist(LbgState st, int64_t n) {
     const int s = blockIdx.y, b = blockIdx.x;
     if (st.done[s]) return;
@@ -76,98 +88,138 @@ static __global__ void __launch_bounds__(64) k_lbg_hist(LbgState st, int64_t n) 
     for (int j = threadIdx.x; j < kMaxK; j += 64) cnt[j] = 0;
     __syncthreads();
     const uint8_t *codes = st.codes + (size_t)s * n;
-    int64_t lo = (int64_t)b * kRowBlock;
-    int64_t hi = lo + kRowBlock < n ? lo + kRowBlock : n;
+    int64_t lo = (int64_t)b * kPartRows;
+    int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
     for (int64_t i = lo + threadIdx.x; i < hi; i += 64) atomicAdd(&cnt[codes[i]], 1u);
     __syncthreads();
-    uint32_t *h = st.hist + ((size_t)s * st.nblk + b) * kMaxK;
+    uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
     for (int j = threadIdx.x; j < kMaxK; j += 64) h[j] = cnt[j];
 }
 
-__device__ __forceinline__ uint32_t tree_depth(uint32_t count) {
-    uint32_t d = 0;
-    while ((uint64_t)count > ((uint64_t)kLeafMax << d)) ++d;
-    return d;
+// Scan step 1: per (column block, segment of kScanSeg parts) sum of the histograms.
+static __global__ void __launch_bounds__(256) k_lbg_scan_seg(LbgState st) {
+    const int s = blockIdx.y, g = blockIdx.x, j = threadIdx.x;
+    if (st.done[s]) return;
+    const int b0 = g * kScanSeg, b1 = (b0 + kScanSeg < st.nparts) ? b0 + kScanSeg : st.nparts;
+    const uint32_t *h = st.hist + ((size_t)s * st.nparts + b0) * kMaxK + j;
+    uint32_t sum = 0;
+    for (int b = b0; b < b1; ++b) sum += h[(size_t)(b - b0) * kMaxK];
+    st.seg[((size_t)s * st.nseg + g) * kMaxK + j] = sum;
 }
 
-// One workgroup of 256 threads per column block; thread j owns cluster j.
-// Turns the histograms into exclusive prefixes over row blocks, derives cluster offsets,
-// tree depths, leaf descriptors, the rank of every empty cluster, and advances the re-seed
-// cursor by the number of empty clusters.
-static __global__ void __launch_bounds__(256) k_lbg_scan(LbgState st, int k) {
+// Scan step 2 ("plan"): one workgroup of 256 threads per column block; thread j owns cluster j.
+// Segment sums -> exclusive prefixes; per cluster: count, first position in perm, first leaf,
+// rank among the empty clusters; per column block: number of leaves and of small clusters, and
+// the re-seed cursor advanced by the number of empty clusters.
+// Leaves: a small cluster (1..1024 members) is one leaf over its whole member list; a large
+// cluster has one leaf per part, unless the streaming kernel sums the large clusters.
+static __global__ void __launch_bounds__(256) k_lbg_plan(LbgState st, int k) {
     const int s = blockIdx.x, j = threadIdx.x;
     if (st.done[s]) return;
-    __shared__ uint32_t sh_cnt[kMaxK], sh_leaf[kMaxK], sh_empty[kMaxK];
+    __shared__ uint32_t sh_cnt[kMaxK], sh_leaf[kMaxK], sh_empty[kMaxK], sh_small[kMaxK];
     uint32_t run = 0;
-    uint32_t *h = st.hist + (size_t)s * st.nblk * kMaxK + j;
-    for (int b = 0; b < st.nblk; ++b) {
-        uint32_t v = h[(size_t)b * kMaxK];
-        h[(size_t)b * kMaxK] = run;
-        run += v;
+    uint32_t *h = st.seg + (size_t)s * st.nseg * kMaxK + j;
+    for (int g0 = 0; g0 < st.nseg; g0 += 8) {
+        uint32_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = (g0 + u < st.nseg) ? h[(size_t)(g0 + u) * kMaxK] : 0u;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (g0 + u < st.nseg) h[(size_t)(g0 + u) * kMaxK] = run;
+            run += v[u];
+        }
     }
     const bool live = j < k;
-    uint32_t cnt = live ? run : 0;
-    uint32_t dep = tree_depth(cnt);
-    uint32_t nl = (live && cnt > 0) ? (1u << dep) : 0u;
-    uint32_t emp = (live && cnt == 0) ? 1u : 0u;
+    const uint32_t cnt = live ? run : 0;
+    const bool small = cnt > 0 && cnt <= (uint32_t)kSeqMax;
+    const bool big = cnt > (uint32_t)kSeqMax;
+    const uint32_t nl = small ? 1u : ((big && !st.stream) ? (uint32_t)st.nparts : 0u);
+    const uint32_t emp = (live && cnt == 0) ? 1u : 0u;
     sh_cnt[j] = cnt;
     sh_leaf[j] = nl;
     sh_empty[j] = emp;
+    sh_small[j] = small ? 1u : 0u;
     __syncthreads();
     // exclusive prefixes over j (k <= 256: a serial walk per thread is cheap and simple)
-    uint32_t pc = 0, pl = 0, pe = 0;
+    uint32_t pc = 0, pl = 0, pe = 0, ps = 0;
     for (int i = 0; i < j; ++i) {
         pc += sh_cnt[i];
         pl += sh_leaf[i];
         pe += sh_empty[i];
+        ps += sh_small[i];
     }
     const size_t sj = (size_t)s * kMaxK + j;
     st.count[sj] = cnt;
     st.start[sj] = pc;
     st.leaf_start[sj] = pl;
-    st.depth[sj] = dep;
     st.empty_rank[sj] = pe;
+    if (small) st.leaf_desc[(size_t)s * st.leaf_cap + pl] = make_uint2(pc, pc + cnt);
     if (j == kMaxK - 1) {
         st.nleaves[s] = (int)(pl + nl);
+        st.nsmall[s] = (int)(ps + (small ? 1u : 0u));
         int u = st.used[s];
         st.ubase[s] = u;
         st.used[s] = u + (int)(pe + emp);
     }
-    // leaf descriptors: leaf l of a depth-d tree is reached by taking bit (d-1-i) of l at level i
-    uint2 *desc = st.leaf_desc + (size_t)s * st.leaf_cap + pl;
-    for (uint32_t l = 0; l < nl; ++l) {
-        uint32_t lo = 0, hi = cnt;
-        for (int bit = (int)dep - 1; bit >= 0; --bit) {
-            uint32_t mid = lo + (hi - lo) / 2;
-            if ((l >> bit) & 1u)
-                lo = mid;
-            else
-                hi = mid;
+}
+
+// Scan step 3: per (column block, segment): histograms -> exclusive prefixes over parts (offset
+// of part b inside cluster j), in place; emits the per-part leaves of the large clusters when
+// they are summed by the gather path.
+static __global__ void __launch_bounds__(256) k_lbg_scan_blocks(LbgState st) {
+    const int s = blockIdx.y, g = blockIdx.x, j = threadIdx.x;
+    if (st.done[s]) return;
+    const int b0 = g * kScanSeg, b1 = (b0 + kScanSeg < st.nparts) ? b0 + kScanSeg : st.nparts;
+    uint32_t *h = st.hist + ((size_t)s * st.nparts + b0) * kMaxK + j;
+    uint32_t run = st.seg[((size_t)s * st.nseg + g) * kMaxK + j];
+    const size_t sj = (size_t)s * kMaxK + j;
+    const bool leaves = !st.stream && st.count[sj] > (uint32_t)kSeqMax;
+    const uint32_t first = st.start[sj];
+    uint2 *desc = st.leaf_desc + (size_t)s * st.leaf_cap + st.leaf_start[sj] + b0;
+    for (int c0 = 0; c0 < b1 - b0; c0 += 8) {
+        uint32_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = (b0 + c0 + u < b1) ? h[(size_t)(c0 + u) * kMaxK] : 0u;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            if (b0 + c0 + u < b1) {
+                h[(size_t)(c0 + u) * kMaxK] = run;
+                if (leaves) desc[c0 + u] = make_uint2(first + run, first + run + v[u]);
+            }
+            run += v[u];
         }
-        desc[l] = make_uint2(pc + lo, pc + hi);
     }
 }
 
-// One wave per (row block, column block): stable ranked scatter of row ids into perm[s].
+// One wave per (part, column block): stable ranked scatter of row ids into perm[s].  When the
+// streaming kernel sums the large clusters only the rows of small clusters are listed.
 static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t n) {
     const int s = blockIdx.y, b = blockIdx.x;
     if (st.done[s]) return;
+    if (st.stream && st.nsmall[s] == 0) return;
     __shared__ uint32_t base[kMaxK];
-    const uint32_t *h = st.hist + ((size_t)s * st.nblk + b) * kMaxK;
+    __shared__ uint8_t listed[kMaxK];
+    const uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
     const uint32_t *start = st.start + (size_t)s * kMaxK;
-    for (int j = threadIdx.x; j < kMaxK; j += 64) base[j] = start[j] + h[j];
+    const uint32_t *count = st.count + (size_t)s * kMaxK;
+    for (int j = threadIdx.x; j < kMaxK; j += 64) {
+        base[j] = start[j] + h[j];
+        listed[j] = (!st.stream || count[j] <= (uint32_t)kSeqMax) ? 1 : 0;
+    }
     __syncthreads();
     const uint8_t *codes = st.codes + (size_t)s * n;
     uint32_t *perm = st.perm + (size_t)s * n;
     const int lane = threadIdx.x;
     const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-    int64_t lo = (int64_t)b * kRowBlock;
-    int64_t hi = lo + kRowBlock < n ? lo + kRowBlock : n;
+    int64_t lo = (int64_t)b * kPartRows;
+    int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
     for (int64_t i0 = lo; i0 < hi; i0 += 64) {
         int64_t i = i0 + lane;
         bool valid = i < hi;
         uint32_t c = valid ? codes[i] : 0u;
+        valid = valid && listed[c];
         uint64_t mask = __ballot(valid);
+        if (mask == 0) continue;  // uniform
 #pragma unroll
         for (int bit = 0; bit < 8; ++bit) {
             bool set = (c >> bit) & 1u;
@@ -211,8 +263,9 @@ static __global__ void __launch_bounds__(256) k_lbg_leafsum(LbgState st, const f
     st.leaf_sum[((size_t)s * st.leaf_cap + leaf) * sd + t] = acc;
 }
 
-// One lane per (cluster, component): combine leaves left + right, divide by the count
-// (src/vector.rs:315-316), or copy the re-seed row for an empty cluster (src/utils.rs:98-101).
+// One lane per (cluster, component): the mean of a small cluster, the sequential fold over the
+// per-part leaves of a large one (gather path), or the re-seed row of an empty cluster
+// (src/vector.rs:315-316, src/utils.rs:98-101).
 static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const float *__restrict__ x,
                                                       int64_t ld, int k, int sd,
                                                       const uint32_t *__restrict__ reseed,
@@ -236,12 +289,155 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const 
         *out = x[(int64_t)r * ld + (int64_t)s * sd + t];
         return;
     }
-    uint32_t nl = 1u << st.depth[sj];
-    float *ls = st.leaf_sum + ((size_t)s * st.leaf_cap + st.leaf_start[sj]) * sd + t;
-    for (uint32_t h = 1; h < nl; h <<= 1)
-        for (uint32_t i = 0; i < nl; i += 2 * h) ls[(size_t)i * sd] = ls[(size_t)i * sd] + ls[(size_t)(i + h) * sd];
-    float nf = __uint2float_rn(cnt);
-    *out = ls[0] / nf;
+    const float *ls = st.leaf_sum + ((size_t)s * st.leaf_cap + st.leaf_start[sj]) * sd + t;
+    float sum;
+    if (cnt <= (uint32_t)kSeqMax) {
+        sum = ls[0];
+    } else {
+        if (st.stream) return;  // k_lbg_combine8 writes the large clusters
+        sum = 0.0f;
+        for (int p = 0; p < st.nparts; ++p) sum = sum + ls[(size_t)p * sd];
+    }
+    *out = sum / __uint2float_rn(cnt);
+}
+
+// ---- streaming sums of the large clusters (sub_dim 8, 4 column blocks per 128-byte line) ------
+// One wave per (part, group of 4 column blocks).  The wave walks its part 64 rows at a time; a
+// lane holds the 128-byte line of its row.  For every column block the rows of the chunk are
+// ranked inside their cluster with wave ballots, and added to the cluster's accumulator in LDS
+// in rank order (round r: the lanes of rank r, all on different clusters) — so every cluster
+// receives its rows of this part in row order, one at a time, starting from 0.0.
+// Emits the part's histogram and the per-part sums; no floating-point atomics.
+static __global__ void __launch_bounds__(64) k_lbg_stream8(LbgState st, const float *__restrict__ x, int64_t n,
+                                                           int64_t ld) {
+    const int g = blockIdx.y, b = blockIdx.x;
+    const int s0 = 4 * g;
+    bool act[4];
+    bool any = false;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        act[q] = st.done[s0 + q] == 0;
+        any |= act[q];
+    }
+    if (!any) return;
+    __shared__ float4 acc[4][kMaxK][2];
+    __shared__ uint32_t cnt[4][kMaxK];
+    const int lane = threadIdx.x;
+    for (int i = lane; i < 4 * kMaxK * 2; i += 64) (&acc[0][0][0])[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = lane; i < 4 * kMaxK; i += 64) (&cnt[0][0])[i] = 0u;
+    __syncthreads();
+    const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    const int64_t lo = (int64_t)b * kPartRows;
+    const int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
+    float4 v[8], vn[8];
+    {
+        const int64_t i = lo + lane;
+        if (i < hi) {
+            const float4 *xr = reinterpret_cast<const float4 *>(x + i * ld + (int64_t)s0 * 8);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) vn[u] = xr[u];
+        }
+    }
+    for (int64_t i0 = lo; i0 < hi; i0 += 64) {
+        const int64_t i = i0 + lane;
+        const bool valid = i < hi;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = vn[u];
+        {
+            const int64_t in = i + 64;  // next chunk, fetched while this one is processed
+            if (in < hi) {
+                const float4 *xr = reinterpret_cast<const float4 *>(x + in * ld + (int64_t)s0 * 8);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) vn[u] = xr[u];
+            }
+        }
+        uint32_t c[4], rank[4];
+        uint32_t maxtot = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            c[q] = 0;
+            rank[q] = 0xFFFFFFFFu;
+            if (!act[q]) continue;  // uniform
+            c[q] = valid ? st.codes[(size_t)(s0 + q) * n + i] : 0u;
+            uint64_t mask = __ballot(valid);
+#pragma unroll
+            for (int bit = 0; bit < 8; ++bit) {
+                bool set = (c[q] >> bit) & 1u;
+                uint64_t bal = __ballot(set);
+                mask &= set ? bal : ~bal;
+            }
+            const uint32_t r = (uint32_t)__popcll(mask & lt);
+            const uint32_t tot = (uint32_t)__popcll(mask);
+            if (valid) {
+                rank[q] = r;
+                if (r == 0) cnt[q][c[q]] += tot;  // one lane per cluster
+                maxtot = tot > maxtot ? tot : maxtot;
+            }
+        }
+        // number of rounds = largest multiplicity of a cluster in this chunk, over the wave
+        uint32_t rounds = maxtot;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            uint32_t o = __shfl_xor(rounds, off);
+            rounds = o > rounds ? o : rounds;
+        }
+        for (uint32_t r = 0; r < rounds; ++r) {
+            float4 a0[4], a1[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (rank[q] == r) {
+                    a0[q] = acc[q][c[q]][0];
+                    a1[q] = acc[q][c[q]][1];
+                }
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (rank[q] == r) {
+                    a0[q].x = a0[q].x + v[2 * q].x;
+                    a0[q].y = a0[q].y + v[2 * q].y;
+                    a0[q].z = a0[q].z + v[2 * q].z;
+                    a0[q].w = a0[q].w + v[2 * q].w;
+                    a1[q].x = a1[q].x + v[2 * q + 1].x;
+                    a1[q].y = a1[q].y + v[2 * q + 1].y;
+                    a1[q].z = a1[q].z + v[2 * q + 1].z;
+                    a1[q].w = a1[q].w + v[2 * q + 1].w;
+                    acc[q][c[q]][0] = a0[q];
+                    acc[q][c[q]][1] = a1[q];
+                }
+            __syncthreads();  // single wave: round r is complete before round r + 1 reads
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        if (!act[q]) continue;
+        float4 *ps = reinterpret_cast<float4 *>(st.part_sum) + ((size_t)(s0 + q) * st.nparts + b) * kMaxK * 2;
+        for (int i = lane; i < kMaxK * 2; i += 64) ps[i] = (&acc[q][0][0])[i];
+        uint32_t *h = st.hist + ((size_t)(s0 + q) * st.nparts + b) * kMaxK;
+        for (int j = lane; j < kMaxK; j += 64) h[j] = cnt[q][j];
+    }
+}
+
+// One lane per (cluster, component): sequential fold of the per-part sums of a large cluster.
+static __global__ void __launch_bounds__(256) k_lbg_combine8(LbgState st, int k, float *__restrict__ cb) {
+    const int s = blockIdx.y;
+    if (st.done[s]) return;
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    const int j = gid / 8, t = gid % 8;
+    if (j >= k) return;
+    const uint32_t cnt = st.count[(size_t)s * kMaxK + j];
+    if (cnt <= (uint32_t)kSeqMax) return;
+    const float *ps = st.part_sum + ((size_t)s * st.nparts * kMaxK + j) * 8 + t;
+    float sum = 0.0f;
+    int p = 0;
+    for (; p + 8 <= st.nparts; p += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = ps[(size_t)(p + u) * kMaxK * 8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum = sum + v[u];
+    }
+    for (; p < st.nparts; ++p) sum = sum + ps[(size_t)p * kMaxK * 8];
+    cb[((size_t)s * k + j) * 8 + t] = sum / __uint2float_rn(cnt);
 }
 
 // Loop control of src/utils.rs:57,104-106, one thread per column block.

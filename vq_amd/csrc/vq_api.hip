@@ -257,7 +257,7 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
-                      &ctx->mfma_tab, &ctx->mfma_list, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
+                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     prof_collect(ctx);
@@ -396,12 +396,19 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
     VQ_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
 
-    const int nblk = (int)((n + vq::kRowBlock - 1) / vq::kRowBlock);
-    const int leaf_cap = (int)(k + n / 512 + 1);
-    VQ_TRY(ensure(ctx, ctx->flags, sizeof(int) * (6 * (size_t)m + 1)));
-    VQ_TRY(ensure(ctx, ctx->tables, sizeof(uint32_t) * 5 * (size_t)m * vq::kMaxK));
-    VQ_TRY(ensure(ctx, ctx->hist, sizeof(uint32_t) * (size_t)m * nblk * vq::kMaxK));
+    const int nparts = (int)((n + vq::kPartRows - 1) / vq::kPartRows);
+    const int nseg = (nparts + vq::kScanSeg - 1) / vq::kScanSeg;
+    // streaming sums of the large clusters: 32-byte sub-vectors, 4 per 128-byte line, aligned rows
+    const bool stream = sd == 8 && m % 4 == 0 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0;
+    const int64_t leaf_cap64 = stream ? (int64_t)k : (int64_t)k * nparts;
+    if (leaf_cap64 * sd > (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * k * sub_dim too large");
+    const int leaf_cap = (int)leaf_cap64;
+    VQ_TRY(ensure(ctx, ctx->flags, sizeof(int) * (7 * (size_t)m + 1)));
+    VQ_TRY(ensure(ctx, ctx->tables, sizeof(uint32_t) * 4 * (size_t)m * vq::kMaxK));
+    VQ_TRY(ensure(ctx, ctx->hist, sizeof(uint32_t) * (size_t)m * nparts * vq::kMaxK));
+    VQ_TRY(ensure(ctx, ctx->seg, sizeof(uint32_t) * (size_t)m * nseg * vq::kMaxK));
     VQ_TRY(ensure(ctx, ctx->perm, sizeof(uint32_t) * (size_t)m * n));
+    if (stream) VQ_TRY(ensure(ctx, ctx->part_sum, sizeof(float) * (size_t)m * nparts * vq::kMaxK * 8));
     VQ_TRY(ensure(ctx, ctx->leaf_desc, sizeof(uint2) * (size_t)m * leaf_cap));
     VQ_TRY(ensure(ctx, ctx->leaf_sum, sizeof(float) * (size_t)m * leaf_cap * sd));
     VQ_TRY(ensure(ctx, ctx->codes, (size_t)m * n));
@@ -416,21 +423,25 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
     S.used = f + 3 * m;
     S.ubase = f + 4 * m;
     S.nleaves = f + 5 * m;
-    S.err = f + 6 * m;
+    S.nsmall = f + 6 * m;
+    S.err = f + 7 * m;
     uint32_t *tb = (uint32_t *)ctx->tables.p;
     const size_t mk = (size_t)m * vq::kMaxK;
     S.count = tb;
     S.start = tb + mk;
     S.leaf_start = tb + 2 * mk;
-    S.depth = tb + 3 * mk;
-    S.empty_rank = tb + 4 * mk;
+    S.empty_rank = tb + 3 * mk;
     S.hist = (uint32_t *)ctx->hist.p;
+    S.seg = (uint32_t *)ctx->seg.p;
     S.perm = (uint32_t *)ctx->perm.p;
     S.leaf_desc = (uint2 *)ctx->leaf_desc.p;
     S.leaf_sum = (float *)ctx->leaf_sum.p;
+    S.part_sum = stream ? (float *)ctx->part_sum.p : nullptr;
     S.codes = (uint8_t *)ctx->codes.p;
-    S.nblk = nblk;
+    S.nparts = nparts;
+    S.nseg = nseg;
     S.leaf_cap = leaf_cap;
+    S.stream = stream ? 1 : 0;
 
     VQ_HIP(ctx, hipMemcpyAsync(ctx->idx.p, h_init_idx, sizeof(uint32_t) * (size_t)m * k,
                                hipMemcpyHostToDevice, st));
@@ -461,23 +472,31 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
             VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd));
         }
         ProfSpan sp(ctx, VQ_PROF_LBG_UPDATE);
-        hipLaunchKernelGGL(vq::k_lbg_hist, dim3(nblk, m), dim3(64), 0, st, S, n);
-        hipLaunchKernelGGL(vq::k_lbg_scan, dim3(m), dim3(256), 0, st, S, k);
-        hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nblk, m), dim3(64), 0, st, S, n);
-        hipLaunchKernelGGL(vq::k_lbg_leafsum, dim3(cdiv((int64_t)leaf_cap * sd, 256), m), dim3(256), 0,
-                           st, S, d_x, n, ld, sd);
+        if (stream)
+            hipLaunchKernelGGL(vq::k_lbg_stream8, dim3(nparts, m / 4), dim3(64), 0, st, S, d_x, n, ld);
+        else
+            hipLaunchKernelGGL(vq::k_lbg_hist, dim3(nparts, m), dim3(64), 0, st, S, n);
+        hipLaunchKernelGGL(vq::k_lbg_scan_seg, dim3(nseg, m), dim3(256), 0, st, S);
+        hipLaunchKernelGGL(vq::k_lbg_plan, dim3(m), dim3(256), 0, st, S, k);
+        hipLaunchKernelGGL(vq::k_lbg_scan_blocks, dim3(nseg, m), dim3(256), 0, st, S);
+        if (stream)
+            hipLaunchKernelGGL(vq::k_lbg_combine8, dim3(cdiv((int64_t)k * 8, 256), m), dim3(256), 0, st, S, k,
+                               d_codebooks);
+        hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nparts, m), dim3(64), 0, st, S, n);
+        hipLaunchKernelGGL(vq::k_lbg_leafsum, dim3(cdiv((int64_t)leaf_cap * sd, 256), m), dim3(256), 0, st, S,
+                           d_x, n, ld, sd);
         hipLaunchKernelGGL(vq::k_lbg_finalize, dim3(cdiv((int64_t)k * sd, 256), m), dim3(256), 0, st, S,
                            d_x, ld, k, sd, (const uint32_t *)ctx->reseed.p, n_reseed, d_codebooks);
         hipLaunchKernelGGL(vq::k_lbg_advance, dim3(cdiv(m, 64)), dim3(64), 0, st, S, m);
         VQ_HIP(ctx, hipGetLastError());
     }
-    std::vector<int> host(6 * (size_t)m + 1);
+    std::vector<int> host(7 * (size_t)m + 1);
     VQ_HIP(ctx, hipMemcpyAsync(host.data(), f, sizeof(int) * host.size(), hipMemcpyDeviceToHost, st));
     VQ_HIP(ctx, hipStreamSynchronize(st));
     prof_collect(ctx);
     if (h_iters_run) memcpy(h_iters_run, host.data() + 2 * m, sizeof(int) * m);
     if (h_reseeds_used) memcpy(h_reseeds_used, host.data() + 3 * m, sizeof(int) * m);
-    if (host[6 * (size_t)m])
+    if (host[7 * (size_t)m])
         return fail(ctx, VQ_ERR_RESEED_EXHAUSTED,
                     "re-seed stream exhausted: pass n_reseed = k*max_iters");
     return VQ_OK;
