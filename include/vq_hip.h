@@ -95,10 +95,12 @@ int32_t vq_timer_stop(vq_ctx *ctx, float *h_ms);
  * accumulators.  vq_prof_read synchronises the stream and returns the summed event time and
  * the number of timed spans of one class. */
 enum vq_prof_class {
-    VQ_PROF_LBG_ASSIGN = 0, /* the assignment kernel of one LBG iteration (utils.rs:59-73) */
+    VQ_PROF_LBG_ASSIGN = 0, /* the assignment kernels of one LBG iteration (utils.rs:59-73) */
     VQ_PROF_LBG_UPDATE = 1, /* the update kernels of one LBG iteration (utils.rs:83-102) */
-    VQ_PROF_ENCODE = 2,     /* the kernel of one vq_assign call */
-    VQ_PROF_CLASSES = 3
+    VQ_PROF_ENCODE = 2,     /* the kernels of one vq_assign call */
+    VQ_PROF_ASSIGN_KERNEL = 3, /* the main assignment kernel alone (matrix-core pass or the
+                                  vector-ALU kernel), in training and in vq_assign */
+    VQ_PROF_CLASSES = 4
 };
 int32_t vq_prof_enable(vq_ctx *ctx, int32_t on);
 int32_t vq_prof_read(vq_ctx *ctx, int32_t cls, double *h_total_ms, int64_t *h_spans);

@@ -16,7 +16,7 @@ ERR_INVALID_ARG, ERR_DIM_MISMATCH, ERR_EMPTY_INPUT = -1, -2, -3
 ERR_UNSUPPORTED, ERR_OOM, ERR_HIP, ERR_RESEED_EXHAUSTED = -4, -5, -6, -7
 
 SQEUCLIDEAN, EUCLIDEAN, COSINE, MANHATTAN = 0, 1, 2, 3
-PROF_LBG_ASSIGN, PROF_LBG_UPDATE, PROF_ENCODE = 0, 1, 2
+PROF_LBG_ASSIGN, PROF_LBG_UPDATE, PROF_ENCODE, PROF_ASSIGN_KERNEL = 0, 1, 2, 3
 
 # every symbol include/vq_hip.h declares: name -> (restype, argtypes)
 _vp, _i32, _i64, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_size_t

@@ -99,7 +99,9 @@ __device__ __forceinline__ int imed3(int a, int b, int c) {
 }
 
 // One wave = TILES tiles of 32 rows, all column blocks.  256 threads = 4 waves.
-template <int SD, bool LBG, int TILES>
+// The sub-vectors of SG consecutive column blocks are loaded together, so that with SG * SD * 4
+// = 128 bytes every line of the rows is fetched once.
+template <int SD, bool LBG, int TILES, int SG>
 __global__ void __launch_bounds__(256) k_assign_mfma(AssignArgs a, MfmaTables tb) {
     constexpr int HS = SD / 2;     // floats per lane of a sub-vector
     extern __shared__ float lds_c2[];  // [m][nb][2][16]
@@ -125,7 +127,27 @@ __global__ void __launch_bounds__(256) k_assign_mfma(AssignArgs a, MfmaTables tb
 #pragma unroll
         for (int w = 0; w < MAXW; ++w) cw[t][w] = 0u;
 
-    for (int s = 0; s < m; ++s) {
+    for (int s0 = 0; s0 < m; s0 += SG) {
+      float xall[TILES][SG][HS];
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) {
+          const int64_t row = row_base + 32 * t + r;
+          if (row < a.n) {
+              const float *xr = a.x + row * a.ld + (int64_t)s0 * SD + h * HS;
+#pragma unroll
+              for (int q = 0; q < SG; ++q)
+#pragma unroll
+                  for (int u = 0; u < HS; ++u) xall[t][q][u] = xr[q * SD + u];
+          } else {
+#pragma unroll
+              for (int q = 0; q < SG; ++q)
+#pragma unroll
+                  for (int u = 0; u < HS; ++u) xall[t][q][u] = 0.0f;
+          }
+      }
+#pragma unroll
+      for (int q = 0; q < SG; ++q) {
+        const int s = s0 + q;
         if constexpr (LBG) {
             if (a.done[s]) continue;
         }
@@ -133,18 +155,11 @@ __global__ void __launch_bounds__(256) k_assign_mfma(AssignArgs a, MfmaTables tb
         int m1[TILES], m2[TILES];
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
-            const int64_t row = row_base + 32 * t + r;
             float p = 0.0f;
-            if (row < a.n) {
-                const float *xr = a.x + row * a.ld + (int64_t)s * SD + h * HS;
 #pragma unroll
-                for (int u = 0; u < HS; ++u) {
-                    xb[t][u] = xr[u];
-                    p = __builtin_fmaf(xb[t][u], xb[t][u], p);
-                }
-            } else {
-#pragma unroll
-                for (int u = 0; u < HS; ++u) xb[t][u] = 0.0f;
+            for (int u = 0; u < HS; ++u) {
+                xb[t][u] = xall[t][q][u];
+                p = __builtin_fmaf(xb[t][u], xb[t][u], p);
             }
             x2[t] = p + __shfl_xor(p, 32);
             m1[t] = 0x7f800000;  // +inf
@@ -213,6 +228,7 @@ __global__ void __launch_bounds__(256) k_assign_mfma(AssignArgs a, MfmaTables tb
             }
         }
     }
+    }  // column-block group
     if constexpr (!LBG) {
         if (packed_out && h == 0) {
 #pragma unroll

@@ -199,6 +199,7 @@ static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t 
     if (st.stream && st.nsmall[s] == 0) return;
     __shared__ uint32_t base[kMaxK];
     __shared__ uint8_t listed[kMaxK];
+    __shared__ uint8_t pcodes[kPartRows];
     const uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
     const uint32_t *start = st.start + (size_t)s * kMaxK;
     const uint32_t *count = st.count + (size_t)s * kMaxK;
@@ -206,17 +207,18 @@ static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t 
         base[j] = start[j] + h[j];
         listed[j] = (!st.stream || count[j] <= (uint32_t)kSeqMax) ? 1 : 0;
     }
-    __syncthreads();
     const uint8_t *codes = st.codes + (size_t)s * n;
     uint32_t *perm = st.perm + (size_t)s * n;
     const int lane = threadIdx.x;
     const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     int64_t lo = (int64_t)b * kPartRows;
     int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
+    for (int64_t i = lo + lane; i < hi; i += 64) pcodes[i - lo] = codes[i];  // one round trip
+    __syncthreads();
     for (int64_t i0 = lo; i0 < hi; i0 += 64) {
         int64_t i = i0 + lane;
         bool valid = i < hi;
-        uint32_t c = valid ? codes[i] : 0u;
+        uint32_t c = valid ? pcodes[i - lo] : 0u;
         valid = valid && listed[c];
         uint64_t mask = __ballot(valid);
         if (mask == 0) continue;  // uniform
@@ -231,9 +233,9 @@ static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t 
         uint32_t tot = (uint32_t)__popcll(mask);
         uint32_t pos = 0;
         if (valid) pos = base[c] + rank;
-        __syncthreads();  // single wave: orders the reads above before the updates below
+        __builtin_amdgcn_wave_barrier();  // one wave, LDS in program order: reads above, updates below
         if (valid && rank == 0) base[c] += tot;
-        __syncthreads();
+        __builtin_amdgcn_wave_barrier();
         if (valid) perm[pos] = (uint32_t)i;
     }
 }
@@ -252,12 +254,26 @@ static __global__ void __launch_bounds__(256) k_lbg_leafsum(LbgState st, const f
     const float *__restrict__ xc = x + (int64_t)s * sd + t;
     float acc = 0.0f;
     uint32_t p = d.x;
-    for (; p + 8 <= d.y; p += 8) {
-        float v[8];
+    // batches of 32 members: the loads of a batch are independent, the adds stay in list order;
+    // the row ids of the next batch are fetched while the current rows are in flight
+    constexpr int B = 32;
+    uint32_t r[B], rn[B];
+    if (p + B <= d.y) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = xc[(int64_t)perm[p + u] * ld];
+        for (int u = 0; u < B; ++u) rn[u] = perm[p + u];
+    }
+    for (; p + B <= d.y; p += B) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) acc = acc + v[u];
+        for (int u = 0; u < B; ++u) r[u] = rn[u];
+        float v[B];
+#pragma unroll
+        for (int u = 0; u < B; ++u) v[u] = xc[(int64_t)r[u] * ld];
+        if (p + 2 * B <= d.y) {
+#pragma unroll
+            for (int u = 0; u < B; ++u) rn[u] = perm[p + B + u];
+        }
+#pragma unroll
+        for (int u = 0; u < B; ++u) acc = acc + v[u];
     }
     for (; p < d.y; ++p) acc = acc + xc[(int64_t)perm[p] * ld];
     st.leaf_sum[((size_t)s * st.leaf_cap + leaf) * sd + t] = acc;
@@ -302,119 +318,104 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const 
 }
 
 // ---- streaming sums of the large clusters (sub_dim 8, 4 column blocks per 128-byte line) ------
-// One wave per (part, group of 4 column blocks).  The wave walks its part 64 rows at a time; a
-// lane holds the 128-byte line of its row.  For every column block the rows of the chunk are
-// ranked inside their cluster with wave ballots, and added to the cluster's accumulator in LDS
-// in rank order (round r: the lanes of rank r, all on different clusters) — so every cluster
-// receives its rows of this part in row order, one at a time, starting from 0.0.
-// Emits the part's histogram and the per-part sums; no floating-point atomics.
-static __global__ void __launch_bounds__(64) k_lbg_stream8(LbgState st, const float *__restrict__ x, int64_t n,
-                                                           int64_t ld) {
+// One workgroup per (part, group of 4 column blocks); wave w of the group owns column block
+// 4g + w, so the four waves together consume whole 128-byte lines of the rows.  A wave walks
+// its part 64 rows at a time; a lane holds the 32-byte sub-vector of its row.  The rows of a
+// chunk are ranked inside their cluster with wave ballots and added to the cluster's
+// accumulator in LDS in rank order (round r: the lanes of rank r, all on different clusters) —
+// so every cluster receives its rows of this part in row order, one at a time, starting from
+// 0.0.  Emits the part's histogram and the per-part sums; no floating-point atomics.
+static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const float *__restrict__ x, int64_t n,
+                                                            int64_t ld) {
     const int g = blockIdx.y, b = blockIdx.x;
-    const int s0 = 4 * g;
-    bool act[4];
-    bool any = false;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        act[q] = st.done[s0 + q] == 0;
-        any |= act[q];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int s = 4 * g + w;
+    __shared__ float4 acc_all[4][kMaxK][2];
+    __shared__ uint32_t cnt_all[4][kMaxK];
+    if (st.done[s]) return;  // uniform per wave; the waves never synchronise with each other
+    float4(*acc)[2] = acc_all[w];
+    uint32_t *cnt = cnt_all[w];
+    for (int i = lane; i < kMaxK; i += 64) {
+        acc[i][0] = make_float4(0.f, 0.f, 0.f, 0.f);
+        acc[i][1] = make_float4(0.f, 0.f, 0.f, 0.f);
+        cnt[i] = 0u;
     }
-    if (!any) return;
-    __shared__ float4 acc[4][kMaxK][2];
-    __shared__ uint32_t cnt[4][kMaxK];
-    const int lane = threadIdx.x;
-    for (int i = lane; i < 4 * kMaxK * 2; i += 64) (&acc[0][0][0])[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int i = lane; i < 4 * kMaxK; i += 64) (&cnt[0][0])[i] = 0u;
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
     const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     const int64_t lo = (int64_t)b * kPartRows;
     const int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
-    float4 v[8], vn[8];
-    {
-        const int64_t i = lo + lane;
-        if (i < hi) {
-            const float4 *xr = reinterpret_cast<const float4 *>(x + i * ld + (int64_t)s0 * 8);
+    const uint8_t *__restrict__ codes = st.codes + (size_t)s * n;
+    // The sub-vectors and codes of the next PF chunks are kept in flight: one chunk's arithmetic
+    // is far shorter than a memory round trip.
+    constexpr int PF = 4;
+    float4 b0[PF], b1[PF];
+    uint32_t bc[PF];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) vn[u] = xr[u];
+    for (int u = 0; u < PF; ++u) {
+        b0[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        b1[u] = b0[u];
+        bc[u] = 0u;
+        const int64_t i = lo + 64 * u + lane;
+        if (i < hi) {
+            const float4 *xr = reinterpret_cast<const float4 *>(x + i * ld + (int64_t)s * 8);
+            b0[u] = xr[0];
+            b1[u] = xr[1];
+            bc[u] = codes[i];
         }
     }
-    for (int64_t i0 = lo; i0 < hi; i0 += 64) {
-        const int64_t i = i0 + lane;
-        const bool valid = i < hi;
+    for (int64_t base = lo; base < hi; base += 64 * PF) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = vn[u];
-        {
-            const int64_t in = i + 64;  // next chunk, fetched while this one is processed
-            if (in < hi) {
-                const float4 *xr = reinterpret_cast<const float4 *>(x + in * ld + (int64_t)s0 * 8);
-#pragma unroll
-                for (int u = 0; u < 8; ++u) vn[u] = xr[u];
+        for (int u = 0; u < PF; ++u) {
+            const int64_t i0 = base + 64 * u;
+            if (i0 >= hi) break;  // uniform
+            const int64_t i = i0 + lane;
+            const bool valid = i < hi;
+            const float4 v0 = b0[u], v1 = b1[u];
+            const uint32_t c = valid ? bc[u] : 0u;
+            {
+                const int64_t in = i + 64 * PF;
+                if (in < hi) {
+                    const float4 *xr = reinterpret_cast<const float4 *>(x + in * ld + (int64_t)s * 8);
+                    b0[u] = xr[0];
+                    b1[u] = xr[1];
+                    bc[u] = codes[in];
+                }
             }
-        }
-        uint32_t c[4], rank[4];
-        uint32_t maxtot = 0;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            c[q] = 0;
-            rank[q] = 0xFFFFFFFFu;
-            if (!act[q]) continue;  // uniform
-            c[q] = valid ? st.codes[(size_t)(s0 + q) * n + i] : 0u;
             uint64_t mask = __ballot(valid);
 #pragma unroll
             for (int bit = 0; bit < 8; ++bit) {
-                bool set = (c[q] >> bit) & 1u;
+                bool set = (c >> bit) & 1u;
                 uint64_t bal = __ballot(set);
                 mask &= set ? bal : ~bal;
             }
-            const uint32_t r = (uint32_t)__popcll(mask & lt);
-            const uint32_t tot = (uint32_t)__popcll(mask);
-            if (valid) {
-                rank[q] = r;
-                if (r == 0) cnt[q][c[q]] += tot;  // one lane per cluster
-                maxtot = tot > maxtot ? tot : maxtot;
+            const uint32_t rank = valid ? (uint32_t)__popcll(mask & lt) : 0xFFFFFFFFu;
+            if (rank == 0) cnt[c] += (uint32_t)__popcll(mask);  // one lane per cluster
+            for (uint32_t r = 0; __any(rank != 0xFFFFFFFFu && rank >= r); ++r) {
+                if (rank == r) {
+                    float4 a0 = acc[c][0], a1 = acc[c][1];
+                    a0.x = a0.x + v0.x;
+                    a0.y = a0.y + v0.y;
+                    a0.z = a0.z + v0.z;
+                    a0.w = a0.w + v0.w;
+                    a1.x = a1.x + v1.x;
+                    a1.y = a1.y + v1.y;
+                    a1.z = a1.z + v1.z;
+                    a1.w = a1.w + v1.w;
+                    acc[c][0] = a0;
+                    acc[c][1] = a1;
+                }
+                // LDS accesses of one wave are performed in program order, so the next round
+                // sees these writes; the barrier below only pins the compiler's schedule (a
+                // fence or s_barrier here would also wait for the row prefetches in flight)
+                __builtin_amdgcn_wave_barrier();
             }
         }
-        // number of rounds = largest multiplicity of a cluster in this chunk, over the wave
-        uint32_t rounds = maxtot;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            uint32_t o = __shfl_xor(rounds, off);
-            rounds = o > rounds ? o : rounds;
-        }
-        for (uint32_t r = 0; r < rounds; ++r) {
-            float4 a0[4], a1[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (rank[q] == r) {
-                    a0[q] = acc[q][c[q]][0];
-                    a1[q] = acc[q][c[q]][1];
-                }
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (rank[q] == r) {
-                    a0[q].x = a0[q].x + v[2 * q].x;
-                    a0[q].y = a0[q].y + v[2 * q].y;
-                    a0[q].z = a0[q].z + v[2 * q].z;
-                    a0[q].w = a0[q].w + v[2 * q].w;
-                    a1[q].x = a1[q].x + v[2 * q + 1].x;
-                    a1[q].y = a1[q].y + v[2 * q + 1].y;
-                    a1[q].z = a1[q].z + v[2 * q + 1].z;
-                    a1[q].w = a1[q].w + v[2 * q + 1].w;
-                    acc[q][c[q]][0] = a0[q];
-                    acc[q][c[q]][1] = a1[q];
-                }
-            __syncthreads();  // single wave: round r is complete before round r + 1 reads
-        }
     }
-    __syncthreads();
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        if (!act[q]) continue;
-        float4 *ps = reinterpret_cast<float4 *>(st.part_sum) + ((size_t)(s0 + q) * st.nparts + b) * kMaxK * 2;
-        for (int i = lane; i < kMaxK * 2; i += 64) ps[i] = (&acc[q][0][0])[i];
-        uint32_t *h = st.hist + ((size_t)(s0 + q) * st.nparts + b) * kMaxK;
-        for (int j = lane; j < kMaxK; j += 64) h[j] = cnt[q][j];
-    }
+    __builtin_amdgcn_wave_barrier();
+    float4 *ps = reinterpret_cast<float4 *>(st.part_sum) + ((size_t)s * st.nparts + b) * kMaxK * 2;
+    for (int i = lane; i < kMaxK * 2; i += 64) ps[i] = (&acc[0][0])[i];
+    uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
+    for (int j = lane; j < kMaxK; j += 64) h[j] = cnt[j];
 }
 
 // One lane per (cluster, component): sequential fold of the per-part sums of a large cluster.

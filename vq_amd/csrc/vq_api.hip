@@ -16,7 +16,7 @@
 #include "assign_mfma.hpp"
 
 #ifndef VQ_MFMA_TILES
-#define VQ_MFMA_TILES 4  // tiles of 32 rows per wave in the matrix-core assignment
+#define VQ_MFMA_TILES 2  // tiles of 32 rows per wave in the matrix-core assignment
 #endif
 #include "lbg_update.hpp"
 
@@ -44,7 +44,10 @@ int32_t launch_static(vq_ctx *ctx, const vq::AssignArgs &a) {
     int64_t tiles = (a.n + 255) / 256;
     int64_t blocks = tiles * (a.m / G);
     if (blocks > 0x7fffffffLL) return fail(ctx, VQ_ERR_UNSUPPORTED, "grid too large");
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, ctx->stream, a);
+    {
+        ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, ctx->stream, a);
+    }
     VQ_HIP(ctx, hipGetLastError());
     return VQ_OK;
 }
@@ -105,11 +108,15 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
     vq::MfmaTables tb{atab, c2perm, maxc2, list, count, nb};
     const size_t lds = sizeof(float) * n_c2;
     constexpr int TILES = VQ_MFMA_TILES;
-    auto kern = vq::k_assign_mfma<SD, LBG, TILES>;
+    // 4 column blocks of 8 floats = one 128-byte line per row
+    auto kern = (a.m % 4 == 0) ? vq::k_assign_mfma<SD, LBG, TILES, 4> : vq::k_assign_mfma<SD, LBG, TILES, 1>;
     if (lds > 48 * 1024)
         VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kern, dim3(cdiv(a.n, 4 * 32 * TILES)), dim3(256), lds, ctx->stream, a, tb);
+    {
+        ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
+        hipLaunchKernelGGL(kern, dim3(cdiv(a.n, 4 * 32 * TILES)), dim3(256), lds, ctx->stream, a, tb);
+    }
     hipLaunchKernelGGL((vq::k_assign_recheck<SD, METRIC, LBG>), dim3(1024), dim3(256), 0, ctx->stream, a,
                        (const uint32_t *)list, (const uint32_t *)count);
     VQ_HIP(ctx, hipGetLastError());
@@ -473,7 +480,7 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
         }
         ProfSpan sp(ctx, VQ_PROF_LBG_UPDATE);
         if (stream)
-            hipLaunchKernelGGL(vq::k_lbg_stream8, dim3(nparts, m / 4), dim3(64), 0, st, S, d_x, n, ld);
+            hipLaunchKernelGGL(vq::k_lbg_stream8, dim3(nparts, m / 4), dim3(256), 0, st, S, d_x, n, ld);
         else
             hipLaunchKernelGGL(vq::k_lbg_hist, dim3(nparts, m), dim3(64), 0, st, S, n);
         hipLaunchKernelGGL(vq::k_lbg_scan_seg, dim3(nseg, m), dim3(256), 0, st, S);
