@@ -232,3 +232,49 @@ def test_lbg_fit_same_result_on_both_assignment_paths(ctx):
     assert np.array_equal(it_a, it_b) and np.array_equal(used_a, used_b)
     want = O.pq_fit(x, m, k, iters, init, reseed)
     assert np.array_equal(b.view(np.uint32), want["codebooks"].view(np.uint32))
+
+
+@pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN])
+@pytest.mark.parametrize("n,m,sd,k,kind", [
+    (3000, 1, 256, 256, "normal"), (1000, 2, 64, 100, "uniform"), (513, 4, 16, 33, "grid"),
+    (700, 1, 128, 256, "offset"), (300, 1, 24, 7, "same"), (640, 1, 256, 64, "nonfinite"),
+    (257, 3, 32, 1, "normal"),
+])
+def test_wide_mfma_path_equals_oracle_and_valu_path(ctx, metric, n, m, sd, k, kind):
+    """sub_dim a multiple of 8 above 8 (RVQ stages use the full dimension): chunked matrix-core
+    contraction + exact re-check must give the oracle's codes bit for bit."""
+    rng = np.random.default_rng(n + k + sd)
+    dim = sd * m
+    if kind == "uniform":
+        x, cb = rng.random((n, dim), dtype=F), rng.random((m, k, sd), dtype=F)
+    elif kind == "grid":
+        x = np.round(rng.standard_normal((n, dim))).astype(F)
+        cb = np.round(rng.standard_normal((m, k, sd))).astype(F)
+    elif kind == "offset":
+        x = (100 + rng.random((n, dim))).astype(F)
+        cb = (100 + rng.random((m, k, sd))).astype(F)
+    elif kind == "same":
+        x = np.tile(rng.standard_normal((1, dim)).astype(F), (n, 1))
+        cb = np.tile(x[:1].reshape(m, 1, sd), (1, k, 1)).copy()
+    elif kind == "nonfinite":
+        x, cb = rng.random((n, dim), dtype=F), rng.random((m, k, sd), dtype=F)
+        x[::7, 3] = np.inf
+        x[1::11, 9] = np.nan
+        x[2::13, 20] = 1e30
+        cb[0, 5, 2] = np.nan
+        cb[0, 9, 1] = -np.inf
+    else:
+        x, cb = rng.standard_normal((n, dim)).astype(F), rng.standard_normal((m, k, sd)).astype(F)
+    dx, dcb = ctx.to_device(x), ctx.to_device(cb)
+    with np.errstate(all="ignore"):
+        want = O.pq_encode(metric, x, cb).astype(np.uint8)
+    ctx.set_assign_path(0)
+    got = gpu_encode(ctx, metric, dx, n, dim, m, k, dcb)
+    frac = ctx.last_recheck_count() / float(n * m)
+    ctx.set_assign_path(1)
+    valu = gpu_encode(ctx, metric, dx, n, dim, m, k, dcb)
+    ctx.set_assign_path(0)
+    assert np.array_equal(valu, want)
+    assert np.array_equal(got, want)
+    if kind in ("normal", "uniform") and k > 1:
+        assert frac < 0.05, frac  # the matrix-core pass decides almost every row itself

@@ -180,3 +180,90 @@ static __global__ void __launch_bounds__(256) k_crosscov_reduce(const double *__
 }
 
 }  // namespace vq
+
+// ---- rotation on the matrix cores ------------------------------------------------------------
+// y[i][a] = sum_b R[a][b] * x[i][b] for dim a multiple of 32, at most 256: D = R * X^T in tiles of
+// 32 output dimensions x 32 rows with v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate).
+namespace vq {
+
+typedef float rot_floatx16 __attribute__((ext_vector_type(16)));
+
+// rtab[kc][b][lane][u] = R[32 b + lane % 32][8 kc + 4 (lane / 32) + u]   (MFMA A-operand order)
+static __global__ void __launch_bounds__(256) k_rotate_prep(const float *__restrict__ R, int dim,
+                                                            float *__restrict__ rtab) {
+    const int nb = dim / 32, nkc = dim / 8;
+    const int total = nkc * nb * 64 * 4;
+    for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
+        const int u = e % 4, lane = (e / 4) % 64, b = (e / 256) % nb, kc = e / (256 * nb);
+        rtab[e] = R[(size_t)(32 * b + lane % 32) * dim + 8 * kc + 4 * (lane / 32) + u];
+    }
+}
+
+// grid ceil(n/128); 256 threads = 4 waves, one tile of 32 rows per wave.
+static __global__ void __launch_bounds__(256) k_rotate_mfma(const float *__restrict__ x, int64_t n, int64_t ld,
+                                                            int dim, const float *__restrict__ rtab,
+                                                            float *__restrict__ y) {
+    constexpr int NBMAX = 8;
+    __shared__ float4 lds_a[2][NBMAX * 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int nb = dim / 32, nkc = dim / 8;
+    const int64_t row = ((int64_t)blockIdx.x * 4 + wave) * 32 + r;
+    const bool valid = row < n;
+    const float4 *ag = reinterpret_cast<const float4 *>(rtab);
+    const int chunk4 = nb * 64;
+    for (int i = threadIdx.x; i < chunk4; i += 256) lds_a[0][i] = ag[i];
+    __syncthreads();
+    rot_floatx16 acc[NBMAX];
+#pragma unroll
+    for (int b = 0; b < NBMAX; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[b][v] = 0.0f;
+    const float *xr = x + (valid ? row : 0) * ld + 4 * h;
+    for (int kc = 0; kc < nkc; ++kc) {
+        const int cur = kc & 1;
+        float4 pre[2];
+        const bool more = kc + 1 < nkc;
+        if (more) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                int i = threadIdx.x + 256 * q;
+                if (i < chunk4) pre[q] = ag[(size_t)(kc + 1) * chunk4 + i];
+            }
+        }
+        float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (valid) xv = *reinterpret_cast<const float4 *>(xr + kc * 8);
+#pragma unroll
+        for (int b = 0; b < NBMAX; ++b) {
+            if (b < nb) {
+                const float4 av = lds_a[cur][b * 64 + lane];
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, xv.x, acc[b], 0, 0, 0);
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, xv.y, acc[b], 0, 0, 0);
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, xv.z, acc[b], 0, 0, 0);
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, xv.w, acc[b], 0, 0, 0);
+            }
+        }
+        if (more) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                int i = threadIdx.x + 256 * q;
+                if (i < chunk4) lds_a[cur ^ 1][i] = pre[q];
+            }
+        }
+        __syncthreads();
+    }
+    if (!valid) return;
+    // register v of block b holds output dimension 32 b + 8 (v / 4) + 4 h + v % 4 of this lane's row
+    float *yr = y + row * dim + 4 * h;
+#pragma unroll
+    for (int b = 0; b < NBMAX; ++b) {
+        if (b < nb) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+                *reinterpret_cast<float4 *>(yr + 32 * b + 8 * g) =
+                    make_float4(acc[b][4 * g], acc[b][4 * g + 1], acc[b][4 * g + 2], acc[b][4 * g + 3]);
+        }
+    }
+}
+
+}  // namespace vq

@@ -123,6 +123,44 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
     return VQ_OK;
 }
 
+// Wide column blocks (sub_dim a multiple of 8 above 8): chunked contraction, same two passes.
+template <int METRIC, bool LBG>
+int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
+    const int nb = (a.k + 31) / 32, nkc = sd / 8;
+    const size_t n_atab = (size_t)a.m * nkc * nb * 64 * 4, n_c2 = (size_t)a.m * nb * 32;
+    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + a.m) + 64));
+    VQ_TRY(ensure(ctx, ctx->mfma_list, sizeof(uint32_t) * ((size_t)a.n * a.m + 4)));
+    float *atab = (float *)ctx->mfma_tab.p;
+    float *c2perm = atab + n_atab;
+    float *maxc2 = c2perm + n_c2;
+    uint32_t *count = (uint32_t *)ctx->mfma_list.p;
+    uint32_t *list = count + 4;
+    hipLaunchKernelGGL(vq::k_mfma_wide_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, sd, atab,
+                       c2perm, maxc2, count);
+    // bound on matrix accumulation + the reference's own rounding: (sd + 16) * 2^-21 per unit of
+    // ||x||^2 + max ||c||^2 (about 2^-16.4 at sd = 8, the constant of the narrow kernel)
+    vq::MfmaWideTables tb{atab, c2perm, maxc2, list, count, nb, sd, (float)(sd + 16) * 4.76837158203125e-07f};
+    {
+        ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
+        hipLaunchKernelGGL((vq::k_assign_mfma_wide<LBG>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0,
+                           ctx->stream, a, tb);
+    }
+    hipLaunchKernelGGL((vq::k_assign_recheck_dyn<METRIC, LBG>), dim3(1024), dim3(256), 0, ctx->stream, a, sd,
+                       (const uint32_t *)list, (const uint32_t *)count);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+template <int METRIC, bool LBG>
+bool mfma_wide_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
+    if (ctx->assign_path != 0) return false;
+    if (METRIC != vq::M_SQ && METRIC != vq::M_EUCLID) return false;
+    if (sd < 16 || sd % 8 != 0 || a.k > 256 || a.m > 65535) return false;
+    // float4 row loads
+    if (a.ld % 4 != 0 || (reinterpret_cast<uintptr_t>(a.x) & 15) != 0) return false;
+    return (int64_t)a.n * a.m < (1LL << 32);
+}
+
 template <int METRIC, bool LBG>
 bool mfma_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     if (ctx->assign_path != 0) return false;
@@ -138,6 +176,10 @@ int32_t launch_assign(vq_ctx *ctx, int metric, const vq::AssignArgs &a, int sd) 
         return launch_mfma<8, vq::M_SQ, LBG>(ctx, a);
     if (metric == VQ_EUCLIDEAN && mfma_applicable<vq::M_EUCLID, LBG>(ctx, a, sd))
         return launch_mfma<8, vq::M_EUCLID, LBG>(ctx, a);
+    if (metric == VQ_SQEUCLIDEAN && mfma_wide_applicable<vq::M_SQ, LBG>(ctx, a, sd))
+        return launch_mfma_wide<vq::M_SQ, LBG>(ctx, a, sd);
+    if (metric == VQ_EUCLIDEAN && mfma_wide_applicable<vq::M_EUCLID, LBG>(ctx, a, sd))
+        return launch_mfma_wide<vq::M_EUCLID, LBG>(ctx, a, sd);
     switch (metric) {
     case VQ_SQEUCLIDEAN: return launch_assign_m<vq::M_SQ, LBG>(ctx, a, sd);
     case VQ_EUCLIDEAN: return launch_assign_m<vq::M_EUCLID, LBG>(ctx, a, sd);

@@ -95,9 +95,20 @@ int32_t vq_rotate(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t 
     if (!ctx) return VQ_ERR_INVALID_ARG;
     if (n == 0) return VQ_OK;
     if (!d_x || !d_R || !d_y || n < 0 || dim <= 0 || ld < dim) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    // matrix-core kernel: dim a multiple of 32 up to 256, rows and output 16-byte aligned
+    if (dim % 32 == 0 && dim <= 256 && ld % 4 == 0 &&
+        ((reinterpret_cast<uintptr_t>(d_x) | reinterpret_cast<uintptr_t>(d_y)) & 15) == 0) {
+        VQ_TRY(ensure(ctx, ctx->tmp_f, sizeof(float) * (size_t)dim * dim));
+        hipLaunchKernelGGL(vq::k_rotate_prep, dim3(cdiv((int64_t)dim * dim, 256)), dim3(256), 0, ctx->stream,
+                           d_R, dim, (float *)ctx->tmp_f.p);
+        hipLaunchKernelGGL(vq::k_rotate_mfma, dim3(cdiv(n, 128)), dim3(256), 0, ctx->stream, d_x, n, ld, dim,
+                           (const float *)ctx->tmp_f.p, d_y);
+        VQ_HIP(ctx, hipGetLastError());
+        return VQ_OK;
+    }
     size_t lds = sizeof(float) * 64 * ((size_t)dim + 1);
     if (lds > 160 * 1024) return fail(ctx, VQ_ERR_UNSUPPORTED, "rotation: dim %d too large", dim);
-    VQ_HIP(ctx, hipSetDevice(ctx->device));
     if (lds > 48 * 1024)
         VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(vq::k_rotate_generic),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
