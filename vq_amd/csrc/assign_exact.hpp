@@ -353,3 +353,230 @@ __global__ void __launch_bounds__(256) k_assign_dyn(AssignArgs a, int sd) {
 }
 
 }  // namespace vq
+
+// ---------------------------------------------------------------------------------------------
+// Exact assignment for wide column blocks: one lane = up to 4 centroids, one wave = 8 rows.
+// The wave keeps its 8 rows in LDS (read back as broadcasts) and every lane walks the codebook
+// rows of its centroids, so each (row, centroid) distance is still one sequential f32 chain in
+// the reference's order.  The argmin over centroids is a lexicographic (distance, index) minimum,
+// which is exactly "strict '<', lowest index wins"; a NaN never wins unless it sits at index 0.
+// Rows come either from a contiguous range (LISTED = false, grid.y = column block) or from the
+// list of undecided pairs left by the matrix-core pass (LISTED = true).
+namespace vq {
+
+constexpr int kWideRows = 8;
+
+template <int METRIC>
+__device__ __forceinline__ void wide_step(float &acc, float xv, float cv) {
+    if constexpr (METRIC == M_COS) {
+        float p = xv * cv;
+        acc = acc + p;
+    } else if constexpr (METRIC == M_L1) {
+        float d = xv - cv;
+        acc = acc + fabsf(d);
+    } else {
+        float d = xv - cv;
+        float p = d * d;
+        acc = acc + p;
+    }
+}
+
+// Distances of the wave's rows (in lds_x, row stride sd) to the centroids of block s, then the
+// reference argmin per row.  rows[i] < 0 marks an unused slot.  Lane 0 returns the codes.
+template <int METRIC, bool VEC>
+__device__ __forceinline__ void wide_argmin(const AssignArgs &a, int sd, int s, const float *lds_x, int lane,
+                                            int (&best_out)[kWideRows]) {
+    const int k = a.k;
+    const float *__restrict__ cb = a.cb + (size_t)s * k * sd;
+    float acc[4][kWideRows];
+    float sa[kWideRows];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int i = 0; i < kWideRows; ++i) acc[q][i] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kWideRows; ++i) sa[i] = 0.0f;
+    const float *cq[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        int j = lane + 64 * q;
+        cq[q] = cb + (size_t)(j < k ? j : 0) * sd;
+    }
+    int t = 0;
+    if constexpr (VEC) {
+        for (; t + 4 <= sd; t += 4) {
+            float4 cv[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) cv[q] = *reinterpret_cast<const float4 *>(cq[q] + t);
+#pragma unroll
+            for (int i = 0; i < kWideRows; ++i) {
+                const float4 xv = *reinterpret_cast<const float4 *>(lds_x + i * sd + t);
+                if constexpr (METRIC == M_COS) {
+                    float p;
+                    p = xv.x * xv.x; sa[i] = sa[i] + p;
+                    p = xv.y * xv.y; sa[i] = sa[i] + p;
+                    p = xv.z * xv.z; sa[i] = sa[i] + p;
+                    p = xv.w * xv.w; sa[i] = sa[i] + p;
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    wide_step<METRIC>(acc[q][i], xv.x, cv[q].x);
+                    wide_step<METRIC>(acc[q][i], xv.y, cv[q].y);
+                    wide_step<METRIC>(acc[q][i], xv.z, cv[q].z);
+                    wide_step<METRIC>(acc[q][i], xv.w, cv[q].w);
+                }
+            }
+        }
+    }
+    for (; t < sd; ++t) {
+        float cv[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) cv[q] = cq[q][t];
+#pragma unroll
+        for (int i = 0; i < kWideRows; ++i) {
+            const float xv = lds_x[i * sd + t];
+            if constexpr (METRIC == M_COS) {
+                float p = xv * xv;
+                sa[i] = sa[i] + p;
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) wide_step<METRIC>(acc[q][i], xv, cv[q]);
+        }
+    }
+    const float inf = __builtin_inff();
+#pragma unroll
+    for (int i = 0; i < kWideRows; ++i) {
+        float bd = inf, d0 = 0.0f;
+        int bi = 0x7fffffff;
+        float dq[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int j = lane + 64 * q;
+            float d = acc[q][i];
+            if constexpr (METRIC == M_COS) {
+                const float na = sqrtf(sa[i]);
+                const float nb = (j < k) ? a.cnorm[(size_t)s * k + j] : 1.0f;
+                const float den = na * nb;
+                const float qq = d / den;
+                d = 1.0f - qq;
+                d = (na == 0.0f || nb == 0.0f) ? 1.0f : d;
+            }
+            if (q == 0) d0 = d;  // lane 0 holds the distance of centroid 0
+            const bool nan = !(d == d);
+            d = (j < k && !nan) ? d : inf;
+            dq[q] = d;
+            if (j < k && d < bd) {  // ascending j inside the lane: strict '<' keeps the first
+                bd = d;
+                bi = j;
+            }
+        }
+        if (bi == 0x7fffffff) bi = lane;  // all +inf in this lane: lowest index of the lane
+        if (lane >= k) bi = 0x7fffffff;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float od = __shfl_xor(bd, off);
+            const int oi = __shfl_xor(bi, off);
+            const bool take = (od < bd) || (od == bd && oi < bi);
+            bd = take ? od : bd;
+            bi = take ? oi : bi;
+        }
+        if constexpr (METRIC == M_EUCLID) {
+            // first index whose root equals the root of the smallest squared distance
+            const float sr = sqrtf(bd);
+            int fi = 0x7fffffff;
+#pragma unroll
+            for (int q = 3; q >= 0; --q) {
+                const int j = lane + 64 * q;
+                if (j < k && sqrtf(dq[q]) == sr) fi = j;
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const int oi = __shfl_xor(fi, off);
+                fi = oi < fi ? oi : fi;
+            }
+            bi = fi;
+        }
+        const float d0b = __shfl(d0, 0);
+        if (!(d0b == d0b)) bi = 0;  // NaN at index 0 is never displaced
+        best_out[i] = bi;
+    }
+}
+
+template <int METRIC, bool LBG, bool LISTED, bool VEC>
+__global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd, const uint32_t *__restrict__ list,
+                                                           const uint32_t *__restrict__ list_count) {
+    extern __shared__ float lds_wide[];  // 4 waves x 8 rows x sd
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float *lds_x = lds_wide + (size_t)wave * kWideRows * sd;
+    const int64_t total = LISTED ? (int64_t)*list_count : a.n;
+    const int64_t groups = (total + kWideRows - 1) / kWideRows;
+    for (int64_t grp = (int64_t)blockIdx.x * 4 + wave; grp < groups; grp += (int64_t)gridDim.x * 4) {
+        int64_t rows[kWideRows];
+        int ss[kWideRows];
+#pragma unroll
+        for (int i = 0; i < kWideRows; ++i) {
+            const int64_t e = grp * kWideRows + i;
+            rows[i] = -1;
+            ss[i] = LISTED ? -1 : (int)blockIdx.y;
+            if (e < total) {
+                if constexpr (LISTED) {
+                    const uint32_t v = list[e];
+                    rows[i] = v / (uint32_t)a.m;
+                    ss[i] = (int)(v % (uint32_t)a.m);
+                } else {
+                    rows[i] = e;
+                }
+            }
+        }
+        if constexpr (LBG && !LISTED) {
+            if (a.done[blockIdx.y]) return;
+        }
+        // sub-groups of slots that share the column block (always one group when not LISTED)
+        bool pending[kWideRows];
+#pragma unroll
+        for (int i = 0; i < kWideRows; ++i) pending[i] = rows[i] >= 0;
+        for (;;) {
+            int s = -1;
+#pragma unroll
+            for (int i = kWideRows - 1; i >= 0; --i)
+                if (pending[i]) s = ss[i];
+            if (s < 0) break;
+            // stage the rows of this sub-group (unused slots repeat a valid row)
+            int64_t fill = -1;
+#pragma unroll
+            for (int i = 0; i < kWideRows; ++i)
+                if (pending[i] && ss[i] == s && fill < 0) fill = rows[i];
+#pragma unroll
+            for (int i = 0; i < kWideRows; ++i) {
+                const int64_t rr = (pending[i] && ss[i] == s) ? rows[i] : fill;
+                const float *xr = a.x + rr * a.ld + (int64_t)s * sd;
+                for (int t = lane; t < sd; t += 64) lds_x[i * sd + t] = xr[t];
+            }
+            __builtin_amdgcn_wave_barrier();
+            int best[kWideRows];
+            wide_argmin<METRIC, VEC>(a, sd, s, lds_x, lane, best);
+            __builtin_amdgcn_wave_barrier();
+            if (lane == 0) {
+#pragma unroll
+                for (int i = 0; i < kWideRows; ++i) {
+                    if (pending[i] && ss[i] == s) {
+                        if constexpr (LBG) {
+                            uint8_t *p = a.codes + (size_t)s * a.n + rows[i];
+                            if (*p != (uint8_t)best[i]) {
+                                *p = (uint8_t)best[i];
+                                a.changed[s] = 1;
+                            }
+                        } else {
+                            a.codes[rows[i] * a.m + s] = (uint8_t)best[i];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kWideRows; ++i)
+                if (ss[i] == s) pending[i] = false;
+        }
+    }
+}
+
+}  // namespace vq

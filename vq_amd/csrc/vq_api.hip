@@ -6,6 +6,7 @@
 
 #include <algorithm>
 #include <cstdarg>
+#include <type_traits>
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -32,6 +33,10 @@ using namespace vqh;
 namespace {
 
 // ---- assignment dispatch -------------------------------------------------------------------
+
+template <int METRIC, bool LBG>
+int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const uint32_t *list,
+                          const uint32_t *count);
 
 template <int SD, int G, int METRIC, bool LBG>
 int32_t launch_static(vq_ctx *ctx, const vq::AssignArgs &a) {
@@ -85,6 +90,10 @@ int32_t launch_assign_m(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
         }
     }
     if (a.m > 65535) return fail(ctx, VQ_ERR_UNSUPPORTED, "m too large for the generic kernel");
+    if (sd >= 24) {
+        ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
+        return launch_wide_exact<METRIC, LBG>(ctx, a, sd, nullptr, nullptr);
+    }
     hipLaunchKernelGGL((vq::k_assign_dyn<METRIC, LBG>), dim3(cdiv(a.n, 256), (unsigned)a.m),
                        dim3(256), 0, ctx->stream, a, sd);
     VQ_HIP(ctx, hipGetLastError());
@@ -123,6 +132,32 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
     return VQ_OK;
 }
 
+// Exact assignment for wide column blocks, on a row range (list == nullptr) or on the list of
+// undecided pairs of the matrix-core pass.
+template <int METRIC, bool LBG>
+int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const uint32_t *list,
+                          const uint32_t *count) {
+    const size_t lds = sizeof(float) * 4 * vq::kWideRows * (size_t)sd;
+    if (lds > 160 * 1024) return fail(ctx, VQ_ERR_UNSUPPORTED, "sub_dim %d too large", sd);
+    const bool vec = sd % 4 == 0 && (reinterpret_cast<uintptr_t>(a.cb) & 15) == 0;
+    const bool listed = list != nullptr;
+    auto pick = [&](auto L, auto V) {
+        constexpr bool LISTED = decltype(L)::value, VEC = decltype(V)::value;
+        return reinterpret_cast<const void *>(vq::k_assign_wide_exact<METRIC, LBG, LISTED, VEC>);
+    };
+    const void *kern = listed ? (vec ? pick(std::true_type{}, std::true_type{}) : pick(std::true_type{}, std::false_type{}))
+                              : (vec ? pick(std::false_type{}, std::true_type{}) : pick(std::false_type{}, std::false_type{}));
+    if (lds > 48 * 1024)
+        VQ_HIP(ctx, hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    const int64_t groups = (a.n + vq::kWideRows - 1) / vq::kWideRows;
+    dim3 grid(listed ? 2048u : (unsigned)std::min<int64_t>((groups + 3) / 4, 1 << 20), listed ? 1u : (unsigned)a.m);
+    vq::AssignArgs aa = a;
+    int sdv = sd;
+    void *args[] = {&aa, &sdv, (void *)&list, (void *)&count};
+    VQ_HIP(ctx, hipLaunchKernel(kern, grid, dim3(256), args, lds, ctx->stream));
+    return VQ_OK;
+}
+
 // Wide column blocks (sub_dim a multiple of 8 above 8): chunked contraction, same two passes.
 template <int METRIC, bool LBG>
 int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
@@ -145,10 +180,8 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
         hipLaunchKernelGGL((vq::k_assign_mfma_wide<LBG>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0,
                            ctx->stream, a, tb);
     }
-    hipLaunchKernelGGL((vq::k_assign_recheck_dyn<METRIC, LBG>), dim3(1024), dim3(256), 0, ctx->stream, a, sd,
-                       (const uint32_t *)list, (const uint32_t *)count);
     VQ_HIP(ctx, hipGetLastError());
-    return VQ_OK;
+    return launch_wide_exact<METRIC, LBG>(ctx, a, sd, list, count);
 }
 
 template <int METRIC, bool LBG>
