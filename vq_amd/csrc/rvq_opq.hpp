@@ -21,17 +21,29 @@ static __global__ void __launch_bounds__(256) k_residual_sub(float *__restrict__
 }
 
 // norms[i] = sqrt(sum_t x[i][t]^2), sequential f32 order (src/rvq.rs:134-135).
-static __global__ void __launch_bounds__(256) k_row_norms(const float *__restrict__ x, int64_t n, int64_t ld,
+// One wave = 64 rows.  The rows are read coalesced, 64 columns at a time, into a padded LDS tile;
+// each lane then walks its own row of the tile, so the per-row sum stays one sequential chain.
+static __global__ void __launch_bounds__(64) k_row_norms(const float *__restrict__ x, int64_t n, int64_t ld,
                                                    int dim, float *__restrict__ norms) {
-    int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (row >= n) return;
-    const float *p = x + row * ld;
+    __shared__ float tile[64][65];
+    const int lane = threadIdx.x;
+    const int64_t row0 = (int64_t)blockIdx.x * 64;
     float acc = 0.0f;
-    for (int t = 0; t < dim; ++t) {
-        float q = p[t] * p[t];
-        acc = acc + q;
+    for (int c0 = 0; c0 < dim; c0 += 64) {
+        const int w = (dim - c0 < 64) ? (dim - c0) : 64;
+        __syncthreads();
+        for (int r = 0; r < 64; ++r) {
+            const int64_t row = row0 + r;
+            if (row < n && lane < w) tile[r][lane] = x[row * ld + c0 + lane];
+        }
+        __syncthreads();
+        for (int t = 0; t < w; ++t) {
+            float v = tile[lane][t];
+            float q = v * v;
+            acc = acc + q;
+        }
     }
-    norms[row] = sqrtf(acc);
+    if (row0 + lane < n) norms[row0 + lane] = sqrtf(acc);
 }
 
 // Fixed-shape two-level sum of n floats in f64: every workgroup sums a contiguous slice with a
@@ -53,35 +65,35 @@ static __global__ void __launch_bounds__(256) k_sum_f64(const float *__restrict_
     if (threadIdx.x == 0) out[blockIdx.x] = sh[0];
 }
 
-// One stage of ResidualQuantizer::quantize for every row still active (src/rvq.rs:200-207):
-// sum += c; residual -= c; stop the row when ||residual|| < epsilon.
+// One stage of ResidualQuantizer::quantize for every row still active (src/rvq.rs:200-202):
+// sum += c; residual -= c.  One lane per element.
 static __global__ void __launch_bounds__(256) k_rvq_stage_apply(float *__restrict__ res, float *__restrict__ sum,
                                                          int64_t n, int dim, const float *__restrict__ cb,
                                                          const uint8_t *__restrict__ stage_codes,
                                                          uint8_t *__restrict__ codes_out, int stages,
-                                                         int stage, uint8_t *__restrict__ active,
-                                                         uint8_t *__restrict__ used, float epsilon) {
+                                                         int stage, const uint8_t *__restrict__ active,
+                                                         uint8_t *__restrict__ used) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n * dim) return;
+    const int64_t row = i / dim;
+    const int t = (int)(i % dim);
+    const bool on = active[row] != 0;
+    const int code = on ? stage_codes[row] : 0;
+    if (t == 0) {
+        codes_out[row * stages + stage] = (uint8_t)code;
+        if (on) used[row] = (uint8_t)(stage + 1);
+    }
+    if (!on) return;
+    const float c = cb[(size_t)code * dim + t];
+    sum[i] = sum[i] + c;
+    res[i] = res[i] - c;
+}
+
+// The row stops when ||residual|| < epsilon (src/rvq.rs:204-207).
+static __global__ void __launch_bounds__(256) k_rvq_stage_stop(const float *__restrict__ norms, int64_t n,
+                                                        float epsilon, uint8_t *__restrict__ active) {
     int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (row >= n) return;
-    if (!active[row]) {
-        codes_out[row * stages + stage] = 0;
-        return;
-    }
-    int code = stage_codes[row];
-    codes_out[row * stages + stage] = (uint8_t)code;
-    const float *c = cb + (size_t)code * dim;
-    float *r = res + row * dim;
-    float *s = sum + row * dim;
-    float acc = 0.0f;
-    for (int t = 0; t < dim; ++t) {
-        s[t] = s[t] + c[t];
-        float v = r[t] - c[t];
-        r[t] = v;
-        float q = v * v;
-        acc = acc + q;
-    }
-    used[row] = (uint8_t)(stage + 1);
-    if (sqrtf(acc) < epsilon) active[row] = 0;
+    if (row < n && active[row] && norms[row] < epsilon) active[row] = 0;
 }
 
 static __global__ void __launch_bounds__(256) k_f32_to_f16(const float *__restrict__ in, int64_t count,

@@ -37,7 +37,7 @@ int32_t vq_mean_l2norm(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int
     VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * ((size_t)blocks + 1)));
     float *norms = (float *)ctx->tmp_a.p;
     double *part = (double *)ctx->tmp_b.p;
-    hipLaunchKernelGGL(vq::k_row_norms, dim3(cdiv(n, 256)), dim3(256), 0, ctx->stream, d_x, n, ld, dim, norms);
+    hipLaunchKernelGGL(vq::k_row_norms, dim3(cdiv(n, 64)), dim3(64), 0, ctx->stream, d_x, n, ld, dim, norms);
     hipLaunchKernelGGL(vq::k_sum_f64, dim3(blocks), dim3(256), 0, ctx->stream, norms,
                        (const double *)nullptr, n, per_block, part);
     hipLaunchKernelGGL(vq::k_sum_f64, dim3(1), dim3(256), 0, ctx->stream, (const float *)nullptr, part,
@@ -62,6 +62,8 @@ int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, 
     VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(float) * (size_t)n * dim));   // residual
     VQ_TRY(ensure(ctx, ctx->tmp_d, sizeof(float) * (size_t)n * dim));   // running sum
     VQ_TRY(ensure(ctx, ctx->tmp_e, (size_t)n * 3 + 16));                // stage codes, active, used
+    VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(float) * (size_t)n));         // row norms
+    float *norms = (float *)ctx->tmp_a.p;
     float *res = (float *)ctx->tmp_c.p;
     float *sum = (float *)ctx->tmp_d.p;
     uint8_t *stage_codes = (uint8_t *)ctx->tmp_e.p;
@@ -78,8 +80,14 @@ int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, 
             hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, stage_codes, n, (uint8_t)0);
         else
             VQ_TRY(assign_codes(ctx, metric, res, n, dim, 1, dim, k, cb, stage_codes));
-        hipLaunchKernelGGL(vq::k_rvq_stage_apply, dim3(cdiv(n, 256)), dim3(256), 0, st, res, sum, n, dim, cb,
-                           stage_codes, d_codes, stages, s, active, used, epsilon);
+        hipLaunchKernelGGL(vq::k_rvq_stage_apply, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, res, sum, n, dim,
+                           cb, stage_codes, d_codes, stages, s, active, used);
+        if (epsilon > 0.0f) {  // a norm is never below a non-positive threshold
+            hipLaunchKernelGGL(vq::k_row_norms, dim3(cdiv(n, 64)), dim3(64), 0, st, res, n, (int64_t)dim, dim,
+                               norms);
+            hipLaunchKernelGGL(vq::k_rvq_stage_stop, dim3(cdiv(n, 256)), dim3(256), 0, st, norms, n, epsilon,
+                               active);
+        }
     }
     if (d_stages_used)
         VQ_HIP(ctx, hipMemcpyAsync(d_stages_used, used, (size_t)n, hipMemcpyDeviceToDevice, st));
