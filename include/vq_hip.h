@@ -63,7 +63,8 @@ int32_t vq_ctx_sync(vq_ctx *ctx);
 void *vq_ctx_stream(vq_ctx *ctx);
 
 /* Which kernels decide the squared-L2 / Euclidean assignment where both exist:
- *   0 (default)  matrix-core pass with an exact re-check of every undecided (row, block) pair
+ *   0 (default)  matrix-core scores (bf16-split operands for 8-float column blocks, fp32 operands
+ *                for wider ones) with an exact re-check of every undecided (row, block) pair
  *   1            the all-vector-ALU kernel in the reference's operation order
  * Both give bit-identical codes; the switch exists for measurement and tests. */
 int32_t vq_ctx_set_assign_path(vq_ctx *ctx, int32_t path);

@@ -29,6 +29,14 @@ struct AssignArgs {
     const int *done;      // LBG mode: blocks with done[s] != 0 are skipped
 };
 
+// Called by the lanes of a wave that changed a code.  Every store to one address is serialised
+// in its L2 channel and a million rows may change in a pass, so one lane of the wave stores, and
+// only when it still reads 0 (a stale 0 from the vector cache costs a store, nothing else).
+__device__ __forceinline__ void mark_changed(int *flag) {
+    const unsigned long long active = __ballot(1);
+    if ((int)__lane_id() == __ffsll(active) - 1 && *flag == 0) *flag = 1;
+}
+
 // sqrt(sum of squares) of every centroid, sequential order (map_sum, src/distances.rs:66-69,144)
 static __global__ void k_centroid_norms(const float *__restrict__ cb, int64_t total, int sd,
                                  float *__restrict__ out) {
@@ -242,7 +250,7 @@ __global__ void __launch_bounds__(256) k_assign_static(AssignArgs a) {
             uint8_t *p = a.codes + (size_t)s * a.n + row;
             if (*p != (uint8_t)best) {
                 *p = (uint8_t)best;
-                a.changed[s] = 1;
+                mark_changed(a.changed + s);
             }
         } else {
             if constexpr (G == 4)
@@ -345,7 +353,7 @@ __global__ void __launch_bounds__(256) k_assign_dyn(AssignArgs a, int sd) {
         uint8_t *p = a.codes + (size_t)s * a.n + row;
         if (*p != (uint8_t)best) {
             *p = (uint8_t)best;
-            a.changed[s] = 1;
+            mark_changed(a.changed + s);
         }
     } else {
         a.codes[row * a.m + s] = (uint8_t)best;
@@ -564,7 +572,7 @@ __global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd,
                             uint8_t *p = a.codes + (size_t)s * a.n + rows[i];
                             if (*p != (uint8_t)best[i]) {
                                 *p = (uint8_t)best[i];
-                                a.changed[s] = 1;
+                                mark_changed(a.changed + s);
                             }
                         } else {
                             a.codes[rows[i] * a.m + s] = (uint8_t)best[i];

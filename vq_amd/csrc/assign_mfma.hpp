@@ -1,20 +1,19 @@
 // Nearest-centroid assignment for squared-L2 / Euclidean on the matrix cores, exact by re-check.
 //
-// Pass 1 (k_assign_mfma): for a tile of 32 rows and one column block, the scores
-//     s[j] = ||c_j||^2 + ||x||^2 - 2 x.c_j
-// of 32 centroids at a time come from v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate; the
-// accumulator starts at ||c_j||^2 + ||x||^2, the products carry -2 c_j).  The running smallest and
-// second-smallest score of every row are kept with the centroid index packed into the 8 low
-// mantissa bits (one v_and_or, one v_med3, one v_min per score).
-// The matrix form rounds differently from the reference's sequential (x-c)^2 sum, so a row is
-// only decided here when its two best scores are further apart than a bound on every error
-// involved (matrix accumulation, the packed bits, the reference's own rounding):
-//     gap > 2^-14 |second| + 2^-16 (||x||^2 + max_j ||c_j||^2)
-// Then the smallest exact distance is provably the same centroid.  Every other (row, block)
-// pair — exact ties, near ties, sqrt collisions under Euclidean, non-finite values — is appended
-// to a list and decided by pass 2.
-// Pass 2 (k_assign_recheck): the reference-order argmin of assign_exact.hpp on the listed pairs.
-// The result is therefore bit-identical to the all-VALU path for every input.
+// The scores  s[j] = ||c_j||^2 + ||x||^2 - 2 x.c_j  of 32 rows against 32 centroids at a time come
+// out of the matrix cores.  The running smallest and second-smallest score of every row are kept
+// with the centroid index packed into the 8 low mantissa bits (one v_and_or per score, then five
+// v_min3 / v_med3 per four scores).  The matrix form rounds differently from the reference's
+// sequential (x-c)^2 sum, so a row is only decided from the scores when its two best are further
+// apart than a bound on every error involved (operand splitting, matrix accumulation, the packed
+// bits, the reference's own rounding).  Then the smallest exact distance is provably the same
+// centroid.  Every other (row, block) pair — exact ties, near ties, sqrt collisions under
+// Euclidean, non-finite values — is decided by the reference-order argmin, so the result is
+// bit-identical to the all-VALU path for every input.
+//
+// 8-float column blocks (k_assign_mfma_bf): bf16 matrix cores with split operands; the undecided
+// rows are resolved inside the same wave.  Wider blocks (k_assign_mfma_wide): fp32 matrix cores;
+// the undecided pairs are listed for the exact kernel of assign_exact.hpp.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -26,50 +25,124 @@ namespace vq {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 // Score of the padding centroids that fill the last block of 32; a row whose best score is not
-// well below it is sent to the exact pass.
+// well below it is decided by the exact path.
 constexpr float kPadScore = 1e30f;
 
-struct MfmaTables {
-    const float *atab;     // [m][nb][64][SD/2]  -2*c in MFMA A-operand order
-    const float *c2perm;   // [m][nb][2][16]     ||c||^2 in accumulator order (kPadScore for padding)
+// Scores are compared through their bit patterns as signed integers: for non-negative floats
+// that is the float order, a slightly negative score (cancellation) still sorts below every
+// positive one, and integer min / med3 need no NaN canonicalisation.  Two negative scores sort
+// in reverse, which only happens inside the error bound, i.e. for pairs that are re-checked.
+__device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
+__device__ __forceinline__ int imax(int a, int b) { return a > b ? a : b; }
+__device__ __forceinline__ int imed3(int a, int b, int c) {
+    return imax(imin(a, b), imin(imax(a, b), c));
+}
+// v_min3_i32 by name: the compiler otherwise splits the chain of smallest keys into pairs of v_min_i32.
+__device__ __forceinline__ int imin3(int a, int b, int c) {
+    int r;
+    asm("v_min3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Four new keys into the running (smallest, second smallest): 5 operations.
+// second smallest of {m1, m2, x, y} with m1 <= m2 is min(m2, med3(m1, x, y)).
+__device__ __forceinline__ void top2_push4(int &m1, int &m2, int k0, int k1, int k2, int k3) {
+    const int ta = imed3(m1, k0, k1);
+    const int a1 = imin3(m1, k0, k1);
+    const int tb = imed3(a1, k2, k3);
+    m1 = imin3(a1, k2, k3);
+    m2 = imin3(m2, ta, tb);
+}
+
+// ---------------------------------------------------------------------------------------------
+// 8-float column blocks on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16, 4x the fp32 rate).
+//
+// Every fp32 operand is split into two bf16 numbers, v = vh + vl + e with |e| <= 2^-16 |v|
+// (round-to-nearest-even twice).  With a = -2c the 16 contraction slots of two instructions hold
+//     instruction 1:  ah . xh  (slots 0-7)   ah . xl  (slots 8-15)
+//     instruction 2:  al . xh  (slots 0-7)   1 . (three bf16 parts of ||x||^2)  (slots 8-10)
+// and the accumulator starts at ||c||^2, so the result is the score ||c||^2 + ||x||^2 - 2 x.c with
+// an error of at most 3 * 2^-16 * sum|a_t||x_t| <= 3 * 2^-16 (||x||^2 + ||c||^2) from the dropped
+// terms (a ex, x ea, al xl) plus at most 2^-17.9 (||x||^2 + ||c||^2) from the fp32 accumulation of
+// the 2 x 17 addends.  Two candidates compared: below 2^-13.2 (||x||^2 + max ||c||^2); the test
+// uses 2^-13, plus 2^-14 |second| for the packed bits and the reference's own rounding.  bf16
+// keeps the fp32 exponent range, so no scaling is needed; non-finite values fail the test.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kStatSlots = 64;    // counters of undecided pairs, one 128-byte line apart
+constexpr int kStatStride = 32;
+
+struct MfmaBfTables {
+    const u32x4 *atab;     // [m][nb][2][64]  A operands of the two instructions, lane order
+    const float *c2perm;   // [m][nb][2][16]  ||c||^2 in accumulator order (kPadScore for padding)
     const float *maxc2;    // [m]
-    uint32_t *list;        // flagged pairs: row*m + s
-    uint32_t *list_count;  // 1
+    uint32_t *stat;        // [kStatSlots * kStatStride]  pairs decided by the exact path (measurement)
     int nb;                // ceil(k/32)
 };
 
-// Builds the tables from the codebooks.  One thread per (s, padded centroid).
-template <int SD>
-__global__ void __launch_bounds__(256) k_mfma_prep(const float *__restrict__ cb, int m, int k, int nb,
-                                                   float *__restrict__ atab, float *__restrict__ c2perm,
-                                                   float *__restrict__ maxc2, uint32_t *__restrict__ list_count) {
-    constexpr int HS = SD / 2;
+// float -> bf16 bits, round to nearest even (NaN stays NaN).
+__host__ __device__ __forceinline__ uint32_t bf16_rne_bits(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
+
+// two floats -> packed bf16 pair (lo = first), round to nearest even
+__device__ __forceinline__ uint32_t bf16_pack2(float a, float b) {
+    floatx2 f = {a, b};
+    bf16x2 h = __builtin_convertvector(f, bf16x2);
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// Tables for k_assign_mfma_bf.  One thread per (s, padded centroid).
+static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__restrict__ cb, int m, int k, int nb,
+                                                             u32x4 *__restrict__ atab, float *__restrict__ c2perm,
+                                                             float *__restrict__ maxc2, uint32_t *__restrict__ stat) {
     const int s = blockIdx.x;
     __shared__ float sh_max[256];
+    if (s == 0 && threadIdx.x < kStatSlots) stat[threadIdx.x * kStatStride] = 0u;
     float mx = 0.0f;
     for (int j = threadIdx.x; j < nb * 32; j += 256) {
         const int b = j / 32, i = j % 32;
         float c2 = kPadScore;  // padding centroids: finite, so that index bits can be packed in
-        float c[SD];
+        float c[8];
         if (j < k) {
             c2 = 0.0f;
 #pragma unroll
-            for (int t = 0; t < SD; ++t) {
-                c[t] = cb[((size_t)s * k + j) * SD + t];
+            for (int t = 0; t < 8; ++t) {
+                c[t] = cb[((size_t)s * k + j) * 8 + t];
                 c2 = __builtin_fmaf(c[t], c[t], c2);
             }
             mx = fmaxf(mx, c2);
             if (!(c2 == c2)) mx = c2;  // a NaN poisons the bound on purpose
         } else {
 #pragma unroll
-            for (int t = 0; t < SD; ++t) c[t] = 0.0f;
+            for (int t = 0; t < 8; ++t) c[t] = 0.0f;
         }
-        // A operand: lane = i + 32*h holds dims [h*HS, (h+1)*HS)
+        uint32_t hb[8], lb[8];
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
+        for (int t = 0; t < 8; ++t) {
+            const float a = -2.0f * c[t];
+            hb[t] = bf16_rne_bits(a);
+            lb[t] = bf16_rne_bits(a - bf16_bits_to_float(hb[t]));
+        }
+        u32x4 ah, al;
 #pragma unroll
-            for (int t = 0; t < HS; ++t)
-                atab[(((size_t)s * nb + b) * 64 + i + 32 * h) * HS + t] = -2.0f * c[h * HS + t];
+        for (int w = 0; w < 4; ++w) {
+            ah[w] = hb[2 * w] | (hb[2 * w + 1] << 16);
+            al[w] = lb[2 * w] | (lb[2 * w + 1] << 16);
+        }
+        const u32x4 ones = {0x3f803f80u, 0x00003f80u, 0u, 0u};  // 1, 1, 1, 0, ...
+        u32x4 *dst = atab + ((size_t)s * nb + b) * 128;
+        dst[i] = ah;
+        dst[32 + i] = ah;
+        dst[64 + i] = al;
+        dst[96 + i] = ones;
         // accumulator order: lane half h, register v <-> centroid 8*(v/4) + 4*h + v%4
         const int hh = (i / 4) % 2, v = (i / 8) * 4 + i % 4;
         c2perm[(((size_t)s * nb + b) * 2 + hh) * 16 + v] = c2;
@@ -84,93 +157,151 @@ __global__ void __launch_bounds__(256) k_mfma_prep(const float *__restrict__ cb,
             if (!(r == r)) break;
         }
         maxc2[s] = r;
-        if (s == 0) *list_count = 0;
     }
 }
 
-// Scores are compared through their bit patterns as signed integers: for non-negative floats
-// that is the float order, a slightly negative score (cancellation) still sorts below every
-// positive one, and integer min / med3 need no NaN canonicalisation.  Two negative scores sort
-// in reverse, which only happens inside the error bound, i.e. for pairs that are re-checked.
-__device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
-__device__ __forceinline__ int imax(int a, int b) { return a > b ? a : b; }
-__device__ __forceinline__ int imed3(int a, int b, int c) {
-    return imax(imin(a, b), imin(imax(a, b), c));
+// The reference's argmin of one row's sub-vector (8 floats, the same in every lane) over the k
+// centroids of a block, by the whole wave: lane l takes centroids l, l + 64, ...; the smallest
+// (distance, index) pair wins, which is the reference's strict '<' scan (src/utils.rs:63-70,
+// src/pq.rs:166-174).  A NaN distance is never chosen unless it is centroid 0's, which is never
+// replaced.  Euclidean compares the roots, as the reference does.
+template <int METRIC>
+__device__ __forceinline__ int exact_argmin8_wave(const float (&xs)[8], const float *__restrict__ cb, int k,
+                                                  int lane) {
+    const float inf = __builtin_inff();
+    float bd = inf, d0 = 0.0f;
+    int bi = 0x7fffffff;
+    for (int j0 = 0; j0 < k; j0 += 256) {
+        // the four loads of a lane are issued together: one memory round trip per 256 centroids
+        float4 c0[4], c1[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int j = j0 + lane + 64 * q;
+            const float4 *cp = reinterpret_cast<const float4 *>(cb + (size_t)(j < k ? j : 0) * 8);
+            c0[q] = cp[0];
+            c1[q] = cp[1];
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int j = j0 + lane + 64 * q;
+            const float c[8] = {c0[q].x, c0[q].y, c0[q].z, c0[q].w, c1[q].x, c1[q].y, c1[q].z, c1[q].w};
+            float d = d_sq<8>(xs, c);
+            if constexpr (METRIC == M_EUCLID) d = sqrtf(d);
+            if (j == 0) d0 = d;
+            d = (d == d) ? d : inf;
+            if (j < k && (d < bd || bi == 0x7fffffff)) {  // ascending j inside the lane: strict '<' keeps the first
+                bd = d;
+                bi = j;
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float od = __shfl_xor(bd, off);
+        const int oi = __shfl_xor(bi, off);
+        const bool take = (od < bd) || (od == bd && oi < bi);
+        bd = take ? od : bd;
+        bi = take ? oi : bi;
+    }
+    d0 = __shfl(d0, 0);
+    return (d0 == d0) ? bi : 0;
 }
 
-// One wave = TILES tiles of 32 rows, all column blocks.  256 threads = 4 waves.
-// The sub-vectors of SG consecutive column blocks are loaded together, so that with SG * SD * 4
-// = 128 bytes every line of the rows is fetched once.
-template <int SD, bool LBG, int TILES, int SG>
-__global__ void __launch_bounds__(256) k_assign_mfma(AssignArgs a, MfmaTables tb) {
-    constexpr int HS = SD / 2;     // floats per lane of a sub-vector
-    extern __shared__ float lds_c2[];  // [m][nb][2][16]
+// One wave = TILES tiles of 32 rows and SG consecutive column blocks of 8 floats (SG = 4: one
+// 128-byte line of every row).  256 threads = 4 waves; grid = (row tiles, groups of column blocks),
+// so that the waves are short enough for the last round of workgroups not to leave the chip idle.
+template <int METRIC, bool LBG, int TILES, int SG>
+__global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
+    constexpr int SD = 8;
+    extern __shared__ float lds_c2[];  // [SG][nb][2][16]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int nb = tb.nb, m = a.m;
-    for (int i = threadIdx.x; i < m * nb * 32; i += 256) lds_c2[i] = tb.c2perm[i];
+    const int s0 = blockIdx.y * SG;
+    for (int i = threadIdx.x; i < SG * nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s0 * nb * 32 + i];
     __syncthreads();
     const int64_t row_base = ((int64_t)blockIdx.x * 4 + wave) * (32 * TILES);
     if (row_base >= a.n) return;
 
-    // index bits of the 16 accumulator registers of this lane half
     uint32_t cvh[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) cvh[v] = (uint32_t)(8 * (v / 4) + 4 * h + v % 4);
 
-    // encode mode: the codes of a row are collected in registers and stored once per row
-    constexpr int MAXW = 4;  // up to 16 column blocks packed
-    const bool packed_out = !LBG && (m % 4 == 0) && (m <= 4 * MAXW);
-    uint32_t cw[TILES][MAXW];
+    float xall[TILES][SG][SD];
+    uint8_t old[TILES][SG];
+    uint32_t cw[TILES];
+    uint32_t n_exact = 0;
 #pragma unroll
-    for (int t = 0; t < TILES; ++t)
+    for (int t = 0; t < TILES; ++t) {
+        const int64_t row = row_base + 32 * t + r;
+        cw[t] = 0u;
+        if (row < a.n) {
+            const float *xr = a.x + row * a.ld + (int64_t)s0 * SD;
 #pragma unroll
-        for (int w = 0; w < MAXW; ++w) cw[t][w] = 0u;
-
-    for (int s0 = 0; s0 < m; s0 += SG) {
-      float xall[TILES][SG][HS];
+            for (int q = 0; q < SG; ++q)
 #pragma unroll
-      for (int t = 0; t < TILES; ++t) {
-          const int64_t row = row_base + 32 * t + r;
-          if (row < a.n) {
-              const float *xr = a.x + row * a.ld + (int64_t)s0 * SD + h * HS;
+                for (int u = 0; u < SD; ++u) xall[t][q][u] = xr[q * SD + u];
+        } else {
 #pragma unroll
-              for (int q = 0; q < SG; ++q)
+            for (int q = 0; q < SG; ++q)
 #pragma unroll
-                  for (int u = 0; u < HS; ++u) xall[t][q][u] = xr[q * SD + u];
-          } else {
+                for (int u = 0; u < SD; ++u) xall[t][q][u] = 0.0f;
+        }
+        if constexpr (LBG) {
 #pragma unroll
-              for (int q = 0; q < SG; ++q)
+            for (int q = 0; q < SG; ++q)
+                old[t][q] = (row < a.n && h == 0) ? a.codes[(size_t)(s0 + q) * a.n + row] : (uint8_t)0;
+        }
+    }
 #pragma unroll
-                  for (int u = 0; u < HS; ++u) xall[t][q][u] = 0.0f;
-          }
-      }
-#pragma unroll
-      for (int q = 0; q < SG; ++q) {
+    for (int q = 0; q < SG; ++q) {
         const int s = s0 + q;
         if constexpr (LBG) {
             if (a.done[s]) continue;
         }
-        float xb[TILES][HS], x2[TILES];
+        u32x4 b1[TILES], b2[TILES];
+        float x2[TILES];
         int m1[TILES], m2[TILES];
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
             float p = 0.0f;
+            uint32_t hb[4];
+            float lo[SD];
 #pragma unroll
-            for (int u = 0; u < HS; ++u) {
-                xb[t][u] = xall[t][q][u];
-                p = __builtin_fmaf(xb[t][u], xb[t][u], p);
+            for (int u = 0; u < SD; ++u) p = __builtin_fmaf(xall[t][q][u], xall[t][q][u], p);
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                hb[w] = bf16_pack2(xall[t][q][2 * w], xall[t][q][2 * w + 1]);
+                lo[2 * w] = xall[t][q][2 * w] - __uint_as_float(hb[w] << 16);
+                lo[2 * w + 1] = xall[t][q][2 * w + 1] - __uint_as_float(hb[w] & 0xffff0000u);
             }
-            x2[t] = p + __shfl_xor(p, 32);
+            x2[t] = p;
+            // ||x||^2 in three bf16 parts (exact to 2^-24)
+            const uint32_t p0 = bf16_pack2(p, 0.0f);
+            const float r1 = p - __uint_as_float(p0 << 16);
+            const uint32_t p1 = bf16_pack2(r1, 0.0f);
+            const float r2 = r1 - __uint_as_float(p1 << 16);
+            const uint32_t p2 = bf16_pack2(r2, 0.0f);
+            const uint32_t xparts[4] = {(p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu, 0u, 0u};
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t lw = bf16_pack2(lo[2 * w], lo[2 * w + 1]);
+                b1[t][w] = h ? lw : hb[w];
+                b2[t][w] = h ? xparts[w] : hb[w];
+            }
             m1[t] = 0x7f800000;  // +inf
             m2[t] = 0x7f800000;
         }
-        const float *ap = tb.atab + ((size_t)s * nb * 64 + lane) * HS;
-        const float *cp = lds_c2 + ((size_t)s * nb * 2 + h) * 16;
+        const u32x4 *ap = tb.atab + (size_t)s * nb * 128 + lane;
+        const float *cp = lds_c2 + ((size_t)q * nb * 2 + h) * 16;
+        u32x4 a1 = ap[0], a2 = ap[64];
         for (int b = 0; b < nb; ++b) {
-            float av[HS], c2v[16];
-#pragma unroll
-            for (int u = 0; u < HS; ++u) av[u] = ap[(size_t)b * 64 * HS + u];
+            const u32x4 a1c = a1, a2c = a2;
+            if (b + 1 < nb) {
+                a1 = ap[(size_t)(b + 1) * 128];
+                a2 = ap[(size_t)(b + 1) * 128 + 64];
+            }
+            floatx16 c2v;
 #pragma unroll
             for (int v = 0; v < 16; ++v) c2v[v] = cp[b * 32 + v];
             uint32_t idxb[16];
@@ -178,22 +309,21 @@ __global__ void __launch_bounds__(256) k_assign_mfma(AssignArgs a, MfmaTables tb
             for (int v = 0; v < 16; ++v) idxb[v] = cvh[v] | ((uint32_t)b << 5);
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
-                floatx16 acc;
+                floatx16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    __builtin_bit_cast(bf16x8, a1c), __builtin_bit_cast(bf16x8, b1[t]), c2v, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                    __builtin_bit_cast(bf16x8, a2c), __builtin_bit_cast(bf16x8, b2[t]), acc, 0, 0, 0);
+                int key[16];
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[v] = c2v[v] + x2[t];
+                for (int v = 0; v < 16; ++v)
+                    key[v] = (int)((__float_as_uint(acc[v]) & 0xFFFFFF00u) | idxb[v]);
 #pragma unroll
-                for (int u = 0; u < HS; ++u)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u], xb[t][u], acc, 0, 0, 0);
-                // running smallest / second smallest with the centroid index in the low 8 bits
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    int key = (int)((__float_as_uint(acc[v]) & 0xFFFFFF00u) | idxb[v]);
-                    m2[t] = imed3(m1[t], m2[t], key);
-                    m1[t] = imin(m1[t], key);
-                }
+                for (int v = 0; v < 16; v += 4)
+                    top2_push4(m1[t], m2[t], key[v], key[v + 1], key[v + 2], key[v + 3]);
             }
         }
         const float mc2 = tb.maxc2[s];
+        const float *cb_s = a.cb + (size_t)s * a.k * SD;
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
             // the partner lane (other half) saw the other 16 centroids of every block
@@ -201,100 +331,50 @@ __global__ void __launch_bounds__(256) k_assign_mfma(AssignArgs a, MfmaTables tb
             const float s1 = __int_as_float(imin(m1[t], o1));
             const float s2 = __int_as_float(imin(imax(m1[t], o1), imin(m2[t], o2)));
             const int64_t row = row_base + 32 * t + r;
-            if (h == 0 && row < a.n) {
-                float bound = x2[t] + mc2;
-                float margin = 6.103515625e-05f * fabsf(s2) + 1.52587890625e-05f * bound;
-                bool sure = (s2 - s1) > margin;  // false for NaN / inf-inf
-                sure = sure && (bound < 1e29f) && (s1 < 1e29f);
-                if (sure) {
-                    uint8_t code = (uint8_t)(__float_as_uint(s1) & 0xFFu);
-                    if constexpr (LBG) {
-                        uint8_t *p = a.codes + (size_t)s * a.n + row;
-                        if (*p != code) {
-                            *p = code;
-                            a.changed[s] = 1;
-                        }
-                    } else if (packed_out) {
+            const bool mine = h == 0 && row < a.n;
+            const float bound = x2[t] + mc2;
+            const float margin = 6.103515625e-05f * fabsf(s2) + 1.220703125e-04f * bound;
+            bool sure = (s2 - s1) > margin;  // false for NaN / inf-inf
+            sure = sure && (bound < 1e29f) && (s1 < 1e29f);
+            int code = (int)(__float_as_uint(s1) & 0xFFu);
+            // undecided rows: the reference-order argmin, one row at a time by the whole wave
+            unsigned long long todo = __ballot(mine && !sure);
+            n_exact += (uint32_t)__popcll(todo);
+            while (todo) {
+                const int src = __builtin_amdgcn_readfirstlane(__ffsll(todo) - 1);
+                float xs[SD];
 #pragma unroll
-                        for (int w = 0; w < MAXW; ++w)
-                            if (w == (s >> 2)) cw[t][w] |= (uint32_t)code << (8 * (s & 3));
-                    } else {
-                        a.codes[row * m + s] = code;
+                for (int u = 0; u < SD; ++u)
+                    xs[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xall[t][q][u]), src));
+                const int best = exact_argmin8_wave<METRIC>(xs, cb_s, a.k, lane);
+                if (lane == src) code = best;
+                todo &= todo - 1;
+            }
+            if (mine) {
+                if constexpr (LBG) {
+                    if (old[t][q] != (uint8_t)code) {
+                        a.codes[(size_t)s * a.n + row] = (uint8_t)code;
+                        mark_changed(a.changed + s);
                     }
+                } else if (SG == 4) {
+                    cw[t] |= (uint32_t)code << (8 * q);
                 } else {
-                    uint32_t pos = atomicAdd(tb.list_count, 1u);
-                    tb.list[pos] = (uint32_t)(row * m + s);
+                    a.codes[row * m + s] = (uint8_t)code;
                 }
             }
         }
     }
-    }  // column-block group
-    if constexpr (!LBG) {
-        if (packed_out && h == 0) {
+    if constexpr (!LBG && SG == 4) {
+        if (h == 0) {
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
                 const int64_t row = row_base + 32 * t + r;
-                if (row < a.n) {
-                    uint32_t *dst = reinterpret_cast<uint32_t *>(a.codes + row * m);
-#pragma unroll
-                    for (int w = 0; w < MAXW; ++w)
-                        if (w < m / 4) dst[w] = cw[t][w];
-                }
+                if (row < a.n) *reinterpret_cast<uint32_t *>(a.codes + row * m + s0) = cw[t];
             }
         }
     }
-}
-
-// Pass 2: exact reference-order argmin for the listed (row, block) pairs.  One lane per pair.
-template <int SD, int METRIC, bool LBG>
-__global__ void __launch_bounds__(256) k_assign_recheck(AssignArgs a, const uint32_t *__restrict__ list,
-                                                        const uint32_t *__restrict__ list_count) {
-    const uint32_t count = *list_count;
-    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < count; i += gridDim.x * 256) {
-        const uint32_t e = list[i];
-        const int64_t row = e / (uint32_t)a.m;
-        const int s = (int)(e % (uint32_t)a.m);
-        float x[SD], c[SD];
-        const float *xr = a.x + row * a.ld + (int64_t)s * SD;
-#pragma unroll
-        for (int t = 0; t < SD; ++t) x[t] = xr[t];
-        const float *cb = a.cb + (size_t)s * a.k * SD;
-        int best = 0;
-#pragma unroll
-        for (int t = 0; t < SD; ++t) c[t] = cb[t];
-        float bd = d_sq<SD>(x, c), pd = __builtin_inff();
-        for (int j = 1; j < a.k; ++j) {
-#pragma unroll
-            for (int t = 0; t < SD; ++t) c[t] = cb[(size_t)j * SD + t];
-            float d = d_sq<SD>(x, c);
-            bool u = d < bd;
-            if constexpr (METRIC == M_EUCLID) pd = u ? bd : pd;
-            bd = u ? d : bd;
-            best = u ? j : best;
-        }
-        if constexpr (METRIC == M_EUCLID) {
-            float sr = sqrtf(bd);
-            if (sqrtf(pd) == sr) {
-                for (int j = 0; j < best; ++j) {
-#pragma unroll
-                    for (int t = 0; t < SD; ++t) c[t] = cb[(size_t)j * SD + t];
-                    if (sqrtf(d_sq<SD>(x, c)) == sr) {
-                        best = j;
-                        break;
-                    }
-                }
-            }
-        }
-        if constexpr (LBG) {
-            uint8_t *p = a.codes + (size_t)s * a.n + row;
-            if (*p != (uint8_t)best) {
-                *p = (uint8_t)best;
-                a.changed[s] = 1;
-            }
-        } else {
-            a.codes[row * a.m + s] = (uint8_t)best;
-        }
-    }
+    if (lane == 0 && n_exact)
+        atomicAdd(tb.stat + ((blockIdx.x * 4 + wave) & (kStatSlots - 1)) * kStatStride, n_exact);
 }
 
 }  // namespace vq
@@ -454,7 +534,7 @@ __global__ void __launch_bounds__(256) k_assign_mfma_wide(AssignArgs a, MfmaWide
                 uint8_t *pc = a.codes + (size_t)s * a.n + row;
                 if (*pc != code) {
                     *pc = code;
-                    a.changed[s] = 1;
+                    mark_changed(a.changed + s);
                 }
             } else {
                 a.codes[row * a.m + s] = code;
@@ -462,60 +542,6 @@ __global__ void __launch_bounds__(256) k_assign_mfma_wide(AssignArgs a, MfmaWide
         } else {
             const uint32_t pos = atomicAdd(tb.list_count, 1u);
             tb.list[pos] = (uint32_t)(row * a.m + s);
-        }
-    }
-}
-
-// Pass 2 for any sub_dim: exact reference-order argmin for the listed pairs, one lane per pair.
-template <int METRIC, bool LBG>
-__global__ void __launch_bounds__(256) k_assign_recheck_dyn(AssignArgs a, int sd, const uint32_t *__restrict__ list,
-                                                            const uint32_t *__restrict__ list_count) {
-    const uint32_t count = *list_count;
-    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < count; i += gridDim.x * 256) {
-        const uint32_t e = list[i];
-        const int64_t row = e / (uint32_t)a.m;
-        const int s = (int)(e % (uint32_t)a.m);
-        const float *__restrict__ xr = a.x + row * a.ld + (int64_t)s * sd;
-        const float *__restrict__ cb = a.cb + (size_t)s * a.k * sd;
-        int best = 0;
-        float bd = 0.0f, pd = __builtin_inff();
-        for (int j = 0; j < a.k; ++j) {
-            float acc = 0.0f;
-            for (int t = 0; t < sd; ++t) {
-                float d = xr[t] - cb[(size_t)j * sd + t];
-                float q = d * d;
-                acc = acc + q;
-            }
-            bool u = (j == 0) || (acc < bd);
-            if constexpr (METRIC == M_EUCLID) pd = (u && j != 0) ? bd : pd;
-            bd = u ? acc : bd;
-            best = u ? j : best;
-        }
-        if constexpr (METRIC == M_EUCLID) {
-            float sr = sqrtf(bd);
-            if (sqrtf(pd) == sr) {
-                for (int j = 0; j < best; ++j) {
-                    float acc = 0.0f;
-                    for (int t = 0; t < sd; ++t) {
-                        float d = xr[t] - cb[(size_t)j * sd + t];
-                        float q = d * d;
-                        acc = acc + q;
-                    }
-                    if (sqrtf(acc) == sr) {
-                        best = j;
-                        break;
-                    }
-                }
-            }
-        }
-        if constexpr (LBG) {
-            uint8_t *p = a.codes + (size_t)s * a.n + row;
-            if (*p != (uint8_t)best) {
-                *p = (uint8_t)best;
-                a.changed[s] = 1;
-            }
-        } else {
-            a.codes[row * a.m + s] = (uint8_t)best;
         }
     }
 }

@@ -23,7 +23,8 @@ struct vq_ctx {
     std::string err;
     // grow-only device workspace
     DevBuf flags, tables, hist, seg, part_sum, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;
-    DevBuf mfma_tab, mfma_list;  // tables and re-check list of the matrix-core assignment
+    DevBuf mfma_tab, mfma_list, mfma_stat;  // tables, re-check list and counters of the matrix-core assignment
+    int recheck_src = 0;         // where the last pass counted its undecided pairs: 1 mfma_stat, 2 mfma_list
     int assign_path = 0;         // 0 = matrix cores where a kernel exists, 1 = vector ALU only
     DevBuf tmp_a, tmp_b, tmp_c, tmp_d, tmp_e, tmp_f;  // scratch of the RVQ / OPQ / TSVQ entry points
     // optional per-kernel-class timing (HIP events on the stream)

@@ -100,35 +100,34 @@ int32_t launch_assign_m(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     return VQ_OK;
 }
 
-// Matrix-core pass + exact re-check of the undecided pairs (assign_mfma.hpp).
-template <int SD, int METRIC, bool LBG>
+// 8-float column blocks: bf16-split scores on the matrix cores, undecided rows resolved in the
+// same kernel by the reference-order argmin (assign_mfma.hpp).
+template <int METRIC, bool LBG>
 int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
     const int nb = (a.k + 31) / 32;
-    const size_t n_atab = (size_t)a.m * nb * 64 * (SD / 2), n_c2 = (size_t)a.m * nb * 32;
+    // A operands: 2 x 64 lanes x 16 bytes per (s, block of 32 centroids)
+    const size_t n_atab = (size_t)a.m * nb * 512, n_c2 = (size_t)a.m * nb * 32;
     VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + a.m) + 64));
-    VQ_TRY(ensure(ctx, ctx->mfma_list, sizeof(uint32_t) * ((size_t)a.n * a.m + 4)));
+    VQ_TRY(ensure(ctx, ctx->mfma_stat, sizeof(uint32_t) * vq::kStatSlots * vq::kStatStride));
     float *atab = (float *)ctx->mfma_tab.p;
     float *c2perm = atab + n_atab;
     float *maxc2 = c2perm + n_c2;
-    uint32_t *count = (uint32_t *)ctx->mfma_list.p;
-    uint32_t *list = count + 4;
-    hipLaunchKernelGGL((vq::k_mfma_prep<SD>), dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, atab,
-                       c2perm, maxc2, count);
-    vq::MfmaTables tb{atab, c2perm, maxc2, list, count, nb};
-    const size_t lds = sizeof(float) * n_c2;
+    uint32_t *stat = (uint32_t *)ctx->mfma_stat.p;
     constexpr int TILES = VQ_MFMA_TILES;
+    hipLaunchKernelGGL(vq::k_mfma_bf_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb,
+                       (vq::u32x4 *)atab, c2perm, maxc2, stat);
+    vq::MfmaBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, stat, nb};
     // 4 column blocks of 8 floats = one 128-byte line per row
-    auto kern = (a.m % 4 == 0) ? vq::k_assign_mfma<SD, LBG, TILES, 4> : vq::k_assign_mfma<SD, LBG, TILES, 1>;
-    if (lds > 48 * 1024)
-        VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    const bool g4 = a.m % 4 == 0;
+    auto kern = g4 ? vq::k_assign_mfma_bf<METRIC, LBG, TILES, 4> : vq::k_assign_mfma_bf<METRIC, LBG, TILES, 1>;
+    const size_t lds = sizeof(float) * (g4 ? 4 : 1) * nb * 32;
     {
         ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
-        hipLaunchKernelGGL(kern, dim3(cdiv(a.n, 4 * 32 * TILES)), dim3(256), lds, ctx->stream, a, tb);
+        hipLaunchKernelGGL(kern, dim3(cdiv(a.n, 4 * 32 * TILES), g4 ? a.m / 4 : a.m), dim3(256), lds, ctx->stream,
+                           a, tb);
     }
-    hipLaunchKernelGGL((vq::k_assign_recheck<SD, METRIC, LBG>), dim3(1024), dim3(256), 0, ctx->stream, a,
-                       (const uint32_t *)list, (const uint32_t *)count);
     VQ_HIP(ctx, hipGetLastError());
+    ctx->recheck_src = 1;
     return VQ_OK;
 }
 
@@ -181,12 +180,13 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
                            ctx->stream, a, tb);
     }
     VQ_HIP(ctx, hipGetLastError());
+    ctx->recheck_src = 2;
     return launch_wide_exact<METRIC, LBG>(ctx, a, sd, list, count);
 }
 
 template <int METRIC, bool LBG>
 bool mfma_wide_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
-    if (ctx->assign_path != 0) return false;
+    if (ctx->assign_path == 1) return false;
     if (METRIC != vq::M_SQ && METRIC != vq::M_EUCLID) return false;
     if (sd < 16 || sd % 8 != 0 || a.k > 256 || a.m > 65535) return false;
     // float4 row loads
@@ -196,19 +196,18 @@ bool mfma_wide_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
 
 template <int METRIC, bool LBG>
 bool mfma_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
-    if (ctx->assign_path != 0) return false;
+    if (ctx->assign_path == 1) return false;
     if (METRIC != vq::M_SQ && METRIC != vq::M_EUCLID) return false;
-    if (sd != 8) return false;
-    // tables must fit LDS; tiny inputs gain nothing
-    return (size_t)a.m * ((a.k + 31) / 32) * 32 * sizeof(float) <= 64 * 1024 && (int64_t)a.n * a.m < (1LL << 32);
+    if (sd != 8 || (reinterpret_cast<uintptr_t>(a.cb) & 15) != 0) return false;  // float4 centroid loads
+    return a.k <= 256;
 }
 
 template <bool LBG>
 int32_t launch_assign(vq_ctx *ctx, int metric, const vq::AssignArgs &a, int sd) {
     if (metric == VQ_SQEUCLIDEAN && mfma_applicable<vq::M_SQ, LBG>(ctx, a, sd))
-        return launch_mfma<8, vq::M_SQ, LBG>(ctx, a);
+        return launch_mfma<vq::M_SQ, LBG>(ctx, a);
     if (metric == VQ_EUCLIDEAN && mfma_applicable<vq::M_EUCLID, LBG>(ctx, a, sd))
-        return launch_mfma<8, vq::M_EUCLID, LBG>(ctx, a);
+        return launch_mfma<vq::M_EUCLID, LBG>(ctx, a);
     if (metric == VQ_SQEUCLIDEAN && mfma_wide_applicable<vq::M_SQ, LBG>(ctx, a, sd))
         return launch_mfma_wide<vq::M_SQ, LBG>(ctx, a, sd);
     if (metric == VQ_EUCLIDEAN && mfma_wide_applicable<vq::M_EUCLID, LBG>(ctx, a, sd))
@@ -339,7 +338,7 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     (void)hipStreamSynchronize(ctx->stream);
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
-                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
+                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     prof_collect(ctx);
@@ -414,9 +413,16 @@ int32_t vq_ctx_set_assign_path(vq_ctx *ctx, int32_t path) {
 int32_t vq_ctx_last_recheck_count(vq_ctx *ctx, uint32_t *h_count) {
     if (!ctx || !h_count) return VQ_ERR_INVALID_ARG;
     *h_count = 0;
-    if (!ctx->mfma_list.p) return VQ_OK;
-    VQ_HIP(ctx, hipMemcpyAsync(h_count, ctx->mfma_list.p, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
-    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (ctx->recheck_src == 1) {
+        uint32_t h[vq::kStatSlots * vq::kStatStride];
+        VQ_HIP(ctx, hipMemcpyAsync(h, ctx->mfma_stat.p, sizeof(h), hipMemcpyDeviceToHost, ctx->stream));
+        VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        for (int i = 0; i < vq::kStatSlots; ++i) *h_count += h[i * vq::kStatStride];
+    } else if (ctx->recheck_src == 2) {
+        VQ_HIP(ctx, hipMemcpyAsync(h_count, ctx->mfma_list.p, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                                   ctx->stream));
+        VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    }
     return VQ_OK;
 }
 
