@@ -279,6 +279,62 @@ static __global__ void __launch_bounds__(256) k_lbg_leafsum(LbgState st, const f
     st.leaf_sum[((size_t)s * st.leaf_cap + leaf) * sd + t] = acc;
 }
 
+// Narrow column blocks (sub_dim a power of two up to 32): one wave per leaf.  A lane-per-component
+// walk as above leaves most of the wave idle and pays one memory round trip per 32 members; here
+// the 64 lanes fetch up to 2048 / sub_dim members at a time into LDS (row ids first, then the
+// sub-vectors, all loads of a chunk in flight together), and lanes 0..sub_dim-1 add them in list
+// order.
+constexpr int kLeafStage = 2048;  // floats staged per wave
+
+static __global__ void __launch_bounds__(256) k_lbg_leafsum_wave(LbgState st, const float *__restrict__ x,
+                                                                 int64_t n, int64_t ld, int sd, int sd_shift) {
+    const int s = blockIdx.y;
+    if (st.done[s]) return;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int64_t leaf = (int64_t)blockIdx.x * 4 + w;
+    if (leaf >= st.nleaves[s]) return;  // uniform per wave; the waves never synchronise
+    __shared__ float stage_all[4][kLeafStage];
+    float *stage = stage_all[w];
+    const uint2 d = st.leaf_desc[(size_t)s * st.leaf_cap + leaf];
+    const uint32_t *__restrict__ perm = st.perm + (size_t)s * n;
+    const float *__restrict__ xs = x + (int64_t)s * sd;
+    const uint32_t chunk = (uint32_t)(kLeafStage >> sd_shift);  // members per chunk
+    constexpr int E = kLeafStage / 64;                          // elements per lane and chunk
+    float acc = 0.0f;
+    for (uint32_t p = d.x; p < d.y; p += chunk) {
+        const uint32_t cm = (d.y - p < chunk) ? d.y - p : chunk;
+        const uint32_t tot = cm << sd_shift;
+        uint32_t row[E];
+        float v[E];
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+            const uint32_t e = (uint32_t)lane + 64u * i;
+            row[i] = (e < tot) ? perm[p + (e >> sd_shift)] : 0u;
+        }
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+            const uint32_t e = (uint32_t)lane + 64u * i;
+            v[i] = (e < tot) ? xs[(int64_t)row[i] * ld + (e & (uint32_t)(sd - 1))] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < E; ++i) stage[lane + 64 * i] = v[i];
+        __builtin_amdgcn_wave_barrier();
+        if (lane < sd) {
+            uint32_t mbr = 0;
+            for (; mbr + 8 <= cm; mbr += 8) {
+                float t[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) t[u] = stage[((mbr + u) << sd_shift) + lane];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) acc = acc + t[u];
+            }
+            for (; mbr < cm; ++mbr) acc = acc + stage[(mbr << sd_shift) + lane];
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (lane < sd) st.leaf_sum[((size_t)s * st.leaf_cap + leaf) * sd + lane] = acc;
+}
+
 // One lane per (cluster, component): the mean of a small cluster, the sequential fold over the
 // per-part leaves of a large one (gather path), or the re-seed row of an empty cluster
 // (src/vector.rs:315-316, src/utils.rs:98-101).
@@ -321,27 +377,28 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const 
 // One workgroup per (part, group of 4 column blocks); wave w of the group owns column block
 // 4g + w, so the four waves together consume whole 128-byte lines of the rows.  A wave walks
 // its part 64 rows at a time; a lane holds the 32-byte sub-vector of its row.  The rows of a
-// chunk are ranked inside their cluster with wave ballots and added to the cluster's
-// accumulator in LDS in rank order (round r: the lanes of rank r, all on different clusters) —
-// so every cluster receives its rows of this part in row order, one at a time, starting from
-// 0.0.  Emits the part's histogram and the per-part sums; no floating-point atomics.
+// chunk are added to their cluster's accumulator in LDS in rounds: in every round the lowest
+// pending lane of each cluster adds its row — so every cluster receives its rows of this part
+// in row order, one at a time, starting from 0.0.  Emits the part's histogram and the per-part sums; no floating-point atomics.
 static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const float *__restrict__ x, int64_t n,
                                                             int64_t ld) {
     const int g = blockIdx.y, b = blockIdx.x;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int s = 4 * g + w;
-    __shared__ float4 acc_all[4][kMaxK][2];
+    __shared__ float4 acc_lo[4][kMaxK], acc_hi[4][kMaxK];  // components 0-3 and 4-7 of every cluster
     __shared__ uint32_t cnt_all[4][kMaxK];
+    __shared__ uint32_t tag_all[4][kMaxK];
     if (st.done[s]) return;  // uniform per wave; the waves never synchronise with each other
-    float4(*acc)[2] = acc_all[w];
+    float4 *alo = acc_lo[w], *ahi = acc_hi[w];
     uint32_t *cnt = cnt_all[w];
+    uint32_t *tag = tag_all[w];
     for (int i = lane; i < kMaxK; i += 64) {
-        acc[i][0] = make_float4(0.f, 0.f, 0.f, 0.f);
-        acc[i][1] = make_float4(0.f, 0.f, 0.f, 0.f);
+        alo[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        ahi[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         cnt[i] = 0u;
+        tag[i] = 0xFFFFFFFFu;
     }
     __builtin_amdgcn_wave_barrier();
-    const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     const int64_t lo = (int64_t)b * kPartRows;
     const int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
     const uint8_t *__restrict__ codes = st.codes + (size_t)s * n;
@@ -369,9 +426,9 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
             const int64_t i0 = base + 64 * u;
             if (i0 >= hi) break;  // uniform
             const int64_t i = i0 + lane;
-            const bool valid = i < hi;
+            bool pending = i < hi;
             const float4 v0 = b0[u], v1 = b1[u];
-            const uint32_t c = valid ? bc[u] : 0u;
+            const uint32_t c = pending ? bc[u] : 0u;
             {
                 const int64_t in = i + 64 * PF;
                 if (in < hi) {
@@ -381,18 +438,16 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
                     bc[u] = codes[in];
                 }
             }
-            uint64_t mask = __ballot(valid);
-#pragma unroll
-            for (int bit = 0; bit < 8; ++bit) {
-                bool set = (c >> bit) & 1u;
-                uint64_t bal = __ballot(set);
-                mask &= set ? bal : ~bal;
-            }
-            const uint32_t rank = valid ? (uint32_t)__popcll(mask & lt) : 0xFFFFFFFFu;
-            if (rank == 0) cnt[c] += (uint32_t)__popcll(mask);  // one lane per cluster
-            for (uint32_t r = 0; __any(rank != 0xFFFFFFFFu && rank >= r); ++r) {
-                if (rank == r) {
-                    float4 a0 = acc[c][0], a1 = acc[c][1];
+            // Rounds: among the pending lanes of a cluster the lowest lane (= the earliest row)
+            // claims the cluster's tag with an LDS atomic min, adds its row, releases the tag.
+            // LDS operations of one wave are performed in program order, so the next round sees
+            // these writes; the wave barriers only pin the compiler's schedule (a fence or
+            // s_barrier here would also wait for the row prefetches in flight).
+            while (__any(pending)) {
+                if (pending) atomicMin(&tag[c], (uint32_t)lane);
+                __builtin_amdgcn_wave_barrier();
+                if (pending && tag[c] == (uint32_t)lane) {
+                    float4 a0 = alo[c], a1 = ahi[c];
                     a0.x = a0.x + v0.x;
                     a0.y = a0.y + v0.y;
                     a0.z = a0.z + v0.z;
@@ -401,19 +456,19 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
                     a1.y = a1.y + v1.y;
                     a1.z = a1.z + v1.z;
                     a1.w = a1.w + v1.w;
-                    acc[c][0] = a0;
-                    acc[c][1] = a1;
+                    alo[c] = a0;
+                    ahi[c] = a1;
+                    cnt[c] += 1u;
+                    tag[c] = 0xFFFFFFFFu;
+                    pending = false;
                 }
-                // LDS accesses of one wave are performed in program order, so the next round
-                // sees these writes; the barrier below only pins the compiler's schedule (a
-                // fence or s_barrier here would also wait for the row prefetches in flight)
                 __builtin_amdgcn_wave_barrier();
             }
         }
     }
     __builtin_amdgcn_wave_barrier();
     float4 *ps = reinterpret_cast<float4 *>(st.part_sum) + ((size_t)s * st.nparts + b) * kMaxK * 2;
-    for (int i = lane; i < kMaxK * 2; i += 64) ps[i] = (&acc[0][0])[i];
+    for (int i = lane; i < kMaxK * 2; i += 64) ps[i] = (i & 1) ? ahi[i >> 1] : alo[i >> 1];
     uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
     for (int j = lane; j < kMaxK; j += 64) h[j] = cnt[j];
 }

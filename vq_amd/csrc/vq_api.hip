@@ -571,8 +571,15 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
             hipLaunchKernelGGL(vq::k_lbg_combine8, dim3(cdiv((int64_t)k * 8, 256), m), dim3(256), 0, st, S, k,
                                d_codebooks);
         hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nparts, m), dim3(64), 0, st, S, n);
-        hipLaunchKernelGGL(vq::k_lbg_leafsum, dim3(cdiv((int64_t)leaf_cap * sd, 256), m), dim3(256), 0, st, S,
-                           d_x, n, ld, sd);
+        if (sd <= 32 && (sd & (sd - 1)) == 0) {
+            int shift = 0;
+            while ((1 << shift) < sd) ++shift;
+            hipLaunchKernelGGL(vq::k_lbg_leafsum_wave, dim3(cdiv(leaf_cap, 4), m), dim3(256), 0, st, S, d_x, n,
+                               ld, sd, shift);
+        } else {
+            hipLaunchKernelGGL(vq::k_lbg_leafsum, dim3(cdiv((int64_t)leaf_cap * sd, 256), m), dim3(256), 0, st,
+                               S, d_x, n, ld, sd);
+        }
         hipLaunchKernelGGL(vq::k_lbg_finalize, dim3(cdiv((int64_t)k * sd, 256), m), dim3(256), 0, st, S,
                            d_x, ld, k, sd, (const uint32_t *)ctx->reseed.p, n_reseed, d_codebooks);
         hipLaunchKernelGGL(vq::k_lbg_advance, dim3(cdiv(m, 64)), dim3(64), 0, st, S, m);
