@@ -377,9 +377,10 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const 
 // One workgroup per (part, group of 4 column blocks); wave w of the group owns column block
 // 4g + w, so the four waves together consume whole 128-byte lines of the rows.  A wave walks
 // its part 64 rows at a time; a lane holds the 32-byte sub-vector of its row.  The rows of a
-// chunk are added to their cluster's accumulator in LDS in rounds: in every round the lowest
-// pending lane of each cluster adds its row — so every cluster receives its rows of this part
-// in row order, one at a time, starting from 0.0.  Emits the part's histogram and the per-part sums; no floating-point atomics.
+// chunk are ranked inside their cluster with wave ballots and added to the cluster's
+// accumulator in LDS in rank order (round r: the lanes of rank r, all on different clusters) —
+// so every cluster receives its rows of this part in row order, one at a time, starting from
+// 0.0.  Emits the part's histogram and the per-part sums; no floating-point atomics.
 static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const float *__restrict__ x, int64_t n,
                                                             int64_t ld) {
     const int g = blockIdx.y, b = blockIdx.x;
@@ -387,16 +388,15 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
     const int s = 4 * g + w;
     __shared__ float4 acc_lo[4][kMaxK], acc_hi[4][kMaxK];  // components 0-3 and 4-7 of every cluster
     __shared__ uint32_t cnt_all[4][kMaxK];
-    __shared__ uint32_t tag_all[4][kMaxK];
     if (st.done[s]) return;  // uniform per wave; the waves never synchronise with each other
     float4 *alo = acc_lo[w], *ahi = acc_hi[w];
     uint32_t *cnt = cnt_all[w];
-    uint32_t *tag = tag_all[w];
+    const uint32_t lt_lo = (lane >= 32) ? 0xFFFFFFFFu : ((1u << lane) - 1u);
+    const uint32_t lt_hi = (lane <= 32) ? 0u : ((1u << (lane - 32)) - 1u);
     for (int i = lane; i < kMaxK; i += 64) {
         alo[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         ahi[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         cnt[i] = 0u;
-        tag[i] = 0xFFFFFFFFu;
     }
     __builtin_amdgcn_wave_barrier();
     const int64_t lo = (int64_t)b * kPartRows;
@@ -407,46 +407,62 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
     constexpr int PF = 4;
     float4 b0[PF], b1[PF];
     uint32_t bc[PF];
+    const float *xp = x + (lo + lane) * ld + (int64_t)s * 8;  // row of this lane in the chunk being fetched
+    const uint8_t *cp = codes + lo + lane;
+    const int64_t xstep = 64 * ld;
+    int left = (int)(hi - lo) - lane;  // rows from this lane's row of the fetched chunk to the end of the part
 #pragma unroll
     for (int u = 0; u < PF; ++u) {
         b0[u] = make_float4(0.f, 0.f, 0.f, 0.f);
         b1[u] = b0[u];
         bc[u] = 0u;
-        const int64_t i = lo + 64 * u + lane;
-        if (i < hi) {
-            const float4 *xr = reinterpret_cast<const float4 *>(x + i * ld + (int64_t)s * 8);
-            b0[u] = xr[0];
-            b1[u] = xr[1];
-            bc[u] = codes[i];
+        if (left > 0) {
+            b0[u] = reinterpret_cast<const float4 *>(xp)[0];
+            b1[u] = reinterpret_cast<const float4 *>(xp)[1];
+            bc[u] = *cp;
         }
+        xp += xstep;
+        cp += 64;
+        left -= 64;
     }
-    for (int64_t base = lo; base < hi; base += 64 * PF) {
+    int mine = (int)(hi - lo) - lane;  // > 0 while this lane's row of the current chunk exists
+    for (int base = 0; base < (int)(hi - lo); base += 64 * PF) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
-            const int64_t i0 = base + 64 * u;
-            if (i0 >= hi) break;  // uniform
-            const int64_t i = i0 + lane;
-            bool pending = i < hi;
+            if (base + 64 * u >= (int)(hi - lo)) break;  // uniform
+            bool pending = mine > 0;
+            mine -= 64;
             const float4 v0 = b0[u], v1 = b1[u];
             const uint32_t c = pending ? bc[u] : 0u;
-            {
-                const int64_t in = i + 64 * PF;
-                if (in < hi) {
-                    const float4 *xr = reinterpret_cast<const float4 *>(x + in * ld + (int64_t)s * 8);
-                    b0[u] = xr[0];
-                    b1[u] = xr[1];
-                    bc[u] = codes[in];
-                }
+            if (left > 0) {
+                b0[u] = reinterpret_cast<const float4 *>(xp)[0];
+                b1[u] = reinterpret_cast<const float4 *>(xp)[1];
+                bc[u] = *cp;
             }
-            // Rounds: among the pending lanes of a cluster the lowest lane (= the earliest row)
-            // claims the cluster's tag with an LDS atomic min, adds its row, releases the tag.
-            // LDS operations of one wave are performed in program order, so the next round sees
-            // these writes; the wave barriers only pin the compiler's schedule (a fence or
-            // s_barrier here would also wait for the row prefetches in flight).
-            while (__any(pending)) {
-                if (pending) atomicMin(&tag[c], (uint32_t)lane);
-                __builtin_amdgcn_wave_barrier();
-                if (pending && tag[c] == (uint32_t)lane) {
+            xp += xstep;
+            cp += 64;
+            left -= 64;
+            // Lanes of the same cluster, found with one wave ballot per code bit: a lane differs
+            // from lane j when some bit of its code differs from j's bit in the ballot.
+            const unsigned long long vb = __ballot(pending);
+            uint32_t bad_lo = ~(uint32_t)vb, bad_hi = ~(uint32_t)(vb >> 32);
+#pragma unroll
+            for (int bit = 0; bit < 8; bit += 2) {
+                const int sp0 = (int)(c << (31 - bit)) >> 31, sp1 = (int)(c << (30 - bit)) >> 31;  // 0 or -1
+                const unsigned long long bal0 = __ballot(sp0 != 0), bal1 = __ballot(sp1 != 0);
+                bad_lo = bad_lo | ((uint32_t)bal0 ^ (uint32_t)sp0) | ((uint32_t)bal1 ^ (uint32_t)sp1);
+                bad_hi = bad_hi | ((uint32_t)(bal0 >> 32) ^ (uint32_t)sp0) | ((uint32_t)(bal1 >> 32) ^ (uint32_t)sp1);
+            }
+            const uint32_t same_lo = ~bad_lo, same_hi = ~bad_hi;
+            const uint32_t rank =
+                pending ? (uint32_t)(__popc(same_lo & lt_lo) + __popc(same_hi & lt_hi)) : 0xFFFFFFFFu;
+            if (rank == 0) atomicAdd(&cnt[c], (uint32_t)(__popc(same_lo) + __popc(same_hi)));  // one lane per cluster
+            // Round r: the lanes of rank r (all on different clusters) add their rows.  LDS
+            // operations of one wave are performed in program order, so the next round sees these
+            // writes; the wave barrier only pins the compiler's schedule (a fence or s_barrier
+            // here would also wait for the row prefetches in flight).
+            for (uint32_t r = 0; __any(rank != 0xFFFFFFFFu && rank >= r); ++r) {
+                if (rank == r) {
                     float4 a0 = alo[c], a1 = ahi[c];
                     a0.x = a0.x + v0.x;
                     a0.y = a0.y + v0.y;
@@ -458,9 +474,6 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
                     a1.w = a1.w + v1.w;
                     alo[c] = a0;
                     ahi[c] = a1;
-                    cnt[c] += 1u;
-                    tag[c] = 0xFFFFFFFFu;
-                    pending = false;
                 }
                 __builtin_amdgcn_wave_barrier();
             }
