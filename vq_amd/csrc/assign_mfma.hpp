@@ -44,6 +44,20 @@ __device__ __forceinline__ int imin3(int a, int b, int c) {
     return r;
 }
 
+// (score bits & keep) | tag as one v_and_or_b32 with the tag in a scalar register: keep must be a
+// vector register the compiler cannot see through (with a literal mask it emits a v_and with the
+// literal and a v_or with the scalar operand, twice the issue time).  Left to the compiler rather
+// than written as inline assembly so that it inserts the wait states between a matrix
+// instruction and the first read of its result.
+__device__ __forceinline__ uint32_t opaque_vgpr(uint32_t value) {
+    uint32_t r;
+    asm volatile("v_mov_b32 %0, %1" : "=v"(r) : "s"(value));
+    return r;
+}
+__device__ __forceinline__ int pack_tag(float score, uint32_t keep, uint32_t tag) {
+    return (int)((__float_as_uint(score) & keep) | tag);
+}
+
 // Four new keys into the running (smallest, second smallest): 5 operations.
 // second smallest of {m1, m2, x, y} with m1 <= m2 is min(m2, med3(m1, x, y)).
 __device__ __forceinline__ void top2_push4(int &m1, int &m2, int k0, int k1, int k2, int k3) {
@@ -211,21 +225,21 @@ __device__ __forceinline__ int exact_argmin8_wave(const float (&xs)[8], const fl
 // 128-byte line of every row).  256 threads = 4 waves; grid = (row tiles, groups of column blocks),
 // so that the waves are short enough for the last round of workgroups not to leave the chip idle.
 template <int METRIC, bool LBG, int TILES, int SG>
-__global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
+__global__ void __launch_bounds__(256, (TILES * SG <= 4) ? 4 : 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
     constexpr int SD = 8;
     extern __shared__ float lds_c2[];  // [SG][nb][2][16]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int nb = tb.nb, m = a.m;
-    const int s0 = blockIdx.y * SG;
+    // consecutive workgroups take the column-block groups of the same rows, so that the lines of
+    // those rows are shared through the L2 while they are hot
+    const int ngroups = m / SG;
+    const int s0 = (int)(blockIdx.x % (unsigned)ngroups) * SG;
+    const int64_t tile_id = blockIdx.x / (unsigned)ngroups;
     for (int i = threadIdx.x; i < SG * nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s0 * nb * 32 + i];
     __syncthreads();
-    const int64_t row_base = ((int64_t)blockIdx.x * 4 + wave) * (32 * TILES);
+    const int64_t row_base = (tile_id * 4 + wave) * (32 * TILES);
     if (row_base >= a.n) return;
-
-    uint32_t cvh[16];
-#pragma unroll
-    for (int v = 0; v < 16; ++v) cvh[v] = (uint32_t)(8 * (v / 4) + 4 * h + v % 4);
 
     float xall[TILES][SG][SD];
     uint8_t old[TILES][SG];
@@ -294,19 +308,13 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
         }
         const u32x4 *ap = tb.atab + (size_t)s * nb * 128 + lane;
         const float *cp = lds_c2 + ((size_t)q * nb * 2 + h) * 16;
-        u32x4 a1 = ap[0], a2 = ap[64];
-        for (int b = 0; b < nb; ++b) {
-            const u32x4 a1c = a1, a2c = a2;
-            if (b + 1 < nb) {
-                a1 = ap[(size_t)(b + 1) * 128];
-                a2 = ap[(size_t)(b + 1) * 128 + 64];
-            }
+        // One block of 32 centroids against the TILES row tiles.  The packed index leaves out the
+        // lane half (bit 2), so it is the same in every lane and lives in scalar registers.
+        const uint32_t keep = opaque_vgpr(0xFFFFFF00u);
+        auto block = [&](int b, const u32x4 &a1c, const u32x4 &a2c) {
             floatx16 c2v;
 #pragma unroll
             for (int v = 0; v < 16; ++v) c2v[v] = cp[b * 32 + v];
-            uint32_t idxb[16];
-#pragma unroll
-            for (int v = 0; v < 16; ++v) idxb[v] = cvh[v] | ((uint32_t)b << 5);
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
                 floatx16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
@@ -316,10 +324,30 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
                 int key[16];
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
-                    key[v] = (int)((__float_as_uint(acc[v]) & 0xFFFFFF00u) | idxb[v]);
+                    key[v] = pack_tag(acc[v], keep, (uint32_t)(32 * b + 8 * (v / 4) + v % 4));
 #pragma unroll
                 for (int v = 0; v < 16; v += 4)
                     top2_push4(m1[t], m2[t], key[v], key[v + 1], key[v + 2], key[v + 3]);
+            }
+        };
+        // A operands of the next block are fetched while the current one is scored (two buffers)
+        u32x4 pa1 = ap[0], pa2 = ap[64], qa1 = pa1, qa2 = pa2;
+        if (nb > 1) {
+            qa1 = ap[128];
+            qa2 = ap[128 + 64];
+        }
+        for (int b = 0; b < nb; b += 2) {
+            block(b, pa1, pa2);
+            if (b + 2 < nb) {
+                pa1 = ap[(size_t)(b + 2) * 128];
+                pa2 = ap[(size_t)(b + 2) * 128 + 64];
+            }
+            if (b + 1 < nb) {
+                block(b + 1, qa1, qa2);
+                if (b + 3 < nb) {
+                    qa1 = ap[(size_t)(b + 3) * 128];
+                    qa2 = ap[(size_t)(b + 3) * 128 + 64];
+                }
             }
         }
         const float mc2 = tb.maxc2[s];
@@ -327,6 +355,8 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
             // the partner lane (other half) saw the other 16 centroids of every block
+            m1[t] |= 4 * h;  // bit 2 of the centroid index: the lane half
+            m2[t] |= 4 * h;
             int o1 = __shfl_xor(m1[t], 32), o2 = __shfl_xor(m2[t], 32);
             const float s1 = __int_as_float(imin(m1[t], o1));
             const float s2 = __int_as_float(imin(imax(m1[t], o1), imin(m2[t], o2)));
@@ -356,7 +386,7 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
                         a.codes[(size_t)s * a.n + row] = (uint8_t)code;
                         mark_changed(a.changed + s);
                     }
-                } else if (SG == 4) {
+                } else if (SG == 4 || SG == 2) {
                     cw[t] |= (uint32_t)code << (8 * q);
                 } else {
                     a.codes[row * m + s] = (uint8_t)code;
@@ -364,17 +394,22 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
             }
         }
     }
-    if constexpr (!LBG && SG == 4) {
+    if constexpr (!LBG && (SG == 4 || SG == 2)) {
         if (h == 0) {
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
                 const int64_t row = row_base + 32 * t + r;
-                if (row < a.n) *reinterpret_cast<uint32_t *>(a.codes + row * m + s0) = cw[t];
+                if (row < a.n) {
+                    if constexpr (SG == 4)
+                        *reinterpret_cast<uint32_t *>(a.codes + row * m + s0) = cw[t];
+                    else
+                        *reinterpret_cast<uint16_t *>(a.codes + row * m + s0) = (uint16_t)cw[t];
+                }
             }
         }
     }
     if (lane == 0 && n_exact)
-        atomicAdd(tb.stat + ((blockIdx.x * 4 + wave) & (kStatSlots - 1)) * kStatStride, n_exact);
+        atomicAdd(tb.stat + ((tile_id * 4 + wave) & (kStatSlots - 1)) * kStatStride, n_exact);
 }
 
 }  // namespace vq

@@ -335,6 +335,80 @@ static __global__ void __launch_bounds__(256) k_lbg_leafsum_wave(LbgState st, co
     if (lane < sd) st.leaf_sum[((size_t)s * st.leaf_cap + leaf) * sd + lane] = acc;
 }
 
+// Few, long leaves (the small clusters beside the streaming kernel: up to 1024 members each): one
+// workgroup per leaf.  All 256 threads fetch the members of a chunk (row ids, then 16-byte pieces
+// of the sub-vectors, every load of the chunk in flight together) and store them transposed in
+// LDS; lanes 0..sub_dim-1 of wave 0 then add them in list order, four members per LDS read.  The
+// chain of dependent adds is the only serial part left.
+constexpr int kLeafWgFloats = 8192;  // floats staged per chunk
+
+static __global__ void __launch_bounds__(256) k_lbg_leafsum_wg(LbgState st, const float *__restrict__ x, int64_t n,
+                                                               int64_t ld, int sd, int sd_shift) {
+    const int s = blockIdx.y;
+    if (st.done[s]) return;
+    const int64_t leaf = blockIdx.x;
+    if (leaf >= st.nleaves[s]) return;  // uniform per workgroup
+    __shared__ float stage[kLeafWgFloats + 4 * 32];
+    const int tid = threadIdx.x;
+    const uint2 d = st.leaf_desc[(size_t)s * st.leaf_cap + leaf];
+    const uint32_t *__restrict__ perm = st.perm + (size_t)s * n;
+    const float *__restrict__ xs = x + (int64_t)s * sd;
+    const uint32_t chunk = (uint32_t)(kLeafWgFloats >> sd_shift);  // members per chunk, a multiple of 4
+    const uint32_t stride = chunk + 4;                             // floats per component row in LDS
+    const int pshift = sd_shift - 2;                               // 16-byte pieces per member: 1 << pshift
+    constexpr int E = kLeafWgFloats / 4 / 256;                     // pieces per thread and chunk
+    float acc = 0.0f;
+    for (uint32_t p = d.x; p < d.y; p += chunk) {
+        const uint32_t cm = (d.y - p < chunk) ? d.y - p : chunk;
+        const uint32_t tot = cm << pshift;
+        uint32_t row[E];
+        float4 v[E];
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+            const uint32_t e = (uint32_t)tid + 256u * i;
+            row[i] = (e < tot) ? perm[p + (e >> pshift)] : 0u;
+        }
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+            const uint32_t e = (uint32_t)tid + 256u * i;
+            const uint32_t piece = e & ((1u << pshift) - 1u);
+            v[i] = (e < tot) ? *reinterpret_cast<const float4 *>(xs + (int64_t)row[i] * ld + 4 * piece)
+                             : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        __syncthreads();  // the previous chunk has been added
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+            const uint32_t e = (uint32_t)tid + 256u * i;
+            if (e < tot) {
+                const uint32_t mbr = e >> pshift, t0 = 4 * (e & ((1u << pshift) - 1u));
+                stage[(t0 + 0) * stride + mbr] = v[i].x;
+                stage[(t0 + 1) * stride + mbr] = v[i].y;
+                stage[(t0 + 2) * stride + mbr] = v[i].z;
+                stage[(t0 + 3) * stride + mbr] = v[i].w;
+            }
+        }
+        __syncthreads();
+        if (tid < sd) {
+            const float *mine = stage + (size_t)tid * stride;
+            uint32_t mbr = 0;
+            for (; mbr + 16 <= cm; mbr += 16) {
+                float4 q[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) q[u] = *reinterpret_cast<const float4 *>(mine + mbr + 4 * u);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    acc = acc + q[u].x;
+                    acc = acc + q[u].y;
+                    acc = acc + q[u].z;
+                    acc = acc + q[u].w;
+                }
+            }
+            for (; mbr < cm; ++mbr) acc = acc + mine[mbr];
+        }
+    }
+    if (tid < sd) st.leaf_sum[((size_t)s * st.leaf_cap + leaf) * sd + tid] = acc;
+}
+
 // One lane per (cluster, component): the mean of a small cluster, the sequential fold over the
 // per-part leaves of a large one (gather path), or the re-seed row of an empty cluster
 // (src/vector.rs:315-316, src/utils.rs:98-101).

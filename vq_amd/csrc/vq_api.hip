@@ -19,6 +19,9 @@
 #ifndef VQ_MFMA_TILES
 #define VQ_MFMA_TILES 2  // tiles of 32 rows per wave in the matrix-core assignment
 #endif
+#ifndef VQ_MFMA_SG
+#define VQ_MFMA_SG 2     // column blocks of 8 floats per wave (2: 64 bytes of each row, 4 waves per SIMD)
+#endif
 #include "lbg_update.hpp"
 
 namespace vqh {
@@ -118,13 +121,16 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
                        (vq::u32x4 *)atab, c2perm, maxc2, stat);
     vq::MfmaBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, stat, nb};
     // 4 column blocks of 8 floats = one 128-byte line per row
-    const bool g4 = a.m % 4 == 0;
-    auto kern = g4 ? vq::k_assign_mfma_bf<METRIC, LBG, TILES, 4> : vq::k_assign_mfma_bf<METRIC, LBG, TILES, 1>;
-    const size_t lds = sizeof(float) * (g4 ? 4 : 1) * nb * 32;
+    constexpr int SG = VQ_MFMA_SG;
+    const bool grouped = a.m % SG == 0;
+    auto kern = grouped ? vq::k_assign_mfma_bf<METRIC, LBG, TILES, SG> : vq::k_assign_mfma_bf<METRIC, LBG, TILES, 1>;
+    const int sg = grouped ? SG : 1;
+    const size_t lds = sizeof(float) * sg * nb * 32;
+    const int64_t blocks = cdiv(a.n, 4 * 32 * TILES) * (a.m / sg);
+    if (blocks >= (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * m too large for one launch");
     {
         ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
-        hipLaunchKernelGGL(kern, dim3(cdiv(a.n, 4 * 32 * TILES), g4 ? a.m / 4 : a.m), dim3(256), lds, ctx->stream,
-                           a, tb);
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, ctx->stream, a, tb);
     }
     VQ_HIP(ctx, hipGetLastError());
     ctx->recheck_src = 1;
@@ -571,9 +577,14 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
             hipLaunchKernelGGL(vq::k_lbg_combine8, dim3(cdiv((int64_t)k * 8, 256), m), dim3(256), 0, st, S, k,
                                d_codebooks);
         hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nparts, m), dim3(64), 0, st, S, n);
-        if (sd <= 32 && (sd & (sd - 1)) == 0) {
-            int shift = 0;
-            while ((1 << shift) < sd) ++shift;
+        int shift = 0;
+        while ((1 << shift) < sd) ++shift;
+        if (stream && sd >= 4 && sd <= 32 && (1 << shift) == sd && ld % 4 == 0 &&
+            (reinterpret_cast<uintptr_t>(d_x) & 15) == 0) {
+            // leaves are the few clusters of up to 1024 members beside the streaming kernel
+            hipLaunchKernelGGL(vq::k_lbg_leafsum_wg, dim3(leaf_cap, m), dim3(256), 0, st, S, d_x, n, ld, sd,
+                               shift);
+        } else if (sd <= 32 && (1 << shift) == sd) {
             hipLaunchKernelGGL(vq::k_lbg_leafsum_wave, dim3(cdiv(leaf_cap, 4), m), dim3(256), 0, st, S, d_x, n,
                                ld, sd, shift);
         } else {
