@@ -92,7 +92,7 @@ constexpr int kStatStride = 32;
 struct MfmaBfTables {
     const u32x4 *atab;     // [m][nb][2][64]  A operands of the two instructions, lane order
     const float *c2perm;   // [m][nb][2][16]  ||c||^2 in accumulator order (kPadScore for padding)
-    const float *maxc2;    // [m]
+    const float *maxc2;    // [m]  largest ||c||^2 of the column block (NaN if any is NaN)
     uint32_t *stat;        // [kStatSlots * kStatStride]  pairs decided by the exact path (measurement)
     int nb;                // ceil(k/32)
 };
@@ -113,15 +113,16 @@ __device__ __forceinline__ uint32_t bf16_pack2(float a, float b) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
-// Tables for k_assign_mfma_bf.  One thread per (s, padded centroid).
+// Tables for k_assign_mfma_bf.  One workgroup per column block s, one thread per padded centroid
+// (k <= 256); maxc2[s] = largest ||c||^2 of the block (NaN if any is NaN).
 static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__restrict__ cb, int m, int k, int nb,
                                                              u32x4 *__restrict__ atab, float *__restrict__ c2perm,
                                                              float *__restrict__ maxc2, uint32_t *__restrict__ stat) {
-    const int s = blockIdx.x;
-    __shared__ float sh_max[256];
-    if (s == 0 && threadIdx.x < kStatSlots) stat[threadIdx.x * kStatStride] = 0u;
+    const int s = blockIdx.x, j = threadIdx.x;
+    __shared__ float sh_max[4];
+    if (s == 0 && j < kStatSlots) stat[j * kStatStride] = 0u;
     float mx = 0.0f;
-    for (int j = threadIdx.x; j < nb * 32; j += 256) {
+    if (j < nb * 32) {
         const int b = j / 32, i = j % 32;
         float c2 = kPadScore;  // padding centroids: finite, so that index bits can be packed in
         float c[8];
@@ -132,8 +133,7 @@ static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__rest
                 c[t] = cb[((size_t)s * k + j) * 8 + t];
                 c2 = __builtin_fmaf(c[t], c[t], c2);
             }
-            mx = fmaxf(mx, c2);
-            if (!(c2 == c2)) mx = c2;  // a NaN poisons the bound on purpose
+            mx = c2;
         } else {
 #pragma unroll
             for (int t = 0; t < 8; ++t) c[t] = 0.0f;
@@ -161,14 +161,20 @@ static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__rest
         const int hh = (i / 4) % 2, v = (i / 8) * 4 + i % 4;
         c2perm[(((size_t)s * nb + b) * 2 + hh) * 16 + v] = c2;
     }
-    sh_max[threadIdx.x] = mx;
+    // largest ||c||^2; a NaN poisons the bound on purpose
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float o = __shfl_xor(mx, off);
+        mx = (mx == mx && o == o) ? fmaxf(mx, o) : __builtin_nanf("");
+    }
+    if ((j & 63) == 0) sh_max[j >> 6] = mx;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        float r = 0.0f;
-        for (int i = 0; i < 256; ++i) {
-            float v = sh_max[i];
-            r = (v == v) ? fmaxf(r, v) : v;
-            if (!(r == r)) break;
+    if (j == 0) {
+        float r = sh_max[0];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            const float o = sh_max[w];
+            r = (r == r && o == o) ? fmaxf(r, o) : __builtin_nanf("");
         }
         maxc2[s] = r;
     }

@@ -222,6 +222,19 @@ static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t 
         valid = valid && listed[c];
         uint64_t mask = __ballot(valid);
         if (mask == 0) continue;  // uniform
+        if (__popcll(mask) <= 4) {
+            // few listed rows (the small clusters beside the streaming kernel): one lane at a time,
+            // in lane = row order; LDS operations of one wave are performed in program order
+            for (uint64_t mm = mask; mm; mm &= mm - 1) {
+                if (lane == __ffsll((unsigned long long)mm) - 1) {
+                    const uint32_t pos = base[c];
+                    base[c] = pos + 1;
+                    perm[pos] = (uint32_t)i;
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+            continue;
+        }
 #pragma unroll
         for (int bit = 0; bit < 8; ++bit) {
             bool set = (c >> bit) & 1u;
