@@ -478,8 +478,6 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
     if (st.done[s]) return;  // uniform per wave; the waves never synchronise with each other
     float4 *alo = acc_lo[w], *ahi = acc_hi[w];
     uint32_t *cnt = cnt_all[w];
-    const uint32_t lt_lo = (lane >= 32) ? 0xFFFFFFFFu : ((1u << lane) - 1u);
-    const uint32_t lt_hi = (lane <= 32) ? 0u : ((1u << (lane - 32)) - 1u);
     for (int i = lane; i < kMaxK; i += 64) {
         alo[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         ahi[i] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -494,41 +492,54 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
     constexpr int PF = 4;
     float4 b0[PF], b1[PF];
     uint32_t bc[PF];
-    const float *xp = x + (lo + lane) * ld + (int64_t)s * 8;  // row of this lane in the chunk being fetched
-    const uint8_t *cp = codes + lo + lane;
-    const int64_t xstep = 64 * ld;
-    int left = (int)(hi - lo) - lane;  // rows from this lane's row of the fetched chunk to the end of the part
+    // Lanes 2p and 2p+1 fetch the two 16-byte halves of row p of the chunk (b0) and of row 32 + p
+    // (b1): one load instruction touches each 64-byte piece of a line once instead of twice.  The
+    // neighbours then swap a half, so that lane 2p owns row p and lane 2p + 1 owns row 32 + p.
+    const int pr = lane >> 1, hf = lane & 1;
+    const int ridx = hf ? 32 + pr : pr;  // this lane's row of a chunk
+    const float *xp = x + (lo + pr) * ld + (int64_t)s * 8 + 4 * hf;
+    const uint8_t *cp = codes + lo + ridx;
+    const int64_t xstep = 64 * ld, xhalf = 32 * ld;
+    const int rows = (int)(hi - lo);
+    int fetched = 0;  // first row of the chunk being fetched
 #pragma unroll
     for (int u = 0; u < PF; ++u) {
         b0[u] = make_float4(0.f, 0.f, 0.f, 0.f);
         b1[u] = b0[u];
         bc[u] = 0u;
-        if (left > 0) {
-            b0[u] = reinterpret_cast<const float4 *>(xp)[0];
-            b1[u] = reinterpret_cast<const float4 *>(xp)[1];
-            bc[u] = *cp;
-        }
+        if (fetched + pr < rows) b0[u] = *reinterpret_cast<const float4 *>(xp);
+        if (fetched + 32 + pr < rows) b1[u] = *reinterpret_cast<const float4 *>(xp + xhalf);
+        if (fetched + ridx < rows) bc[u] = *cp;
         xp += xstep;
         cp += 64;
-        left -= 64;
+        fetched += 64;
     }
-    int mine = (int)(hi - lo) - lane;  // > 0 while this lane's row of the current chunk exists
-    for (int base = 0; base < (int)(hi - lo); base += 64 * PF) {
+    // lanes whose row comes before this lane's row
+    const unsigned long long even = 0x5555555555555555ull, below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    const unsigned long long ltm = hf ? (even | (~even & below)) : (even & below);
+    const uint32_t lt_lo = (uint32_t)ltm, lt_hi = (uint32_t)(ltm >> 32);
+    for (int base = 0; base < rows; base += 64 * PF) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
-            if (base + 64 * u >= (int)(hi - lo)) break;  // uniform
-            bool pending = mine > 0;
-            mine -= 64;
-            const float4 v0 = b0[u], v1 = b1[u];
+            if (base + 64 * u >= rows) break;  // uniform
+            bool pending = base + 64 * u + ridx < rows;
+            const float4 fa = b0[u], fb = b1[u];
             const uint32_t c = pending ? bc[u] : 0u;
-            if (left > 0) {
-                b0[u] = reinterpret_cast<const float4 *>(xp)[0];
-                b1[u] = reinterpret_cast<const float4 *>(xp)[1];
-                bc[u] = *cp;
-            }
+            if (fetched + pr < rows) b0[u] = *reinterpret_cast<const float4 *>(xp);
+            if (fetched + 32 + pr < rows) b1[u] = *reinterpret_cast<const float4 *>(xp + xhalf);
+            if (fetched + ridx < rows) bc[u] = *cp;
             xp += xstep;
             cp += 64;
-            left -= 64;
+            fetched += 64;
+            // swap: the even lane sends its half of row 32 + p, the odd lane its half of row p
+            const float4 snd = hf ? fa : fb;
+            float4 rcv;
+            rcv.x = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(snd.x), 0xB1, 0xF, 0xF, true));
+            rcv.y = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(snd.y), 0xB1, 0xF, 0xF, true));
+            rcv.z = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(snd.z), 0xB1, 0xF, 0xF, true));
+            rcv.w = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(snd.w), 0xB1, 0xF, 0xF, true));
+            const float4 v0 = hf ? rcv : fa;  // components 0-3 of this lane's row
+            const float4 v1 = hf ? fb : rcv;  // components 4-7
             // Lanes of the same cluster, found with one wave ballot per code bit: a lane differs
             // from lane j when some bit of its code differs from j's bit in the ballot.
             const unsigned long long vb = __ballot(pending);
