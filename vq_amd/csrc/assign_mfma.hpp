@@ -237,11 +237,15 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 4) ? 4 : 3) k_assign_mfma_
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int nb = tb.nb, m = a.m;
-    // consecutive workgroups take the column-block groups of the same rows, so that the lines of
-    // those rows are shared through the L2 while they are hot
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: workgroups id, id + 8,
+    // id + 16, ... (the same XCD, dispatched close together) take the column-block groups of one
+    // row tile, so that the lines of those rows are fetched into one L2 once and the code bytes
+    // of a row are merged there before they are written back.
     const int ngroups = m / SG;
-    const int s0 = (int)(blockIdx.x % (unsigned)ngroups) * SG;
-    const int64_t tile_id = blockIdx.x / (unsigned)ngroups;
+    const unsigned per_chunk = 8u * (unsigned)ngroups;
+    const unsigned chunk_id = blockIdx.x / per_chunk, rem = blockIdx.x % per_chunk;
+    const int s0 = (int)(rem / 8u) * SG;
+    const int64_t tile_id = (int64_t)chunk_id * 8 + (rem % 8u);
     for (int i = threadIdx.x; i < SG * nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s0 * nb * 32 + i];
     __syncthreads();
     const int64_t row_base = (tile_id * 4 + wave) * (32 * TILES);

@@ -126,7 +126,7 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
     auto kern = grouped ? vq::k_assign_mfma_bf<METRIC, LBG, TILES, SG> : vq::k_assign_mfma_bf<METRIC, LBG, TILES, 1>;
     const int sg = grouped ? SG : 1;
     const size_t lds = sizeof(float) * sg * nb * 32;
-    const int64_t blocks = cdiv(a.n, 4 * 32 * TILES) * (a.m / sg);
+    const int64_t blocks = cdiv(cdiv(a.n, 4 * 32 * TILES), 8) * 8 * (a.m / sg);  // tiles in chunks of 8
     if (blocks >= (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * m too large for one launch");
     {
         ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
