@@ -79,7 +79,8 @@ def test_equal_variances_take_the_last_dimension(ctx):
 
 
 @pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN, O.COSINE, O.MANHATTAN])
-@pytest.mark.parametrize("n,dim,depth", [(4000, 16, 6), (1000, 10, 3), (777, 128, 8)])
+@pytest.mark.parametrize("n,dim,depth", [(4000, 16, 6), (1000, 10, 3), (777, 128, 8), (1500, 32, 5),
+                                         (1300, 64, 7), (900, 96, 4)])
 def test_descent_matches_oracle(ctx, metric, n, dim, depth):
     rng = np.random.default_rng(n + metric)
     x = data.unit_rows(n, dim, seed=3) if dim == 128 else rng.standard_normal((n, dim)).astype(F)

@@ -274,6 +274,138 @@ __global__ void __launch_bounds__(256) k_tsvq_descend(const float *__restrict__ 
     leaf[row] = node;
 }
 
+// The same walk with the row held in registers (DIM a multiple of 32 up to 128).  One wave = 64
+// rows: the rows are read with whole-line loads through a small padded LDS tile, so every byte of
+// the input is fetched once; the two child centroids of a lane's node are read 64 bytes at a
+// time, the next piece in flight while the current one is accumulated.  The sums stay one
+// sequential chain per (row, child), as in the reference.
+template <int METRIC>
+__device__ __forceinline__ void tsvq_step(float &al, float &ar, float xv, float cl, float cr) {
+    if constexpr (METRIC == M_COS) {
+        float pl = xv * cl, pr = xv * cr;
+        al = al + pl;
+        ar = ar + pr;
+    } else if constexpr (METRIC == M_L1) {
+        float dl = xv - cl, dr = xv - cr;
+        al = al + fabsf(dl);
+        ar = ar + fabsf(dr);
+    } else {
+        float dl = xv - cl, dr = xv - cr;
+        float pl = dl * dl, pr = dr * dr;
+        al = al + pl;
+        ar = ar + pr;
+    }
+}
+
+template <int METRIC, int DIM>
+__global__ void __launch_bounds__(64) k_tsvq_descend_reg(const float *__restrict__ x, int64_t n, int64_t ld,
+                                                         const float *__restrict__ cen,
+                                                         const float *__restrict__ cnorm,
+                                                         const int *__restrict__ left,
+                                                         const int *__restrict__ right,
+                                                         int *__restrict__ leaf) {
+    constexpr int CH = 32;
+    __shared__ float tile[64 * (CH + 4)];
+    const int lane = threadIdx.x;
+    const int64_t row0 = (int64_t)blockIdx.x * 64;
+    float xr[DIM];
+#pragma unroll
+    for (int c = 0; c < DIM / CH; ++c) {
+        float4 v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int e = lane + 64 * i, r = e >> 3, pc = e & 7;
+            const int64_t row = row0 + r;
+            v[i] = (row < n) ? *reinterpret_cast<const float4 *>(x + row * ld + c * CH + pc * 4)
+                             : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        __builtin_amdgcn_wave_barrier();  // one wave: LDS accesses are performed in program order
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int e = lane + 64 * i, r = e >> 3, pc = e & 7;
+            *reinterpret_cast<float4 *>(&tile[r * (CH + 4) + pc * 4]) = v[i];
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const float4 t4 = *reinterpret_cast<const float4 *>(&tile[lane * (CH + 4) + q * 4]);
+            xr[c * CH + q * 4 + 0] = t4.x;
+            xr[c * CH + q * 4 + 1] = t4.y;
+            xr[c * CH + q * 4 + 2] = t4.z;
+            xr[c * CH + q * 4 + 3] = t4.w;
+        }
+    }
+    float na = 0.0f;
+    if constexpr (METRIC == M_COS) {
+        float sa = 0.0f;
+#pragma unroll
+        for (int t = 0; t < DIM; ++t) {
+            float p = xr[t] * xr[t];
+            sa = sa + p;
+        }
+        na = sqrtf(sa);
+    }
+    int node = 0;
+    bool active = row0 + lane < n;
+    while (__any(active)) {
+        int l = -1, r = -1;
+        if (active) {
+            l = left[node];
+            r = right[node];
+        }
+        if (l >= 0 && r >= 0) {
+            const float4 *pl = reinterpret_cast<const float4 *>(cen + (size_t)l * DIM);
+            const float4 *pr = reinterpret_cast<const float4 *>(cen + (size_t)r * DIM);
+            float al = 0.0f, ar = 0.0f;
+            float4 bl[2][4], br[2][4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                bl[0][q] = pl[q];
+                br[0][q] = pr[q];
+            }
+#pragma unroll
+            for (int c = 0; c < DIM / 16; ++c) {
+                if (c + 1 < DIM / 16) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        bl[(c + 1) & 1][q] = pl[(c + 1) * 4 + q];
+                        br[(c + 1) & 1][q] = pr[(c + 1) * 4 + q];
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 a = bl[c & 1][q], b = br[c & 1][q];
+                    tsvq_step<METRIC>(al, ar, xr[c * 16 + q * 4 + 0], a.x, b.x);
+                    tsvq_step<METRIC>(al, ar, xr[c * 16 + q * 4 + 1], a.y, b.y);
+                    tsvq_step<METRIC>(al, ar, xr[c * 16 + q * 4 + 2], a.z, b.z);
+                    tsvq_step<METRIC>(al, ar, xr[c * 16 + q * 4 + 3], a.w, b.w);
+                }
+            }
+            float dl, dr;
+            if constexpr (METRIC == M_COS) {
+                float nl = cnorm[l], nr = cnorm[r];
+                float ql = al / (na * nl), qr = ar / (na * nr);
+                dl = (na == 0.0f || nl == 0.0f) ? 1.0f : 1.0f - ql;
+                dr = (na == 0.0f || nr == 0.0f) ? 1.0f : 1.0f - qr;
+            } else if constexpr (METRIC == M_EUCLID) {
+                dl = sqrtf(al);
+                dr = sqrtf(ar);
+            } else {
+                dl = al;
+                dr = ar;
+            }
+            node = (dl <= dr) ? l : r;
+        } else if (l >= 0) {
+            node = l;
+        } else if (r >= 0) {
+            node = r;
+        } else {
+            active = false;
+        }
+    }
+    if (row0 + lane < n) leaf[row0 + lane] = node;
+}
+
 // out[i][t] = f16(centroid[leaf[i]][t])   (src/tsvq.rs:242-248)
 static __global__ void __launch_bounds__(256) k_tsvq_decode_f16(const int *__restrict__ leaf, int64_t n, int dim,
                                                          const float *__restrict__ cen,

@@ -403,6 +403,31 @@ int32_t vq_tsvq_descend(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n
     if (ld < tree->dim)
         return fail(ctx, VQ_ERR_DIM_MISMATCH, "Dimension mismatch: expected %d, got %lld", tree->dim, (long long)ld);
     VQ_HIP(ctx, hipSetDevice(ctx->device));
+    // rows in registers: dim a multiple of 32 up to 128, 16-byte aligned rows
+    if (tree->dim % 32 == 0 && tree->dim <= 128 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0) {
+        dim3 g(cdiv(n, 64)), b(64);
+#define DESC_REG(M, D)                                                                                \
+    hipLaunchKernelGGL((vq::k_tsvq_descend_reg<M, D>), g, b, 0, ctx->stream, d_x, n, ld,              \
+                       tree->d_centroids, tree->d_cnorm, tree->d_left, tree->d_right, d_leaf)
+#define DESC_DIM(M)                                                                                   \
+    switch (tree->dim) {                                                                              \
+    case 32: DESC_REG(M, 32); break;                                                                  \
+    case 64: DESC_REG(M, 64); break;                                                                  \
+    case 96: DESC_REG(M, 96); break;                                                                  \
+    default: DESC_REG(M, 128); break;                                                                 \
+    }
+        switch (metric) {
+        case VQ_SQEUCLIDEAN: DESC_DIM(vq::M_SQ); break;
+        case VQ_EUCLIDEAN: DESC_DIM(vq::M_EUCLID); break;
+        case VQ_COSINE: DESC_DIM(vq::M_COS); break;
+        case VQ_MANHATTAN: DESC_DIM(vq::M_L1); break;
+        default: return fail(ctx, VQ_ERR_UNSUPPORTED, "metric %d has no kernel", metric);
+        }
+#undef DESC_DIM
+#undef DESC_REG
+        VQ_HIP(ctx, hipGetLastError());
+        return VQ_OK;
+    }
     dim3 grid(cdiv(n, 256)), block(256);
 #define DESC(M)                                                                                       \
     hipLaunchKernelGGL((vq::k_tsvq_descend<M>), grid, block, 0, ctx->stream, d_x, n, ld, tree->dim,   \
