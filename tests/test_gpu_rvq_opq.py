@@ -126,7 +126,7 @@ def test_rotate_matches_matrix_product(ctx, n, dim):
     assert np.array_equal(dy.download(), x)  # identity is exact (opq.rs:119-121)
 
 
-@pytest.mark.parametrize("n,dim", [(1000, 10), (5000, 128), (2049, 32)])
+@pytest.mark.parametrize("n,dim", [(1000, 10), (5000, 128), (2049, 32), (4099, 16), (2050, 80), (777, 20)])
 def test_cross_cov_matches_f64_product(ctx, n, dim):
     rng = np.random.default_rng(n)
     x = rng.standard_normal((n, dim)).astype(F)

@@ -182,6 +182,56 @@ static __global__ void __launch_bounds__(256) k_crosscov_partial(const float *__
     }
 }
 
+// The same partial sums on the f64 matrix cores (v_mfma_f64_16x16x4_f64) for dim = 16 * NT <= 128.
+// One wave owns the 16 output rows [16 ti, 16 ti + 16) of a chunk and all NT column tiles; a
+// contraction step takes 4 rows: lane l supplies y[row + l/16][16 ti + l%16] and, per column
+// tile, x[row + l/16][16 tj + l%16], converted to f64 (the products are then exact).  The result
+// register v of lane l is A[16 ti + 4 v + l/16][16 tj + l%16].  Fixed order: deterministic.
+typedef double doublex4 __attribute__((ext_vector_type(4)));
+
+template <int NT>
+__global__ void __launch_bounds__(256) k_crosscov_mfma(const float *__restrict__ yr, const float *__restrict__ x,
+                                                       int64_t n, int64_t rows_per_chunk,
+                                                       double *__restrict__ part) {
+    constexpr int DIM = 16 * NT;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int ti = blockIdx.y * 4 + w;
+    if (ti >= NT) return;
+    const int kk = lane >> 4, jj = lane & 15;
+    const int64_t lo = (int64_t)blockIdx.x * rows_per_chunk;
+    const int64_t hi = lo + rows_per_chunk < n ? lo + rows_per_chunk : n;
+    doublex4 acc[NT];
+#pragma unroll
+    for (int tj = 0; tj < NT; ++tj) acc[tj] = doublex4{0.0, 0.0, 0.0, 0.0};
+    const float *yp = yr + (lo + kk) * DIM + 16 * ti + jj;
+    const float *xp = x + (lo + kk) * DIM + jj;
+    float a = 0.0f, b[NT];
+    bool valid = lo + kk < hi;
+    a = valid ? *yp : 0.0f;
+#pragma unroll
+    for (int tj = 0; tj < NT; ++tj) b[tj] = valid ? xp[16 * tj] : 0.0f;
+    for (int64_t r = lo; r < hi; r += 4) {
+        const float ac = a;
+        float bc[NT];
+#pragma unroll
+        for (int tj = 0; tj < NT; ++tj) bc[tj] = b[tj];
+        yp += 4 * DIM;
+        xp += 4 * DIM;
+        valid = r + 4 + kk < hi;  // the next step's operands are fetched while this one is multiplied
+        a = valid ? *yp : 0.0f;
+#pragma unroll
+        for (int tj = 0; tj < NT; ++tj) b[tj] = valid ? xp[16 * tj] : 0.0f;
+#pragma unroll
+        for (int tj = 0; tj < NT; ++tj)
+            acc[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64((double)ac, (double)bc[tj], acc[tj], 0, 0, 0);
+    }
+    double *out = part + (size_t)blockIdx.x * DIM * DIM;
+#pragma unroll
+    for (int tj = 0; tj < NT; ++tj)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) out[(size_t)(16 * ti + 4 * v + kk) * DIM + 16 * tj + jj] = acc[tj][v];
+}
+
 static __global__ void __launch_bounds__(256) k_crosscov_reduce(const double *__restrict__ part, int chunks,
                                                          int total, double *__restrict__ out) {
     int e = blockIdx.x * 256 + threadIdx.x;

@@ -137,9 +137,29 @@ int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n,
     const int total = dim * dim;
     VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(double) * (size_t)chunks * total));
     VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * (size_t)total));
-    size_t lds = sizeof(float) * 2 * 32 * (size_t)dim;
-    hipLaunchKernelGGL(vq::k_crosscov_partial, dim3(chunks), dim3(256), lds, ctx->stream, d_y, d_x, n, dim,
-                       rows_per_chunk, (double *)ctx->tmp_a.p);
+    if (dim % 16 == 0) {
+        const int nt = dim / 16;
+        const dim3 grid(chunks, (nt + 3) / 4);
+        double *part = (double *)ctx->tmp_a.p;
+#define CROSSCOV(NT)                                                                                 \
+    hipLaunchKernelGGL((vq::k_crosscov_mfma<NT>), grid, dim3(256), 0, ctx->stream, d_y, d_x, n,     \
+                       rows_per_chunk, part)
+        switch (nt) {
+        case 1: CROSSCOV(1); break;
+        case 2: CROSSCOV(2); break;
+        case 3: CROSSCOV(3); break;
+        case 4: CROSSCOV(4); break;
+        case 5: CROSSCOV(5); break;
+        case 6: CROSSCOV(6); break;
+        case 7: CROSSCOV(7); break;
+        default: CROSSCOV(8); break;
+        }
+#undef CROSSCOV
+    } else {
+        size_t lds = sizeof(float) * 2 * 32 * (size_t)dim;
+        hipLaunchKernelGGL(vq::k_crosscov_partial, dim3(chunks), dim3(256), lds, ctx->stream, d_y, d_x, n, dim,
+                           rows_per_chunk, (double *)ctx->tmp_a.p);
+    }
     hipLaunchKernelGGL(vq::k_crosscov_reduce, dim3(cdiv(total, 256)), dim3(256), 0, ctx->stream,
                        (const double *)ctx->tmp_a.p, chunks, total, (double *)ctx->tmp_b.p);
     VQ_HIP(ctx, hipGetLastError());
