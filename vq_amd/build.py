@@ -51,7 +51,7 @@ HOST_LIB = os.path.join(HERE, "libvqhost.so")
 
 def build_host(verbose=False):
     """Compiles the C++ host mirror (plain g++: it only needs the C ABI) and links it to libvqhip."""
-    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-Wall",
+    cmd = ["g++", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-Wall",
            os.path.join(HERE, "host", "vq_host_c.cpp"), "-o", HOST_LIB,
            "-L" + HERE, "-lvqhip", "-Wl,-rpath,$ORIGIN"]
     if verbose:

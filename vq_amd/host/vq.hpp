@@ -350,47 +350,53 @@ private:
 // R = V U^T for A = U S V^T, by a cyclic one-sided Jacobi SVD in f64; row-major dim x dim.
 inline void procrustes_rotation(const std::vector<double> &A, size_t dim, std::vector<double> &R) {
     const size_t n = dim;
-    std::vector<double> U(A), V(n * n, 0.0);
-    for (size_t i = 0; i < n; ++i) V[i * n + i] = 1.0;
+    // columns of U and V are kept as contiguous rows (Ut, Vt): every inner loop is unit-stride
+    std::vector<double> Ut(n * n), Vt(n * n, 0.0);
+    for (size_t i = 0; i < n; ++i) {
+        Vt[i * n + i] = 1.0;
+        for (size_t j = 0; j < n; ++j) Ut[j * n + i] = A[i * n + j];
+    }
     for (int sweep = 0; sweep < 60; ++sweep) {
         double off = 0.0;
         for (size_t p = 0; p + 1 < n; ++p)
             for (size_t q = p + 1; q < n; ++q) {
+                double *up = &Ut[p * n], *uq = &Ut[q * n];
                 double alpha = 0, beta = 0, gamma = 0;
                 for (size_t i = 0; i < n; ++i) {
-                    alpha += U[i * n + p] * U[i * n + p];
-                    beta += U[i * n + q] * U[i * n + q];
-                    gamma += U[i * n + p] * U[i * n + q];
+                    alpha += up[i] * up[i];
+                    beta += uq[i] * uq[i];
+                    gamma += up[i] * uq[i];
                 }
                 if (gamma == 0.0) continue;
                 off = std::max(off, std::fabs(gamma) / std::sqrt(alpha * beta + 1e-300));
                 double zeta = (beta - alpha) / (2.0 * gamma);
                 double t = (zeta >= 0 ? 1.0 : -1.0) / (std::fabs(zeta) + std::sqrt(1.0 + zeta * zeta));
                 double c = 1.0 / std::sqrt(1.0 + t * t), s = c * t;
+                double *vp = &Vt[p * n], *vq = &Vt[q * n];
                 for (size_t i = 0; i < n; ++i) {
-                    double up = U[i * n + p], uq = U[i * n + q];
-                    U[i * n + p] = c * up - s * uq;
-                    U[i * n + q] = s * up + c * uq;
-                    double vp = V[i * n + p], vq = V[i * n + q];
-                    V[i * n + p] = c * vp - s * vq;
-                    V[i * n + q] = s * vp + c * vq;
+                    double a = up[i], b = uq[i];
+                    up[i] = c * a - s * b;
+                    uq[i] = s * a + c * b;
+                    double d = vp[i], e = vq[i];
+                    vp[i] = c * d - s * e;
+                    vq[i] = s * d + c * e;
                 }
             }
         if (off < 1e-15) break;
     }
     for (size_t j = 0; j < n; ++j) {
         double s = 0;
-        for (size_t i = 0; i < n; ++i) s += U[i * n + j] * U[i * n + j];
+        for (size_t i = 0; i < n; ++i) s += Ut[j * n + i] * Ut[j * n + i];
         s = std::sqrt(s);
         if (s > 0)
-            for (size_t i = 0; i < n; ++i) U[i * n + j] /= s;
+            for (size_t i = 0; i < n; ++i) Ut[j * n + i] /= s;
     }
+    // R[i][j] = sum_l V[i][l] U[j][l], l ascending
     R.assign(n * n, 0.0);
-    for (size_t i = 0; i < n; ++i)
-        for (size_t j = 0; j < n; ++j) {
-            double acc = 0;
-            for (size_t l = 0; l < n; ++l) acc += V[i * n + l] * U[j * n + l];
-            R[i * n + j] = acc;
+    for (size_t l = 0; l < n; ++l)
+        for (size_t i = 0; i < n; ++i) {
+            const double v = Vt[l * n + i];
+            for (size_t j = 0; j < n; ++j) R[i * n + j] += v * Ut[l * n + j];
         }
 }
 
