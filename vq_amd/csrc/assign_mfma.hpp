@@ -231,7 +231,7 @@ __device__ __forceinline__ int exact_argmin8_wave(const float (&xs)[8], const fl
 // 128-byte line of every row).  256 threads = 4 waves; grid = (row tiles, groups of column blocks),
 // so that the waves are short enough for the last round of workgroups not to leave the chip idle.
 template <int METRIC, bool LBG, int TILES, int SG>
-__global__ void __launch_bounds__(256, (TILES * SG <= 4) ? 4 : 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
+__global__ void __launch_bounds__(256, (TILES * SG <= 2) ? 5 : (TILES * SG <= 4) ? 4 : 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
     constexpr int SD = 8;
     extern __shared__ float lds_c2[];  // [SG][nb][2][16]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -589,6 +589,288 @@ __global__ void __launch_bounds__(256) k_assign_mfma_wide(AssignArgs a, MfmaWide
             tb.list[pos] = (uint32_t)(row * a.m + s);
         }
     }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Wide column blocks on the bf16 matrix cores: the operand split of k_assign_mfma_bf applied to
+// every chunk of 8 dimensions (two instructions per chunk and tile of 32 centroids; the three
+// bf16 parts of the chunk's share of ||x||^2 ride in the spare slots of the second one).
+// A workgroup = 128 rows; wave w takes the row tiles {2 (w&1), 2 (w&1) + 1} and the centroid tiles
+// [4 (w>>1), 4 (w>>1) + 4): 8 accumulator tiles (128 registers), every A operand read from LDS
+// feeds two matrix instructions.  The A operands of a chunk (16 KB for 256 centroids) are staged
+// in LDS once per workgroup, double-buffered; the rows and the next A chunk are fetched one chunk
+// ahead.  The two waves that share rows merge their (smallest, second smallest) through LDS.
+// Error of a score: 3 * 2^-16 (split, as above) + (34 * sd/8 + 16) * 2^-24 (fp32 accumulation of
+// 2 x 17 addends per chunk), per unit of ||x||^2 + ||c||^2; twice that for two candidates.
+struct MfmaWideBfTables {
+    const u32x4 *atab;     // [m][sd/8][nb][2][64]
+    const float *c2perm;   // [m][nb][2][16]
+    const float *maxc2;    // [m]
+    uint32_t *list;
+    uint32_t *list_count;
+    int nb;
+    int sd;
+    float kappa;           // error-bound coefficient on (||x||^2 + max ||c||^2)
+};
+
+// One workgroup per column block s, one thread per padded centroid (k <= 256).
+static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *__restrict__ cb, int m, int k, int nb,
+                                                                  int sd, u32x4 *__restrict__ atab,
+                                                                  float *__restrict__ c2perm,
+                                                                  float *__restrict__ maxc2,
+                                                                  uint32_t *__restrict__ list_count) {
+    const int s = blockIdx.x, j = threadIdx.x;
+    const int nkc = sd / 8;
+    __shared__ float sh_max[4];
+    float mx = 0.0f;
+    if (j < nb * 32) {
+        const int b = j / 32, i = j % 32;
+        const float *c = cb + ((size_t)s * k + j) * sd;
+        float c2 = kPadScore;
+        if (j < k) {
+            c2 = 0.0f;
+            for (int t = 0; t < sd; ++t) c2 = __builtin_fmaf(c[t], c[t], c2);
+            mx = c2;
+        }
+        const u32x4 ones = {0x3f803f80u, 0x00003f80u, 0u, 0u};
+        for (int kc = 0; kc < nkc; ++kc) {
+            u32x4 ah, al;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                uint32_t hb[2], lb[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float a = (j < k) ? -2.0f * c[kc * 8 + 2 * w + e] : 0.0f;
+                    hb[e] = bf16_rne_bits(a);
+                    lb[e] = bf16_rne_bits(a - bf16_bits_to_float(hb[e]));
+                }
+                ah[w] = hb[0] | (hb[1] << 16);
+                al[w] = lb[0] | (lb[1] << 16);
+            }
+            u32x4 *dst = atab + (((size_t)s * nkc + kc) * nb + b) * 128;
+            dst[i] = ah;
+            dst[32 + i] = ah;
+            dst[64 + i] = al;
+            dst[96 + i] = ones;
+        }
+        const int hh = (i / 4) % 2, v = (i / 8) * 4 + i % 4;
+        c2perm[(((size_t)s * nb + b) * 2 + hh) * 16 + v] = c2;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float o = __shfl_xor(mx, off);
+        mx = (mx == mx && o == o) ? fmaxf(mx, o) : __builtin_nanf("");
+    }
+    if ((j & 63) == 0) sh_max[j >> 6] = mx;
+    __syncthreads();
+    if (j == 0) {
+        float r = sh_max[0];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            const float o = sh_max[w];
+            r = (r == r && o == o) ? fmaxf(r, o) : __builtin_nanf("");
+        }
+        maxc2[s] = r;
+        if (s == 0) *list_count = 0;
+    }
+}
+
+// LDS writes of this wave done, then the workgroup barrier; vector-memory loads stay in flight
+// (__syncthreads would wait for the prefetches as well).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// grid (ceil(n/128), m); 256 threads = 4 waves.
+template <bool LBG>
+__global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, MfmaWideBfTables tb) {
+    constexpr int NBMAX = 8;
+    __shared__ u32x4 lds_a[2][NBMAX * 128];  // 2 x 16 KB
+    __shared__ float lds_c2[NBMAX * 32];
+    __shared__ int lds_top[2][2][2][32];     // [row pair][row tile][m1 | m2][row] of the upper centroid half
+    __shared__ uint32_t wg_list[128];
+    __shared__ uint32_t wg_count, wg_base;
+    const int s = blockIdx.y;
+    if constexpr (LBG) {
+        if (a.done[s]) return;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int rp = wave & 1, ch = wave >> 1;
+    const int nb = tb.nb, sd = tb.sd, nkc = sd / 8;
+    const u32x4 *ag = tb.atab + (size_t)s * nkc * nb * 128;
+    const int chunk16 = nb * 128;  // 16-byte pieces per chunk
+    for (int i = threadIdx.x; i < nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s * nb * 32 + i];
+    for (int i = threadIdx.x; i < chunk16; i += 256) lds_a[0][i] = ag[i];
+    if (threadIdx.x == 0) wg_count = 0;
+    __syncthreads();
+
+    int64_t row[2];
+    bool valid[2];
+    const float *xr[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        row[t] = (int64_t)blockIdx.x * 128 + (2 * rp + t) * 32 + r;
+        valid[t] = row[t] < a.n;
+        xr[t] = a.x + (valid[t] ? row[t] : 0) * a.ld + (int64_t)s * sd;
+    }
+    floatx16 acc[2][4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int b = 4 * ch + c;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float c2 = (b < nb) ? lds_c2[(b * 2 + h) * 16 + v] : kPadScore;
+            acc[0][c][v] = c2;
+            acc[1][c][v] = c2;
+        }
+    }
+    float4 xn[2][2];  // the next chunk of the rows
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        xn[t][0] = valid[t] ? *reinterpret_cast<const float4 *>(xr[t]) : make_float4(0.f, 0.f, 0.f, 0.f);
+        xn[t][1] = valid[t] ? *reinterpret_cast<const float4 *>(xr[t] + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float x2[2] = {0.0f, 0.0f};
+    for (int kc = 0; kc < nkc; ++kc) {
+        const int cur = kc & 1;
+        const bool more = kc + 1 < nkc;
+        // operands of this chunk from the rows fetched one chunk ago
+        u32x4 b1[2], b2[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const float xv[8] = {xn[t][0].x, xn[t][0].y, xn[t][0].z, xn[t][0].w,
+                                 xn[t][1].x, xn[t][1].y, xn[t][1].z, xn[t][1].w};
+            float p = 0.0f;
+            uint32_t hb[4];
+            float lo[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                hb[w] = bf16_pack2(xv[2 * w], xv[2 * w + 1]);
+                lo[2 * w] = xv[2 * w] - __uint_as_float(hb[w] << 16);
+                lo[2 * w + 1] = xv[2 * w + 1] - __uint_as_float(hb[w] & 0xffff0000u);
+            }
+            x2[t] += p;
+            const uint32_t p0 = bf16_pack2(p, 0.0f);
+            const float r1 = p - __uint_as_float(p0 << 16);
+            const uint32_t p1 = bf16_pack2(r1, 0.0f);
+            const float r2 = r1 - __uint_as_float(p1 << 16);
+            const uint32_t p2 = bf16_pack2(r2, 0.0f);
+            const uint32_t xparts[4] = {(p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu, 0u, 0u};
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t lw = bf16_pack2(lo[2 * w], lo[2 * w + 1]);
+                b1[t][w] = h ? lw : hb[w];
+                b2[t][w] = h ? xparts[w] : hb[w];
+            }
+        }
+        // fetch the next chunk: rows into registers, A operands into registers then LDS
+        u32x4 pre[4];
+        if (more) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (valid[t]) {
+                    xn[t][0] = *reinterpret_cast<const float4 *>(xr[t] + (kc + 1) * 8);
+                    xn[t][1] = *reinterpret_cast<const float4 *>(xr[t] + (kc + 1) * 8 + 4);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i = threadIdx.x + 256 * q;
+                if (i < chunk16) pre[q] = ag[(size_t)(kc + 1) * chunk16 + i];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int b = 4 * ch + c;
+            if (b < nb) {
+                const u32x4 a1 = lds_a[cur][b * 128 + lane], a2 = lds_a[cur][b * 128 + 64 + lane];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8, a1), __builtin_bit_cast(bf16x8, b1[t]), acc[t][c], 0, 0, 0);
+                    acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8, a2), __builtin_bit_cast(bf16x8, b2[t]), acc[t][c], 0, 0, 0);
+                }
+            }
+        }
+        if (more) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i = threadIdx.x + 256 * q;
+                if (i < chunk16) lds_a[cur ^ 1][i] = pre[q];
+            }
+        }
+        lds_barrier();
+    }
+    // smallest and second smallest score of this wave's centroid tiles
+    int m1[2], m2[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        m1[t] = 0x7f800000;
+        m2[t] = 0x7f800000;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int b = 4 * ch + c;
+            if (b < nb) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const uint32_t idx = (uint32_t)(32 * b + 8 * (v / 4) + 4 * h + v % 4);
+                    const int key = (int)((__float_as_uint(acc[t][c][v]) & 0xFFFFFF00u) | idx);
+                    m2[t] = imed3(m1[t], m2[t], key);
+                    m1[t] = imin(m1[t], key);
+                }
+            }
+        }
+        const int o1 = __shfl_xor(m1[t], 32), o2 = __shfl_xor(m2[t], 32);
+        const int n1 = imin(m1[t], o1);
+        m2[t] = imin(imax(m1[t], o1), imin(m2[t], o2));
+        m1[t] = n1;
+    }
+    if (ch == 1 && h == 0) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            lds_top[rp][t][0][r] = m1[t];
+            lds_top[rp][t][1][r] = m2[t];
+        }
+    }
+    __syncthreads();
+    if (ch == 0 && h == 0) {
+        const float mc2 = tb.maxc2[s];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int o1 = lds_top[rp][t][0][r], o2 = lds_top[rp][t][1][r];
+            const float s1 = __int_as_float(imin(m1[t], o1));
+            const float s2 = __int_as_float(imin(imax(m1[t], o1), imin(m2[t], o2)));
+            if (valid[t]) {
+                const float bound = x2[t] + mc2;
+                const float margin = 6.103515625e-05f * fabsf(s2) + tb.kappa * bound;
+                bool sure = (s2 - s1) > margin;
+                sure = sure && (bound < 1e29f) && (s1 < 1e29f);
+                if (sure) {
+                    const uint8_t code = (uint8_t)(__float_as_uint(s1) & 0xFFu);
+                    if constexpr (LBG) {
+                        uint8_t *pc = a.codes + (size_t)s * a.n + row[t];
+                        if (*pc != code) {
+                            *pc = code;
+                            mark_changed(a.changed + s);
+                        }
+                    } else {
+                        a.codes[row[t] * a.m + s] = code;
+                    }
+                } else {
+                    wg_list[atomicAdd(&wg_count, 1u)] = (uint32_t)(row[t] * a.m + s);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t cnt = wg_count;
+    if (cnt == 0) return;
+    if (threadIdx.x == 0) wg_base = atomicAdd(tb.list_count, cnt);
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < cnt; i += 256) tb.list[wg_base + i] = wg_list[i];
 }
 
 }  // namespace vq

@@ -163,11 +163,12 @@ int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const ui
     return VQ_OK;
 }
 
-// Wide column blocks (sub_dim a multiple of 8 above 8): chunked contraction, same two passes.
+// Wide column blocks (sub_dim a multiple of 8 above 8): chunked contraction on the bf16 matrix
+// cores with split operands, undecided pairs listed for the exact kernel.
 template <int METRIC, bool LBG>
 int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     const int nb = (a.k + 31) / 32, nkc = sd / 8;
-    const size_t n_atab = (size_t)a.m * nkc * nb * 64 * 4, n_c2 = (size_t)a.m * nb * 32;
+    const size_t n_atab = (size_t)a.m * nkc * nb * 128 * 4, n_c2 = (size_t)a.m * nb * 32;  // floats
     VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + a.m) + 64));
     VQ_TRY(ensure(ctx, ctx->mfma_list, sizeof(uint32_t) * ((size_t)a.n * a.m + 4)));
     float *atab = (float *)ctx->mfma_tab.p;
@@ -175,14 +176,14 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     float *maxc2 = c2perm + n_c2;
     uint32_t *count = (uint32_t *)ctx->mfma_list.p;
     uint32_t *list = count + 4;
-    hipLaunchKernelGGL(vq::k_mfma_wide_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, sd, atab,
-                       c2perm, maxc2, count);
-    // bound on matrix accumulation + the reference's own rounding: (sd + 16) * 2^-21 per unit of
-    // ||x||^2 + max ||c||^2 (about 2^-16.4 at sd = 8, the constant of the narrow kernel)
-    vq::MfmaWideTables tb{atab, c2perm, maxc2, list, count, nb, sd, (float)(sd + 16) * 4.76837158203125e-07f};
+    hipLaunchKernelGGL(vq::k_mfma_wide_bf_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, sd,
+                       (vq::u32x4 *)atab, c2perm, maxc2, count);
+    // two candidates, each: operand split 3 * 2^-16, fp32 accumulation (34 per chunk + 16) * 2^-24
+    const float kappa = 2.0f * (3.0f * 1.52587890625e-05f + (34.0f * nkc + 16.0f) * 5.9604644775390625e-08f);
+    vq::MfmaWideBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, list, count, nb, sd, kappa};
     {
         ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
-        hipLaunchKernelGGL((vq::k_assign_mfma_wide<LBG>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0,
+        hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0,
                            ctx->stream, a, tb);
     }
     VQ_HIP(ctx, hipGetLastError());
