@@ -174,6 +174,110 @@ static __global__ void k_seg_middles(const float *__restrict__ sorted, const uin
     }
 }
 
+// ---- middle values by radix select ---------------------------------------------------------
+// The reference sorts the split column and takes values[c/2] (and values[c/2 - 1] for an even
+// count, src/tsvq.rs:108-117); only those two order statistics are needed.  Floats are mapped to
+// unsigned keys of the same order; four passes of 8 bits narrow each target down: a pass counts,
+// per segment and target, the keys that share the target's known high bits by their next byte
+// (LDS histograms per workgroup, flushed with integer atomics), then one thread per (segment,
+// target) picks the byte whose bin holds the target's rank.
+struct SegSelect {
+    uint32_t prefix;  // known high bits of the key (low bits zero)
+    uint32_t rank;    // rank of the target among the keys that share the prefix
+};
+
+__device__ __forceinline__ uint32_t float_order_key(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float float_from_order_key(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+static __global__ void k_seg_select_init(const uint2 *__restrict__ seg_range, int nseg, SegSelect *__restrict__ sel,
+                                         uint32_t *__restrict__ hist) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nseg * 512) hist[i] = 0u;
+    if (i < nseg) {
+        const uint2 r = seg_range[i];
+        const uint32_t c = r.y - r.x;
+        sel[2 * i] = SegSelect{0u, (c % 2 == 0) ? c / 2 - 1 : c / 2};
+        sel[2 * i + 1] = SegSelect{0u, c / 2};
+    }
+}
+
+// One workgroup per 4096 positions; pass = 0..3 looks at key bits [31 - 8 pass, 24 - 8 pass].
+static __global__ void __launch_bounds__(256) k_seg_select_hist(const float *__restrict__ vals, int64_t n,
+                                                                const uint2 *__restrict__ seg_range, int nseg,
+                                                                const SegSelect *__restrict__ sel, int pass,
+                                                                uint32_t *__restrict__ hist) {
+    __shared__ uint32_t lh[512];
+    const int64_t lo = (int64_t)blockIdx.x * 4096;
+    const int64_t hi = lo + 4096 < n ? lo + 4096 : n;
+    const int shift = 24 - 8 * pass;
+    const uint32_t high_mask = pass == 0 ? 0u : (0xFFFFFFFFu << (shift + 8));
+    // segments are sorted by position and disjoint: walk the ones that overlap this chunk
+    int g = 0;
+    {
+        int a = 0, b = nseg;  // first segment whose end is beyond lo
+        while (a < b) {
+            const int mid = (a + b) >> 1;
+            if (seg_range[mid].y <= (uint32_t)lo) a = mid + 1; else b = mid;
+        }
+        g = a;
+    }
+    for (; g < nseg; ++g) {
+        const uint2 r = seg_range[g];
+        if ((int64_t)r.x >= hi) break;
+        const int64_t from = (int64_t)r.x > lo ? (int64_t)r.x : lo, to = (int64_t)r.y < hi ? (int64_t)r.y : hi;
+        const uint32_t p0 = sel[2 * g].prefix, p1 = sel[2 * g + 1].prefix;
+        __syncthreads();
+        lh[threadIdx.x] = 0u;
+        lh[256 + threadIdx.x] = 0u;
+        __syncthreads();
+        for (int64_t p = from + threadIdx.x; p < to; p += 256) {
+            const uint32_t key = float_order_key(vals[p]);
+            const uint32_t byte = (key >> shift) & 255u;
+            if ((key & high_mask) == p0) atomicAdd(&lh[byte], 1u);
+            if ((key & high_mask) == p1) atomicAdd(&lh[256 + byte], 1u);
+        }
+        __syncthreads();
+        uint32_t *gh = hist + (size_t)g * 512;
+        if (lh[threadIdx.x]) atomicAdd(&gh[threadIdx.x], lh[threadIdx.x]);
+        if (lh[256 + threadIdx.x]) atomicAdd(&gh[256 + threadIdx.x], lh[256 + threadIdx.x]);
+    }
+}
+
+// One thread per (segment, target): the byte whose bin holds the rank; clears the bins.
+static __global__ void k_seg_select_pick(uint32_t *__restrict__ hist, SegSelect *__restrict__ sel, int nseg,
+                                         int pass) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= 2 * nseg) return;
+    uint32_t *h = hist + (size_t)i * 256;
+    SegSelect s = sel[i];
+    uint32_t byte = 255u;
+    bool found = false;
+    for (uint32_t b = 0; b < 256u; ++b) {
+        const uint32_t c = h[b];
+        h[b] = 0u;
+        if (!found) {
+            if (s.rank < c) {
+                byte = b;
+                found = true;
+            } else {
+                s.rank -= c;
+            }
+        }
+    }
+    s.prefix |= byte << (24 - 8 * pass);
+    sel[i] = s;
+}
+
+static __global__ void k_seg_select_out(const SegSelect *__restrict__ sel, int nseg, float *__restrict__ mids) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < 2 * nseg) mids[i] = float_from_order_key(sel[i].prefix);
+}
+
 // ---- descent -------------------------------------------------------------------------------
 template <int METRIC>
 __device__ __forceinline__ float tsvq_dist(const float *__restrict__ xr, const float *__restrict__ c,

@@ -85,7 +85,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     VQ_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
 
-    // workspace: two row-id lists, column values (+sorted), flags, scan
+    // workspace: two row-id lists, column values, flags, scan
     VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(uint32_t) * (size_t)n));
     VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(uint32_t) * (size_t)n));
     VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(float) * (size_t)n));
@@ -93,7 +93,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     VQ_TRY(ensure(ctx, ctx->tmp_e, sizeof(uint32_t) * (size_t)n));
     VQ_TRY(ensure(ctx, ctx->tmp_f, sizeof(uint32_t) * (size_t)n));
     uint32_t *perm = (uint32_t *)ctx->tmp_a.p, *perm2 = (uint32_t *)ctx->tmp_b.p;
-    float *vals = (float *)ctx->tmp_c.p, *sorted = (float *)ctx->tmp_d.p;
+    float *vals = (float *)ctx->tmp_c.p;
     uint32_t *flags = (uint32_t *)ctx->tmp_e.p, *scan = (uint32_t *)ctx->tmp_f.p;
     hipLaunchKernelGGL(vq::k_iota_u32, dim3(cdiv(n, 256)), dim3(256), 0, st, perm, n);
 
@@ -192,7 +192,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             std::copy_n(T->h_centroids.data() + (size_t)level[split[i]].node * dim, dim,
                         smeans.data() + (size_t)i * dim);
         void *d_range = nullptr, *d_smeans = nullptr, *d_var = nullptr, *d_sdim = nullptr, *d_mids = nullptr,
-             *d_median = nullptr, *d_nleft = nullptr, *d_begin = nullptr, *d_end = nullptr;
+             *d_median = nullptr, *d_nleft = nullptr, *d_sel = nullptr, *d_hist = nullptr;
         auto free_split = [&]() {
             (void)hipFree(d_range);
             (void)hipFree(d_smeans);
@@ -201,8 +201,8 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             (void)hipFree(d_mids);
             (void)hipFree(d_median);
             (void)hipFree(d_nleft);
-            (void)hipFree(d_begin);
-            (void)hipFree(d_end);
+            (void)hipFree(d_sel);
+            (void)hipFree(d_hist);
         };
 #define SP_HIP(call)                                                                              \
     do {                                                                                          \
@@ -223,8 +223,8 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         SP_HIP(hipMalloc(&d_mids, sizeof(float) * 2 * ns));
         SP_HIP(hipMalloc(&d_median, sizeof(float) * ns));
         SP_HIP(hipMalloc(&d_nleft, sizeof(uint32_t) * ns));
-        SP_HIP(hipMalloc(&d_begin, sizeof(uint32_t) * ns));
-        SP_HIP(hipMalloc(&d_end, sizeof(uint32_t) * ns));
+        SP_HIP(hipMalloc(&d_sel, sizeof(vq::SegSelect) * 2 * ns));
+        SP_HIP(hipMalloc(&d_hist, sizeof(uint32_t) * 512 * (size_t)ns));
         SP_HIP(hipMemcpyAsync(d_range, range.data(), sizeof(uint2) * ns, hipMemcpyHostToDevice, st));
         SP_HIP(hipMemcpyAsync(d_smeans, smeans.data(), sizeof(float) * (size_t)ns * dim, hipMemcpyHostToDevice, st));
         // per-dimension sums of squared deviations (src/tsvq.rs:88-99)
@@ -245,29 +245,19 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             sdim[i] = best;
         }
         SP_HIP(hipMemcpyAsync(d_sdim, sdim.data(), sizeof(int) * ns, hipMemcpyHostToDevice, st));
-        // split column, segmented sort, middle values (src/tsvq.rs:109-117)
+        // split column, middle values by radix select (src/tsvq.rs:109-117)
         hipLaunchKernelGGL(vq::k_seg_gather_col, dim3(cdiv(n, 256)), dim3(256), 0, st, perm, n,
                            (const uint2 *)d_range, ns, (const int *)d_sdim, d_x, ld, vals);
-        std::vector<uint32_t> begin(ns), end(ns);
-        for (int i = 0; i < ns; ++i) {
-            begin[i] = range[i].x;
-            end[i] = range[i].y;
+        hipLaunchKernelGGL(vq::k_seg_select_init, dim3(cdiv((int64_t)ns * 512, 256)), dim3(256), 0, st,
+                           (const uint2 *)d_range, ns, (vq::SegSelect *)d_sel, (uint32_t *)d_hist);
+        for (int pass = 0; pass < 4; ++pass) {
+            hipLaunchKernelGGL(vq::k_seg_select_hist, dim3(cdiv(n, 4096)), dim3(256), 0, st, (const float *)vals, n,
+                               (const uint2 *)d_range, ns, (const vq::SegSelect *)d_sel, pass, (uint32_t *)d_hist);
+            hipLaunchKernelGGL(vq::k_seg_select_pick, dim3(cdiv(2 * ns, 64)), dim3(64), 0, st, (uint32_t *)d_hist,
+                               (vq::SegSelect *)d_sel, ns, pass);
         }
-        SP_HIP(hipMemcpyAsync(d_begin, begin.data(), sizeof(uint32_t) * ns, hipMemcpyHostToDevice, st));
-        SP_HIP(hipMemcpyAsync(d_end, end.data(), sizeof(uint32_t) * ns, hipMemcpyHostToDevice, st));
-        size_t need = 0;
-        SP_HIP(rocprim::segmented_radix_sort_keys(nullptr, need, vals, sorted, (unsigned)n, (unsigned)ns,
-                                                  (const uint32_t *)d_begin, (const uint32_t *)d_end, 0, 32, st));
-        if (need > rp_cap) {
-            (void)hipFree(rp_tmp);
-            rp_tmp = nullptr;
-            SP_HIP(hipMalloc(&rp_tmp, need));
-            rp_cap = need;
-        }
-        SP_HIP(rocprim::segmented_radix_sort_keys(rp_tmp, need, vals, sorted, (unsigned)n, (unsigned)ns,
-                                                  (const uint32_t *)d_begin, (const uint32_t *)d_end, 0, 32, st));
-        hipLaunchKernelGGL(vq::k_seg_middles, dim3(cdiv(ns, 64)), dim3(64), 0, st, sorted,
-                           (const uint2 *)d_range, ns, (float *)d_mids);
+        hipLaunchKernelGGL(vq::k_seg_select_out, dim3(cdiv(2 * ns, 64)), dim3(64), 0, st,
+                           (const vq::SegSelect *)d_sel, ns, (float *)d_mids);
         SP_HIP(hipGetLastError());
         std::vector<float> mids(2 * (size_t)ns), median(ns);
         SP_HIP(hipMemcpyAsync(mids.data(), d_mids, sizeof(float) * 2 * ns, hipMemcpyDeviceToHost, st));
@@ -285,7 +275,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         // stable partition by `<= median` (src/tsvq.rs:120-123)
         hipLaunchKernelGGL(vq::k_seg_flags, dim3(cdiv(n, 256)), dim3(256), 0, st, vals, n, (const uint2 *)d_range,
                            ns, (const float *)d_median, flags);
-        need = 0;
+        size_t need = 0;
         SP_HIP(rocprim::exclusive_scan(nullptr, need, flags, scan, 0u, (size_t)n, rocprim::plus<uint32_t>(), st));
         if (need > rp_cap) {
             (void)hipFree(rp_tmp);
