@@ -92,6 +92,110 @@ static __global__ void __launch_bounds__(64) k_seg_variance(const uint32_t *__re
     var[(size_t)g * dim + t] = acc;
 }
 
+// The same sums with the memory traffic taken off the chain of dependent adds.  One workgroup of
+// 1024 threads per segment: all threads fetch rows (16-byte pieces, whole rows contiguous) eight
+// chunks ahead into registers and hand them over through two LDS tiles; threads 0..dim-1 add the
+// rows of the current tile in order.  A chunk is 8192 / dim rows; about 512 rows (256 KB at
+// dim = 128) are in flight per workgroup, which is what one chain of adds consumes per memory
+// round trip.  The barrier waits for LDS only, so the loads in flight are not drained.
+constexpr int kVarStage = 8192;  // floats per LDS tile
+constexpr int kVarAhead = 8;     // chunks in flight
+
+__device__ __forceinline__ void lds_only_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+static __global__ void __launch_bounds__(1024) k_seg_variance_wg(const uint32_t *__restrict__ perm,
+                                                                const uint2 *__restrict__ seg_range,
+                                                                const float *__restrict__ means, int64_t first,
+                                                                const float *__restrict__ x, int64_t ld, int dim,
+                                                                float *__restrict__ var) {
+    __shared__ float4 tile[2][kVarStage / 4];
+    const int g = blockIdx.x, tid = threadIdx.x;
+    const uint2 range = seg_range[g];
+    const uint32_t count = range.y - range.x;
+    const int ppr = dim / 4;                  // 16-byte pieces per row
+    const int R = kVarStage / dim;            // rows per chunk
+    const int pieces = R * ppr;               // pieces per chunk (<= 2048)
+    const int nch = (int)((count + R - 1) / R);
+    // this thread's two pieces of every chunk
+    int rr[2], pc[2];
+    bool has[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int e = tid + 1024 * j;
+        has[j] = e < pieces;
+        rr[j] = has[j] ? e / ppr : 0;
+        pc[j] = has[j] ? e % ppr : 0;
+    }
+    const uint32_t *pm = perm + range.x;
+    uint32_t idr[kVarAhead][2];
+    float4 xrg[kVarAhead][2];
+    auto load_ids = [&](int chunk, uint32_t (&dst)[2]) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t m = (uint32_t)chunk * R + rr[j];
+            dst[j] = (chunk < nch && has[j] && m < count) ? pm[m] : 0xFFFFFFFFu;
+        }
+    };
+    auto load_rows = [&](const uint32_t (&ids)[2], float4 (&dst)[2]) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            dst[j] = (ids[j] != 0xFFFFFFFFu) ? *reinterpret_cast<const float4 *>(x + (int64_t)ids[j] * ld + 4 * pc[j])
+                                             : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    auto store_tile = [&](int buf, const float4 (&src)[2]) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            if (has[j]) tile[buf][rr[j] * ppr + pc[j]] = src[j];
+    };
+    // prologue: ids of chunks 0..15, rows of chunks 0..7, chunk 0 in LDS
+#pragma unroll
+    for (int u = 0; u < kVarAhead; ++u) load_ids(u, idr[u]);
+#pragma unroll
+    for (int u = 0; u < kVarAhead; ++u) {
+        load_rows(idr[u], xrg[u]);
+        load_ids(u + kVarAhead, idr[u]);
+    }
+    store_tile(0, xrg[0]);
+    lds_only_barrier();
+    const float mu = (tid < dim) ? means[(first + g) * dim + tid] : 0.0f;
+    float acc = 0.0f;
+    for (int base = 0; base < nch; base += kVarAhead) {
+#pragma unroll
+        for (int u = 0; u < kVarAhead; ++u) {
+            const int i = base + u;
+            if (i >= nch) break;  // uniform
+            // rows of chunk i + 8 into the slot chunk i has left, ids of chunk i + 16 behind them
+            load_rows(idr[u], xrg[u]);
+            load_ids(i + 2 * kVarAhead, idr[u]);
+            // chunk i + 1 (fetched seven iterations ago) into the other tile
+            if (i + 1 < nch) store_tile((i + 1) & 1, xrg[(u + 1) % kVarAhead]);
+            if (tid < dim) {
+                const float *t = reinterpret_cast<const float *>(tile[i & 1]) + tid;
+                const int rows = (int)(((uint32_t)(i + 1) * R <= count) ? R : count - (uint32_t)i * R);
+                int r = 0;
+                for (; r + 8 <= rows; r += 8) {
+                    float v[8];
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) v[q] = t[(r + q) * dim];
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) {
+                        const float d = v[q] - mu;
+                        const float p = d * d;
+                        acc = acc + p;
+                    }
+                }
+                for (; r < rows; ++r) {
+                    const float d = t[r * dim] - mu;
+                    const float p = d * d;
+                    acc = acc + p;
+                }
+            }
+            lds_only_barrier();
+        }
+    }
+    if (tid < dim) var[(size_t)g * dim + tid] = acc;
+}
+
 __device__ __forceinline__ int find_segment(const uint2 *__restrict__ seg_range, int nseg, uint32_t p) {
     // segments are sorted by position and disjoint; returns -1 when p lies in none
     int lo = 0, hi = nseg - 1;

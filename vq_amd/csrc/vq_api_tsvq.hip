@@ -228,9 +228,13 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         SP_HIP(hipMemcpyAsync(d_range, range.data(), sizeof(uint2) * ns, hipMemcpyHostToDevice, st));
         SP_HIP(hipMemcpyAsync(d_smeans, smeans.data(), sizeof(float) * (size_t)ns * dim, hipMemcpyHostToDevice, st));
         // per-dimension sums of squared deviations (src/tsvq.rs:88-99)
-        hipLaunchKernelGGL(vq::k_seg_variance, dim3(cdiv((int64_t)ns * dim, 64)), dim3(64), 0, st, perm,
-                           (const uint2 *)d_range, ns, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
-                           (float *)d_var);
+        if (dim % 4 == 0 && dim <= 1024 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0)
+            hipLaunchKernelGGL(vq::k_seg_variance_wg, dim3(ns), dim3(1024), 0, st, perm, (const uint2 *)d_range,
+                               (const float *)d_smeans, (int64_t)0, d_x, ld, dim, (float *)d_var);
+        else
+            hipLaunchKernelGGL(vq::k_seg_variance, dim3(cdiv((int64_t)ns * dim, 64)), dim3(64), 0, st, perm,
+                               (const uint2 *)d_range, ns, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
+                               (float *)d_var);
         SP_HIP(hipGetLastError());
         std::vector<float> var((size_t)ns * dim);
         SP_HIP(hipMemcpyAsync(var.data(), d_var, sizeof(float) * (size_t)ns * dim, hipMemcpyDeviceToHost, st));
