@@ -103,6 +103,28 @@ constexpr int kVarAhead = 8;     // chunks in flight
 
 __device__ __forceinline__ void lds_only_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// acc + sum over the rows of one LDS tile of (v - mu)^2, in row order, for one component.
+__device__ __forceinline__ float seg_variance_chunk(const float *t, int rows, int dim, float mu, float acc) {
+    int r = 0;
+    for (; r + 8 <= rows; r += 8) {
+        float v[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) v[q] = t[(r + q) * dim];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const float d = v[q] - mu;
+            const float p = d * d;
+            acc = acc + p;
+        }
+    }
+    for (; r < rows; ++r) {
+        const float d = t[r * dim] - mu;
+        const float p = d * d;
+        acc = acc + p;
+    }
+    return acc;
+}
+
 static __global__ void __launch_bounds__(1024) k_seg_variance_wg(const uint32_t *__restrict__ perm,
                                                                 const uint2 *__restrict__ seg_range,
                                                                 const float *__restrict__ means, int64_t first,
@@ -126,73 +148,68 @@ static __global__ void __launch_bounds__(1024) k_seg_variance_wg(const uint32_t 
         rr[j] = has[j] ? e / ppr : 0;
         pc[j] = has[j] ? e % ppr : 0;
     }
-    const uint32_t *pm = perm + range.x;
-    uint32_t idr[kVarAhead][2];
-    float4 xrg[kVarAhead][2];
-    auto load_ids = [&](int chunk, uint32_t (&dst)[2]) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const uint32_t m = (uint32_t)chunk * R + rr[j];
-            dst[j] = (chunk < nch && has[j] && m < count) ? pm[m] : 0xFFFFFFFFu;
-        }
-    };
-    auto load_rows = [&](const uint32_t (&ids)[2], float4 (&dst)[2]) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-            dst[j] = (ids[j] != 0xFFFFFFFFu) ? *reinterpret_cast<const float4 *>(x + (int64_t)ids[j] * ld + 4 * pc[j])
-                                             : make_float4(0.f, 0.f, 0.f, 0.f);
-    };
-    auto store_tile = [&](int buf, const float4 (&src)[2]) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-            if (has[j]) tile[buf][rr[j] * ppr + pc[j]] = src[j];
-    };
-    // prologue: ids of chunks 0..15, rows of chunks 0..7, chunk 0 in LDS
-#pragma unroll
-    for (int u = 0; u < kVarAhead; ++u) load_ids(u, idr[u]);
-#pragma unroll
-    for (int u = 0; u < kVarAhead; ++u) {
-        load_rows(idr[u], xrg[u]);
-        load_ids(u + kVarAhead, idr[u]);
+    if (count == 0) {  // uniform
+        if (tid < dim) var[(size_t)g * dim + tid] = 0.0f;
+        return;
     }
-    store_tile(0, xrg[0]);
+    const uint32_t *pm = perm + range.x;
+    // Loads are unconditional (positions clamped into the segment; surplus rows are fetched and
+    // never read): loads under a branch would make the compiler wait for every outstanding load
+    // at each use instead of counting them.  The rings are plain arrays with constant indices.
+    // (Eight named slots instead of an array: an array of this size is left in scratch memory.)
+    const float *xp0 = x + 4 * pc[0], *xp1 = x + 4 * pc[1];
+#define VAR_DECL(S) uint32_t ida_##S, idb_##S; float4 xa_##S, xb_##S;
+    VAR_DECL(0) VAR_DECL(1) VAR_DECL(2) VAR_DECL(3) VAR_DECL(4) VAR_DECL(5) VAR_DECL(6) VAR_DECL(7)
+#define VAR_IDS(S, chunk)                                                     \
+    {                                                                         \
+        const uint32_t m0 = (uint32_t)(chunk) * R + rr[0], m1 = (uint32_t)(chunk) * R + rr[1]; \
+        ida_##S = pm[m0 < count ? m0 : count - 1];                            \
+        idb_##S = pm[m1 < count ? m1 : count - 1];                            \
+    }
+#define VAR_ROWS(S)                                                           \
+    {                                                                         \
+        xa_##S = *reinterpret_cast<const float4 *>(xp0 + (int64_t)ida_##S * ld); \
+        xb_##S = *reinterpret_cast<const float4 *>(xp1 + (int64_t)idb_##S * ld); \
+    }
+#define VAR_STORE(buf, S)                                                     \
+    {                                                                         \
+        if (has[0]) tile[buf][rr[0] * ppr + pc[0]] = xa_##S;                  \
+        if (has[1]) tile[buf][rr[1] * ppr + pc[1]] = xb_##S;                  \
+    }
+    // prologue: ids of chunks 0..15, rows of chunks 0..7, chunk 0 in LDS
+    VAR_IDS(0, 0) VAR_IDS(1, 1) VAR_IDS(2, 2) VAR_IDS(3, 3) VAR_IDS(4, 4) VAR_IDS(5, 5) VAR_IDS(6, 6) VAR_IDS(7, 7)
+#define VAR_PRO(S) VAR_ROWS(S) VAR_IDS(S, S + kVarAhead)
+    VAR_PRO(0) VAR_PRO(1) VAR_PRO(2) VAR_PRO(3) VAR_PRO(4) VAR_PRO(5) VAR_PRO(6) VAR_PRO(7)
+    VAR_STORE(0, 0)
     lds_only_barrier();
     const float mu = (tid < dim) ? means[(first + g) * dim + tid] : 0.0f;
     float acc = 0.0f;
-    for (int base = 0; base < nch; base += kVarAhead) {
-#pragma unroll
-        for (int u = 0; u < kVarAhead; ++u) {
-            const int i = base + u;
-            if (i >= nch) break;  // uniform
-            // rows of chunk i + 8 into the slot chunk i has left, ids of chunk i + 16 behind them
-            load_rows(idr[u], xrg[u]);
-            load_ids(i + 2 * kVarAhead, idr[u]);
-            // chunk i + 1 (fetched seven iterations ago) into the other tile
-            if (i + 1 < nch) store_tile((i + 1) & 1, xrg[(u + 1) % kVarAhead]);
-            if (tid < dim) {
-                const float *t = reinterpret_cast<const float *>(tile[i & 1]) + tid;
-                const int rows = (int)(((uint32_t)(i + 1) * R <= count) ? R : count - (uint32_t)i * R);
-                int r = 0;
-                for (; r + 8 <= rows; r += 8) {
-                    float v[8];
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) v[q] = t[(r + q) * dim];
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) {
-                        const float d = v[q] - mu;
-                        const float p = d * d;
-                        acc = acc + p;
-                    }
-                }
-                for (; r < rows; ++r) {
-                    const float d = t[r * dim] - mu;
-                    const float p = d * d;
-                    acc = acc + p;
-                }
-            }
-            lds_only_barrier();
-        }
+    // One step: rows of chunk i + 8 into the slot chunk i has left, ids of chunk i + 16 behind
+    // them; chunk i + 1 (fetched seven steps ago) into the other tile; chunk i added.  Chunks past
+    // the end run empty, so every thread reaches every barrier.
+#define VAR_STEP(S, SN)                                                       \
+    {                                                                         \
+        const int i = base + S;                                               \
+        VAR_ROWS(S)                                                           \
+        VAR_IDS(S, i + 2 * kVarAhead)                                         \
+        VAR_STORE((i + 1) & 1, SN)                                            \
+        if (tid < dim && i < nch) {                                           \
+            const float *t = reinterpret_cast<const float *>(tile[i & 1]) + tid; \
+            const int rows = (int)(((uint32_t)(i + 1) * R <= count) ? R : count - (uint32_t)i * R); \
+            acc = seg_variance_chunk(t, rows, dim, mu, acc);                  \
+        }                                                                     \
+        lds_only_barrier();                                                   \
     }
+    for (int base = 0; base < nch; base += kVarAhead) {
+        VAR_STEP(0, 1) VAR_STEP(1, 2) VAR_STEP(2, 3) VAR_STEP(3, 4)
+        VAR_STEP(4, 5) VAR_STEP(5, 6) VAR_STEP(6, 7) VAR_STEP(7, 0)
+    }
+#undef VAR_DECL
+#undef VAR_PRO
+#undef VAR_STEP
+#undef VAR_IDS
+#undef VAR_ROWS
+#undef VAR_STORE
     if (tid < dim) var[(size_t)g * dim + tid] = acc;
 }
 
