@@ -606,7 +606,7 @@ __global__ void __launch_bounds__(256) k_assign_mfma_wide(AssignArgs a, MfmaWide
 struct MfmaWideBfTables {
     const u32x4 *atab;     // [m][sd/8][nb][2][64]
     const float *c2perm;   // [m][nb][2][16]
-    const float *maxc2;    // [m]
+    const float *blockmax; // [m][nb]  largest ||c||^2 per block of 32 centroids (NaN if any is NaN)
     uint32_t *list;
     uint32_t *list_count;
     int nb;
@@ -614,65 +614,67 @@ struct MfmaWideBfTables {
     float kappa;           // error-bound coefficient on (||x||^2 + max ||c||^2)
 };
 
-// One workgroup per column block s, one thread per padded centroid (k <= 256).
+// One workgroup per (column block s, block b of 32 centroids): thread (i, g) = (tid % 32, tid / 32)
+// writes the chunks kc = g, g + 8, ... of centroid 32 b + i and sums their share of ||c||^2; the
+// eight shares are added in g order.  blockmax[s][b] = largest ||c||^2 of the block (NaN stays).
 static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *__restrict__ cb, int m, int k, int nb,
                                                                   int sd, u32x4 *__restrict__ atab,
                                                                   float *__restrict__ c2perm,
-                                                                  float *__restrict__ maxc2,
+                                                                  float *__restrict__ blockmax,
                                                                   uint32_t *__restrict__ list_count) {
-    const int s = blockIdx.x, j = threadIdx.x;
+    const int s = blockIdx.x, b = blockIdx.y;
+    const int i = threadIdx.x & 31, g = threadIdx.x >> 5;
+    const int j = b * 32 + i;
     const int nkc = sd / 8;
-    __shared__ float sh_max[4];
-    float mx = 0.0f;
-    if (j < nb * 32) {
-        const int b = j / 32, i = j % 32;
-        const float *c = cb + ((size_t)s * k + j) * sd;
-        float c2 = kPadScore;
-        if (j < k) {
-            c2 = 0.0f;
-            for (int t = 0; t < sd; ++t) c2 = __builtin_fmaf(c[t], c[t], c2);
-            mx = c2;
-        }
-        const u32x4 ones = {0x3f803f80u, 0x00003f80u, 0u, 0u};
-        for (int kc = 0; kc < nkc; ++kc) {
-            u32x4 ah, al;
+    __shared__ float part[8][32];
+    const float *c = cb + ((size_t)s * k + (j < k ? j : 0)) * sd;
+    const u32x4 ones = {0x3f803f80u, 0x00003f80u, 0u, 0u};
+    float p = 0.0f;
+    for (int kc = g; kc < nkc; kc += 8) {
+        const float4 v0 = *reinterpret_cast<const float4 *>(c + kc * 8);
+        const float4 v1 = *reinterpret_cast<const float4 *>(c + kc * 8 + 4);
+        const float cv[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+        u32x4 ah, al;
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                uint32_t hb[2], lb[2];
+        for (int w = 0; w < 4; ++w) {
+            uint32_t hb[2], lb[2];
 #pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    const float a = (j < k) ? -2.0f * c[kc * 8 + 2 * w + e] : 0.0f;
-                    hb[e] = bf16_rne_bits(a);
-                    lb[e] = bf16_rne_bits(a - bf16_bits_to_float(hb[e]));
-                }
-                ah[w] = hb[0] | (hb[1] << 16);
-                al[w] = lb[0] | (lb[1] << 16);
+            for (int e = 0; e < 2; ++e) {
+                const float x = cv[2 * w + e];
+                p = __builtin_fmaf(x, x, p);
+                const float a = (j < k) ? -2.0f * x : 0.0f;
+                hb[e] = bf16_rne_bits(a);
+                lb[e] = bf16_rne_bits(a - bf16_bits_to_float(hb[e]));
             }
-            u32x4 *dst = atab + (((size_t)s * nkc + kc) * nb + b) * 128;
-            dst[i] = ah;
-            dst[32 + i] = ah;
-            dst[64 + i] = al;
-            dst[96 + i] = ones;
+            ah[w] = hb[0] | (hb[1] << 16);
+            al[w] = lb[0] | (lb[1] << 16);
+        }
+        u32x4 *dst = atab + (((size_t)s * nkc + kc) * nb + b) * 128;
+        dst[i] = ah;
+        dst[32 + i] = ah;
+        dst[64 + i] = al;
+        dst[96 + i] = ones;
+    }
+    part[g][i] = p;
+    __syncthreads();
+    if (g == 0) {
+        float c2 = 0.0f;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) c2 = c2 + part[q][i];
+        float mx = c2;
+        if (j >= k) {
+            c2 = kPadScore;
+            mx = 0.0f;
         }
         const int hh = (i / 4) % 2, v = (i / 8) * 4 + i % 4;
         c2perm[(((size_t)s * nb + b) * 2 + hh) * 16 + v] = c2;
-    }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const float o = __shfl_xor(mx, off);
-        mx = (mx == mx && o == o) ? fmaxf(mx, o) : __builtin_nanf("");
-    }
-    if ((j & 63) == 0) sh_max[j >> 6] = mx;
-    __syncthreads();
-    if (j == 0) {
-        float r = sh_max[0];
-#pragma unroll
-        for (int w = 1; w < 4; ++w) {
-            const float o = sh_max[w];
-            r = (r == r && o == o) ? fmaxf(r, o) : __builtin_nanf("");
+        for (int off = 16; off > 0; off >>= 1) {
+            const float o = __shfl_xor(mx, off);
+            mx = (mx == mx && o == o) ? fmaxf(mx, o) : __builtin_nanf("");
         }
-        maxc2[s] = r;
-        if (s == 0) *list_count = 0;
+        if (i == 0) blockmax[(size_t)s * nb + b] = mx;
+        if (s == 0 && b == 0 && i == 0) *list_count = 0;
     }
 }
 
@@ -837,7 +839,11 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     }
     __syncthreads();
     if (ch == 0 && h == 0) {
-        const float mc2 = tb.maxc2[s];
+        float mc2 = 0.0f;  // largest ||c||^2 of the column block; a NaN stays
+        for (int b = 0; b < nb; ++b) {
+            const float o = tb.blockmax[(size_t)s * nb + b];
+            mc2 = (mc2 == mc2 && o == o) ? fmaxf(mc2, o) : __builtin_nanf("");
+        }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int o1 = lds_top[rp][t][0][r], o2 = lds_top[rp][t][1][r];

@@ -169,14 +169,14 @@ template <int METRIC, bool LBG>
 int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     const int nb = (a.k + 31) / 32, nkc = sd / 8;
     const size_t n_atab = (size_t)a.m * nkc * nb * 128 * 4, n_c2 = (size_t)a.m * nb * 32;  // floats
-    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + a.m) + 64));
+    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + (size_t)a.m * nb) + 64));
     VQ_TRY(ensure(ctx, ctx->mfma_list, sizeof(uint32_t) * ((size_t)a.n * a.m + 4)));
     float *atab = (float *)ctx->mfma_tab.p;
     float *c2perm = atab + n_atab;
-    float *maxc2 = c2perm + n_c2;
+    float *maxc2 = c2perm + n_c2;  // per block of 32 centroids
     uint32_t *count = (uint32_t *)ctx->mfma_list.p;
     uint32_t *list = count + 4;
-    hipLaunchKernelGGL(vq::k_mfma_wide_bf_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, sd,
+    hipLaunchKernelGGL(vq::k_mfma_wide_bf_prep, dim3(a.m, nb), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, sd,
                        (vq::u32x4 *)atab, c2perm, maxc2, count);
     // two candidates, each: operand split 3 * 2^-16, fp32 accumulation (34 per chunk + 16) * 2^-24
     const float kappa = 2.0f * (3.0f * 1.52587890625e-05f + (34.0f * nkc + 16.0f) * 5.9604644775390625e-08f);
@@ -196,8 +196,9 @@ bool mfma_wide_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     if (ctx->assign_path == 1) return false;
     if (METRIC != vq::M_SQ && METRIC != vq::M_EUCLID) return false;
     if (sd < 16 || sd % 8 != 0 || a.k > 256 || a.m > 65535) return false;
-    // float4 row loads
-    if (a.ld % 4 != 0 || (reinterpret_cast<uintptr_t>(a.x) & 15) != 0) return false;
+    // float4 row and centroid loads
+    if (a.ld % 4 != 0 || ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.cb)) & 15) != 0)
+        return false;
     return (int64_t)a.n * a.m < (1LL << 32);
 }
 
