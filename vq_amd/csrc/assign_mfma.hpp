@@ -12,8 +12,8 @@
 // bit-identical to the all-VALU path for every input.
 //
 // 8-float column blocks (k_assign_mfma_bf): bf16 matrix cores with split operands; the undecided
-// rows are resolved inside the same wave.  Wider blocks (k_assign_mfma_wide): fp32 matrix cores;
-// the undecided pairs are listed for the exact kernel of assign_exact.hpp.
+// rows are resolved inside the same wave.  Wider blocks (k_assign_mfma_wide_bf): the same split
+// per chunk of 8 dimensions; the undecided pairs are listed for the exact kernel of assign_exact.hpp.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -426,171 +426,7 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 2) ? 5 : (TILES * SG <= 4)
 
 // =============================================================================================
 // Wide column blocks (sub_dim a multiple of 8, up to the full dimension: RVQ stages).
-// Same two-pass scheme; the contraction over sub_dim is a loop over chunks of 8 dimensions with
-// the scores of all 8 blocks of 32 centroids kept in accumulators (128 registers per lane), the
-// -2c operand of a chunk staged once per workgroup in LDS and shared by its 4 waves.
 namespace vq {
-
-struct MfmaWideTables {
-    const float *atab;     // [m][sd/8][nb][64][4]  -2*c in MFMA A-operand order, chunk-major
-    const float *c2perm;   // [m][nb][2][16]
-    const float *maxc2;    // [m]
-    uint32_t *list;
-    uint32_t *list_count;
-    int nb;
-    int sd;
-    float kappa;           // error-bound coefficient on (||x||^2 + max ||c||^2)
-};
-
-static __global__ void __launch_bounds__(256) k_mfma_wide_prep(const float *__restrict__ cb, int m, int k, int nb,
-                                                               int sd, float *__restrict__ atab,
-                                                               float *__restrict__ c2perm,
-                                                               float *__restrict__ maxc2,
-                                                               uint32_t *__restrict__ list_count) {
-    const int s = blockIdx.x;
-    const int nkc = sd / 8;
-    __shared__ float sh_max[256];
-    float mx = 0.0f;
-    for (int j = threadIdx.x; j < nb * 32; j += 256) {
-        const int b = j / 32, i = j % 32;
-        const float *c = cb + ((size_t)s * k + j) * sd;
-        float c2 = kPadScore;
-        if (j < k) {
-            c2 = 0.0f;
-            for (int t = 0; t < sd; ++t) c2 = __builtin_fmaf(c[t], c[t], c2);
-            mx = fmaxf(mx, c2);
-            if (!(c2 == c2)) mx = c2;
-        }
-        for (int kc = 0; kc < nkc; ++kc)
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    atab[((((size_t)s * nkc + kc) * nb + b) * 64 + i + 32 * h) * 4 + u] =
-                        (j < k) ? -2.0f * c[kc * 8 + 4 * h + u] : 0.0f;
-        const int hh = (i / 4) % 2, v = (i / 8) * 4 + i % 4;
-        c2perm[(((size_t)s * nb + b) * 2 + hh) * 16 + v] = c2;
-    }
-    sh_max[threadIdx.x] = mx;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        float r = 0.0f;
-        for (int i = 0; i < 256; ++i) {
-            float v = sh_max[i];
-            r = (v == v) ? fmaxf(r, v) : v;
-            if (!(r == r)) break;
-        }
-        maxc2[s] = r;
-        if (s == 0) *list_count = 0;
-    }
-}
-
-// grid (ceil(n/128), m); 256 threads = 4 waves, one tile of 32 rows per wave.
-template <bool LBG>
-__global__ void __launch_bounds__(256) k_assign_mfma_wide(AssignArgs a, MfmaWideTables tb) {
-    constexpr int NBMAX = 8;
-    __shared__ float4 lds_a[2][NBMAX * 64];
-    __shared__ float lds_c2[NBMAX * 32];
-    const int s = blockIdx.y;
-    if constexpr (LBG) {
-        if (a.done[s]) return;
-    }
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r = lane & 31, h = lane >> 5;
-    const int nb = tb.nb, sd = tb.sd, nkc = sd / 8;
-    const int64_t row = ((int64_t)blockIdx.x * 4 + wave) * 32 + r;
-    const bool valid = row < a.n;
-    const float4 *ag = reinterpret_cast<const float4 *>(tb.atab) + (size_t)s * nkc * nb * 64;
-    const int chunk4 = nb * 64;  // float4 per chunk
-    for (int i = threadIdx.x; i < nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s * nb * 32 + i];
-    for (int i = threadIdx.x; i < chunk4; i += 256) lds_a[0][i] = ag[i];
-    __syncthreads();
-
-    floatx16 acc[NBMAX];
-#pragma unroll
-    for (int b = 0; b < NBMAX; ++b)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[b][v] = 0.0f;
-    const float *xr = a.x + (valid ? row : 0) * a.ld + (int64_t)s * sd + 4 * h;
-    float p = 0.0f;
-    for (int kc = 0; kc < nkc; ++kc) {
-        const int cur = kc & 1;
-        // fetch the next chunk of the -2c operand while this one is used
-        float4 pre[2];
-        const bool more = kc + 1 < nkc;
-        if (more) {
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                int i = threadIdx.x + 256 * q;
-                if (i < chunk4) pre[q] = ag[(size_t)(kc + 1) * chunk4 + i];
-            }
-        }
-        float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (valid) xv = *reinterpret_cast<const float4 *>(xr + kc * 8);
-        p = __builtin_fmaf(xv.x, xv.x, p);
-        p = __builtin_fmaf(xv.y, xv.y, p);
-        p = __builtin_fmaf(xv.z, xv.z, p);
-        p = __builtin_fmaf(xv.w, xv.w, p);
-#pragma unroll
-        for (int b = 0; b < NBMAX; ++b) {
-            if (b < nb) {
-                const float4 av = lds_a[cur][b * 64 + lane];
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, xv.x, acc[b], 0, 0, 0);
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, xv.y, acc[b], 0, 0, 0);
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, xv.z, acc[b], 0, 0, 0);
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, xv.w, acc[b], 0, 0, 0);
-            }
-        }
-        if (more) {
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                int i = threadIdx.x + 256 * q;
-                if (i < chunk4) lds_a[cur ^ 1][i] = pre[q];
-            }
-        }
-        __syncthreads();
-    }
-    const float x2 = p + __shfl_xor(p, 32);
-    int m1 = 0x7f800000, m2 = 0x7f800000;
-#pragma unroll
-    for (int b = 0; b < NBMAX; ++b) {
-        if (b < nb) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const float sc = acc[b][v] + (lds_c2[(b * 2 + h) * 16 + v] + x2);
-                const uint32_t idx = (uint32_t)(32 * b + 8 * (v / 4) + 4 * h + v % 4);
-                const int key = (int)((__float_as_uint(sc) & 0xFFFFFF00u) | idx);
-                m2 = imed3(m1, m2, key);
-                m1 = imin(m1, key);
-            }
-        }
-    }
-    const int o1 = __shfl_xor(m1, 32), o2 = __shfl_xor(m2, 32);
-    const float s1 = __int_as_float(imin(m1, o1));
-    const float s2 = __int_as_float(imin(imax(m1, o1), imin(m2, o2)));
-    if (h == 0 && valid) {
-        const float bound = x2 + tb.maxc2[s];
-        const float margin = 6.103515625e-05f * fabsf(s2) + tb.kappa * bound;
-        bool sure = (s2 - s1) > margin;
-        sure = sure && (bound < 1e29f) && (s1 < 1e29f);
-        if (sure) {
-            const uint8_t code = (uint8_t)(__float_as_uint(s1) & 0xFFu);
-            if constexpr (LBG) {
-                uint8_t *pc = a.codes + (size_t)s * a.n + row;
-                if (*pc != code) {
-                    *pc = code;
-                    mark_changed(a.changed + s);
-                }
-            } else {
-                a.codes[row * a.m + s] = code;
-            }
-        } else {
-            const uint32_t pos = atomicAdd(tb.list_count, 1u);
-            tb.list[pos] = (uint32_t)(row * a.m + s);
-        }
-    }
-}
-
 
 // ---------------------------------------------------------------------------------------------
 // Wide column blocks on the bf16 matrix cores: the operand split of k_assign_mfma_bf applied to
