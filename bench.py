@@ -47,7 +47,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel on the workload's rows (3 launches): the "
                          "known-size kernel the FETCH_SIZE / WRITE_SIZE counters are scaled by")
-    ap.add_argument("--cpu-sample", type=int, default=100_000,
+    ap.add_argument("--cpu-sample", type=int, default=1_000_000,
                     help="rows of the CPU-baseline sample (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
