@@ -72,11 +72,13 @@ __device__ __forceinline__ void top2_push4(int &m1, int &m2, int k0, int k1, int
 // 8-float column blocks on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16, 4x the fp32 rate).
 //
 // Every fp32 operand is split into two bf16 numbers, v = vh + vl + e with |e| <= 2^-16 |v|
-// (round-to-nearest-even twice).  With a = -2c the 16 contraction slots of two instructions hold
-//     instruction 1:  ah . xh  (slots 0-7)   ah . xl  (slots 8-15)
-//     instruction 2:  al . xh  (slots 0-7)   1 . (three bf16 parts of ||x||^2)  (slots 8-10)
-// and the accumulator starts at ||c||^2, so the result is the score ||c||^2 + ||x||^2 - 2 x.c with
-// an error of at most 3 * 2^-16 * sum|a_t||x_t| <= 3 * 2^-16 (||x||^2 + ||c||^2) from the dropped
+// (round-to-nearest-even twice).  With a = -2c, the lanes of half h = lane / 32 own dimensions
+// [4h, 4h + 4) of the block and the 8 contraction slots of that half hold
+//     instruction 1:  ah . xh  (4 slots)   ah . xl  (4 slots)
+//     instruction 2:  al . xh  (4 slots)   1 . (three bf16 parts of the half's share of ||x||^2)
+// so a lane loads and splits only its own 16 bytes of the row, both halves do the same work, and
+// the accumulator starts at ||c||^2: the result is the score ||c||^2 + ||x||^2 - 2 x.c with an
+// error of at most 3 * 2^-16 * sum|a_t||x_t| <= 3 * 2^-16 (||x||^2 + ||c||^2) from the dropped
 // terms (a ex, x ea, al xl) plus at most 2^-17.9 (||x||^2 + ||c||^2) from the fp32 accumulation of
 // the 2 x 17 addends.  Two candidates compared: below 2^-13.2 (||x||^2 + max ||c||^2); the test
 // uses 2^-13, plus 2^-14 |second| for the packed bits and the reference's own rounding.  bf16
@@ -145,18 +147,15 @@ static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__rest
             hb[t] = bf16_rne_bits(a);
             lb[t] = bf16_rne_bits(a - bf16_bits_to_float(hb[t]));
         }
-        u32x4 ah, al;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            ah[w] = hb[2 * w] | (hb[2 * w + 1] << 16);
-            al[w] = lb[2 * w] | (lb[2 * w + 1] << 16);
-        }
-        const u32x4 ones = {0x3f803f80u, 0x00003f80u, 0u, 0u};  // 1, 1, 1, 0, ...
+        // lane i + 32 h: instruction 1 {ah[4h..4h+3], ah[4h..4h+3]}, instruction 2 {al[4h..4h+3], 1, 1, 1, 0}
         u32x4 *dst = atab + ((size_t)s * nb + b) * 128;
-        dst[i] = ah;
-        dst[32 + i] = ah;
-        dst[64 + i] = al;
-        dst[96 + i] = ones;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t ah0 = hb[4 * h] | (hb[4 * h + 1] << 16), ah1 = hb[4 * h + 2] | (hb[4 * h + 3] << 16);
+            const uint32_t al0 = lb[4 * h] | (lb[4 * h + 1] << 16), al1 = lb[4 * h + 2] | (lb[4 * h + 3] << 16);
+            dst[32 * h + i] = u32x4{ah0, ah1, ah0, ah1};
+            dst[64 + 32 * h + i] = u32x4{al0, al1, 0x3f803f80u, 0x00003f80u};
+        }
         // accumulator order: lane half h, register v <-> centroid 8*(v/4) + 4*h + v%4
         const int hh = (i / 4) % 2, v = (i / 8) * 4 + i % 4;
         c2perm[(((size_t)s * nb + b) * 2 + hh) * 16 + v] = c2;
@@ -231,7 +230,7 @@ __device__ __forceinline__ int exact_argmin8_wave(const float (&xs)[8], const fl
 // 128-byte line of every row).  256 threads = 4 waves; grid = (row tiles, groups of column blocks),
 // so that the waves are short enough for the last round of workgroups not to leave the chip idle.
 template <int METRIC, bool LBG, int TILES, int SG>
-__global__ void __launch_bounds__(256, (TILES * SG <= 2) ? 5 : (TILES * SG <= 4) ? 4 : 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
+__global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
     constexpr int SD = 8;
     extern __shared__ float lds_c2[];  // [SG][nb][2][16]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -251,7 +250,7 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 2) ? 5 : (TILES * SG <= 4)
     const int64_t row_base = (tile_id * 4 + wave) * (32 * TILES);
     if (row_base >= a.n) return;
 
-    float xall[TILES][SG][SD];
+    float xall[TILES][SG][4];  // this lane's dimensions [4h, 4h + 4) of every block
     uint8_t old[TILES][SG];
     uint32_t cw[TILES];
     uint32_t n_exact = 0;
@@ -260,16 +259,16 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 2) ? 5 : (TILES * SG <= 4)
         const int64_t row = row_base + 32 * t + r;
         cw[t] = 0u;
         if (row < a.n) {
-            const float *xr = a.x + row * a.ld + (int64_t)s0 * SD;
+            const float *xr = a.x + row * a.ld + (int64_t)s0 * SD + 4 * h;
 #pragma unroll
             for (int q = 0; q < SG; ++q)
 #pragma unroll
-                for (int u = 0; u < SD; ++u) xall[t][q][u] = xr[q * SD + u];
+                for (int u = 0; u < 4; ++u) xall[t][q][u] = xr[q * SD + u];
         } else {
 #pragma unroll
             for (int q = 0; q < SG; ++q)
 #pragma unroll
-                for (int u = 0; u < SD; ++u) xall[t][q][u] = 0.0f;
+                for (int u = 0; u < 4; ++u) xall[t][q][u] = 0.0f;
         }
         if constexpr (LBG) {
 #pragma unroll
@@ -288,31 +287,22 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 2) ? 5 : (TILES * SG <= 4)
         int m1[TILES], m2[TILES];
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
+            const float *xv = xall[t][q];
             float p = 0.0f;
-            uint32_t hb[4];
-            float lo[SD];
 #pragma unroll
-            for (int u = 0; u < SD; ++u) p = __builtin_fmaf(xall[t][q][u], xall[t][q][u], p);
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                hb[w] = bf16_pack2(xall[t][q][2 * w], xall[t][q][2 * w + 1]);
-                lo[2 * w] = xall[t][q][2 * w] - __uint_as_float(hb[w] << 16);
-                lo[2 * w + 1] = xall[t][q][2 * w + 1] - __uint_as_float(hb[w] & 0xffff0000u);
-            }
-            x2[t] = p;
-            // ||x||^2 in three bf16 parts (exact to 2^-24)
+            for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
+            const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
+            const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
+            const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
+            // this half's share of ||x||^2 in three bf16 parts (exact to 2^-24)
             const uint32_t p0 = bf16_pack2(p, 0.0f);
             const float r1 = p - __uint_as_float(p0 << 16);
             const uint32_t p1 = bf16_pack2(r1, 0.0f);
             const float r2 = r1 - __uint_as_float(p1 << 16);
             const uint32_t p2 = bf16_pack2(r2, 0.0f);
-            const uint32_t xparts[4] = {(p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu, 0u, 0u};
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const uint32_t lw = bf16_pack2(lo[2 * w], lo[2 * w + 1]);
-                b1[t][w] = h ? lw : hb[w];
-                b2[t][w] = h ? xparts[w] : hb[w];
-            }
+            b1[t] = u32x4{h01, h23, l01, l23};
+            b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu};
+            x2[t] = p + __shfl_xor(p, 32);
             m1[t] = 0x7f800000;  // +inf
             m2[t] = 0x7f800000;
         }
@@ -382,10 +372,12 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 2) ? 5 : (TILES * SG <= 4)
             n_exact += (uint32_t)__popcll(todo);
             while (todo) {
                 const int src = __builtin_amdgcn_readfirstlane(__ffsll(todo) - 1);
-                float xs[SD];
+                float xs[SD];  // the row's 8 floats: dimensions 0-3 from lane src, 4-7 from lane src + 32
 #pragma unroll
-                for (int u = 0; u < SD; ++u)
+                for (int u = 0; u < 4; ++u) {
                     xs[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xall[t][q][u]), src));
+                    xs[4 + u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xall[t][q][u]), src + 32));
+                }
                 const int best = exact_argmin8_wave<METRIC>(xs, cb_s, a.k, lane);
                 if (lane == src) code = best;
                 todo &= todo - 1;

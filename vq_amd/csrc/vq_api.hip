@@ -20,7 +20,7 @@
 #define VQ_MFMA_TILES 2  // tiles of 32 rows per wave in the matrix-core assignment
 #endif
 #ifndef VQ_MFMA_SG
-#define VQ_MFMA_SG 2     // column blocks of 8 floats per wave (2: 64 bytes of each row, 4 waves per SIMD)
+#define VQ_MFMA_SG 4     // column blocks of 8 floats per wave (4: one 128-byte line of each row)
 #endif
 #include "lbg_update.hpp"
 
