@@ -422,8 +422,9 @@ namespace vq {
 
 // ---------------------------------------------------------------------------------------------
 // Wide column blocks on the bf16 matrix cores: the operand split of k_assign_mfma_bf applied to
-// every chunk of 8 dimensions (two instructions per chunk and tile of 32 centroids; the three
-// bf16 parts of the chunk's share of ||x||^2 ride in the spare slots of the second one).
+// every chunk of 8 dimensions (two instructions per chunk and tile of 32 centroids; each lane half
+// owns 4 of the 8 dimensions, the three bf16 parts of its share of ||x||^2 ride in the spare slots
+// of the second instruction).
 // A workgroup = 128 rows; wave w takes the row tiles {2 (w&1), 2 (w&1) + 1} and the centroid tiles
 // [4 (w>>1), 4 (w>>1) + 4): 8 accumulator tiles (128 registers), every A operand read from LDS
 // feeds two matrix instructions.  The A operands of a chunk (16 KB for 256 centroids) are staged
@@ -456,13 +457,12 @@ static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *_
     const int nkc = sd / 8;
     __shared__ float part[8][32];
     const float *c = cb + ((size_t)s * k + (j < k ? j : 0)) * sd;
-    const u32x4 ones = {0x3f803f80u, 0x00003f80u, 0u, 0u};
     float p = 0.0f;
     for (int kc = g; kc < nkc; kc += 8) {
         const float4 v0 = *reinterpret_cast<const float4 *>(c + kc * 8);
         const float4 v1 = *reinterpret_cast<const float4 *>(c + kc * 8 + 4);
         const float cv[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-        u32x4 ah, al;
+        uint32_t hw[4], lw[4];  // packed pairs of the high and low parts
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             uint32_t hb[2], lb[2];
@@ -474,14 +474,16 @@ static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *_
                 hb[e] = bf16_rne_bits(a);
                 lb[e] = bf16_rne_bits(a - bf16_bits_to_float(hb[e]));
             }
-            ah[w] = hb[0] | (hb[1] << 16);
-            al[w] = lb[0] | (lb[1] << 16);
+            hw[w] = hb[0] | (hb[1] << 16);
+            lw[w] = lb[0] | (lb[1] << 16);
         }
+        // lane i + 32 h: instruction 1 {ah[4h..4h+3], ah[4h..4h+3]}, instruction 2 {al[4h..4h+3], 1, 1, 1, 0}
         u32x4 *dst = atab + (((size_t)s * nkc + kc) * nb + b) * 128;
-        dst[i] = ah;
-        dst[32 + i] = ah;
-        dst[64 + i] = al;
-        dst[96 + i] = ones;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            dst[32 * h + i] = u32x4{hw[2 * h], hw[2 * h + 1], hw[2 * h], hw[2 * h + 1]};
+            dst[64 + 32 * h + i] = u32x4{lw[2 * h], lw[2 * h + 1], 0x3f803f80u, 0x00003f80u};
+        }
     }
     part[g][i] = p;
     __syncthreads();
@@ -541,7 +543,7 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     for (int t = 0; t < 2; ++t) {
         row[t] = (int64_t)blockIdx.x * 128 + (2 * rp + t) * 32 + r;
         valid[t] = row[t] < a.n;
-        xr[t] = a.x + (valid[t] ? row[t] : 0) * a.ld + (int64_t)s * sd;
+        xr[t] = a.x + (valid[t] ? row[t] : 0) * a.ld + (int64_t)s * sd + 4 * h;  // this half's 4 dimensions
     }
     floatx16 acc[2][4];
 #pragma unroll
@@ -554,12 +556,12 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
             acc[1][c][v] = c2;
         }
     }
-    float4 xn[2][2];  // the next chunk of the rows
+    // Loads are unconditional (a row past the end reads row 0 and is never stored; A pieces past
+    // the chunk are clamped): loads under a branch make the compiler wait for every outstanding
+    // load at each use instead of counting them.
+    float4 xn[2];  // the next chunk of the rows
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        xn[t][0] = valid[t] ? *reinterpret_cast<const float4 *>(xr[t]) : make_float4(0.f, 0.f, 0.f, 0.f);
-        xn[t][1] = valid[t] ? *reinterpret_cast<const float4 *>(xr[t] + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
+    for (int t = 0; t < 2; ++t) xn[t] = *reinterpret_cast<const float4 *>(xr[t]);
     float x2[2] = {0.0f, 0.0f};
     for (int kc = 0; kc < nkc; ++kc) {
         const int cur = kc & 1;
@@ -568,48 +570,31 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         u32x4 b1[2], b2[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const float xv[8] = {xn[t][0].x, xn[t][0].y, xn[t][0].z, xn[t][0].w,
-                                 xn[t][1].x, xn[t][1].y, xn[t][1].z, xn[t][1].w};
+            const float xv[4] = {xn[t].x, xn[t].y, xn[t].z, xn[t].w};
             float p = 0.0f;
-            uint32_t hb[4];
-            float lo[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                hb[w] = bf16_pack2(xv[2 * w], xv[2 * w + 1]);
-                lo[2 * w] = xv[2 * w] - __uint_as_float(hb[w] << 16);
-                lo[2 * w + 1] = xv[2 * w + 1] - __uint_as_float(hb[w] & 0xffff0000u);
-            }
+            for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
+            const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
+            const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
+            const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
             x2[t] += p;
             const uint32_t p0 = bf16_pack2(p, 0.0f);
             const float r1 = p - __uint_as_float(p0 << 16);
             const uint32_t p1 = bf16_pack2(r1, 0.0f);
             const float r2 = r1 - __uint_as_float(p1 << 16);
             const uint32_t p2 = bf16_pack2(r2, 0.0f);
-            const uint32_t xparts[4] = {(p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu, 0u, 0u};
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const uint32_t lw = bf16_pack2(lo[2 * w], lo[2 * w + 1]);
-                b1[t][w] = h ? lw : hb[w];
-                b2[t][w] = h ? xparts[w] : hb[w];
-            }
+            b1[t] = u32x4{h01, h23, l01, l23};
+            b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu};
         }
         // fetch the next chunk: rows into registers, A operands into registers then LDS
         u32x4 pre[4];
-        if (more) {
+        const int nx = more ? kc + 1 : kc;
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                if (valid[t]) {
-                    xn[t][0] = *reinterpret_cast<const float4 *>(xr[t] + (kc + 1) * 8);
-                    xn[t][1] = *reinterpret_cast<const float4 *>(xr[t] + (kc + 1) * 8 + 4);
-                }
-            }
+        for (int t = 0; t < 2; ++t) xn[t] = *reinterpret_cast<const float4 *>(xr[t] + nx * 8);
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int i = threadIdx.x + 256 * q;
-                if (i < chunk16) pre[q] = ag[(size_t)(kc + 1) * chunk16 + i];
-            }
+        for (int q = 0; q < 4; ++q) {
+            const int i = threadIdx.x + 256 * q;
+            pre[q] = ag[(size_t)nx * chunk16 + (i < chunk16 ? i : chunk16 - 1)];
         }
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -634,6 +619,8 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         }
         lds_barrier();
     }
+    x2[0] += __shfl_xor(x2[0], 32);  // both halves' shares of ||x||^2
+    x2[1] += __shfl_xor(x2[1], 32);
     // smallest and second smallest score of this wave's centroid tiles
     int m1[2], m2[2];
 #pragma unroll
