@@ -192,7 +192,7 @@ def test_mfma_path_equals_oracle_and_valu_path(ctx, metric, n, m, k, kind):
     elif kind == "grid":
         x = np.round(rng.standard_normal((n, dim))).astype(F)
         cb = np.round(rng.standard_normal((m, k, 8))).astype(F)
-    elif kind == "offset":  # far from the origin: the error bound is large, most pairs re-checked
+    elif kind == "offset":  # far from the origin: scored relative to the block's centre, so still few re-checks
         x = (1000 + rng.random((n, dim))).astype(F)
         cb = (1000 + rng.random((m, k, 8))).astype(F)
     elif kind == "same":
@@ -219,7 +219,7 @@ def test_mfma_path_equals_oracle_and_valu_path(ctx, metric, n, m, k, kind):
     ctx.set_assign_path(0)
     assert np.array_equal(valu, want)
     assert np.array_equal(got, want)
-    if kind in ("normal", "uniform") and k > 1:
+    if kind in ("normal", "uniform", "offset") and k > 1:
         assert frac < 0.05, frac  # the matrix-core pass decides almost every row itself
 
 
@@ -279,5 +279,5 @@ def test_wide_mfma_path_equals_oracle_and_valu_path(ctx, metric, n, m, sd, k, ki
     ctx.set_assign_path(0)
     assert np.array_equal(valu, want)
     assert np.array_equal(got, want)
-    if kind in ("normal", "uniform") and k > 1:
+    if kind in ("normal", "uniform", "offset") and k > 1:
         assert frac < 0.05, frac  # the matrix-core pass decides almost every row itself

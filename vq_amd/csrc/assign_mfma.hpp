@@ -83,6 +83,9 @@ __device__ __forceinline__ void top2_push4(int &m1, int &m2, int k0, int k1, int
 // the 2 x 17 addends.  Two candidates compared: below 2^-13.2 (||x||^2 + max ||c||^2); the test
 // uses 2^-13, plus 2^-14 |second| for the packed bits and the reference's own rounding.  bf16
 // keeps the fp32 exponent range, so no scaling is needed; non-finite values fail the test.
+// x and c here are the row and the centroid minus the block's centre mu (rounded to fp32): the
+// rounding of the two differences moves a squared distance by at most 2^-22 (||x||^2 + ||c||^2),
+// far inside the slack between 2^-13.2 and 2^-13, and the bound itself shrinks with the norms.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
@@ -94,7 +97,8 @@ constexpr int kStatStride = 32;
 struct MfmaBfTables {
     const u32x4 *atab;     // [m][nb][2][64]  A operands of the two instructions, lane order
     const float *c2perm;   // [m][nb][2][16]  ||c||^2 in accumulator order (kPadScore for padding)
-    const float *maxc2;    // [m]  largest ||c||^2 of the column block (NaN if any is NaN)
+    const float *maxc2;    // [m]  largest ||c - mu||^2 of the column block (NaN if any is NaN)
+    const float *mu;       // [m][8]  the block's centre: mean of its centroids
     uint32_t *stat;        // [kStatSlots * kStatStride]  pairs decided by the exact path (measurement)
     int nb;                // ceil(k/32)
 };
@@ -116,29 +120,48 @@ __device__ __forceinline__ uint32_t bf16_pack2(float a, float b) {
 }
 
 // Tables for k_assign_mfma_bf.  One workgroup per column block s, one thread per padded centroid
-// (k <= 256); maxc2[s] = largest ||c||^2 of the block (NaN if any is NaN).
+// (k <= 256).  Rows and centroids are scored relative to mu[s] = mean of the block's centroids
+// (distances do not change under a common shift, the bound on the score error, which is
+// proportional to ||x - mu||^2 + ||c - mu||^2, does); maxc2[s] = largest ||c - mu||^2 of the
+// block (NaN if any is NaN).
 static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__restrict__ cb, int m, int k, int nb,
                                                              u32x4 *__restrict__ atab, float *__restrict__ c2perm,
-                                                             float *__restrict__ maxc2, uint32_t *__restrict__ stat) {
+                                                             float *__restrict__ maxc2, float *__restrict__ mu,
+                                                             uint32_t *__restrict__ stat) {
     const int s = blockIdx.x, j = threadIdx.x;
     __shared__ float sh_max[4];
+    __shared__ float sh_mu[4][8];
     if (s == 0 && j < kStatSlots) stat[j * kStatStride] = 0u;
+    float c[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) c[t] = (j < k) ? cb[((size_t)s * k + j) * 8 + t] : 0.0f;
+    // centre: sum of c / 256 (no overflow for k <= 256), then * 256 / k
+    float centre[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        float v = c[t] * 0.00390625f;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+        if ((j & 63) == 0) sh_mu[j >> 6][t] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        centre[t] = (((sh_mu[0][t] + sh_mu[1][t]) + sh_mu[2][t]) + sh_mu[3][t]) * (256.0f / (float)k);
+        if (j == 0) mu[s * 8 + t] = centre[t];
+    }
     float mx = 0.0f;
     if (j < nb * 32) {
         const int b = j / 32, i = j % 32;
         float c2 = kPadScore;  // padding centroids: finite, so that index bits can be packed in
-        float c[8];
         if (j < k) {
             c2 = 0.0f;
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                c[t] = cb[((size_t)s * k + j) * 8 + t];
+                c[t] -= centre[t];
                 c2 = __builtin_fmaf(c[t], c[t], c2);
             }
             mx = c2;
-        } else {
-#pragma unroll
-            for (int t = 0; t < 8; ++t) c[t] = 0.0f;
         }
         uint32_t hb[8], lb[8];
 #pragma unroll
@@ -232,7 +255,7 @@ __device__ __forceinline__ int exact_argmin8_wave(const float (&xs)[8], const fl
 template <int METRIC, bool LBG, int TILES, int SG>
 __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
     constexpr int SD = 8;
-    extern __shared__ float lds_c2[];  // [SG][nb][2][16]
+    extern __shared__ float lds_c2[];  // [SG][nb][2][16], then the centres [SG][8]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int nb = tb.nb, m = a.m;
@@ -246,6 +269,8 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
     const int s0 = (int)(rem / 8u) * SG;
     const int64_t tile_id = (int64_t)chunk_id * 8 + (rem % 8u);
     for (int i = threadIdx.x; i < SG * nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s0 * nb * 32 + i];
+    float *lds_mu = lds_c2 + SG * nb * 32;
+    if (threadIdx.x < SG * 8) lds_mu[threadIdx.x] = tb.mu[(size_t)s0 * 8 + threadIdx.x];
     __syncthreads();
     const int64_t row_base = (tile_id * 4 + wave) * (32 * TILES);
     if (row_base >= a.n) return;
@@ -287,7 +312,9 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
         int m1[TILES], m2[TILES];
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
-            const float *xv = xall[t][q];
+            float xv[4];  // relative to the block's centre
+#pragma unroll
+            for (int u = 0; u < 4; ++u) xv[u] = xall[t][q][u] - lds_mu[q * 8 + 4 * h + u];
             float p = 0.0f;
 #pragma unroll
             for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
@@ -431,11 +458,16 @@ namespace vq {
 // in LDS once per workgroup, double-buffered; the rows and the next A chunk are fetched one chunk
 // ahead.  The two waves that share rows merge their (smallest, second smallest) through LDS.
 // Error of a score: 3 * 2^-16 (split, as above) + (34 * sd/8 + 16) * 2^-24 (fp32 accumulation of
-// 2 x 17 addends per chunk), per unit of ||x||^2 + ||c||^2; twice that for two candidates.
+// 2 x 17 addends per chunk) + 2^-22 (rounding of x - mu and c - mu), per unit of
+// ||x - mu||^2 + ||c - mu||^2; twice that for two candidates.
+constexpr int kWideCentreMax = 2048;  // widest column block whose centre is staged in LDS
+
 struct MfmaWideBfTables {
     const u32x4 *atab;     // [m][sd/8][nb][2][64]
     const float *c2perm;   // [m][nb][2][16]
-    const float *blockmax; // [m][nb]  largest ||c||^2 per block of 32 centroids (NaN if any is NaN)
+    const float *blockmax; // [m][nb]  largest ||c - mu||^2 per block of 32 centroids (NaN if any is NaN)
+    const float *mu;       // [m][sd]  centre of every column block: mean of its centroids
+    const int *shifted;    // [m]  0: the centre is not used
     uint32_t *list;
     uint32_t *list_count;
     int nb;
@@ -446,7 +478,61 @@ struct MfmaWideBfTables {
 // One workgroup per (column block s, block b of 32 centroids): thread (i, g) = (tid % 32, tid / 32)
 // writes the chunks kc = g, g + 8, ... of centroid 32 b + i and sums their share of ||c||^2; the
 // eight shares are added in g order.  blockmax[s][b] = largest ||c||^2 of the block (NaN stays).
-static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *__restrict__ cb, int m, int k, int nb,
+// mu[s][t] = mean over the k <= 256 centroids of column block s (sum of c / 256, then * 256 / k:
+// no overflow).  Rows and centroids are scored relative to it, as in k_mfma_bf_prep, when that
+// shrinks the norms the error bound is proportional to: k_mfma_wide_bf_prep sets shifted[s] = 0
+// and ignores the centre if ||mu||^2 is no more than a quarter of the mean ||c||^2 (or the block
+// is wider than kWideCentreMax), and the assignment kernel then skips the subtraction.  Grid (m, ceil(sd / 32)); thread (i, g) =
+// (tid % 32, tid / 32) adds the centroids g, g + 8, ... of dimension 32 y + i; norms[s][y] =
+// this slice's share of {||mu||^2, mean ||c||^2}.
+static __global__ void __launch_bounds__(256) k_block_centres(const float *__restrict__ cb, int k, int sd,
+                                                              float *__restrict__ mu, float2 *__restrict__ norms) {
+    const int s = blockIdx.x, y = blockIdx.y;
+    const int i = threadIdx.x & 31, g = threadIdx.x >> 5;
+    const int t = 32 * y + i;
+    __shared__ float part[2][8][32];
+    float acc = 0.0f, sq = 0.0f;
+    if (t < sd) {
+        const float *c = cb + (size_t)s * k * sd + t;
+        float v[32];  // k <= 256: all of the thread's loads are in flight together
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+            const int j = g + 8 * u;
+            v[u] = c[(size_t)(j < k ? j : 0) * sd];
+        }
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+            const float w = (g + 8 * u < k) ? v[u] * 0.00390625f : 0.0f;
+            acc += w;
+            sq = __builtin_fmaf(w, w, sq);
+        }
+    }
+    part[0][g][i] = acc;
+    part[1][g][i] = sq;
+    __syncthreads();
+    if (g == 0) {
+        float a = 0.0f, q = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            a += part[0][u][i];
+            q += part[1][u][i];
+        }
+        const float ctr = a * (256.0f / (float)k);
+        if (t < sd) mu[(size_t)s * sd + t] = ctr;
+        float mm = (t < sd) ? ctr * ctr : 0.0f, cc = q * (65536.0f / (float)k);
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) {
+            mm += __shfl_xor(mm, off);
+            cc += __shfl_xor(cc, off);
+        }
+        if (i == 0) norms[(size_t)s * gridDim.y + y] = make_float2(mm, cc);
+    }
+}
+
+static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *__restrict__ cb,
+                                                                  const float *__restrict__ mu,
+                                                                  const float2 *__restrict__ norms,
+                                                                  int *__restrict__ shifted, int m, int k, int nb,
                                                                   int sd, u32x4 *__restrict__ atab,
                                                                   float *__restrict__ c2perm,
                                                                   float *__restrict__ blockmax,
@@ -456,12 +542,27 @@ static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *_
     const int j = b * 32 + i;
     const int nkc = sd / 8;
     __shared__ float part[8][32];
+    // the same decision in every workgroup of the column block (same values, same order)
+    float mm = 0.0f, cc = 0.0f;
+    for (int y = 0; y < (sd + 31) / 32; ++y) {
+        const float2 v = norms[(size_t)s * ((sd + 31) / 32) + y];
+        mm += v.x;
+        cc += v.y;
+    }
+    const bool on = mm > 0.25f * cc && mm < 1e30f && sd <= kWideCentreMax;  // false for NaN
+    if (b == 0 && threadIdx.x == 0) shifted[s] = on ? 1 : 0;
     const float *c = cb + ((size_t)s * k + (j < k ? j : 0)) * sd;
     float p = 0.0f;
     for (int kc = g; kc < nkc; kc += 8) {
         const float4 v0 = *reinterpret_cast<const float4 *>(c + kc * 8);
         const float4 v1 = *reinterpret_cast<const float4 *>(c + kc * 8 + 4);
-        const float cv[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+        float4 u0 = make_float4(0.f, 0.f, 0.f, 0.f), u1 = u0;
+        if (on) {
+            u0 = *reinterpret_cast<const float4 *>(mu + (size_t)s * sd + kc * 8);
+            u1 = *reinterpret_cast<const float4 *>(mu + (size_t)s * sd + kc * 8 + 4);
+        }
+        const float cv[8] = {v0.x - u0.x, v0.y - u0.y, v0.z - u0.z, v0.w - u0.w,
+                             v1.x - u1.x, v1.y - u1.y, v1.z - u1.z, v1.w - u1.w};
         uint32_t hw[4], lw[4];  // packed pairs of the high and low parts
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
@@ -518,6 +619,7 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     constexpr int NBMAX = 8;
     __shared__ u32x4 lds_a[2][NBMAX * 128];  // 2 x 16 KB
     __shared__ float lds_c2[NBMAX * 32];
+    __shared__ float lds_mu[kWideCentreMax];
     __shared__ int lds_top[2][2][2][32];     // [row pair][row tile][m1 | m2][row] of the upper centroid half
     __shared__ uint32_t wg_list[128];
     __shared__ uint32_t wg_count, wg_base;
@@ -534,6 +636,8 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     for (int i = threadIdx.x; i < nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s * nb * 32 + i];
     for (int i = threadIdx.x; i < chunk16; i += 256) lds_a[0][i] = ag[i];
     if (threadIdx.x == 0) wg_count = 0;
+    if (tb.shifted[s] != 0)
+        for (int i = threadIdx.x; i < sd; i += 256) lds_mu[i] = tb.mu[(size_t)s * sd + i];
     __syncthreads();
 
     int64_t row[2];
@@ -545,6 +649,7 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         valid[t] = row[t] < a.n;
         xr[t] = a.x + (valid[t] ? row[t] : 0) * a.ld + (int64_t)s * sd + 4 * h;  // this half's 4 dimensions
     }
+    const bool shifted = tb.shifted[s] != 0;  // uniform
     floatx16 acc[2][4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -570,7 +675,14 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         u32x4 b1[2], b2[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const float xv[4] = {xn[t].x, xn[t].y, xn[t].z, xn[t].w};
+            float xv[4] = {xn[t].x, xn[t].y, xn[t].z, xn[t].w};
+            if (shifted) {
+                const float4 mn = *reinterpret_cast<const float4 *>(lds_mu + kc * 8 + 4 * h);
+                xv[0] -= mn.x;
+                xv[1] -= mn.y;
+                xv[2] -= mn.z;
+                xv[3] -= mn.w;
+            }
             float p = 0.0f;
 #pragma unroll
             for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);

@@ -110,22 +110,23 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
     const int nb = (a.k + 31) / 32;
     // A operands: 2 x 64 lanes x 16 bytes per (s, block of 32 centroids)
     const size_t n_atab = (size_t)a.m * nb * 512, n_c2 = (size_t)a.m * nb * 32;
-    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + a.m) + 64));
+    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + 9 * (size_t)a.m) + 64));
     VQ_TRY(ensure(ctx, ctx->mfma_stat, sizeof(uint32_t) * vq::kStatSlots * vq::kStatStride));
     float *atab = (float *)ctx->mfma_tab.p;
     float *c2perm = atab + n_atab;
     float *maxc2 = c2perm + n_c2;
+    float *mu = maxc2 + a.m;
     uint32_t *stat = (uint32_t *)ctx->mfma_stat.p;
     constexpr int TILES = VQ_MFMA_TILES;
     hipLaunchKernelGGL(vq::k_mfma_bf_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb,
-                       (vq::u32x4 *)atab, c2perm, maxc2, stat);
-    vq::MfmaBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, stat, nb};
+                       (vq::u32x4 *)atab, c2perm, maxc2, mu, stat);
+    vq::MfmaBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, mu, stat, nb};
     // 4 column blocks of 8 floats = one 128-byte line per row
     constexpr int SG = VQ_MFMA_SG;
     const bool grouped = a.m % SG == 0;
     auto kern = grouped ? vq::k_assign_mfma_bf<METRIC, LBG, TILES, SG> : vq::k_assign_mfma_bf<METRIC, LBG, TILES, 1>;
     const int sg = grouped ? SG : 1;
-    const size_t lds = sizeof(float) * sg * nb * 32;
+    const size_t lds = sizeof(float) * sg * (nb * 32 + 8);
     const int64_t blocks = cdiv(cdiv(a.n, 4 * 32 * TILES), 8) * 8 * (a.m / sg);  // tiles in chunks of 8
     if (blocks >= (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * m too large for one launch");
     {
@@ -167,20 +168,26 @@ int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const ui
 // cores with split operands, undecided pairs listed for the exact kernel.
 template <int METRIC, bool LBG>
 int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
-    const int nb = (a.k + 31) / 32, nkc = sd / 8;
+    const int nb = (a.k + 31) / 32, nkc = sd / 8, nsl = (sd + 31) / 32;
     const size_t n_atab = (size_t)a.m * nkc * nb * 128 * 4, n_c2 = (size_t)a.m * nb * 32;  // floats
-    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + (size_t)a.m * nb) + 64));
+    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + (size_t)a.m * nb + (size_t)a.m * sd + a.m + 2 * (size_t)a.m * nsl + 8) + 64));
     VQ_TRY(ensure(ctx, ctx->mfma_list, sizeof(uint32_t) * ((size_t)a.n * a.m + 4)));
     float *atab = (float *)ctx->mfma_tab.p;
     float *c2perm = atab + n_atab;
     float *maxc2 = c2perm + n_c2;  // per block of 32 centroids
+    float *mu = maxc2 + (((size_t)a.m * nb + 3) & ~(size_t)3);  // 16-byte aligned: read as float4
     uint32_t *count = (uint32_t *)ctx->mfma_list.p;
     uint32_t *list = count + 4;
-    hipLaunchKernelGGL(vq::k_mfma_wide_bf_prep, dim3(a.m, nb), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, sd,
+    float2 *norms = (float2 *)(mu + (size_t)a.m * sd);  // sd is a multiple of 8: 8-byte aligned
+    int *shifted = (int *)(norms + (size_t)a.m * nsl);
+    hipLaunchKernelGGL(vq::k_block_centres, dim3(a.m, nsl), dim3(256), 0, ctx->stream, a.cb, a.k, sd, mu, norms);
+    hipLaunchKernelGGL(vq::k_mfma_wide_bf_prep, dim3(a.m, nb), dim3(256), 0, ctx->stream, a.cb, mu, norms, shifted,
+                       a.m, a.k, nb, sd,
                        (vq::u32x4 *)atab, c2perm, maxc2, count);
-    // two candidates, each: operand split 3 * 2^-16, fp32 accumulation (34 per chunk + 16) * 2^-24
-    const float kappa = 2.0f * (3.0f * 1.52587890625e-05f + (34.0f * nkc + 16.0f) * 5.9604644775390625e-08f);
-    vq::MfmaWideBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, list, count, nb, sd, kappa};
+    // two candidates, each: operand split 3 * 2^-16, fp32 accumulation (34 per chunk + 16) * 2^-24,
+    // rounding of the differences from the centre 2^-22
+    const float kappa = 2.0f * (3.0f * 1.52587890625e-05f + (34.0f * nkc + 16.0f + 4.0f) * 5.9604644775390625e-08f);
+    vq::MfmaWideBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, mu, shifted, list, count, nb, sd, kappa};
     {
         ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
         hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0,
