@@ -100,7 +100,7 @@ struct MfmaBfTables {
     const float *maxc2;    // [m]  largest ||c - mu||^2 of the column block (NaN if any is NaN)
     const float *mu;       // [m][8]  the block's centre: mean of its centroids
     uint32_t *stat;        // [kStatSlots * kStatStride]  pairs decided by the exact path (measurement)
-    int nb;                // ceil(k/32)
+    int nb;                // blocks of 32 centroids, padded to an even number
 };
 
 // float -> bf16 bits, round to nearest even (NaN stays NaN).
@@ -255,7 +255,7 @@ __device__ __forceinline__ int exact_argmin8_wave(const float (&xs)[8], const fl
 template <int METRIC, bool LBG, int TILES, int SG>
 __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
     constexpr int SD = 8;
-    extern __shared__ float lds_c2[];  // [SG][nb][2][16], then the centres [SG][8]
+    extern __shared__ __attribute__((aligned(16))) float lds_c2[];  // [SG][nb][2][16], the centres [SG][8], maxc2 [SG]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int nb = tb.nb, m = a.m;
@@ -271,47 +271,52 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
     for (int i = threadIdx.x; i < SG * nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s0 * nb * 32 + i];
     float *lds_mu = lds_c2 + SG * nb * 32;
     if (threadIdx.x < SG * 8) lds_mu[threadIdx.x] = tb.mu[(size_t)s0 * 8 + threadIdx.x];
+    if (threadIdx.x < SG) lds_mu[SG * 8 + threadIdx.x] = tb.maxc2[s0 + threadIdx.x];
+    // LBG: the blocks that have converged, read once (the same in every lane)
+    bool skip[SG];
+#pragma unroll
+    for (int q = 0; q < SG; ++q) skip[q] = LBG ? __builtin_amdgcn_readfirstlane(a.done[s0 + q]) != 0 : false;
     __syncthreads();
     const int64_t row_base = (tile_id * 4 + wave) * (32 * TILES);
     if (row_base >= a.n) return;
 
     float xall[TILES][SG][4];  // this lane's dimensions [4h, 4h + 4) of every block
-    uint8_t old[TILES][SG];
     uint32_t cw[TILES];
     uint32_t n_exact = 0;
+    uint32_t chg = 0;  // LBG: bit q set when a code of block s0 + q changed in this lane
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
         const int64_t row = row_base + 32 * t + r;
         cw[t] = 0u;
-        if (row < a.n) {
-            const float *xr = a.x + row * a.ld + (int64_t)s0 * SD + 4 * h;
+        // Unconditional loads (a row past the end reads row 0 and is never stored): loads under a
+        // branch make the compiler wait for every load in flight at each use.
+        const int64_t rc = row < a.n ? row : 0;
+        const float *xr = a.x + rc * a.ld + (int64_t)s0 * SD + 4 * h;
 #pragma unroll
-            for (int q = 0; q < SG; ++q)
+        for (int q = 0; q < SG; ++q)
 #pragma unroll
-                for (int u = 0; u < 4; ++u) xall[t][q][u] = xr[q * SD + u];
-        } else {
-#pragma unroll
-            for (int q = 0; q < SG; ++q)
-#pragma unroll
-                for (int u = 0; u < 4; ++u) xall[t][q][u] = 0.0f;
-        }
-        if constexpr (LBG) {
-#pragma unroll
-            for (int q = 0; q < SG; ++q)
-                old[t][q] = (row < a.n && h == 0) ? a.codes[(size_t)(s0 + q) * a.n + row] : (uint8_t)0;
-        }
+            for (int u = 0; u < 4; ++u) xall[t][q][u] = xr[q * SD + u];
     }
+    const u32x4 *ap = tb.atab + (size_t)s0 * nb * 128 + lane;
+    u32x4 pa1, pa2, qa1, qa2;
+    bool primed = false;
 #pragma unroll
     for (int q = 0; q < SG; ++q) {
         const int s = s0 + q;
-        if constexpr (LBG) {
-            if (a.done[s]) continue;
+        if (skip[q]) {
+            primed = false;
+            continue;
         }
         u32x4 b1[TILES], b2[TILES];
         float x2[TILES];
         int m1[TILES], m2[TILES];
+        uint8_t old[TILES];  // LBG: the rows' current codes, in flight while the block is scored
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
+            if constexpr (LBG) {
+                const int64_t row = row_base + 32 * t + r;
+                old[t] = a.codes[(size_t)s * a.n + (row < a.n ? row : 0)];
+            }
             float xv[4];  // relative to the block's centre
 #pragma unroll
             for (int u = 0; u < 4; ++u) xv[u] = xall[t][q][u] - lds_mu[q * 8 + 4 * h + u];
@@ -333,7 +338,6 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
             m1[t] = 0x7f800000;  // +inf
             m2[t] = 0x7f800000;
         }
-        const u32x4 *ap = tb.atab + (size_t)s * nb * 128 + lane;
         const float *cp = lds_c2 + ((size_t)q * nb * 2 + h) * 16;
         // One block of 32 centroids against the TILES row tiles.  The packed index leaves out the
         // lane half (bit 2), so it is the same in every lane and lives in scalar registers.
@@ -357,27 +361,27 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
                     top2_push4(m1[t], m2[t], key[v], key[v + 1], key[v + 2], key[v + 3]);
             }
         };
-        // A operands of the next block are fetched while the current one is scored (two buffers)
-        u32x4 pa1 = ap[0], pa2 = ap[64], qa1 = pa1, qa2 = pa2;
-        if (nb > 1) {
-            qa1 = ap[128];
-            qa2 = ap[128 + 64];
+        // The A operands of the SG column blocks are one run of SG * nb blocks (nb is even): two
+        // buffers, each refilled two blocks ahead as soon as its block is scored, so the first
+        // blocks of the next column block arrive while this one's rows are decided.
+        const int fb = q * nb;
+        if (!primed) {
+            pa1 = ap[(size_t)fb * 128];
+            pa2 = ap[(size_t)fb * 128 + 64];
+            qa1 = ap[(size_t)(fb + 1) * 128];
+            qa2 = ap[(size_t)(fb + 1) * 128 + 64];
+            primed = true;
         }
         for (int b = 0; b < nb; b += 2) {
             block(b, pa1, pa2);
-            if (b + 2 < nb) {
-                pa1 = ap[(size_t)(b + 2) * 128];
-                pa2 = ap[(size_t)(b + 2) * 128 + 64];
-            }
-            if (b + 1 < nb) {
-                block(b + 1, qa1, qa2);
-                if (b + 3 < nb) {
-                    qa1 = ap[(size_t)(b + 3) * 128];
-                    qa2 = ap[(size_t)(b + 3) * 128 + 64];
-                }
-            }
+            const int f2 = fb + b + 2 < SG * nb ? fb + b + 2 : SG * nb - 2;  // past the end: any valid block
+            pa1 = ap[(size_t)f2 * 128];
+            pa2 = ap[(size_t)f2 * 128 + 64];
+            block(b + 1, qa1, qa2);
+            qa1 = ap[(size_t)(f2 + 1) * 128];
+            qa2 = ap[(size_t)(f2 + 1) * 128 + 64];
         }
-        const float mc2 = tb.maxc2[s];
+        const float mc2 = lds_mu[SG * 8 + q];
         const float *cb_s = a.cb + (size_t)s * a.k * SD;
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
@@ -399,21 +403,20 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
             n_exact += (uint32_t)__popcll(todo);
             while (todo) {
                 const int src = __builtin_amdgcn_readfirstlane(__ffsll(todo) - 1);
-                float xs[SD];  // the row's 8 floats: dimensions 0-3 from lane src, 4-7 from lane src + 32
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    xs[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xall[t][q][u]), src));
-                    xs[4 + u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xall[t][q][u]), src + 32));
-                }
+                // the row's 8 floats, read again (same address in every lane) rather than kept in
+                // registers through the scoring of every block for this rare path
+                const float4 *xp = reinterpret_cast<const float4 *>(a.x + (row_base + 32 * t + src) * a.ld + (int64_t)s * SD);
+                const float4 xa = xp[0], xb = xp[1];
+                const float xs[SD] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
                 const int best = exact_argmin8_wave<METRIC>(xs, cb_s, a.k, lane);
                 if (lane == src) code = best;
                 todo &= todo - 1;
             }
             if (mine) {
                 if constexpr (LBG) {
-                    if (old[t][q] != (uint8_t)code) {
+                    if (old[t] != (uint8_t)code) {
                         a.codes[(size_t)s * a.n + row] = (uint8_t)code;
-                        mark_changed(a.changed + s);
+                        chg |= 1u << q;
                     }
                 } else if (SG == 4 || SG == 2) {
                     cw[t] |= (uint32_t)code << (8 * q);
@@ -435,6 +438,22 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
                         *reinterpret_cast<uint16_t *>(a.codes + row * m + s0) = (uint16_t)cw[t];
                 }
             }
+        }
+    }
+    if constexpr (LBG) {
+        // changed[s]: one lane per wave, once per wave, and only where the flag still reads 0 (every
+        // store to one address is serialised in its L2 channel; a stale 0 from the vector cache
+        // costs a store, nothing else).  The flags are read together: one memory round trip.
+        uint32_t any = 0;
+#pragma unroll
+        for (int q = 0; q < SG; ++q) any |= __any((chg >> q) & 1u) ? (1u << q) : 0u;
+        if (lane == 0 && any) {
+            int cur[SG];
+#pragma unroll
+            for (int q = 0; q < SG; ++q) cur[q] = a.changed[s0 + q];
+#pragma unroll
+            for (int q = 0; q < SG; ++q)
+                if (((any >> q) & 1u) && cur[q] == 0) a.changed[s0 + q] = 1;
         }
     }
     if (lane == 0 && n_exact)

@@ -107,7 +107,7 @@ int32_t launch_assign_m(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
 // same kernel by the reference-order argmin (assign_mfma.hpp).
 template <int METRIC, bool LBG>
 int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
-    const int nb = (a.k + 31) / 32;
+    const int nb = 2 * ((a.k + 63) / 64);  // blocks of 32 centroids, an even number (the kernel scores them in pairs)
     // A operands: 2 x 64 lanes x 16 bytes per (s, block of 32 centroids)
     const size_t n_atab = (size_t)a.m * nb * 512, n_c2 = (size_t)a.m * nb * 32;
     VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + 9 * (size_t)a.m) + 64));
@@ -126,7 +126,7 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
     const bool grouped = a.m % SG == 0;
     auto kern = grouped ? vq::k_assign_mfma_bf<METRIC, LBG, TILES, SG> : vq::k_assign_mfma_bf<METRIC, LBG, TILES, 1>;
     const int sg = grouped ? SG : 1;
-    const size_t lds = sizeof(float) * sg * (nb * 32 + 8);
+    const size_t lds = sizeof(float) * sg * (nb * 32 + 9);
     const int64_t blocks = cdiv(cdiv(a.n, 4 * 32 * TILES), 8) * 8 * (a.m / sg);  // tiles in chunks of 8
     if (blocks >= (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * m too large for one launch");
     {
