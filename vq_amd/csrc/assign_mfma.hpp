@@ -58,6 +58,15 @@ __device__ __forceinline__ int pack_tag(float score, uint32_t keep, uint32_t tag
     return (int)((__float_as_uint(score) & keep) | tag);
 }
 
+// The values of lanes l and l ^ 32 in one vector instruction (v_permlane32_swap: the upper half of
+// the first operand and the lower half of the second change places).  Lanes below 32 get
+// (own, partner), the others (partner, own): for symmetric uses only.
+__device__ __forceinline__ void swap_halves(int v, int &a, int &b) {
+    const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    a = (int)r[0];
+    b = (int)r[1];
+}
+
 // Four new keys into the running (smallest, second smallest): 5 operations.
 // second smallest of {m1, m2, x, y} with m1 <= m2 is min(m2, med3(m1, x, y)).
 __device__ __forceinline__ void top2_push4(int &m1, int &m2, int k0, int k1, int k2, int k3) {
@@ -334,7 +343,9 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
             const uint32_t p2 = bf16_pack2(r2, 0.0f);
             b1[t] = u32x4{h01, h23, l01, l23};
             b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu};
-            x2[t] = p + __shfl_xor(p, 32);
+            int pa, pb;
+            swap_halves(__float_as_int(p), pa, pb);
+            x2[t] = __int_as_float(pa) + __int_as_float(pb);  // lower half's share + upper half's, in both
             m1[t] = 0x7f800000;  // +inf
             m2[t] = 0x7f800000;
         }
@@ -388,9 +399,11 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
             // the partner lane (other half) saw the other 16 centroids of every block
             m1[t] |= 4 * h;  // bit 2 of the centroid index: the lane half
             m2[t] |= 4 * h;
-            int o1 = __shfl_xor(m1[t], 32), o2 = __shfl_xor(m2[t], 32);
-            const float s1 = __int_as_float(imin(m1[t], o1));
-            const float s2 = __int_as_float(imin(imax(m1[t], o1), imin(m2[t], o2)));
+            int f1, g1, f2, g2;
+            swap_halves(m1[t], f1, g1);
+            swap_halves(m2[t], f2, g2);
+            const float s1 = __int_as_float(imin(f1, g1));
+            const float s2 = __int_as_float(imin(imax(f1, g1), imin(f2, g2)));
             const int64_t row = row_base + 32 * t + r;
             const bool mine = h == 0 && row < a.n;
             const float bound = x2[t] + mc2;
