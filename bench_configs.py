@@ -67,6 +67,9 @@ def main():
         enc()
         out["c4_rvq_encode_ms"] = timed(enc)
         out["c4_recheck_fraction_last_stage"] = ctx.last_recheck_count() / n
+        allc, two = ctx.last_recheck_split()
+        out["c4_recheck_all_centroids_fraction"] = allc / n
+        out["c4_recheck_two_candidates_fraction"] = two / n
         one = lambda: ctx.assign(vq_amd.EUCLIDEAN, dx, n, dim, 1, dim, k, dcb.ptr, dcodes)
         ctx.set_assign_path(1)
         one()

@@ -72,6 +72,9 @@ int32_t vq_ctx_set_assign_path(vq_ctx *ctx, int32_t path);
 /* Number of (row, block) pairs the most recent matrix-core assignment pass left to the exact
  * re-check (0 if that path has not run).  Synchronises.  Measurement only. */
 int32_t vq_ctx_last_recheck_count(vq_ctx *ctx, uint32_t *h_count);
+/* The same count split by how the pair was decided: by the reference-order scan over all
+ * centroids, or (wide column blocks only) between the two best-scored candidates. */
+int32_t vq_ctx_last_recheck_split(vq_ctx *ctx, uint32_t *h_all_centroids, uint32_t *h_two_candidates);
 
 int32_t vq_malloc(vq_ctx *ctx, size_t bytes, void **d_ptr);
 int32_t vq_free(vq_ctx *ctx, void *d_ptr);

@@ -28,6 +28,7 @@ SYMBOLS = {
     "vq_ctx_stream": (_vp, [_vp]),
     "vq_ctx_set_assign_path": (_i32, [_vp, _i32]),
     "vq_ctx_last_recheck_count": (_i32, [_vp, C.POINTER(C.c_uint32)]),
+    "vq_ctx_last_recheck_split": (_i32, [_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "vq_malloc": (_i32, [_vp, _sz, C.POINTER(_vp)]),
     "vq_free": (_i32, [_vp, _vp]),
     "vq_h2d": (_i32, [_vp, _vp, _vp, _sz]),
@@ -195,6 +196,12 @@ class Context:
         c = C.c_uint32(0)
         self._check(_lib.vq_ctx_last_recheck_count(self._h, C.byref(c)))
         return c.value
+
+    def last_recheck_split(self):
+        """(pairs decided over all centroids, pairs decided between two candidates)."""
+        a, b = C.c_uint32(0), C.c_uint32(0)
+        self._check(_lib.vq_ctx_last_recheck_split(self._h, C.byref(a), C.byref(b)))
+        return a.value, b.value
 
     def sync(self):
         self._check(_lib.vq_ctx_sync(self._h))

@@ -391,19 +391,19 @@ __device__ __forceinline__ void wide_step(float &acc, float xv, float cv) {
 
 // Distances of the wave's rows (in lds_x, row stride sd) to the centroids of block s, then the
 // reference argmin per row.  rows[i] < 0 marks an unused slot.  Lane 0 returns the codes.
-template <int METRIC, bool VEC>
+template <int METRIC, bool VEC, int NR>
 __device__ __forceinline__ void wide_argmin(const AssignArgs &a, int sd, int s, const float *lds_x, int lane,
-                                            int (&best_out)[kWideRows]) {
+                                            int (&best_out)[NR]) {
     const int k = a.k;
     const float *__restrict__ cb = a.cb + (size_t)s * k * sd;
-    float acc[4][kWideRows];
-    float sa[kWideRows];
+    float acc[4][NR];
+    float sa[NR];
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int i = 0; i < kWideRows; ++i) acc[q][i] = 0.0f;
+        for (int i = 0; i < NR; ++i) acc[q][i] = 0.0f;
 #pragma unroll
-    for (int i = 0; i < kWideRows; ++i) sa[i] = 0.0f;
+    for (int i = 0; i < NR; ++i) sa[i] = 0.0f;
     const float *cq[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
@@ -417,7 +417,7 @@ __device__ __forceinline__ void wide_argmin(const AssignArgs &a, int sd, int s, 
 #pragma unroll
             for (int q = 0; q < 4; ++q) cv[q] = *reinterpret_cast<const float4 *>(cq[q] + t);
 #pragma unroll
-            for (int i = 0; i < kWideRows; ++i) {
+            for (int i = 0; i < NR; ++i) {
                 const float4 xv = *reinterpret_cast<const float4 *>(lds_x + i * sd + t);
                 if constexpr (METRIC == M_COS) {
                     float p;
@@ -441,7 +441,7 @@ __device__ __forceinline__ void wide_argmin(const AssignArgs &a, int sd, int s, 
 #pragma unroll
         for (int q = 0; q < 4; ++q) cv[q] = cq[q][t];
 #pragma unroll
-        for (int i = 0; i < kWideRows; ++i) {
+        for (int i = 0; i < NR; ++i) {
             const float xv = lds_x[i * sd + t];
             if constexpr (METRIC == M_COS) {
                 float p = xv * xv;
@@ -453,7 +453,7 @@ __device__ __forceinline__ void wide_argmin(const AssignArgs &a, int sd, int s, 
     }
     const float inf = __builtin_inff();
 #pragma unroll
-    for (int i = 0; i < kWideRows; ++i) {
+    for (int i = 0; i < NR; ++i) {
         float bd = inf, d0 = 0.0f;
         int bi = 0x7fffffff;
         float dq[4];
@@ -510,20 +510,17 @@ __device__ __forceinline__ void wide_argmin(const AssignArgs &a, int sd, int s, 
     }
 }
 
-template <int METRIC, bool LBG, bool LISTED, bool VEC>
-__global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd, const uint32_t *__restrict__ list,
-                                                           const uint32_t *__restrict__ list_count) {
-    extern __shared__ float lds_wide[];  // 4 waves x 8 rows x sd
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    float *lds_x = lds_wide + (size_t)wave * kWideRows * sd;
-    const int64_t total = LISTED ? (int64_t)*list_count : a.n;
-    const int64_t groups = (total + kWideRows - 1) / kWideRows;
+// The wave's share of the groups of NR rows (or listed pairs).
+template <int METRIC, bool LBG, bool LISTED, bool VEC, int NR>
+__device__ __forceinline__ void wide_exact_groups(const AssignArgs &a, int sd, const uint32_t *__restrict__ list,
+                                                  int64_t total, float *lds_x, int lane, int wave) {
+    const int64_t groups = (total + NR - 1) / NR;
     for (int64_t grp = (int64_t)blockIdx.x * 4 + wave; grp < groups; grp += (int64_t)gridDim.x * 4) {
-        int64_t rows[kWideRows];
-        int ss[kWideRows];
+        int64_t rows[NR];
+        int ss[NR];
 #pragma unroll
-        for (int i = 0; i < kWideRows; ++i) {
-            const int64_t e = grp * kWideRows + i;
+        for (int i = 0; i < NR; ++i) {
+            const int64_t e = grp * NR + i;
             rows[i] = -1;
             ss[i] = LISTED ? -1 : (int)blockIdx.y;
             if (e < total) {
@@ -536,37 +533,34 @@ __global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd,
                 }
             }
         }
-        if constexpr (LBG && !LISTED) {
-            if (a.done[blockIdx.y]) return;
-        }
         // sub-groups of slots that share the column block (always one group when not LISTED)
-        bool pending[kWideRows];
+        bool pending[NR];
 #pragma unroll
-        for (int i = 0; i < kWideRows; ++i) pending[i] = rows[i] >= 0;
+        for (int i = 0; i < NR; ++i) pending[i] = rows[i] >= 0;
         for (;;) {
             int s = -1;
 #pragma unroll
-            for (int i = kWideRows - 1; i >= 0; --i)
+            for (int i = NR - 1; i >= 0; --i)
                 if (pending[i]) s = ss[i];
             if (s < 0) break;
             // stage the rows of this sub-group (unused slots repeat a valid row)
             int64_t fill = -1;
 #pragma unroll
-            for (int i = 0; i < kWideRows; ++i)
+            for (int i = 0; i < NR; ++i)
                 if (pending[i] && ss[i] == s && fill < 0) fill = rows[i];
 #pragma unroll
-            for (int i = 0; i < kWideRows; ++i) {
+            for (int i = 0; i < NR; ++i) {
                 const int64_t rr = (pending[i] && ss[i] == s) ? rows[i] : fill;
                 const float *xr = a.x + rr * a.ld + (int64_t)s * sd;
                 for (int t = lane; t < sd; t += 64) lds_x[i * sd + t] = xr[t];
             }
             __builtin_amdgcn_wave_barrier();
-            int best[kWideRows];
-            wide_argmin<METRIC, VEC>(a, sd, s, lds_x, lane, best);
+            int best[NR];
+            wide_argmin<METRIC, VEC, NR>(a, sd, s, lds_x, lane, best);
             __builtin_amdgcn_wave_barrier();
             if (lane == 0) {
 #pragma unroll
-                for (int i = 0; i < kWideRows; ++i) {
+                for (int i = 0; i < NR; ++i) {
                     if (pending[i] && ss[i] == s) {
                         if constexpr (LBG) {
                             uint8_t *p = a.codes + (size_t)s * a.n + rows[i];
@@ -581,8 +575,79 @@ __global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd,
                 }
             }
 #pragma unroll
-            for (int i = 0; i < kWideRows; ++i)
+            for (int i = 0; i < NR; ++i)
                 if (ss[i] == s) pending[i] = false;
+        }
+    }
+}
+
+template <int METRIC, bool LBG, bool LISTED, bool VEC>
+__global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd, const uint32_t *__restrict__ list,
+                                                           const uint32_t *__restrict__ list_count) {
+    extern __shared__ float lds_wide[];  // 4 waves x 8 rows x sd
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float *lds_x = lds_wide + (size_t)wave * kWideRows * sd;
+    const int64_t total = LISTED ? (int64_t)*list_count : a.n;
+    if constexpr (LBG && !LISTED) {
+        if (a.done[blockIdx.y]) return;
+    }
+    if constexpr (LISTED) {
+        // a short list: one pair per wave, so that the pass is as long as one pair's scan, not eight
+        if (total <= (int64_t)gridDim.x * 4) {
+            wide_exact_groups<METRIC, LBG, LISTED, VEC, 1>(a, sd, list, total, lds_x, lane, wave);
+            return;
+        }
+    }
+    wide_exact_groups<METRIC, LBG, LISTED, VEC, kWideRows>(a, sd, list, total, lds_x, lane, wave);
+}
+
+// Exact decision between two candidate centroids per listed (row, column block) pair — the
+// pairs the matrix-core pass narrowed down to its two best scores.  Lanes 2i and 2i + 1 take
+// candidates c1 and c2 of entry i: each accumulates its distance in the reference's order
+// (sequential over the sub-vector), then the smaller (distance, index) wins, which is the
+// reference's strict '<' scan restricted to the only two centroids that can win it.  Euclidean
+// compares the roots, as the reference does.  Requires sd % 4 == 0 and 16-byte aligned rows
+// and centroids.
+template <int METRIC, bool LBG>
+__global__ void __launch_bounds__(256) k_assign_wide_pair(AssignArgs a, int sd, const uint2 *__restrict__ pairs,
+                                                          const uint32_t *__restrict__ pair_count) {
+    const uint32_t total = *pair_count;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float inf = __builtin_inff();
+    for (uint64_t base = ((uint64_t)blockIdx.x * 4 + wave) * 32; base < total; base += (uint64_t)gridDim.x * 4 * 32) {
+        const uint64_t e = base + (lane >> 1);
+        const bool active = e < total;
+        const uint2 ent = pairs[active ? e : base];
+        const int64_t row = ent.x / (uint32_t)a.m;
+        const int s = (int)(ent.x % (uint32_t)a.m);
+        const int j = (int)((ent.y >> (8 * (lane & 1))) & 0xFFu);
+        const float4 *xp = reinterpret_cast<const float4 *>(a.x + row * a.ld + (int64_t)s * sd);
+        const float4 *cp = reinterpret_cast<const float4 *>(a.cb + ((size_t)s * a.k + j) * sd);
+        float acc = 0.0f;
+#pragma unroll 4
+        for (int t = 0; t < sd / 4; ++t) {
+            const float4 xv = xp[t], cv = cp[t];
+            wide_step<METRIC>(acc, xv.x, cv.x);
+            wide_step<METRIC>(acc, xv.y, cv.y);
+            wide_step<METRIC>(acc, xv.z, cv.z);
+            wide_step<METRIC>(acc, xv.w, cv.w);
+        }
+        float d = acc;
+        if constexpr (METRIC == M_EUCLID) d = sqrtf(d);
+        d = (d == d) ? d : inf;
+        const float od = __shfl_xor(d, 1);
+        const int oj = __shfl_xor(j, 1);
+        const int best = (od < d || (od == d && oj < j)) ? oj : j;
+        if (active && (lane & 1) == 0) {
+            if constexpr (LBG) {
+                uint8_t *p = a.codes + (size_t)s * a.n + row;
+                if (*p != (uint8_t)best) {
+                    *p = (uint8_t)best;
+                    mark_changed(a.changed + s);
+                }
+            } else {
+                a.codes[row * a.m + s] = (uint8_t)best;
+            }
         }
     }
 }

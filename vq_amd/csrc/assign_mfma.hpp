@@ -500,8 +500,9 @@ struct MfmaWideBfTables {
     const float *blockmax; // [m][nb]  largest ||c - mu||^2 per block of 32 centroids (NaN if any is NaN)
     const float *mu;       // [m][sd]  centre of every column block: mean of its centroids
     const int *shifted;    // [m]  0: the centre is not used
-    uint32_t *list;
-    uint32_t *list_count;
+    uint32_t *list;        // undecided pairs (row * m + s) for the exact kernel over all centroids
+    uint32_t *list_count;  // [0] entries of list, [1] entries of pairs
+    uint2 *pairs;          // undecided pairs with only two candidates: {row * m + s, c1 | c2 << 8}
     int nb;
     int sd;
     float kappa;           // error-bound coefficient on (||x||^2 + max ||c||^2)
@@ -637,7 +638,7 @@ static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *_
             mx = (mx == mx && o == o) ? fmaxf(mx, o) : __builtin_nanf("");
         }
         if (i == 0) blockmax[(size_t)s * nb + b] = mx;
-        if (s == 0 && b == 0 && i == 0) *list_count = 0;
+        if (s == 0 && b == 0 && i < 2) list_count[i] = 0;
     }
 }
 
@@ -652,9 +653,10 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     __shared__ u32x4 lds_a[2][NBMAX * 128];  // 2 x 16 KB
     __shared__ float lds_c2[NBMAX * 32];
     __shared__ float lds_mu[kWideCentreMax];
-    __shared__ int lds_top[2][2][2][32];     // [row pair][row tile][m1 | m2][row] of the upper centroid half
+    __shared__ int lds_top[2][2][3][32];     // [row pair][row tile][m1 | m2 | m3][row] of the upper centroid half
     __shared__ uint32_t wg_list[128];
-    __shared__ uint32_t wg_count, wg_base;
+    __shared__ uint2 wg_pairs[128];
+    __shared__ uint32_t wg_count, wg_base, wg_pcount, wg_pbase;
     const int s = blockIdx.y;
     if constexpr (LBG) {
         if (a.done[s]) return;
@@ -667,7 +669,10 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     const int chunk16 = nb * 128;  // 16-byte pieces per chunk
     for (int i = threadIdx.x; i < nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s * nb * 32 + i];
     for (int i = threadIdx.x; i < chunk16; i += 256) lds_a[0][i] = ag[i];
-    if (threadIdx.x == 0) wg_count = 0;
+    if (threadIdx.x == 0) {
+        wg_count = 0;
+        wg_pcount = 0;
+    }
     if (tb.shifted[s] != 0)
         for (int i = threadIdx.x; i < sd; i += 256) lds_mu[i] = tb.mu[(size_t)s * sd + i];
     __syncthreads();
@@ -765,12 +770,18 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     }
     x2[0] += __shfl_xor(x2[0], 32);  // both halves' shares of ||x||^2
     x2[1] += __shfl_xor(x2[1], 32);
-    // smallest and second smallest score of this wave's centroid tiles
-    int m1[2], m2[2];
+    // the three smallest scores of this wave's centroid tiles (index in the low 8 bits)
+    auto push = [](int &m1, int &m2, int &m3, int key) {
+        m3 = imed3(m2, m3, key);
+        m2 = imed3(m1, m2, key);
+        m1 = imin(m1, key);
+    };
+    int m1[2], m2[2], m3[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         m1[t] = 0x7f800000;
         m2[t] = 0x7f800000;
+        m3[t] = 0x7f800000;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const int b = 4 * ch + c;
@@ -778,22 +789,21 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const uint32_t idx = (uint32_t)(32 * b + 8 * (v / 4) + 4 * h + v % 4);
-                    const int key = (int)((__float_as_uint(acc[t][c][v]) & 0xFFFFFF00u) | idx);
-                    m2[t] = imed3(m1[t], m2[t], key);
-                    m1[t] = imin(m1[t], key);
+                    push(m1[t], m2[t], m3[t], (int)((__float_as_uint(acc[t][c][v]) & 0xFFFFFF00u) | idx));
                 }
             }
         }
-        const int o1 = __shfl_xor(m1[t], 32), o2 = __shfl_xor(m2[t], 32);
-        const int n1 = imin(m1[t], o1);
-        m2[t] = imin(imax(m1[t], o1), imin(m2[t], o2));
-        m1[t] = n1;
+        const int o1 = __shfl_xor(m1[t], 32), o2 = __shfl_xor(m2[t], 32), o3 = __shfl_xor(m3[t], 32);
+        push(m1[t], m2[t], m3[t], o1);
+        push(m1[t], m2[t], m3[t], o2);
+        push(m1[t], m2[t], m3[t], o3);
     }
     if (ch == 1 && h == 0) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             lds_top[rp][t][0][r] = m1[t];
             lds_top[rp][t][1][r] = m2[t];
+            lds_top[rp][t][2][r] = m3[t];
         }
     }
     __syncthreads();
@@ -805,14 +815,19 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const int o1 = lds_top[rp][t][0][r], o2 = lds_top[rp][t][1][r];
-            const float s1 = __int_as_float(imin(m1[t], o1));
-            const float s2 = __int_as_float(imin(imax(m1[t], o1), imin(m2[t], o2)));
+            push(m1[t], m2[t], m3[t], lds_top[rp][t][0][r]);
+            push(m1[t], m2[t], m3[t], lds_top[rp][t][1][r]);
+            push(m1[t], m2[t], m3[t], lds_top[rp][t][2][r]);
+            const float s1 = __int_as_float(m1[t]), s2 = __int_as_float(m2[t]), s3 = __int_as_float(m3[t]);
             if (valid[t]) {
                 const float bound = x2[t] + mc2;
-                const float margin = 6.103515625e-05f * fabsf(s2) + tb.kappa * bound;
-                bool sure = (s2 - s1) > margin;
-                sure = sure && (bound < 1e29f) && (s1 < 1e29f);
+                const bool finite = (bound < 1e29f) && (s1 < 1e29f);  // false for NaN
+                const float slack = tb.kappa * bound;
+                // the smallest exact distance is the best-scored centroid's when the second score is
+                // further away than the error bound ...
+                const bool sure = finite && (s2 - s1) > 6.103515625e-05f * fabsf(s2) + slack;
+                // ... and one of the two best-scored centroids' when the third score is
+                const bool two = finite && (s2 < 1e29f) && (s3 - s1) > 6.103515625e-05f * fabsf(s3) + slack;
                 if (sure) {
                     const uint8_t code = (uint8_t)(__float_as_uint(s1) & 0xFFu);
                     if constexpr (LBG) {
@@ -824,6 +839,9 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
                     } else {
                         a.codes[row[t] * a.m + s] = code;
                     }
+                } else if (two) {
+                    wg_pairs[atomicAdd(&wg_pcount, 1u)] = make_uint2(
+                        (uint32_t)(row[t] * a.m + s), (__float_as_uint(s1) & 0xFFu) | ((__float_as_uint(s2) & 0xFFu) << 8));
                 } else {
                     wg_list[atomicAdd(&wg_count, 1u)] = (uint32_t)(row[t] * a.m + s);
                 }
@@ -831,11 +849,15 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         }
     }
     __syncthreads();
-    const uint32_t cnt = wg_count;
-    if (cnt == 0) return;
-    if (threadIdx.x == 0) wg_base = atomicAdd(tb.list_count, cnt);
+    const uint32_t cnt = wg_count, pcnt = wg_pcount;
+    if (cnt == 0 && pcnt == 0) return;
+    if (threadIdx.x == 0) {
+        if (cnt) wg_base = atomicAdd(tb.list_count, cnt);
+        if (pcnt) wg_pbase = atomicAdd(tb.list_count + 1, pcnt);
+    }
     __syncthreads();
     for (uint32_t i = threadIdx.x; i < cnt; i += 256) tb.list[wg_base + i] = wg_list[i];
+    for (uint32_t i = threadIdx.x; i < pcnt; i += 256) tb.pairs[wg_pbase + i] = wg_pairs[i];
 }
 
 }  // namespace vq

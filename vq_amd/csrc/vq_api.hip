@@ -171,13 +171,16 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     const int nb = (a.k + 31) / 32, nkc = sd / 8, nsl = (sd + 31) / 32;
     const size_t n_atab = (size_t)a.m * nkc * nb * 128 * 4, n_c2 = (size_t)a.m * nb * 32;  // floats
     VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + (size_t)a.m * nb + (size_t)a.m * sd + a.m + 2 * (size_t)a.m * nsl + 8) + 64));
-    VQ_TRY(ensure(ctx, ctx->mfma_list, sizeof(uint32_t) * ((size_t)a.n * a.m + 4)));
+    // header (two counts), the list for the all-centroid check, the list for the two-candidate check
+    const size_t n_pairs = (size_t)a.n * a.m;
+    VQ_TRY(ensure(ctx, ctx->mfma_list, sizeof(uint32_t) * (4 + ((n_pairs + 1) & ~(size_t)1) + 2 * n_pairs)));
     float *atab = (float *)ctx->mfma_tab.p;
     float *c2perm = atab + n_atab;
     float *maxc2 = c2perm + n_c2;  // per block of 32 centroids
     float *mu = maxc2 + (((size_t)a.m * nb + 3) & ~(size_t)3);  // 16-byte aligned: read as float4
     uint32_t *count = (uint32_t *)ctx->mfma_list.p;
     uint32_t *list = count + 4;
+    uint2 *pairs = (uint2 *)(list + ((n_pairs + 1) & ~(size_t)1));  // 8-byte aligned
     float2 *norms = (float2 *)(mu + (size_t)a.m * sd);  // sd is a multiple of 8: 8-byte aligned
     int *shifted = (int *)(norms + (size_t)a.m * nsl);
     hipLaunchKernelGGL(vq::k_block_centres, dim3(a.m, nsl), dim3(256), 0, ctx->stream, a.cb, a.k, sd, mu, norms);
@@ -187,7 +190,7 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     // two candidates, each: operand split 3 * 2^-16, fp32 accumulation (34 per chunk + 16) * 2^-24,
     // rounding of the differences from the centre 2^-22
     const float kappa = 2.0f * (3.0f * 1.52587890625e-05f + (34.0f * nkc + 16.0f + 4.0f) * 5.9604644775390625e-08f);
-    vq::MfmaWideBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, mu, shifted, list, count, nb, sd, kappa};
+    vq::MfmaWideBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, mu, shifted, list, count, pairs, nb, sd, kappa};
     {
         ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
         hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0,
@@ -195,6 +198,10 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     }
     VQ_HIP(ctx, hipGetLastError());
     ctx->recheck_src = 2;
+    // undecided pairs with two candidates, then the few that need every centroid
+    hipLaunchKernelGGL((vq::k_assign_wide_pair<METRIC, LBG>), dim3(512), dim3(256), 0, ctx->stream, a, sd,
+                       (const uint2 *)pairs, (const uint32_t *)(count + 1));
+    VQ_HIP(ctx, hipGetLastError());
     return launch_wide_exact<METRIC, LBG>(ctx, a, sd, list, count);
 }
 
@@ -427,16 +434,27 @@ int32_t vq_ctx_set_assign_path(vq_ctx *ctx, int32_t path) {
 
 int32_t vq_ctx_last_recheck_count(vq_ctx *ctx, uint32_t *h_count) {
     if (!ctx || !h_count) return VQ_ERR_INVALID_ARG;
+    uint32_t all = 0, two = 0;
+    const int32_t rc = vq_ctx_last_recheck_split(ctx, &all, &two);
+    *h_count = all + two;
+    return rc;
+}
+
+int32_t vq_ctx_last_recheck_split(vq_ctx *ctx, uint32_t *h_count, uint32_t *h_two) {
+    if (!ctx || !h_count || !h_two) return VQ_ERR_INVALID_ARG;
     *h_count = 0;
+    *h_two = 0;
     if (ctx->recheck_src == 1) {
         uint32_t h[vq::kStatSlots * vq::kStatStride];
         VQ_HIP(ctx, hipMemcpyAsync(h, ctx->mfma_stat.p, sizeof(h), hipMemcpyDeviceToHost, ctx->stream));
         VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
         for (int i = 0; i < vq::kStatSlots; ++i) *h_count += h[i * vq::kStatStride];
     } else if (ctx->recheck_src == 2) {
-        VQ_HIP(ctx, hipMemcpyAsync(h_count, ctx->mfma_list.p, sizeof(uint32_t), hipMemcpyDeviceToHost,
-                                   ctx->stream));
+        uint32_t h[2];  // all-centroid checks, two-candidate checks
+        VQ_HIP(ctx, hipMemcpyAsync(h, ctx->mfma_list.p, sizeof(h), hipMemcpyDeviceToHost, ctx->stream));
         VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        *h_count = h[0];
+        *h_two = h[1];
     }
     return VQ_OK;
 }
