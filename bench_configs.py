@@ -57,7 +57,8 @@ def main():
                 ctx.lbg_fit(dres, n, dim, 1, dim, k, iters, init[st], reseed[st], cbp)
                 ctx.assign(vq_amd.EUCLIDEAN, dres, n, dim, 1, dim, k, cbp, dcodes)
                 ctx.residual_sub(dres, n, dim, dim, k, cbp, dcodes)
-                ctx.mean_l2norm(dres, n, dim, dim)
+                # (epsilon = 0: the mean residual norm, src/rvq.rs:131-141, cannot stop the fit and is skipped,
+                # as the host class does)
 
         rvq_fit()
         out["c4_rvq_fit_ms"] = timed(rvq_fit)
@@ -77,6 +78,9 @@ def main():
         ctx.set_assign_path(0)
         one()
         out["c4_assign_pass_matrix_cores_ms"] = timed(one, 3)
+        norm = lambda: ctx.mean_l2norm(dres, n, dim, dim)
+        norm()
+        out["c4_mean_residual_norm_ms"] = timed(norm, 3)
         del dx, dres, dall, drec
     if "c5" in which:
         n, dim, depth = 1_000_000, 128, 8

@@ -20,6 +20,43 @@ static __global__ void __launch_bounds__(256) k_residual_sub(float *__restrict__
     *p = *p - cb[(size_t)codes[row * code_stride] * dim + t];
 }
 
+// The same, four components per lane (dim and ld multiples of 4, 16-byte aligned pointers); a
+// workgroup covers 1024 consecutive float4 of the n x dim/4 grid.  active == nullptr: every row.
+// codes_out / used (both or neither): RVQ encode bookkeeping of the stage, written by the lane
+// that holds a row's first components (src/rvq.rs:196-202).
+static __global__ void __launch_bounds__(256) k_residual_sub4(float *__restrict__ res, int64_t n, int64_t ld,
+                                                       int dim4, const float *__restrict__ cb,
+                                                       const uint8_t *__restrict__ codes,
+                                                       const uint8_t *__restrict__ active,
+                                                       uint8_t *__restrict__ codes_out, int stages, int stage,
+                                                       uint8_t *__restrict__ used) {
+    const int64_t first = (int64_t)blockIdx.x * 1024;
+    const int64_t row0 = first / dim4;            // uniform
+    const uint32_t rem0 = (uint32_t)(first % dim4);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const uint32_t local = rem0 + threadIdx.x + 256u * u;
+        const int64_t row = row0 + local / (uint32_t)dim4;
+        const uint32_t t4 = local % (uint32_t)dim4;
+        if (row >= n) continue;
+        const bool on = active ? active[row] != 0 : true;
+        const uint32_t code = on ? codes[row] : 0u;
+        if (codes_out && t4 == 0) {
+            codes_out[row * stages + stage] = (uint8_t)code;
+            if (on) used[row] = (uint8_t)(stage + 1);
+        }
+        if (!on) continue;
+        float4 *p = reinterpret_cast<float4 *>(res + row * ld) + t4;
+        const float4 c = reinterpret_cast<const float4 *>(cb + (size_t)code * dim4 * 4)[t4];
+        float4 v = *p;
+        v.x = v.x - c.x;
+        v.y = v.y - c.y;
+        v.z = v.z - c.z;
+        v.w = v.w - c.w;
+        *p = v;
+    }
+}
+
 // norms[i] = sqrt(sum_t x[i][t]^2), sequential f32 order (src/rvq.rs:134-135).
 // One wave = 64 rows.  The rows are read coalesced, 64 columns at a time, into a padded LDS tile;
 // each lane then walks its own row of the tile, so the per-row sum stays one sequential chain.
@@ -28,13 +65,23 @@ static __global__ void __launch_bounds__(64) k_row_norms(const float *__restrict
     __shared__ float tile[64][65];
     const int lane = threadIdx.x;
     const int64_t row0 = (int64_t)blockIdx.x * 64;
+    const int64_t last = n - 1;
     float acc = 0.0f;
     for (int c0 = 0; c0 < dim; c0 += 64) {
         const int w = (dim - c0 < 64) ? (dim - c0) : 64;
+        // Loads are unconditional (clamped to the last row and column, the surplus is never
+        // summed) and issued sixteen at a time: under a branch each one would be waited for.
+        const int col = c0 + (lane < w ? lane : w - 1);
         __syncthreads();
-        for (int r = 0; r < 64; ++r) {
-            const int64_t row = row0 + r;
-            if (row < n && lane < w) tile[r][lane] = x[row * ld + c0 + lane];
+        for (int r0 = 0; r0 < 64; r0 += 16) {
+            float v[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t row = row0 + r0 + r;
+                v[r] = x[(row < n ? row : last) * ld + col];
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tile[r0 + r][lane] = v[r];
         }
         __syncthreads();
         for (int t = 0; t < w; ++t) {
@@ -65,10 +112,11 @@ static __global__ void __launch_bounds__(256) k_sum_f64(const float *__restrict_
     if (threadIdx.x == 0) out[blockIdx.x] = sh[0];
 }
 
-// One stage of ResidualQuantizer::quantize for every row still active (src/rvq.rs:200-202):
-// sum += c; residual -= c.  One lane per element.
-static __global__ void __launch_bounds__(256) k_rvq_stage_apply(float *__restrict__ res, float *__restrict__ sum,
-                                                         int64_t n, int dim, const float *__restrict__ cb,
+// One stage of ResidualQuantizer::quantize for every row still active (src/rvq.rs:200-202), the
+// residual's half: residual -= c; the stage's code and the number of stages used are recorded.
+// The other half (sum += c) is replayed from the codes by k_rvq_recon_f16.  One lane per element.
+static __global__ void __launch_bounds__(256) k_rvq_stage_apply(float *__restrict__ res, int64_t n, int dim,
+                                                         const float *__restrict__ cb,
                                                          const uint8_t *__restrict__ stage_codes,
                                                          uint8_t *__restrict__ codes_out, int stages,
                                                          int stage, const uint8_t *__restrict__ active,
@@ -84,9 +132,59 @@ static __global__ void __launch_bounds__(256) k_rvq_stage_apply(float *__restric
         if (on) used[row] = (uint8_t)(stage + 1);
     }
     if (!on) return;
-    const float c = cb[(size_t)code * dim + t];
-    sum[i] = sum[i] + c;
-    res[i] = res[i] - c;
+    res[i] = res[i] - cb[(size_t)code * dim + t];
+}
+
+// The reconstruction of ResidualQuantizer::quantize from the codes: sum = 0; for every stage the
+// row used, in order, sum = sum + c (src/rvq.rs:183,201); then f16 (src/rvq.rs:212).  One lane
+// per element; the codebooks (stages x k x dim) stay in L2.
+static __global__ void __launch_bounds__(256) k_rvq_recon_f16(int64_t n, int dim, int k,
+                                                       const float *__restrict__ codebooks,
+                                                       const uint8_t *__restrict__ codes, int stages,
+                                                       const uint8_t *__restrict__ used,
+                                                       uint16_t *__restrict__ out) {
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n * dim) return;
+    const int64_t row = i / dim;
+    const int t = (int)(i % dim);
+    const int nst = used[row];
+    float sum = 0.0f;
+    for (int st = 0; st < nst; ++st)
+        sum = sum + codebooks[((size_t)st * k + codes[row * stages + st]) * dim + t];
+    out[i] = __half_as_ushort(__float2half_rn(sum));
+}
+
+// The same, four components per lane (dim a multiple of 4, 16-byte aligned codebooks, 8-byte
+// aligned output).
+static __global__ void __launch_bounds__(256) k_rvq_recon4_f16(int64_t n, int dim4, int k,
+                                                        const float *__restrict__ codebooks,
+                                                        const uint8_t *__restrict__ codes, int stages,
+                                                        const uint8_t *__restrict__ used,
+                                                        uint16_t *__restrict__ out) {
+    const int64_t first = (int64_t)blockIdx.x * 1024;
+    const int64_t row0 = first / dim4;
+    const uint32_t rem0 = (uint32_t)(first % dim4);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const uint32_t local = rem0 + threadIdx.x + 256u * u;
+        const int64_t row = row0 + local / (uint32_t)dim4;
+        const uint32_t t4 = local % (uint32_t)dim4;
+        if (row >= n) continue;
+        const int nst = used[row];
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int st = 0; st < nst; ++st) {
+            const float4 c =
+                reinterpret_cast<const float4 *>(codebooks + ((size_t)st * k + codes[row * stages + st]) * dim4 * 4)[t4];
+            sum.x = sum.x + c.x;
+            sum.y = sum.y + c.y;
+            sum.z = sum.z + c.z;
+            sum.w = sum.w + c.w;
+        }
+        uint2 h;
+        h.x = (uint32_t)__half_as_ushort(__float2half_rn(sum.x)) | ((uint32_t)__half_as_ushort(__float2half_rn(sum.y)) << 16);
+        h.y = (uint32_t)__half_as_ushort(__float2half_rn(sum.z)) | ((uint32_t)__half_as_ushort(__float2half_rn(sum.w)) << 16);
+        reinterpret_cast<uint2 *>(out + row * (int64_t)dim4 * 4)[t4] = h;
+    }
 }
 
 // The row stops when ||residual|| < epsilon (src/rvq.rs:204-207).
@@ -96,18 +194,7 @@ static __global__ void __launch_bounds__(256) k_rvq_stage_stop(const float *__re
     if (row < n && active[row] && norms[row] < epsilon) active[row] = 0;
 }
 
-static __global__ void __launch_bounds__(256) k_f32_to_f16(const float *__restrict__ in, int64_t count,
-                                                    uint16_t *__restrict__ out) {
-    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < count) out[i] = __half_as_ushort(__float2half_rn(in[i]));
-}
-
 static __global__ void __launch_bounds__(256) k_fill_u8(uint8_t *__restrict__ p, int64_t count, uint8_t v) {
-    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < count) p[i] = v;
-}
-
-static __global__ void __launch_bounds__(256) k_fill_f32(float *__restrict__ p, int64_t count, float v) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < count) p[i] = v;
 }

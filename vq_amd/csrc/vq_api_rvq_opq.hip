@@ -20,8 +20,14 @@ int32_t vq_residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_
     if (!d_res || !d_codebook || !d_codes || n < 0 || dim <= 0 || ld < dim || k <= 0 || k > 256)
         return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
     VQ_HIP(ctx, hipSetDevice(ctx->device));
-    hipLaunchKernelGGL(vq::k_residual_sub, dim3(cdiv(n * dim, 256)), dim3(256), 0, ctx->stream, d_res, n,
-                       ld, dim, d_codebook, d_codes, 1);
+    if (dim % 4 == 0 && ld % 4 == 0 &&
+        ((reinterpret_cast<uintptr_t>(d_res) | reinterpret_cast<uintptr_t>(d_codebook)) & 15) == 0)
+        hipLaunchKernelGGL(vq::k_residual_sub4, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, ctx->stream, d_res,
+                           n, ld, dim / 4, d_codebook, d_codes, (const uint8_t *)nullptr, (uint8_t *)nullptr, 0, 0,
+                           (uint8_t *)nullptr);
+    else
+        hipLaunchKernelGGL(vq::k_residual_sub, dim3(cdiv(n * dim, 256)), dim3(256), 0, ctx->stream, d_res, n,
+                           ld, dim, d_codebook, d_codes, 1);
     VQ_HIP(ctx, hipGetLastError());
     return VQ_OK;
 }
@@ -60,18 +66,16 @@ int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, 
     VQ_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
     VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(float) * (size_t)n * dim));   // residual
-    VQ_TRY(ensure(ctx, ctx->tmp_d, sizeof(float) * (size_t)n * dim));   // running sum
     VQ_TRY(ensure(ctx, ctx->tmp_e, (size_t)n * 3 + 16));                // stage codes, active, used
     VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(float) * (size_t)n));         // row norms
     float *norms = (float *)ctx->tmp_a.p;
     float *res = (float *)ctx->tmp_c.p;
-    float *sum = (float *)ctx->tmp_d.p;
     uint8_t *stage_codes = (uint8_t *)ctx->tmp_e.p;
     uint8_t *active = stage_codes + ((n + 3) & ~(int64_t)3);
     uint8_t *used = active + n;
     VQ_HIP(ctx, hipMemcpy2DAsync(res, sizeof(float) * dim, d_x, sizeof(float) * ld, sizeof(float) * dim,
                                  (size_t)n, hipMemcpyDeviceToDevice, st));
-    hipLaunchKernelGGL(vq::k_fill_f32, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, sum, n * dim, 0.0f);
+    const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(d_codebooks) & 15) == 0;
     hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, active, n, (uint8_t)1);
     hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, used, n, (uint8_t)0);
     for (int s = 0; s < stages; ++s) {
@@ -80,8 +84,12 @@ int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, 
             hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, stage_codes, n, (uint8_t)0);
         else
             VQ_TRY(assign_codes(ctx, metric, res, n, dim, 1, dim, k, cb, stage_codes));
-        hipLaunchKernelGGL(vq::k_rvq_stage_apply, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, res, sum, n, dim,
-                           cb, stage_codes, d_codes, stages, s, active, used);
+        if (vec4)
+            hipLaunchKernelGGL(vq::k_residual_sub4, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, st, res, n,
+                               (int64_t)dim, dim / 4, cb, stage_codes, active, d_codes, stages, s, used);
+        else
+            hipLaunchKernelGGL(vq::k_rvq_stage_apply, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, res, n, dim, cb,
+                               stage_codes, d_codes, stages, s, active, used);
         if (epsilon > 0.0f) {  // a norm is never below a non-positive threshold
             hipLaunchKernelGGL(vq::k_row_norms, dim3(cdiv(n, 64)), dim3(64), 0, st, res, n, (int64_t)dim, dim,
                                norms);
@@ -91,9 +99,14 @@ int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, 
     }
     if (d_stages_used)
         VQ_HIP(ctx, hipMemcpyAsync(d_stages_used, used, (size_t)n, hipMemcpyDeviceToDevice, st));
-    if (d_recon_f16)
-        hipLaunchKernelGGL(vq::k_f32_to_f16, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, sum, n * dim,
-                           d_recon_f16);
+    if (d_recon_f16) {
+        if (vec4 && (reinterpret_cast<uintptr_t>(d_recon_f16) & 7) == 0)
+            hipLaunchKernelGGL(vq::k_rvq_recon4_f16, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, st, n, dim / 4, k,
+                               d_codebooks, d_codes, stages, used, d_recon_f16);
+        else
+            hipLaunchKernelGGL(vq::k_rvq_recon_f16, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, n, dim, k,
+                               d_codebooks, d_codes, stages, used, d_recon_f16);
+    }
     VQ_HIP(ctx, hipGetLastError());
     return VQ_OK;
 }

@@ -553,9 +553,11 @@ public:
                                      cb, dcodes.get()));  // rvq.rs:116-125
             dev->check(vq_residual_sub(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)k, cb,
                                        dcodes.get()));  // rvq.rs:127
-            float avg = 0.f;
-            dev->check(vq_mean_l2norm(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, &avg));  // 131-138
-            if (avg < epsilon) break;  // rvq.rs:139-141
+            if (epsilon > 0.f) {  // a mean norm is never below a non-positive (or NaN) threshold
+                float avg = 0.f;
+                dev->check(vq_mean_l2norm(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, &avg));  // 131-138
+                if (avg < epsilon) break;  // rvq.rs:139-141
+            }
         }
         q.stages_ = produced;  // rvq.rs:145
         return q;
