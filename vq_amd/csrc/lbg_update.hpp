@@ -266,29 +266,25 @@ static __global__ void __launch_bounds__(256) k_lbg_leafsum(LbgState st, const f
     const uint32_t *__restrict__ perm = st.perm + (size_t)s * n;
     const float *__restrict__ xc = x + (int64_t)s * sd + t;
     float acc = 0.0f;
-    uint32_t p = d.x;
-    // batches of 32 members: the loads of a batch are independent, the adds stay in list order;
-    // the row ids of the next batch are fetched while the current rows are in flight
-    constexpr int B = 32;
-    uint32_t r[B], rn[B];
-    if (p + B <= d.y) {
+    // Batches of 16 members: the loads of a batch are independent (issued unconditionally, a batch
+    // past the end of the list repeats its last row and is not added), the adds stay in list order;
+    // the row ids of the next batch are fetched while the current rows are in flight.
+    constexpr int B = 16;
+    uint32_t rn[B];
+    const uint32_t lastp = d.y - 1;  // leaves are never empty
 #pragma unroll
-        for (int u = 0; u < B; ++u) rn[u] = perm[p + u];
-    }
-    for (; p + B <= d.y; p += B) {
-#pragma unroll
-        for (int u = 0; u < B; ++u) r[u] = rn[u];
+    for (int u = 0; u < B; ++u) rn[u] = perm[d.x + u < d.y ? d.x + u : lastp];
+    for (uint32_t p = d.x; p < d.y; p += B) {
         float v[B];
 #pragma unroll
-        for (int u = 0; u < B; ++u) v[u] = xc[(int64_t)r[u] * ld];
-        if (p + 2 * B <= d.y) {
+        for (int u = 0; u < B; ++u) v[u] = xc[(int64_t)rn[u] * ld];
 #pragma unroll
-            for (int u = 0; u < B; ++u) rn[u] = perm[p + B + u];
-        }
+        for (int u = 0; u < B; ++u) rn[u] = perm[p + B + u < d.y ? p + B + u : lastp];
+        const uint32_t cnt = d.y - p;  // the same in every lane of the leaf
 #pragma unroll
-        for (int u = 0; u < B; ++u) acc = acc + v[u];
+        for (int u = 0; u < B; ++u)
+            if ((uint32_t)u < cnt) acc = acc + v[u];
     }
-    for (; p < d.y; ++p) acc = acc + xc[(int64_t)perm[p] * ld];
     st.leaf_sum[((size_t)s * st.leaf_cap + leaf) * sd + t] = acc;
 }
 
@@ -454,8 +450,18 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const 
         sum = ls[0];
     } else {
         if (st.stream) return;  // k_lbg_combine8 writes the large clusters
+        // the per-part sums in part order; sixteen loads in flight, the adds one chain
         sum = 0.0f;
-        for (int p = 0; p < st.nparts; ++p) sum = sum + ls[(size_t)p * sd];
+        constexpr int B = 16;
+        const int np = st.nparts;
+        for (int p = 0; p < np; p += B) {
+            float v[B];
+#pragma unroll
+            for (int u = 0; u < B; ++u) v[u] = ls[(size_t)(p + u < np ? p + u : np - 1) * sd];
+#pragma unroll
+            for (int u = 0; u < B; ++u)
+                if (p + u < np) sum = sum + v[u];
+        }
     }
     *out = sum / __uint2float_rn(cnt);
 }
