@@ -103,7 +103,11 @@ static __global__ void __launch_bounds__(256) k_lbg_scan_seg(LbgState st) {
     const int b0 = g * kScanSeg, b1 = (b0 + kScanSeg < st.nparts) ? b0 + kScanSeg : st.nparts;
     const uint32_t *h = st.hist + ((size_t)s * st.nparts + b0) * kMaxK + j;
     uint32_t sum = 0;
-    for (int b = b0; b < b1; ++b) sum += h[(size_t)(b - b0) * kMaxK];
+    uint32_t v[kScanSeg];  // all loads of the segment in flight together
+#pragma unroll
+    for (int u = 0; u < kScanSeg; ++u) v[u] = h[(size_t)(b0 + u < b1 ? u : b1 - 1 - b0) * kMaxK];
+#pragma unroll
+    for (int u = 0; u < kScanSeg; ++u) sum += (b0 + u < b1) ? v[u] : 0u;
     st.seg[((size_t)s * st.nseg + g) * kMaxK + j] = sum;
 }
 
@@ -600,16 +604,19 @@ static __global__ void __launch_bounds__(256) k_lbg_combine8(LbgState st, int k,
     const uint32_t cnt = st.count[(size_t)s * kMaxK + j];
     if (cnt <= (uint32_t)kSeqMax) return;
     const float *ps = st.part_sum + ((size_t)s * st.nparts * kMaxK + j) * 8 + t;
+    // the kernel is a handful of waves: its time is memory round trips, so 32 loads are in flight
+    // at a time (unconditional, clamped to the last part); the adds stay one chain in part order
     float sum = 0.0f;
-    int p = 0;
-    for (; p + 8 <= st.nparts; p += 8) {
-        float v[8];
+    constexpr int B = 32;
+    const int np = st.nparts;
+    for (int p = 0; p < np; p += B) {
+        float v[B];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = ps[(size_t)(p + u) * kMaxK * 8];
+        for (int u = 0; u < B; ++u) v[u] = ps[(size_t)(p + u < np ? p + u : np - 1) * kMaxK * 8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) sum = sum + v[u];
+        for (int u = 0; u < B; ++u)
+            if (p + u < np) sum = sum + v[u];
     }
-    for (; p < st.nparts; ++p) sum = sum + ps[(size_t)p * kMaxK * 8];
     cb[((size_t)s * k + j) * 8 + t] = sum / __uint2float_rn(cnt);
 }
 
