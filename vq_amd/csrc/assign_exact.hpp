@@ -412,6 +412,9 @@ __device__ __forceinline__ void wide_argmin(const AssignArgs &a, int sd, int s, 
     }
     int t = 0;
     if constexpr (VEC) {
+        // (one row per wave is a latency-bound walk over the centroids: more loads in flight)
+        constexpr int kAhead = NR == 1 ? 4 : 1;
+#pragma unroll kAhead
         for (; t + 4 <= sd; t += 4) {
             float4 cv[4];
 #pragma unroll
