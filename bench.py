@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0
 PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X published dense bf16 matrix peak
 # rocprofv3 FETCH_SIZE / WRITE_SIZE of one LBG launch of k_assign_mfma_bf (KiB per dispatch), scaled by
 # the plain copy kernel (FETCH x 2.000, WRITE x 1.000): profiles/pq_fit_encode_1Mx128_mfma_bf16.md
-MEASURED_ASSIGN_TRAFFIC_BYTES = int((261518.0 * 2.000 + 13341.2 * 1.000) * 1024)
+MEASURED_ASSIGN_TRAFFIC_BYTES = int((263174.9 * 2.000 + 12191.5 * 1.000) * 1024)
 
 
 def log(*a):
@@ -117,7 +117,7 @@ def main():
     achieved_tflops = flop_per_launch / (avg_kern_ms * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",
-        "kernel": "k_assign_mfma_bf<*,*,2,2> (bf16-split matrix-core scores + packed-index top-2 + "
+        "kernel": "k_assign_mfma_bf<*,*,2,4> (bf16-split matrix-core scores + packed-index top-2 + "
                   "in-wave exact re-check; LBG passes and the encode pass)",
         "achieved": round(achieved_tflops, 3),
         "peak": PEAK_FP32_MFMA_TFLOPS,
