@@ -92,39 +92,48 @@ static __global__ void __launch_bounds__(64) k_seg_variance(const uint32_t *__re
     var[(size_t)g * dim + t] = acc;
 }
 
-// The same sums with the memory traffic taken off the chain of dependent adds.  One workgroup of
-// 1024 threads per segment: all threads fetch rows (16-byte pieces, whole rows contiguous) eight
-// chunks ahead into registers and hand them over through two LDS tiles; threads 0..dim-1 add the
-// rows of the current tile in order.  A chunk is 8192 / dim rows; about 512 rows (256 KB at
-// dim = 128) are in flight per workgroup, which is what one chain of adds consumes per memory
-// round trip.  The barrier waits for LDS only, so the loads in flight are not drained.
+// The same sums with everything but the adds taken off the chain of dependent adds.  One workgroup
+// of 1024 threads per segment: all threads fetch rows (16-byte pieces, whole rows contiguous)
+// eight chunks ahead into registers, turn them into squared deviations (v - mean)^2 — the same
+// two roundings as in the chain — and hand those over through two LDS tiles; threads 0..dim-1
+// add the squares of the current tile in row order, one add per row.  A chunk is 8192 / dim rows;
+// about 512 rows (256 KB at dim = 128) are in flight per workgroup, which is what one chain of adds
+// consumes per memory round trip.  The barrier waits for LDS only, so the loads in flight are not
+// drained.
 constexpr int kVarStage = 8192;  // floats per LDS tile
 constexpr int kVarAhead = 8;     // chunks in flight
 
 __device__ __forceinline__ void lds_only_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// acc + sum over the rows of one LDS tile of (v - mu)^2, in row order, for one component.
-__device__ __forceinline__ float seg_variance_chunk(const float *t, int rows, int dim, float mu, float acc) {
+// acc + the squares of one component over the rows of one LDS tile, in row order.  DIM > 0: the row
+// stride as a constant, so that the reads pair up with constant offsets and the next sixteen
+// values are on their way while sixteen are added; DIM = 0: any stride.
+template <int DIM>
+__device__ __forceinline__ float seg_variance_chunk(const float *t, int rows, int dim, float acc) {
+    const int stride = DIM > 0 ? DIM : dim;
     int r = 0;
-    for (; r + 8 <= rows; r += 8) {
-        float v[8];
+    if (rows >= 16) {
+        float v[16];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) v[q] = t[(r + q) * dim];
+        for (int q = 0; q < 16; ++q) v[q] = t[q * stride];
+        for (; r + 32 <= rows; r += 16) {
+            float w[16];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const float d = v[q] - mu;
-            const float p = d * d;
-            acc = acc + p;
+            for (int q = 0; q < 16; ++q) w[q] = t[(r + 16 + q) * stride];
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc = acc + v[q];
+#pragma unroll
+            for (int q = 0; q < 16; ++q) v[q] = w[q];
         }
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc = acc + v[q];
+        r += 16;
     }
-    for (; r < rows; ++r) {
-        const float d = t[r * dim] - mu;
-        const float p = d * d;
-        acc = acc + p;
-    }
+    for (; r < rows; ++r) acc = acc + t[r * stride];
     return acc;
 }
 
+template <int DIM>
 static __global__ void __launch_bounds__(1024) k_seg_variance_wg(const uint32_t *__restrict__ perm,
                                                                 const uint2 *__restrict__ seg_range,
                                                                 const float *__restrict__ means, int64_t first,
@@ -158,6 +167,22 @@ static __global__ void __launch_bounds__(1024) k_seg_variance_wg(const uint32_t 
     // at each use instead of counting them.  The rings are plain arrays with constant indices.
     // (Eight named slots instead of an array: an array of this size is left in scratch memory.)
     const float *xp0 = x + 4 * pc[0], *xp1 = x + 4 * pc[1];
+    // the means of this thread's columns
+    const float *mrow = means + (first + g) * dim;
+    const float4 mu0 = *reinterpret_cast<const float4 *>(mrow + 4 * pc[0]);
+    const float4 mu1 = *reinterpret_cast<const float4 *>(mrow + 4 * pc[1]);
+    auto sq_dev = [](float4 v, float4 m) {
+        float4 d, p;
+        d.x = v.x - m.x;
+        d.y = v.y - m.y;
+        d.z = v.z - m.z;
+        d.w = v.w - m.w;
+        p.x = d.x * d.x;
+        p.y = d.y * d.y;
+        p.z = d.z * d.z;
+        p.w = d.w * d.w;
+        return p;
+    };
 #define VAR_DECL(S) uint32_t ida_##S, idb_##S; float4 xa_##S, xb_##S;
     VAR_DECL(0) VAR_DECL(1) VAR_DECL(2) VAR_DECL(3) VAR_DECL(4) VAR_DECL(5) VAR_DECL(6) VAR_DECL(7)
 #define VAR_IDS(S, chunk)                                                     \
@@ -173,8 +198,8 @@ static __global__ void __launch_bounds__(1024) k_seg_variance_wg(const uint32_t 
     }
 #define VAR_STORE(buf, S)                                                     \
     {                                                                         \
-        if (has[0]) tile[buf][rr[0] * ppr + pc[0]] = xa_##S;                  \
-        if (has[1]) tile[buf][rr[1] * ppr + pc[1]] = xb_##S;                  \
+        if (has[0]) tile[buf][rr[0] * ppr + pc[0]] = sq_dev(xa_##S, mu0);     \
+        if (has[1]) tile[buf][rr[1] * ppr + pc[1]] = sq_dev(xb_##S, mu1);     \
     }
     // prologue: ids of chunks 0..15, rows of chunks 0..7, chunk 0 in LDS
     VAR_IDS(0, 0) VAR_IDS(1, 1) VAR_IDS(2, 2) VAR_IDS(3, 3) VAR_IDS(4, 4) VAR_IDS(5, 5) VAR_IDS(6, 6) VAR_IDS(7, 7)
@@ -182,7 +207,6 @@ static __global__ void __launch_bounds__(1024) k_seg_variance_wg(const uint32_t 
     VAR_PRO(0) VAR_PRO(1) VAR_PRO(2) VAR_PRO(3) VAR_PRO(4) VAR_PRO(5) VAR_PRO(6) VAR_PRO(7)
     VAR_STORE(0, 0)
     lds_only_barrier();
-    const float mu = (tid < dim) ? means[(first + g) * dim + tid] : 0.0f;
     float acc = 0.0f;
     // One step: rows of chunk i + 8 into the slot chunk i has left, ids of chunk i + 16 behind
     // them; chunk i + 1 (fetched seven steps ago) into the other tile; chunk i added.  Chunks past
@@ -196,7 +220,7 @@ static __global__ void __launch_bounds__(1024) k_seg_variance_wg(const uint32_t 
         if (tid < dim && i < nch) {                                           \
             const float *t = reinterpret_cast<const float *>(tile[i & 1]) + tid; \
             const int rows = (int)(((uint32_t)(i + 1) * R <= count) ? R : count - (uint32_t)i * R); \
-            acc = seg_variance_chunk(t, rows, dim, mu, acc);                  \
+            acc = seg_variance_chunk<DIM>(t, rows, dim, acc);                 \
         }                                                                     \
         lds_only_barrier();                                                   \
     }

@@ -228,10 +228,19 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         SP_HIP(hipMemcpyAsync(d_range, range.data(), sizeof(uint2) * ns, hipMemcpyHostToDevice, st));
         SP_HIP(hipMemcpyAsync(d_smeans, smeans.data(), sizeof(float) * (size_t)ns * dim, hipMemcpyHostToDevice, st));
         // per-dimension sums of squared deviations (src/tsvq.rs:88-99)
-        if (dim % 4 == 0 && dim <= 1024 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0)
-            hipLaunchKernelGGL(vq::k_seg_variance_wg, dim3(ns), dim3(1024), 0, st, perm, (const uint2 *)d_range,
-                               (const float *)d_smeans, (int64_t)0, d_x, ld, dim, (float *)d_var);
-        else
+        if (dim % 4 == 0 && dim <= 1024 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0) {
+#define VARIANCE_WG(D)                                                                                     \
+    hipLaunchKernelGGL((vq::k_seg_variance_wg<D>), dim3(ns), dim3(1024), 0, st, perm, (const uint2 *)d_range, \
+                       (const float *)d_smeans, (int64_t)0, d_x, ld, dim, (float *)d_var)
+            switch (dim) {  // the common row lengths get constant LDS strides
+            case 32: VARIANCE_WG(32); break;
+            case 64: VARIANCE_WG(64); break;
+            case 128: VARIANCE_WG(128); break;
+            case 256: VARIANCE_WG(256); break;
+            default: VARIANCE_WG(0); break;
+            }
+#undef VARIANCE_WG
+        } else
             hipLaunchKernelGGL(vq::k_seg_variance, dim3(cdiv((int64_t)ns * dim, 64)), dim3(64), 0, st, perm,
                                (const uint2 *)d_range, ns, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
                                (float *)d_var);
