@@ -546,17 +546,31 @@ __device__ __forceinline__ void tsvq_step(float &al, float &ar, float xv, float 
     }
 }
 
+// The centroids of the first kTopNodes nodes (the upper levels of a tree numbered level by level)
+// are staged in LDS: down there the lanes of a wave sit on a handful of nodes, and per-lane
+// global reads of a few distinct lines cost the address unit as much as fully scattered ones.  Row
+// stride DIM + 4: the 16-byte reads of up to 8 nodes at the same offset fall into different banks.
+constexpr int kTopNodes = 31;  // levels 0-4 of a complete tree
+
 template <int METRIC, int DIM>
 __global__ void __launch_bounds__(64) k_tsvq_descend_reg(const float *__restrict__ x, int64_t n, int64_t ld,
                                                          const float *__restrict__ cen,
                                                          const float *__restrict__ cnorm,
                                                          const int *__restrict__ left,
-                                                         const int *__restrict__ right,
+                                                         const int *__restrict__ right, int n_nodes,
                                                          int *__restrict__ leaf) {
     constexpr int CH = 32;
+    constexpr int TS = DIM + 4;
     __shared__ float tile[64 * (CH + 4)];
+    __shared__ float top[kTopNodes * TS];
     const int lane = threadIdx.x;
     const int64_t row0 = (int64_t)blockIdx.x * 64;
+    const int ntop = n_nodes < kTopNodes ? n_nodes : kTopNodes;
+    for (int e = lane; e < ntop * (DIM / 4); e += 64) {
+        const int nd = e / (DIM / 4), pc = e % (DIM / 4);
+        *reinterpret_cast<float4 *>(&top[nd * TS + pc * 4]) =
+            *reinterpret_cast<const float4 *>(cen + (size_t)nd * DIM + pc * 4);
+    }
     float xr[DIM];
 #pragma unroll
     for (int c = 0; c < DIM / CH; ++c) {
@@ -602,7 +616,45 @@ __global__ void __launch_bounds__(64) k_tsvq_descend_reg(const float *__restrict
             l = left[node];
             r = right[node];
         }
-        if (l >= 0 && r >= 0) {
+        const bool both = l >= 0 && r >= 0;
+        // every lane that compares two children finds them in LDS: the whole wave reads there
+        if (!__any(both && (l >= ntop || r >= ntop))) {
+            if (both) {
+                const float *pl = &top[l * TS], *pr = &top[r * TS];
+                float al = 0.0f, ar = 0.0f;
+#pragma unroll
+                for (int q = 0; q < DIM / 4; ++q) {
+                    const float4 a = *reinterpret_cast<const float4 *>(pl + q * 4);
+                    const float4 b = *reinterpret_cast<const float4 *>(pr + q * 4);
+                    tsvq_step<METRIC>(al, ar, xr[q * 4 + 0], a.x, b.x);
+                    tsvq_step<METRIC>(al, ar, xr[q * 4 + 1], a.y, b.y);
+                    tsvq_step<METRIC>(al, ar, xr[q * 4 + 2], a.z, b.z);
+                    tsvq_step<METRIC>(al, ar, xr[q * 4 + 3], a.w, b.w);
+                }
+                float dl, dr;
+                if constexpr (METRIC == M_COS) {
+                    float nl = cnorm[l], nr = cnorm[r];
+                    float ql = al / (na * nl), qr = ar / (na * nr);
+                    dl = (na == 0.0f || nl == 0.0f) ? 1.0f : 1.0f - ql;
+                    dr = (na == 0.0f || nr == 0.0f) ? 1.0f : 1.0f - qr;
+                } else if constexpr (METRIC == M_EUCLID) {
+                    dl = sqrtf(al);
+                    dr = sqrtf(ar);
+                } else {
+                    dl = al;
+                    dr = ar;
+                }
+                node = (dl <= dr) ? l : r;
+            } else if (l >= 0) {
+                node = l;
+            } else if (r >= 0) {
+                node = r;
+            } else {
+                active = false;
+            }
+            continue;
+        }
+        if (both) {
             const float4 *pl = reinterpret_cast<const float4 *>(cen + (size_t)l * DIM);
             const float4 *pr = reinterpret_cast<const float4 *>(cen + (size_t)r * DIM);
             float al = 0.0f, ar = 0.0f;

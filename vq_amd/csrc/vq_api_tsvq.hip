@@ -411,7 +411,8 @@ int32_t vq_tsvq_descend(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n
         dim3 g(cdiv(n, 64)), b(64);
 #define DESC_REG(M, D)                                                                                \
     hipLaunchKernelGGL((vq::k_tsvq_descend_reg<M, D>), g, b, 0, ctx->stream, d_x, n, ld,              \
-                       tree->d_centroids, tree->d_cnorm, tree->d_left, tree->d_right, d_leaf)
+                       tree->d_centroids, tree->d_cnorm, tree->d_left, tree->d_right, (int)tree->h_left.size(),    \
+                       d_leaf)
 #define DESC_DIM(M)                                                                                   \
     switch (tree->dim) {                                                                              \
     case 32: DESC_REG(M, 32); break;                                                                  \
