@@ -550,7 +550,7 @@ __device__ __forceinline__ void tsvq_step(float &al, float &ar, float xv, float 
 // are staged in LDS: down there the lanes of a wave sit on a handful of nodes, and per-lane
 // global reads of a few distinct lines cost the address unit as much as fully scattered ones.  Row
 // stride DIM + 4: the 16-byte reads of up to 8 nodes at the same offset fall into different banks.
-constexpr int kTopNodes = 63;  // levels 0-5 of a complete tree
+constexpr int kTopNodes = 127;  // levels 0-6 of a complete tree
 
 template <int METRIC, int DIM>
 __global__ void __launch_bounds__(256) k_tsvq_descend_reg(const float *__restrict__ x, int64_t n, int64_t ld,
@@ -561,18 +561,14 @@ __global__ void __launch_bounds__(256) k_tsvq_descend_reg(const float *__restric
                                                          int *__restrict__ leaf) {
     constexpr int CH = 32;
     constexpr int TS = DIM + 4;
-    __shared__ float tiles[4][64 * (CH + 4)];
-    __shared__ float top[kTopNodes * TS];
+    // one LDS area: first the four waves' row tiles, then (the rows being in registers) the centroids
+    constexpr int kTileFloats = 64 * (CH + 4), kTopFloats = kTopNodes * TS;
+    __shared__ float lds[(4 * kTileFloats > kTopFloats) ? 4 * kTileFloats : kTopFloats];
     const int lane = threadIdx.x & 63;
-    float *tile = tiles[threadIdx.x >> 6];
+    float *tile = lds + (threadIdx.x >> 6) * kTileFloats;
+    float *top = lds;
     const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64;  // one wave = 64 rows
     const int ntop = n_nodes < kTopNodes ? n_nodes : kTopNodes;
-    for (int e = threadIdx.x; e < ntop * (DIM / 4); e += 256) {
-        const int nd = e / (DIM / 4), pc = e % (DIM / 4);
-        *reinterpret_cast<float4 *>(&top[nd * TS + pc * 4]) =
-            *reinterpret_cast<const float4 *>(cen + (size_t)nd * DIM + pc * 4);
-    }
-    __syncthreads();  // the only point where the four waves meet
     float xr[DIM];
 #pragma unroll
     for (int c = 0; c < DIM / CH; ++c) {
@@ -600,6 +596,13 @@ __global__ void __launch_bounds__(256) k_tsvq_descend_reg(const float *__restric
             xr[c * CH + q * 4 + 3] = t4.w;
         }
     }
+    __syncthreads();  // every wave has its rows: the tiles make room for the centroids
+    for (int e = threadIdx.x; e < ntop * (DIM / 4); e += 256) {
+        const int nd = e / (DIM / 4), pc = e % (DIM / 4);
+        *reinterpret_cast<float4 *>(&top[nd * TS + pc * 4]) =
+            *reinterpret_cast<const float4 *>(cen + (size_t)nd * DIM + pc * 4);
+    }
+    __syncthreads();
     float na = 0.0f;
     if constexpr (METRIC == M_COS) {
         float sa = 0.0f;
