@@ -524,7 +524,7 @@ __global__ void __launch_bounds__(256) k_tsvq_descend(const float *__restrict__ 
 }
 
 // The same walk with the row held in registers (DIM a multiple of 32 up to 128).  One wave = 64
-// rows, four waves per workgroup: the rows are read with whole-line loads through a small padded LDS tile, so every byte of
+// rows, eight waves per workgroup: the rows are read with whole-line loads through a small padded LDS tile, so every byte of
 // the input is fetched once; the two child centroids of a lane's node are read 64 bytes at a
 // time, the next piece in flight while the current one is accumulated.  The sums stay one
 // sequential chain per (row, child), as in the reference.
@@ -550,10 +550,10 @@ __device__ __forceinline__ void tsvq_step(float &al, float &ar, float xv, float 
 // are staged in LDS: down there the lanes of a wave sit on a handful of nodes, and per-lane
 // global reads of a few distinct lines cost the address unit as much as fully scattered ones.  Row
 // stride DIM + 4: the 16-byte reads of up to 8 nodes at the same offset fall into different banks.
-constexpr int kTopNodes = 127;  // levels 0-6 of a complete tree
+constexpr int kTopNodes = 255;  // levels 0-7 of a complete tree
 
 template <int METRIC, int DIM>
-__global__ void __launch_bounds__(256) k_tsvq_descend_reg(const float *__restrict__ x, int64_t n, int64_t ld,
+__global__ void __launch_bounds__(512) k_tsvq_descend_reg(const float *__restrict__ x, int64_t n, int64_t ld,
                                                          const float *__restrict__ cen,
                                                          const float *__restrict__ cnorm,
                                                          const int *__restrict__ left,
@@ -561,13 +561,13 @@ __global__ void __launch_bounds__(256) k_tsvq_descend_reg(const float *__restric
                                                          int *__restrict__ leaf) {
     constexpr int CH = 32;
     constexpr int TS = DIM + 4;
-    // one LDS area: first the four waves' row tiles, then (the rows being in registers) the centroids
+    // one LDS area: first the eight waves' row tiles, then (the rows being in registers) the centroids
     constexpr int kTileFloats = 64 * (CH + 4), kTopFloats = kTopNodes * TS;
-    __shared__ float lds[(4 * kTileFloats > kTopFloats) ? 4 * kTileFloats : kTopFloats];
+    __shared__ float lds[(8 * kTileFloats > kTopFloats) ? 8 * kTileFloats : kTopFloats];
     const int lane = threadIdx.x & 63;
     float *tile = lds + (threadIdx.x >> 6) * kTileFloats;
     float *top = lds;
-    const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 64;  // one wave = 64 rows
+    const int64_t row0 = ((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 64;  // one wave = 64 rows
     const int ntop = n_nodes < kTopNodes ? n_nodes : kTopNodes;
     float xr[DIM];
 #pragma unroll
@@ -597,7 +597,7 @@ __global__ void __launch_bounds__(256) k_tsvq_descend_reg(const float *__restric
         }
     }
     __syncthreads();  // every wave has its rows: the tiles make room for the centroids
-    for (int e = threadIdx.x; e < ntop * (DIM / 4); e += 256) {
+    for (int e = threadIdx.x; e < ntop * (DIM / 4); e += 512) {
         const int nd = e / (DIM / 4), pc = e % (DIM / 4);
         *reinterpret_cast<float4 *>(&top[nd * TS + pc * 4]) =
             *reinterpret_cast<const float4 *>(cen + (size_t)nd * DIM + pc * 4);

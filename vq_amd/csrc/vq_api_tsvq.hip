@@ -408,7 +408,7 @@ int32_t vq_tsvq_descend(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n
     VQ_HIP(ctx, hipSetDevice(ctx->device));
     // rows in registers: dim a multiple of 32 up to 128, 16-byte aligned rows
     if (tree->dim % 32 == 0 && tree->dim <= 128 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0) {
-        dim3 g(cdiv(n, 256)), b(256);
+        dim3 g(cdiv(n, 512)), b(512);
 #define DESC_REG(M, D)                                                                                \
     hipLaunchKernelGGL((vq::k_tsvq_descend_reg<M, D>), g, b, 0, ctx->stream, d_x, n, ld,              \
                        tree->d_centroids, tree->d_cnorm, tree->d_left, tree->d_right, (int)tree->h_left.size(),    \
