@@ -281,3 +281,30 @@ def test_wide_mfma_path_equals_oracle_and_valu_path(ctx, metric, n, m, sd, k, ki
     assert np.array_equal(got, want)
     if kind in ("normal", "uniform", "offset") and k > 1:
         assert frac < 0.05, frac  # the matrix-core pass decides almost every row itself
+
+
+@pytest.mark.parametrize("sd,m,k", [(8, 4, 64), (8, 16, 256), (32, 2, 100), (6, 3, 9)])
+@pytest.mark.parametrize("pad,shift", [(0, 0), (1, 0), (3, 1), (4, 0), (6, 2)])
+def test_rows_with_leading_dimension_and_offset(ctx, sd, m, k, pad, shift):
+    """Rows inside a wider buffer (ld > dim) that starts `shift` floats into the allocation: the
+    matrix-core kernels take 16-byte pieces of the rows where they can and must give the same
+    codes and centroids when the rows are not 16-byte aligned."""
+    n, dim = 3000, sd * m
+    ld = dim + pad + shift
+    rng = np.random.default_rng(sd * 100 + pad * 10 + shift)
+    buf = rng.standard_normal((n, ld)).astype(F)
+    x = np.ascontiguousarray(buf[:, shift:shift + dim])
+    cb = np.ascontiguousarray(x[rng.choice(n, k, replace=False)].reshape(k, m, sd).transpose(1, 0, 2))
+    dbuf, dcb = ctx.to_device(buf), ctx.to_device(cb)
+    dcodes = ctx.empty((n, m), np.uint8)
+    for metric in (O.SQEUCLIDEAN, O.EUCLIDEAN):
+        want = O.pq_encode(metric, x, cb).astype(np.uint8)
+        ctx.assign(metric, dbuf.ptr + 4 * shift, n, ld, m, sd, k, dcb, dcodes)
+        assert np.array_equal(dcodes.download(), want)
+    init, reseed = data.index_streams(n, m, k, 3, seed=pad + shift)
+    w = O.pq_fit(x, m, k, 3, init, reseed)
+    assert w["rc"] == 0
+    dcb2 = ctx.empty((m, k, sd), F)
+    it, _ = ctx.lbg_fit(dbuf.ptr + 4 * shift, n, ld, m, sd, k, 3, init, reseed, dcb2)
+    assert np.array_equal(it, w["iters"])
+    assert np.array_equal(dcb2.download().view(np.uint32), w["codebooks"].view(np.uint32))
