@@ -23,6 +23,7 @@ struct vq_ctx {
     std::string err;
     // grow-only device workspace
     DevBuf flags, tables, hist, seg, part_sum, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;
+    DevBuf tsvq_sq;              // TSVQ build: squared deviations of a level
     DevBuf mfma_tab, mfma_list, mfma_stat;  // tables, re-check list and counters of the matrix-core assignment
     int recheck_src = 0;         // where the last pass counted its undecided pairs: 1 mfma_stat, 2 mfma_list
     int assign_path = 0;         // 0 = matrix cores where a kernel exists, 1 = vector ALU only
