@@ -92,111 +92,123 @@ static __global__ void __launch_bounds__(64) k_seg_variance(const uint32_t *__re
     var[(size_t)g * dim + t] = acc;
 }
 
-// ---- per-dimension sums of squared deviations in two steps (dim a multiple of 16) -------------
+// ---- per-dimension sums of squared deviations in two steps (dim a multiple of 8) --------------
 // Step 1, on the whole GPU: sq = (x - mean)^2, the same two roundings as in the chain, stored so
-// that the 16 consecutive positions of a column sit side by side:
-//   sq16[(lo_g + 16 g) * dim + ((p - lo_g) / 16) * 16 * dim + (c / 16) * 256 + (c % 16) * 16 + (p - lo_g) % 16]
-// (every segment starts on its own group of 16 positions: n + 16 nseg rows of room).
-// Grid (blocks of 64 positions, segments); one lane per (group of 16 positions, column).
-static __global__ void __launch_bounds__(256) k_seg_sqdev16(const uint32_t *__restrict__ perm,
+// that 32 consecutive positions of a column sit side by side:
+//   sq32[(lo_g + 32 g) * dim + ((p - lo_g) / 32) * 32 * dim + (c / 8) * 256 + (c % 8) * 32 + (p - lo_g) % 32]
+// (every segment starts on its own group of 32 positions: n + 32 nseg rows of room).
+// Grid (blocks of 64 positions, segments); one lane per (group of 32 positions, column).
+constexpr int kChainGroup = 32;  // positions per group
+
+static __global__ void __launch_bounds__(256) k_seg_sqdev32(const uint32_t *__restrict__ perm,
                                                             const uint2 *__restrict__ seg_range,
                                                             const float *__restrict__ means, int64_t first,
                                                             const float *__restrict__ x, int64_t ld, int dim,
-                                                            float *__restrict__ sq16) {
+                                                            float *__restrict__ sq32) {
     const int g = blockIdx.y;
     const uint2 range = seg_range[g];
     const uint32_t count = range.y - range.x;
-    const uint32_t P0 = blockIdx.x * 4u;  // first group of 16 of this block
-    if (P0 * 16u >= count) return;
-    const uint32_t nP = (count + 15u) / 16u;
-    const uint32_t groups = nP - P0 < 4u ? nP - P0 : 4u;
+    const uint32_t P0 = blockIdx.x * 2u;  // first group of this block
+    if (P0 * 32u >= count) return;
+    const uint32_t nP = (count + 31u) / 32u;
+    const uint32_t groups = nP - P0 < 2u ? nP - P0 : 2u;
     const float *mrow = means + (first + g) * dim;
-    float *out = sq16 + ((size_t)range.x + 16u * (size_t)g) * dim;
+    float *out = sq32 + ((size_t)range.x + 32u * (size_t)g) * dim;
     const uint32_t *pm = perm + range.x;
     for (uint32_t e = threadIdx.x; e < groups * (uint32_t)dim; e += 256) {
         const uint32_t P = P0 + e / (uint32_t)dim, c = e % (uint32_t)dim;
         const float m = mrow[c];
-        float q[16];
+        float4 *o = reinterpret_cast<float4 *>(out + (size_t)P * 32 * dim + (c / 8u) * 256u + (c % 8u) * 32u);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint32_t p = 16u * P + r;  // past the end: the last row again, never added
-            const float d = x[(int64_t)pm[p < count ? p : count - 1] * ld + c] - m;
-            q[r] = d * d;
+        for (int h = 0; h < 2; ++h) {  // sixteen loads in flight at a time
+            float q[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const uint32_t p = 32u * P + 16u * h + r;  // past the end: the last row again, never added
+                const float d = x[(int64_t)pm[p < count ? p : count - 1] * ld + c] - m;
+                q[r] = d * d;
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[4 * h + r] = make_float4(q[4 * r], q[4 * r + 1], q[4 * r + 2], q[4 * r + 3]);
         }
-        float4 *o = reinterpret_cast<float4 *>(out + (size_t)P * 16 * dim + (c / 16u) * 256u + (c % 16u) * 16u);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = make_float4(q[4 * r], q[4 * r + 1], q[4 * r + 2], q[4 * r + 3]);
     }
 }
 
-// Step 2: the sequential sums.  Grid (segments, dim / 64); a wave owns 16 columns, the four lanes
-// of a quad own one column: lane 4 cc + j loads positions 4j .. 4j+3 of column cc — one 16-byte
-// load per lane moves 16 positions of 16 columns, 1 KB contiguous per wave — and the quad's first
-// lane adds the 16 values in position order, its neighbours' twelve handed over by quad
-// permutes.  A lane can have about 60 loads in flight (the counter of outstanding loads holds no
-// more), so a wave keeps 960 positions in flight: enough to cover a memory round trip of 3 us at
-// 3-4 ns per position, which one 16-byte load per 4 positions (240 in flight) is not.
-constexpr int kChainRing = 60;
+// Step 2: the sequential sums.  Grid (segments, dim / 32); a wave owns 8 columns, eight
+// neighbouring lanes own one column: lane 8 cc + j loads positions 4j .. 4j+3 of column cc of a
+// group — one 16-byte load per lane moves 32 positions of 8 columns, 1 KB contiguous per wave —
+// and the first lane of the eight adds the 32 values in position order, its neighbours' values
+// read through DPP row shifts folded into the adds.  A lane keeps kChainRing loads in flight: 768
+// positions per wave cover a memory round trip of 3 us at 3-4 ns per position with a ring of 96
+// registers; one 16-byte load per 4 positions of a lane's own column could keep 240 in flight at
+// most (the counter of outstanding loads holds 63) and measured 12 ns per position.
+constexpr int kChainRing = 24;
 
-__device__ __forceinline__ float quad_lane(float v, int j) {  // the value of lane j of this lane's quad
-    const int x = __float_as_int(v);
-    const int r = j == 1 ? __builtin_amdgcn_mov_dpp(x, 0x55, 0xF, 0xF, true)
-                : j == 2 ? __builtin_amdgcn_mov_dpp(x, 0xAA, 0xF, 0xF, true)
-                         : __builtin_amdgcn_mov_dpp(x, 0xFF, 0xF, 0xF, true);
-    return __int_as_float(r);
+template <int J>
+__device__ __forceinline__ float lane_ahead(float v) {  // the value of the lane J places up in its row of 16
+    static_assert(J >= 1 && J <= 15, "row shift");
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x100 + J, 0xF, 0xF, true));
 }
 
-static __global__ void __launch_bounds__(256) k_seg_chain16(const float *__restrict__ sq16,
+static __global__ void __launch_bounds__(256) k_seg_chain32(const float *__restrict__ sq32,
                                                            const uint2 *__restrict__ seg_range, int dim,
                                                            float *__restrict__ var) {
     const int g = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int cb = blockIdx.y * 4 + wave;  // block of 16 columns
-    if (cb * 16 >= dim) return;
+    const int cb = blockIdx.y * 4 + wave;  // block of 8 columns
+    if (cb * 8 >= dim) return;
     const uint2 range = seg_range[g];
     const uint32_t count = range.y - range.x;
     float acc = 0.0f;
     if (count > 0) {
-        const uint32_t nP = (count + 15u) / 16u, last = nP - 1u;
-        const size_t stride = (size_t)4 * dim;  // float4 per group of 16 positions
-        const float4 *q = reinterpret_cast<const float4 *>(sq16 + ((size_t)range.x + 16u * (size_t)g) * dim) +
+        const uint32_t nP = (count + 31u) / 32u, last = nP - 1u;
+        const size_t stride = (size_t)8 * dim;  // float4 per group of 32 positions
+        const float4 *q = reinterpret_cast<const float4 *>(sq32 + ((size_t)range.x + 32u * (size_t)g) * dim) +
                           (size_t)cb * 64 + lane;
+        // rem: positions of this group inside the segment (the same in every lane)
+        auto add4 = [&](float a, float b, float c, float d, int rem, int at) {
+            if (rem > at) acc = acc + a;
+            if (rem > at + 1) acc = acc + b;
+            if (rem > at + 2) acc = acc + c;
+            if (rem > at + 3) acc = acc + d;
+        };
+        auto add32 = [&](const float4 &v, int rem) {
+            add4(v.x, v.y, v.z, v.w, rem, 0);
+            add4(lane_ahead<1>(v.x), lane_ahead<1>(v.y), lane_ahead<1>(v.z), lane_ahead<1>(v.w), rem, 4);
+            add4(lane_ahead<2>(v.x), lane_ahead<2>(v.y), lane_ahead<2>(v.z), lane_ahead<2>(v.w), rem, 8);
+            add4(lane_ahead<3>(v.x), lane_ahead<3>(v.y), lane_ahead<3>(v.z), lane_ahead<3>(v.w), rem, 12);
+            add4(lane_ahead<4>(v.x), lane_ahead<4>(v.y), lane_ahead<4>(v.z), lane_ahead<4>(v.w), rem, 16);
+            add4(lane_ahead<5>(v.x), lane_ahead<5>(v.y), lane_ahead<5>(v.z), lane_ahead<5>(v.w), rem, 20);
+            add4(lane_ahead<6>(v.x), lane_ahead<6>(v.y), lane_ahead<6>(v.z), lane_ahead<6>(v.w), rem, 24);
+            add4(lane_ahead<7>(v.x), lane_ahead<7>(v.y), lane_ahead<7>(v.z), lane_ahead<7>(v.w), rem, 28);
+        };
         float4 buf[kChainRing];
 #pragma unroll
-        for (int k = 0; k < kChainRing; ++k) buf[k] = q[(size_t)((uint32_t)k < last ? (uint32_t)k : last) * stride];
-        auto add16 = [&](const float4 &v, int rem) {  // rem: positions of this group inside the segment (uniform)
-            const float4 v1 = make_float4(quad_lane(v.x, 1), quad_lane(v.y, 1), quad_lane(v.z, 1), quad_lane(v.w, 1));
-            const float4 v2 = make_float4(quad_lane(v.x, 2), quad_lane(v.y, 2), quad_lane(v.z, 2), quad_lane(v.w, 2));
-            const float4 v3 = make_float4(quad_lane(v.x, 3), quad_lane(v.y, 3), quad_lane(v.z, 3), quad_lane(v.w, 3));
-            const float e[16] = {v.x,  v.y,  v.z,  v.w,  v1.x, v1.y, v1.z, v1.w,
-                                 v2.x, v2.y, v2.z, v2.w, v3.x, v3.y, v3.z, v3.w};
-            if (rem >= 16) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc = acc + e[r];
-            } else {
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    if (r < rem) acc = acc + e[r];
-            }
-        };
-        const uint32_t full = count / 16u;  // groups with all 16 positions
+        for (int k = 0; k < kChainRing; ++k) {
+            buf[k] = q[(size_t)((uint32_t)k < last ? (uint32_t)k : last) * stride];
+            // the first loads are issued in slot order, as the loop issues them: the loop's waits count
+            // the loads issued after a slot's, and one order on both ways into the loop keeps them exact
+            asm volatile("" ::: "memory");
+        }
+        const uint32_t full = count / 32u;  // groups with all their positions
         uint32_t P = 0;
         for (; P + kChainRing <= full; P += kChainRing) {
 #pragma unroll
             for (int k = 0; k < kChainRing; ++k) {
-                const float4 v = buf[k];
+                // (added first, refilled after: the slot's register is free when its load is issued,
+                // so no copy of the ring is carried around the loop)
+                add32(buf[k], 32);
                 const uint32_t nx = P + kChainRing + k;
                 buf[k] = q[(size_t)(nx < last ? nx : last) * stride];
-                add16(v, 16);
             }
         }
 #pragma unroll
         for (int k = 0; k < kChainRing; ++k) {
-            const int rem = (int)count - 16 * (int)(P + k);
-            if (rem > 0) add16(buf[k], rem);
+            const int rem = (int)count - 32 * (int)(P + k);
+            if (rem > 0) add32(buf[k], rem);
         }
     }
-    if ((lane & 3) == 0) var[(size_t)g * dim + cb * 16 + (lane >> 2)] = acc;
+    if ((lane & 7) == 0) var[(size_t)g * dim + cb * 8 + (lane >> 3)] = acc;
 }
 
 // The same sums with everything but the adds taken off the chain of dependent adds.  One workgroup

@@ -92,11 +92,12 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     VQ_TRY(ensure(ctx, ctx->tmp_d, sizeof(float) * (size_t)n));
     VQ_TRY(ensure(ctx, ctx->tmp_e, sizeof(uint32_t) * (size_t)n));
     VQ_TRY(ensure(ctx, ctx->tmp_f, sizeof(uint32_t) * (size_t)n));
-    // two-step variance (squares on the whole GPU, then the chains): dim a multiple of 16, and room
-    // for a level's squares with every node starting on its own group of 16 positions
-    constexpr int kChainSegs = 4096;  // levels with more nodes than this take the other kernels
-    const bool var_chain = dim % 16 == 0;
-    if (var_chain) VQ_TRY(ensure(ctx, ctx->tsvq_sq, sizeof(float) * ((size_t)n + 16 * (size_t)kChainSegs) * dim));
+    // two-step variance (squares on the whole GPU, then the chains): dim a multiple of 8, and room
+    // for a level's squares with every node starting on its own group of 32 positions
+    constexpr int kChainSegs = 2048;  // levels with more nodes than this take the other kernels
+    const bool var_chain = dim % 8 == 0;
+    if (var_chain)
+        VQ_TRY(ensure(ctx, ctx->tsvq_sq, sizeof(float) * ((size_t)n + vq::kChainGroup * (size_t)kChainSegs) * dim));
     float *d_sq = (float *)ctx->tsvq_sq.p;
     uint32_t *perm = (uint32_t *)ctx->tmp_a.p, *perm2 = (uint32_t *)ctx->tmp_b.p;
     float *vals = (float *)ctx->tmp_c.p;
@@ -237,10 +238,10 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         if (var_chain && ns <= kChainSegs) {
             uint32_t longest = 0;
             for (int i = 0; i < ns; ++i) longest = std::max(longest, range[i].y - range[i].x);
-            hipLaunchKernelGGL(vq::k_seg_sqdev16, dim3((unsigned)cdiv((int64_t)longest, 64), (unsigned)ns), dim3(256),
+            hipLaunchKernelGGL(vq::k_seg_sqdev32, dim3((unsigned)cdiv((int64_t)longest, 64), (unsigned)ns), dim3(256),
                                0, st, perm, (const uint2 *)d_range, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
                                d_sq);
-            hipLaunchKernelGGL(vq::k_seg_chain16, dim3((unsigned)ns, (unsigned)cdiv(dim, 64)), dim3(256), 0, st,
+            hipLaunchKernelGGL(vq::k_seg_chain32, dim3((unsigned)ns, (unsigned)cdiv(dim, 32)), dim3(256), 0, st,
                                (const float *)d_sq, (const uint2 *)d_range, dim, (float *)d_var);
         } else if (dim % 4 == 0 && dim <= 1024 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0) {
 #define VARIANCE_WG(D)                                                                                     \
