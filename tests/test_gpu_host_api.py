@@ -173,3 +173,22 @@ def test_tsvq_on_random_vectors(vq):
         tsvq.quantize(training[0, :4])
     with pytest.raises(vq.VqError, match="Empty input"):
         vq.TSVQ.new(np.zeros((0, 10), F), 3, vq.Distance.Euclidean)
+
+
+def test_rows_as_vectors_and_as_one_array_agree(vq):
+    """`&[Vector<f32>]` (one heap vector per row, packed by the host layer) and a contiguous array
+    (taken as a view) give the same reconstructions; a short row is a "Dimension mismatch" with the
+    lengths the reference's row-by-row check would name."""
+    x = generate_test_data(300, 12)
+    pq = vq.ProductQuantizer.fit(x, 3, 8, 5, vq.Distance.Euclidean, 1)
+    tsvq = vq.TSVQ.new(x, 3, vq.Distance.Manhattan)
+    rvq = vq.ResidualQuantizer.fit(x, 2, 4, 5, 1e-6, vq.Distance.Euclidean, 1)
+    opq = vq.OptimizedProductQuantizer.fit(x, 3, 8, 5, 2, vq.Distance.Euclidean, 1)
+    for q in (pq, tsvq, rvq, opq):
+        a = q.quantize_batch(x)
+        b = q.quantize_batch_vectors(x)
+        assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+        with pytest.raises(vq.VqError, match="Dimension mismatch: expected 12, got 7"):
+            q.quantize_batch_vectors(x, short_row=5, short_len=7)
+        with pytest.raises(vq.VqError, match="Dimension mismatch: expected 12, got 3"):
+            q.quantize_batch_vectors(x, short_row=0, short_len=3)

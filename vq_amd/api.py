@@ -101,6 +101,15 @@ class _Quantizer:
         _check(_h.vqh_quantize_batch(_vp(self._o), _p(x), _i64(x.shape[0]), _i64(x.shape[1]), _p(out)))
         return out.view(np.float16)
 
+    def quantize_batch_vectors(self, data, short_row=-1, short_len=0):
+        """quantize_batch through the reference's shape, one heap-allocated vector per row; row
+        `short_row` (if >= 0) is passed with only `short_len` floats."""
+        x = _rows(data)
+        out = np.zeros(x.shape, np.uint16)
+        _check(_h.vqh_quantize_batch_vectors(_vp(self._o), _p(x), _i64(x.shape[0]), _i64(x.shape[1]),
+                                             _i64(short_row), _i64(short_len), _p(out)))
+        return out.view(np.float16)
+
 
 class ProductQuantizer(_Quantizer):
     @classmethod

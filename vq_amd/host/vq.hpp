@@ -218,18 +218,52 @@ private:
     size_t count_ = 0;
 };
 
-// Packs `&[Vector<f32>]` (one heap allocation per vector, src/vector.rs:150-152) into one
-// row-major buffer and checks that all rows have the same length.
-inline std::vector<float> pack_rows(const std::vector<Vector<float>> &rows, size_t dim) {
-    std::vector<float> flat(rows.size() * dim);
-    for (size_t i = 0; i < rows.size(); ++i) {
-        if (rows[i].len() != dim) throw VqError::DimensionMismatch(dim, rows[i].len());
-        std::memcpy(flat.data() + i * dim, rows[i].data.data(), dim * sizeof(float));
+// `&[Vector<f32>]` as the device wants it: one row-major buffer.  The reference's shape — one
+// heap allocation per vector (src/vector.rs:150-152) — converts implicitly: packed once, lengths
+// checked.  Rows that are contiguous already (a matrix of another library, a memory-mapped file)
+// are taken as a view, without a copy.
+class Rows {
+public:
+    Rows(const std::vector<Vector<float>> &rows) : n_(rows.size()), dim_(rows.empty() ? 0 : rows[0].len()) {
+        own_.resize(n_ * dim_);
+        for (size_t i = 0; i < n_; ++i) {
+            if (rows[i].len() != dim_) {  // reported by expect_dim, in the order a row-by-row check would
+                ragged_ = true;
+                ragged_len_ = rows[i].len();
+                break;
+            }
+            std::memcpy(own_.data() + i * dim_, rows[i].data.data(), dim_ * sizeof(float));
+        }
+        p_ = own_.data();
     }
-    return flat;
-}
+    static Rows view(const float *p, size_t n, size_t dim) {
+        Rows r;
+        r.p_ = p;
+        r.n_ = n;
+        r.dim_ = dim;
+        return r;
+    }
+    bool empty() const { return n_ == 0; }
+    size_t size() const { return n_; }
+    size_t dim() const { return dim_; }  // length of the first row
+    const float *data() const { return p_; }
+    // every row has `dim` floats, or "Dimension mismatch" with the first length that differs
+    void expect_dim(size_t dim) const {
+        if (n_ == 0) return;
+        if (dim_ != dim) throw VqError::DimensionMismatch(dim, dim_);
+        if (ragged_) throw VqError::DimensionMismatch(dim, ragged_len_);
+    }
+
+private:
+    Rows() = default;
+    std::vector<float> own_;
+    const float *p_ = nullptr;
+    size_t n_ = 0, dim_ = 0, ragged_len_ = 0;
+    bool ragged_ = false;
+};
 
 inline std::vector<Vector<f16>> unpack_f16(const std::vector<uint16_t> &flat, size_t n, size_t dim) {
+    if (flat.empty()) return {};
     std::vector<Vector<f16>> out(n);
     for (size_t i = 0; i < n; ++i) {
         out[i].data.resize(dim);
@@ -239,22 +273,22 @@ inline std::vector<Vector<f16>> unpack_f16(const std::vector<uint16_t> &flat, si
 }
 
 // ---- lbg_quantize (src/utils.rs:32-109) --------------------------------------------------------
-inline std::vector<Vector<float>> lbg_quantize(const std::vector<Vector<float>> &data, size_t k,
+inline std::vector<Vector<float>> lbg_quantize(const Rows &data, size_t k,
                                                size_t max_iters, uint64_t seed,
                                                const IndexStreams *streams = nullptr,
                                                std::shared_ptr<Device> dev = Device::shared()) {
     size_t n = data.size();
     if (k == 0) throw VqError::InvalidParameter("k must be greater than 0");
     if (n < k) throw VqError::InvalidParameter("Not enough data points for k clusters");
-    size_t dim = data[0].len();
-    std::vector<float> flat = pack_rows(data, dim);
+    size_t dim = data.dim();
+    data.expect_dim(dim);
     IndexStreams own;
     if (!streams) {
         own = IndexStreams::from_seed(seed, 1, n, k, max_iters);
         streams = &own;
     }
     DeviceBuffer<float> dx(dev, n * dim), dcb(dev, k * dim);
-    dx.upload(flat.data(), flat.size());
+    dx.upload(data.data(), n * dim);
     dev->check(vq_lbg_fit(dev->ctx(), dx.get(), (int64_t)n, (int64_t)dim, 1, (int32_t)dim, (int32_t)k,
                           (int32_t)max_iters, streams->init.data(), streams->reseed.data(),
                           streams->n_reseed, dcb.get(), nullptr, nullptr));
@@ -268,12 +302,12 @@ inline std::vector<Vector<float>> lbg_quantize(const std::vector<Vector<float>> 
 class ProductQuantizer {
 public:
     // src/pq.rs:79-129
-    static ProductQuantizer fit(const std::vector<Vector<float>> &training_data, size_t m, size_t k,
+    static ProductQuantizer fit(const Rows &training_data, size_t m, size_t k,
                                 size_t max_iters, Distance distance, uint64_t seed,
                                 const IndexStreams *streams = nullptr,
                                 std::shared_ptr<Device> dev = Device::shared()) {
         if (training_data.empty()) throw VqError::EmptyInput();
-        size_t n = training_data[0].len();
+        size_t n = training_data.dim();
         if (n < m) throw VqError::InvalidParameter("Data dimension must be at least m");
         if (n % m != 0) throw VqError::InvalidParameter("Data dimension must be divisible by m");
         size_t rows = training_data.size();
@@ -285,14 +319,15 @@ public:
         pq.k_ = k;
         pq.sub_dim_ = n / m;
         pq.distance_ = distance;
-        std::vector<float> flat = pack_rows(training_data, n);
+        training_data.expect_dim(n);
+        const float *flat = training_data.data();
         IndexStreams own;
         if (!streams) {
             own = IndexStreams::from_seed(seed, m, rows, k, max_iters);
             streams = &own;
         }
         DeviceBuffer<float> dx(dev, rows * n);
-        dx.upload(flat.data(), flat.size());
+        dx.upload(flat, dx.size());
         pq.codebooks_ = DeviceBuffer<float>(dev, m * k * pq.sub_dim_);
         dev->check(vq_lbg_fit(dev->ctx(), dx.get(), (int64_t)rows, (int64_t)n, (int32_t)m, (int32_t)pq.sub_dim_,
                               (int32_t)k, (int32_t)max_iters, streams->init.data(), streams->reseed.data(),
@@ -303,31 +338,38 @@ public:
     // src/pq.rs:146-187
     Vector<f16> quantize(const Vector<float> &vector) const {
         if (vector.len() != sub_dim_ * m_) throw VqError::DimensionMismatch(sub_dim_ * m_, vector.len());
-        return quantize_batch({vector})[0];
+        return quantize_batch(std::vector<Vector<float>>{vector})[0];
     }
 
-    std::vector<Vector<f16>> quantize_batch(const std::vector<Vector<float>> &vectors) const {
+    std::vector<Vector<f16>> quantize_batch(const Rows &vectors) const {
+        return unpack_f16(quantize_batch_flat(vectors), vectors.size(), sub_dim_ * m_);
+    }
+
+    // the same reconstructions as one row-major n x dim array of f16 bit patterns
+    std::vector<uint16_t> quantize_batch_flat(const Rows &vectors) const {
         size_t dim = sub_dim_ * m_, n = vectors.size();
         if (n == 0) return {};
-        std::vector<float> flat = pack_rows(vectors, dim);
+        vectors.expect_dim(dim);
+        const float *flat = vectors.data();
         DeviceBuffer<float> dx(dev_, n * dim);
-        dx.upload(flat.data(), flat.size());
+        dx.upload(flat, dx.size());
         DeviceBuffer<uint8_t> dcodes(dev_, n * m_);
         DeviceBuffer<uint16_t> dout(dev_, n * dim);
         dev_->check(vq_assign(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim, (int32_t)m_,
                               (int32_t)sub_dim_, (int32_t)k_, codebooks_.get(), dcodes.get()));
         dev_->check(vq_decode_f16(dev_->ctx(), dcodes.get(), (int64_t)n, (int32_t)m_, (int32_t)sub_dim_,
                                   (int32_t)k_, codebooks_.get(), dout.get()));
-        return unpack_f16(dout.to_host(), n, dim);
+        return dout.to_host();
     }
 
     // The integer codes the reference keeps only as `best_index` (src/pq.rs:166-174): n x m bytes.
-    std::vector<uint8_t> encode(const std::vector<Vector<float>> &vectors) const {
+    std::vector<uint8_t> encode(const Rows &vectors) const {
         size_t dim = sub_dim_ * m_, n = vectors.size();
         if (n == 0) return {};
-        std::vector<float> flat = pack_rows(vectors, dim);
+        vectors.expect_dim(dim);
+        const float *flat = vectors.data();
         DeviceBuffer<float> dx(dev_, n * dim);
-        dx.upload(flat.data(), flat.size());
+        dx.upload(flat, dx.size());
         DeviceBuffer<uint8_t> dcodes(dev_, n * m_);
         dev_->check(vq_assign(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim, (int32_t)m_,
                               (int32_t)sub_dim_, (int32_t)k_, codebooks_.get(), dcodes.get()));
@@ -404,12 +446,12 @@ inline void procrustes_rotation(const std::vector<double> &A, size_t dim, std::v
 class OptimizedProductQuantizer {
 public:
     // src/opq.rs:90-205
-    static OptimizedProductQuantizer fit(const std::vector<Vector<float>> &training_data, size_t m, size_t k,
+    static OptimizedProductQuantizer fit(const Rows &training_data, size_t m, size_t k,
                                          size_t max_iters, size_t opq_iters, Distance distance, uint64_t seed,
                                          const IndexStreams *streams = nullptr,
                                          std::shared_ptr<Device> dev = Device::shared()) {
         if (training_data.empty()) throw VqError::EmptyInput();
-        size_t dim = training_data[0].len();
+        size_t dim = training_data.dim();
         if (dim < m) throw VqError::InvalidParameter("Dimension must be at least m");
         if (dim % m != 0) throw VqError::InvalidParameter("Dimension must be divisible by m");
         size_t n = training_data.size(), sd = dim / m;
@@ -423,7 +465,8 @@ public:
         q.dim_ = dim;
         q.distance_ = distance;
         const int32_t metric = distance.abi_metric();
-        std::vector<float> flat = pack_rows(training_data, dim);
+        training_data.expect_dim(dim);
+        const float *flat = training_data.data();
         IndexStreams own;
         if (!streams) {  // the same streams in every outer iteration (opq.rs:140 re-seeds seed + i)
             own = IndexStreams::from_seed(seed, m, n, k, max_iters);
@@ -432,7 +475,7 @@ public:
         vq_ctx *c = dev->ctx();
         DeviceBuffer<float> dx(dev, n * dim), drot(dev, n * dim), drec(dev, n * dim);
         DeviceBuffer<uint8_t> dcodes(dev, n * m);
-        dx.upload(flat.data(), flat.size());
+        dx.upload(flat, dx.size());
         dev->check(vq_copy_f32(c, drot.get(), dx.get(), (int64_t)(n * dim)));  // opq.rs:121
         q.codebooks_ = DeviceBuffer<float>(dev, m * k * sd);
         q.rotation_.assign(dim * dim, 0.f);
@@ -462,20 +505,24 @@ public:
     // src/opq.rs:222-264
     Vector<f16> quantize(const Vector<float> &vector) const {
         if (vector.len() != dim_) throw VqError::DimensionMismatch(dim_, vector.len());
-        return quantize_batch({vector})[0];
+        return quantize_batch(std::vector<Vector<float>>{vector})[0];
     }
 
-    std::vector<Vector<f16>> quantize_batch(const std::vector<Vector<float>> &vectors) const {
+    std::vector<Vector<f16>> quantize_batch(const Rows &vectors) const {
+        return unpack_f16(quantize_batch_flat(vectors), vectors.size(), dim_);
+    }
+
+    std::vector<uint16_t> quantize_batch_flat(const Rows &vectors) const {
         size_t n = vectors.size();
         if (n == 0) return {};
         DeviceBuffer<uint8_t> dcodes = encode_device(vectors);
         DeviceBuffer<uint16_t> dout(dev_, n * dim_);
         dev_->check(vq_decode_f16(dev_->ctx(), dcodes.get(), (int64_t)n, (int32_t)m_, (int32_t)sub_dim_,
                                   (int32_t)k_, codebooks_.get(), dout.get()));
-        return unpack_f16(dout.to_host(), n, dim_);
+        return dout.to_host();
     }
 
-    std::vector<uint8_t> encode(const std::vector<Vector<float>> &vectors) const {
+    std::vector<uint8_t> encode(const Rows &vectors) const {
         if (vectors.empty()) return {};
         return encode_device(vectors).to_host();
     }
@@ -484,11 +531,12 @@ public:
     const std::vector<float> &rotation() const { return rotation_; }  // row-major dim x dim
 
 private:
-    DeviceBuffer<uint8_t> encode_device(const std::vector<Vector<float>> &vectors) const {
+    DeviceBuffer<uint8_t> encode_device(const Rows &vectors) const {
         size_t n = vectors.size();
-        std::vector<float> flat = pack_rows(vectors, dim_);
+        vectors.expect_dim(dim_);
+        const float *flat = vectors.data();
         DeviceBuffer<float> dx(dev_, n * dim_), dy(dev_, n * dim_);
-        dx.upload(flat.data(), flat.size());
+        dx.upload(flat, dx.size());
         DeviceBuffer<uint8_t> dcodes(dev_, n * m_);
         vq_ctx *c = dev_->ctx();
         dev_->check(vq_rotate(c, dx.get(), (int64_t)n, (int64_t)dim_, (int32_t)dim_, d_rotation_.get(), dy.get()));
@@ -508,12 +556,12 @@ private:
 class ResidualQuantizer {
 public:
     // src/rvq.rs:87-154
-    static ResidualQuantizer fit(const std::vector<Vector<float>> &training_data, size_t stages, size_t k,
+    static ResidualQuantizer fit(const Rows &training_data, size_t stages, size_t k,
                                  size_t max_iters, float epsilon, Distance distance, uint64_t seed,
                                  const IndexStreams *streams = nullptr,
                                  std::shared_ptr<Device> dev = Device::shared()) {
         if (training_data.empty()) throw VqError::EmptyInput();
-        size_t dim = training_data[0].len(), n = training_data.size();
+        size_t dim = training_data.dim(), n = training_data.size();
         if (stages > 0) {
             if (k == 0) throw VqError::InvalidParameter("k must be greater than 0");
             if (n < k) throw VqError::InvalidParameter("Not enough data points for k clusters");
@@ -525,7 +573,8 @@ public:
         q.epsilon_ = epsilon;
         q.distance_ = distance;
         const int32_t metric = distance.abi_metric();
-        std::vector<float> flat = pack_rows(training_data, dim);
+        training_data.expect_dim(dim);
+        const float *flat = training_data.data();
         IndexStreams own;
         if (!streams) {
             own = IndexStreams::from_seed(seed, stages, n, k, max_iters);
@@ -534,7 +583,7 @@ public:
         vq_ctx *c = dev->ctx();
         DeviceBuffer<float> dx(dev, n * dim), dres(dev, n * dim);
         DeviceBuffer<uint8_t> dcodes(dev, n + 16);
-        dx.upload(flat.data(), flat.size());
+        dx.upload(flat, dx.size());
         dev->check(vq_copy_f32(c, dres.get(), dx.get(), (int64_t)(n * dim)));  // rvq.rs:103
         q.codebooks_ = DeviceBuffer<float>(dev, std::max<size_t>(stages * k * dim, 1));
         std::vector<uint8_t> zeros(n, 0);
@@ -566,23 +615,27 @@ public:
     // src/rvq.rs:171-215
     Vector<f16> quantize(const Vector<float> &vector) const {
         if (vector.len() != dim_) throw VqError::DimensionMismatch(dim_, vector.len());
-        return quantize_batch({vector})[0];
+        return quantize_batch(std::vector<Vector<float>>{vector})[0];
     }
 
-    std::vector<Vector<f16>> quantize_batch(const std::vector<Vector<float>> &vectors,
-                                            std::vector<uint8_t> *codes = nullptr) const {
+    std::vector<Vector<f16>> quantize_batch(const Rows &vectors, std::vector<uint8_t> *codes = nullptr) const {
+        return unpack_f16(quantize_batch_flat(vectors, codes), vectors.size(), dim_);
+    }
+
+    std::vector<uint16_t> quantize_batch_flat(const Rows &vectors, std::vector<uint8_t> *codes = nullptr) const {
         size_t n = vectors.size();
         if (n == 0) return {};
-        std::vector<float> flat = pack_rows(vectors, dim_);
+        vectors.expect_dim(dim_);
+        const float *flat = vectors.data();
         DeviceBuffer<float> dx(dev_, n * dim_);
-        dx.upload(flat.data(), flat.size());
+        dx.upload(flat, dx.size());
         DeviceBuffer<uint8_t> dcodes(dev_, std::max<size_t>(n * stages_, 1));
         DeviceBuffer<uint16_t> dout(dev_, n * dim_);
         dev_->check(vq_rvq_encode(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim_,
                                   (int32_t)dim_, (int32_t)stages_, (int32_t)std::max<size_t>(k_, 1),
                                   codebooks_.get(), epsilon_, dcodes.get(), nullptr, dout.get()));
         if (codes) *codes = dcodes.to_host();
-        return unpack_f16(dout.to_host(), n, dim_);
+        return dout.to_host();
     }
 
     size_t stages() const { return stages_; }
@@ -606,17 +659,18 @@ public:
     Distance distance;  // `pub distance`, src/tsvq.rs:193
 
     // TSVQ::new, src/tsvq.rs:209-215
-    static TSVQ create(const std::vector<Vector<float>> &training_data, size_t max_depth, Distance distance,
+    static TSVQ create(const Rows &training_data, size_t max_depth, Distance distance,
                        std::shared_ptr<Device> dev = Device::shared()) {
         if (training_data.empty()) throw VqError::EmptyInput();
-        size_t dim = training_data[0].len(), n = training_data.size();
-        std::vector<float> flat = pack_rows(training_data, dim);
+        size_t dim = training_data.dim(), n = training_data.size();
+        training_data.expect_dim(dim);
+        const float *flat = training_data.data();
         TSVQ t;
         t.dev_ = dev;
         t.distance = distance;
         t.dim_ = dim;
         DeviceBuffer<float> dx(dev, n * dim);
-        dx.upload(flat.data(), flat.size());
+        dx.upload(flat, dx.size());
         vq_tree *tree = nullptr;
         dev->check(vq_tsvq_build(dev->ctx(), dx.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)max_depth,
                                  &tree));
@@ -628,23 +682,27 @@ public:
     // src/tsvq.rs:231-249
     Vector<f16> quantize(const Vector<float> &vector) const {
         if (vector.len() != dim_) throw VqError::DimensionMismatch(dim_, vector.len());
-        return quantize_batch({vector})[0];
+        return quantize_batch(std::vector<Vector<float>>{vector})[0];
     }
 
-    std::vector<Vector<f16>> quantize_batch(const std::vector<Vector<float>> &vectors,
-                                            std::vector<int32_t> *leaves = nullptr) const {
+    std::vector<Vector<f16>> quantize_batch(const Rows &vectors, std::vector<int32_t> *leaves = nullptr) const {
+        return unpack_f16(quantize_batch_flat(vectors, leaves), vectors.size(), dim_);
+    }
+
+    std::vector<uint16_t> quantize_batch_flat(const Rows &vectors, std::vector<int32_t> *leaves = nullptr) const {
         size_t n = vectors.size();
         if (n == 0) return {};
-        std::vector<float> flat = pack_rows(vectors, dim_);
+        vectors.expect_dim(dim_);
+        const float *flat = vectors.data();
         DeviceBuffer<float> dx(dev_, n * dim_);
-        dx.upload(flat.data(), flat.size());
+        dx.upload(flat, dx.size());
         DeviceBuffer<int32_t> dleaf(dev_, n);
         DeviceBuffer<uint16_t> dout(dev_, n * dim_);
         dev_->check(vq_tsvq_descend(dev_->ctx(), distance.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim_,
                                     tree_.get(), dleaf.get()));
         dev_->check(vq_tsvq_decode_f16(dev_->ctx(), tree_.get(), dleaf.get(), (int64_t)n, dout.get()));
         if (leaves) *leaves = dleaf.to_host();
-        return unpack_f16(dout.to_host(), n, dim_);
+        return dout.to_host();
     }
 
     int32_t n_nodes() const {

@@ -20,11 +20,10 @@ struct Obj {
     int64_t dim = 0;
 };
 
-std::vector<vq::Vector<float>> rows_of(const float *x, int64_t n, int64_t dim) {
-    std::vector<vq::Vector<float>> v((size_t)n);
-    for (int64_t i = 0; i < n; ++i) v[(size_t)i].data.assign(x + i * dim, x + (i + 1) * dim);
-    return v;
-}
+// The caller's rows are one contiguous array already: a view, no per-row vectors.  (The conversion
+// from the reference's `&[Vector<f32>]` shape is exercised by vqh_quantize, which goes through
+// `quantize(&Vector<f32>)`.)
+vq::Rows rows_of(const float *x, int64_t n, int64_t dim) { return vq::Rows::view(x, (size_t)n, (size_t)dim); }
 
 vq::IndexStreams streams_of(const uint32_t *init, size_t n_init, const uint32_t *reseed, size_t problems,
                             int32_t n_reseed) {
@@ -49,10 +48,8 @@ int guarded(F &&f) {
     }
 }
 
-void flatten(const std::vector<vq::Vector<vq::f16>> &q, uint16_t *out) {
-    size_t o = 0;
-    for (const auto &v : q)
-        for (const auto &h : v.data) out[o++] = h.bits;
+void flatten(const std::vector<uint16_t> &q, uint16_t *out) {
+    if (!q.empty()) std::memcpy(out, q.data(), q.size() * sizeof(uint16_t));
 }
 }  // namespace
 
@@ -155,11 +152,33 @@ int vqh_quantize_batch(void *obj, const float *x, int64_t n, int64_t dim, uint16
         Obj *o = (Obj *)obj;
         auto rows = rows_of(x, n, dim);
         switch (o->kind) {
-        case 1: flatten(o->pq->quantize_batch(rows), out); break;
-        case 2: flatten(o->opq->quantize_batch(rows), out); break;
-        case 3: flatten(o->rvq->quantize_batch(rows), out); break;
-        default: flatten(o->tsvq->quantize_batch(rows), out); break;
+        case 1: flatten(o->pq->quantize_batch_flat(rows), out); break;
+        case 2: flatten(o->opq->quantize_batch_flat(rows), out); break;
+        case 3: flatten(o->rvq->quantize_batch_flat(rows), out); break;
+        default: flatten(o->tsvq->quantize_batch_flat(rows), out); break;
         }
+    });
+}
+
+// The same through the reference's own shape, one heap-allocated Vector<f32> per row
+// (`&[Vector<f32>]` -> Vec<Vector<f16>>); row `short_row` (if >= 0) is cut to `short_len` floats.
+int vqh_quantize_batch_vectors(void *obj, const float *x, int64_t n, int64_t dim, int64_t short_row,
+                               int64_t short_len, uint16_t *out) {
+    return guarded([&] {
+        Obj *o = (Obj *)obj;
+        std::vector<vq::Vector<float>> rows((size_t)n);
+        for (int64_t i = 0; i < n; ++i)
+            rows[(size_t)i].data.assign(x + i * dim, x + i * dim + (i == short_row ? short_len : dim));
+        std::vector<vq::Vector<vq::f16>> q;
+        switch (o->kind) {
+        case 1: q = o->pq->quantize_batch(rows); break;
+        case 2: q = o->opq->quantize_batch(rows); break;
+        case 3: q = o->rvq->quantize_batch(rows); break;
+        default: q = o->tsvq->quantize_batch(rows); break;
+        }
+        size_t at = 0;
+        for (const auto &v : q)
+            for (const auto &h : v.data) out[at++] = h.bits;
     });
 }
 
@@ -172,7 +191,7 @@ int vqh_encode(void *obj, const float *x, int64_t n, int64_t dim, uint8_t *codes
         switch (o->kind) {
         case 1: c = o->pq->encode(rows); break;
         case 2: c = o->opq->encode(rows); break;
-        case 3: o->rvq->quantize_batch(rows, &c); break;
+        case 3: o->rvq->quantize_batch_flat(rows, &c); break;
         default: throw vq::VqError::InvalidParameter("TSVQ has leaves, not codes");
         }
         std::memcpy(codes, c.data(), c.size());
@@ -184,7 +203,7 @@ int vqh_leaves(void *obj, const float *x, int64_t n, int64_t dim, int32_t *leave
         Obj *o = (Obj *)obj;
         if (o->kind != 4) throw vq::VqError::InvalidParameter("not a TSVQ");
         std::vector<int32_t> l;
-        o->tsvq->quantize_batch(rows_of(x, n, dim), &l);
+        o->tsvq->quantize_batch_flat(rows_of(x, n, dim), &l);
         std::memcpy(leaves, l.data(), l.size() * sizeof(int32_t));
     });
 }
