@@ -55,6 +55,10 @@ def assert_same_tree(got, want):
     (20000, 8, 2, "normal"),   # nodes above 1024 rows -> midpoint-tree means
     (1, 4, 3, "normal"),
     (700, 6, 0, "normal"),     # max_depth 0: the root is a leaf
+    (30000, 32, 9, "normal"),  # dim a multiple of 8: squares on the whole GPU, then the chains
+    (12345, 128, 7, "normal"), # node sizes that are no multiples of 32
+    (9000, 64, 13, "normal"),  # deep: levels with more than 2048 nodes take the lane-per-sum kernel
+    (5000, 24, 5, "grid"),     # dim 24, tied variances and medians
 ])
 def test_build_matches_oracle(ctx, n, dim, depth, kind):
     rng = np.random.default_rng(n + depth)
