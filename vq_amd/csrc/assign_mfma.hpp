@@ -745,18 +745,34 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
             const int i = threadIdx.x + 256 * q;
             pre[q] = ag[(size_t)nx * chunk16 + (i < chunk16 ? i : chunk16 - 1)];
         }
+        // the A operands of the wave's four centroid tiles are read from LDS together (a tile past
+        // the last block reads the last block and is not multiplied): one LDS round trip per
+        // chunk instead of one per tile
+        u32x4 a1[4], a2[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            const int b = 4 * ch + c;
-            if (b < nb) {
-                const u32x4 a1 = lds_a[cur][b * 128 + lane], a2 = lds_a[cur][b * 128 + 64 + lane];
+            const int b = 4 * ch + c < nb ? 4 * ch + c : nb - 1;
+            a1[c] = lds_a[cur][b * 128 + lane];
+            a2[c] = lds_a[cur][b * 128 + 64 + lane];
+        }
+        // first instruction of every accumulator tile, then the second: the two instructions of a
+        // tile depend on each other and are kept seven others apart
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
+        for (int c = 0; c < 4; ++c) {
+            if (4 * ch + c < nb) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
                     acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8, a1), __builtin_bit_cast(bf16x8, b1[t]), acc[t][c], 0, 0, 0);
+                        __builtin_bit_cast(bf16x8, a1[c]), __builtin_bit_cast(bf16x8, b1[t]), acc[t][c], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (4 * ch + c < nb) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
                     acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8, a2), __builtin_bit_cast(bf16x8, b2[t]), acc[t][c], 0, 0, 0);
-                }
+                        __builtin_bit_cast(bf16x8, a2[c]), __builtin_bit_cast(bf16x8, b2[t]), acc[t][c], 0, 0, 0);
             }
         }
         if (more) {
