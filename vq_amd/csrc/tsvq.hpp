@@ -423,21 +423,6 @@ static __global__ void __launch_bounds__(256) k_iota_u32(uint32_t *__restrict__ 
     if (i < n) p[i] = (uint32_t)i;
 }
 
-// mids[2g], mids[2g+1] = the two middle values of the sorted segment g (equal for odd counts)
-static __global__ void k_seg_middles(const float *__restrict__ sorted, const uint2 *__restrict__ seg_range,
-                              int nseg, float *__restrict__ mids) {
-    int g = blockIdx.x * blockDim.x + threadIdx.x;
-    if (g >= nseg) return;
-    uint2 r = seg_range[g];
-    uint32_t c = r.y - r.x;
-    if (c % 2 == 0) {
-        mids[2 * g] = sorted[r.x + c / 2 - 1];
-        mids[2 * g + 1] = sorted[r.x + c / 2];
-    } else {
-        mids[2 * g] = mids[2 * g + 1] = sorted[r.x + c / 2];
-    }
-}
-
 // ---- middle values by radix select ---------------------------------------------------------
 // The reference sorts the split column and takes values[c/2] (and values[c/2 - 1] for an even
 // count, src/tsvq.rs:108-117); only those two order statistics are needed.  Floats are mapped to
