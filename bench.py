@@ -52,7 +52,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
-            "(the path shards by rows, see DESIGN.md, but no multi-GPU code is built).")
+            "(the path would shard by rows, one exchange of per-part sums per LBG iteration, "
+            "but no multi-GPU code is built).")
         sys.exit(2)
 
     import vq_amd
