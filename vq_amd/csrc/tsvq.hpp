@@ -138,7 +138,7 @@ static __global__ void __launch_bounds__(256) k_seg_sqdev32(const uint32_t *__re
 // neighbouring lanes own one column: lane 8 cc + j loads positions 4j .. 4j+3 of column cc of a
 // group — one 16-byte load per lane moves 32 positions of 8 columns, 1 KB contiguous per wave —
 // and the first lane of the eight adds the 32 values in position order, its neighbours' values
-// read through DPP row shifts folded into the adds.  A lane keeps kChainRing loads in flight: 768
+// fetched by DPP row-shift moves.  A lane keeps kChainRing loads in flight: 768
 // positions per wave cover a memory round trip of 3 us at 3-4 ns per position with a ring of 96
 // registers; one 16-byte load per 4 positions of a lane's own column could keep 240 in flight at
 // most (the counter of outstanding loads holds 63) and measured 12 ns per position.
@@ -147,7 +147,13 @@ constexpr int kChainRing = 24;
 template <int J>
 __device__ __forceinline__ float lane_ahead(float v) {  // the value of the lane J places up in its row of 16
     static_assert(J >= 1 && J <= 15, "row shift");
-    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x100 + J, 0xF, 0xF, true));
+    float r = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x100 + J, 0xF, 0xF, true));
+    // The move stays a move (the compiler would fold it into the add as a DPP operand): an add
+    // with a DPP operand has a longer latency than a plain one, and the adds are one dependent
+    // chain, while the moves are independent and issue in its shadow (measured: 11 -> 8.6 cycles
+    // per position).
+    asm volatile("" : "+v"(r));
+    return r;
 }
 
 static __global__ void __launch_bounds__(256) k_seg_chain32(const float *__restrict__ sq32,
