@@ -105,7 +105,7 @@ def main():
         streams = data.index_streams(n, m, k, iters, seed=1)
         t0 = time.perf_counter()
         q = api.OptimizedProductQuantizer.fit(x, m, k, iters, outer, api.Distance.Euclidean, 0, streams=streams)
-        out["c3_opq_fit_host_classes_ms_incl_pack_upload_and_host_svd"] = (time.perf_counter() - t0) * 1e3
+        out["c3_opq_fit_host_classes_ms_incl_pack_and_upload"] = (time.perf_counter() - t0) * 1e3
         R = q.rotation().astype(np.float64)
         out["c3_rotation_orthogonality_err"] = float(np.abs(R.T @ R - np.eye(dim)).max())
         dx = ctx.to_device(x)

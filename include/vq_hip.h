@@ -186,6 +186,11 @@ int32_t vq_rotate(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t 
  * src/opq.rs:172-179, accumulated in f64 in a fixed order.  dim <= 128.  Synchronises. */
 int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n, int32_t dim, double *h_A);
 
+/* h_R = V U^T for h_A = U S V^T (both dim x dim, row-major, host memory): the rotation update of
+ * src/opq.rs:180-183, by a one-sided Jacobi SVD in f64 on the device.  dim even, 2 <= dim <= 128.
+ * Synchronises. */
+int32_t vq_procrustes_rotation(vq_ctx *ctx, const double *h_A, int32_t dim, double *h_R);
+
 /* ---- tree-structured VQ (src/tsvq.rs) ------------------------------------------------------ */
 
 typedef struct vq_tree vq_tree;

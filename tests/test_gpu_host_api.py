@@ -112,7 +112,7 @@ def test_opq_first_outer_iteration_matches_oracle(vq):
     want = O.opq_fit(O.EUCLIDEAN, x, m, k, iters, 1, *streams)
     # codebooks of the first outer iteration are trained on un-rotated data: bit-exact
     assert np.array_equal(got.codebooks(), want["codebooks"])
-    # the rotation goes through a host SVD in both: equal to f32 rounding
+    # the rotation goes through a Jacobi SVD in both (device here, host there): equal to f32 rounding
     assert np.allclose(got.rotation(), want["rotation"], atol=2e-6)
     # three outer iterations: same reconstruction quality as the oracle's run (1e-3 relative)
     got3 = vq.OptimizedProductQuantizer.fit(x, m, k, iters, 3, vq.Distance.Euclidean, 0, streams=streams)

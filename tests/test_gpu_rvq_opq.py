@@ -138,6 +138,34 @@ def test_cross_cov_matches_f64_product(ctx, n, dim):
     assert np.array_equal(A, ctx.cross_cov(ctx.to_device(y), ctx.to_device(x), n, dim))
 
 
+@pytest.mark.parametrize("dim", [2, 4, 10, 16, 64, 128])
+def test_procrustes_rotation_is_the_polar_factor(ctx, dim):
+    """The device rotation update (src/opq.rs:180-183: R = V U^T of svd(A)) against what the
+    mathematics fixes: R is orthogonal, R A is symmetric positive semi-definite with trace equal
+    to the nuclear norm of A, an orthogonal A gives A^T; and against the oracle's host SVD."""
+    rng = np.random.default_rng(dim)
+    A = (rng.standard_normal((dim, dim)) @ np.diag(rng.uniform(0.1, 50.0, dim))
+         @ rng.standard_normal((dim, dim))).astype(F).astype(np.float64)
+    R = ctx.procrustes_rotation(A)
+    assert np.allclose(R.T @ R, np.eye(dim), atol=1e-11)
+    P = R @ A
+    assert np.allclose(P, P.T, atol=1e-9 * np.abs(A).max())
+    assert np.linalg.eigvalsh((P + P.T) / 2).min() > -1e-9 * np.abs(A).max()
+    assert abs(np.trace(P) - np.linalg.svd(A, compute_uv=False).sum()) <= 1e-10 * np.abs(P).sum()
+    assert np.allclose(R, O.procrustes(A), atol=1e-9)
+    Q, _ = np.linalg.qr(rng.standard_normal((dim, dim)))
+    assert np.allclose(ctx.procrustes_rotation(Q), Q.T, atol=1e-12)
+    # a zero matrix has no unit singular vectors: zero comes back, as from the host routine
+    assert np.array_equal(ctx.procrustes_rotation(np.zeros((dim, dim))), O.procrustes(np.zeros((dim, dim))))
+
+
+def test_procrustes_rotation_rejects_sizes_outside_the_kernel(ctx):
+    import vq_amd
+    for dim in (3, 130):
+        with pytest.raises(vq_amd.VqError):
+            ctx.procrustes_rotation(np.eye(dim))
+
+
 def test_opq_outer_iteration_stepwise(ctx):
     """One OPQ outer iteration (src/opq.rs:124-195) on the GPU, every step checked against the
     oracle on identical inputs; the rotation's rounding is the only tolerance."""

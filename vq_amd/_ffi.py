@@ -29,6 +29,7 @@ SYMBOLS = {
     "vq_ctx_set_assign_path": (_i32, [_vp, _i32]),
     "vq_ctx_last_recheck_count": (_i32, [_vp, C.POINTER(C.c_uint32)]),
     "vq_ctx_last_recheck_split": (_i32, [_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
+    "vq_procrustes_rotation": (_i32, [_vp, _vp, _i32, _vp]),
     "vq_malloc": (_i32, [_vp, _sz, C.POINTER(_vp)]),
     "vq_free": (_i32, [_vp, _vp]),
     "vq_h2d": (_i32, [_vp, _vp, _vp, _sz]),
@@ -274,6 +275,12 @@ class Context:
         A = np.empty((dim, dim), np.float64)
         self._check(_lib.vq_cross_cov(self._h, d_y.ptr, d_x.ptr, n, dim, A.ctypes.data))
         return A
+
+    def procrustes_rotation(self, A):
+        A = np.ascontiguousarray(A, np.float64)
+        R = np.empty_like(A)
+        self._check(_lib.vq_procrustes_rotation(self._h, A.ctypes.data, A.shape[0], R.ctypes.data))
+        return R
 
     # -- tree-structured VQ --------------------------------------------------------------------
     def tsvq_build(self, d_x, n, ld, dim, max_depth):

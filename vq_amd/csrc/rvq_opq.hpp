@@ -416,3 +416,194 @@ static __global__ void __launch_bounds__(256) k_rotate_mfma(const float *__restr
 }
 
 }  // namespace vq
+
+// ---- orthogonal Procrustes (src/opq.rs:180-183) -------------------------------------------------
+// R = V U^T for A = U S V^T by a one-sided Jacobi SVD in f64.  The columns of A are made orthogonal
+// by plane rotations; V is the product of those rotations.  The rotations depend on the columns of
+// A only, never on V, so the work is split in three:
+//   k_jacobi_sweeps      one workgroup, the columns of A as rows of ut in LDS (n <= 128, n even:
+//                        133 KB).  A round rotates n / 2 disjoint pairs at once, sixteen lanes per
+//                        pair (round-robin pairing: n - 1 rounds are a sweep over all pairs), and
+//                        writes each rotation (c, s) to a list.  Sweeps stop when no pair is
+//                        further from orthogonal than 1e-15, as in the host routine.
+//   k_jacobi_accumulate  replays the list on V, one wave per row of V: lane g holds the two
+//                        entries that pair g of the round rotates, and the entries move one lane
+//                        along after every round as the pairing does, so nothing leaves registers.
+//   k_jacobi_product     out = V U^T with the columns of U scaled to unit length.
+// Pair g of round r is (a, b) = ((r + g) mod (n - 1), (r - g) mod (n - 1)), pair 0 is (r, n - 1);
+// its rotation maps (a, b) to (c a - s b, s a + c b).
+namespace vq {
+
+constexpr int kJacobiMax = 128;
+constexpr int kJacobiSweeps = 60;
+constexpr int kJacobiStride = kJacobiMax + 16;  // rows one apart are half the LDS banks apart
+
+// the value of the lane that a DPP control names (quad permutation, row mirror ...)
+template <int CTRL> __device__ __forceinline__ double dpp_f64(double v) {
+    const long long bits = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)bits, CTRL, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(bits >> 32), CTRL, 0xf, 0xf, false);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
+}
+// sum over the LANES (4, 8 or 16) adjacent lanes of a pair, in every one of them
+template <int LANES> __device__ __forceinline__ double pair_sum(double v) {
+    v += dpp_f64<0xB1>(v);  // quad_perm [1,0,3,2]
+    v += dpp_f64<0x4E>(v);  // quad_perm [2,3,0,1]
+    if (LANES >= 8) v += dpp_f64<0x141>(v);   // row_half_mirror: the other quad of the eight
+    if (LANES == 16) v += dpp_f64<0x128>(v);  // row_ror 8: the other eight of the sixteen
+    return v;
+}
+// 1 / x and 1 / sqrt(x) to within a few ulp for positive normal x: the hardware's estimate and two
+// Newton steps (the rotations need c^2 + s^2 = 1 to rounding, not correctly rounded quotients)
+__device__ __forceinline__ double rcp_newton(double x) {
+    double r = __builtin_amdgcn_rcp(x);
+    r = fma(fma(-x, r, 1.0), r, r);
+    return fma(fma(-x, r, 1.0), r, r);
+}
+__device__ __forceinline__ double rsq_newton(double x) {
+    double y = __builtin_amdgcn_rsq(x);
+    y = fma(fma(-x * y, y, 1.0), 0.5 * y, y);
+    return fma(fma(-x * y, y, 1.0), 0.5 * y, y);
+}
+
+// LANES lanes per pair, 64 * LANES threads; a lane holds 128 / LANES entries of both rows.  Rows
+// are kJacobiMax long whatever n is: the entries from n on are zero and stay zero.
+template <int LANES>
+static __global__ void __launch_bounds__(64 * LANES) k_jacobi_sweeps(const double *__restrict__ A, int n,
+                                                                      double2 *__restrict__ rot,
+                                                                      int *__restrict__ n_rounds,
+                                                                      double *__restrict__ uhat) {
+    extern __shared__ __attribute__((aligned(16))) double ut[];  // n rows of stride kJacobiStride
+    __shared__ int unfinished;
+    constexpr int S = kJacobiStride, NT = 64 * LANES, PER = kJacobiMax / (2 * LANES);
+    const int tid = threadIdx.x, pair = tid / LANES, sub = tid % LANES;
+    for (int e = tid; e < n * kJacobiMax; e += NT) {
+        const int j = e / kJacobiMax, i = e % kJacobiMax;
+        ut[j * S + i] = i < n ? A[(size_t)i * n + j] : 0.0;  // row j of ut = column j of A
+    }
+    if (tid == 0) unfinished = 0;
+    __syncthreads();
+    const int half = n / 2;
+    int round = 0;
+    for (int sweep = 0; sweep < kJacobiSweeps; ++sweep) {
+        for (int r = 0; r < n - 1; ++r, ++round) {
+            if (pair < half) {
+                const int p = (r + pair) % (n - 1);
+                const int q = pair == 0 ? n - 1 : (r - pair + (n - 1)) % (n - 1);
+                double2 *up = reinterpret_cast<double2 *>(ut + p * S) + sub;
+                double2 *uq = reinterpret_cast<double2 *>(ut + q * S) + sub;
+                double2 a[PER], b[PER];
+#pragma unroll
+                for (int j = 0; j < PER; ++j) {
+                    a[j] = up[LANES * j];
+                    b[j] = uq[LANES * j];
+                }
+                double alpha = 0.0, beta = 0.0, gamma = 0.0;
+#pragma unroll
+                for (int j = 0; j < PER; ++j) {
+                    alpha = fma(a[j].x, a[j].x, alpha);
+                    beta = fma(b[j].x, b[j].x, beta);
+                    gamma = fma(a[j].x, b[j].x, gamma);
+                    alpha = fma(a[j].y, a[j].y, alpha);
+                    beta = fma(b[j].y, b[j].y, beta);
+                    gamma = fma(a[j].y, b[j].y, gamma);
+                }
+                alpha = pair_sum<LANES>(alpha);
+                beta = pair_sum<LANES>(beta);
+                gamma = pair_sum<LANES>(gamma);
+                // the pair counts as orthogonal below a cosine of 1e-16 and is left alone; a
+                // cosine of 1e-15 or more asks for another sweep (the host routine's test)
+                const double g2 = gamma * gamma, ab = alpha * beta;
+                double c = 1.0, s = 0.0;
+                if (g2 > 1e-32 * ab) {  // the same in the lanes of a pair
+                    if (sub == 0 && g2 >= 1e-30 * ab) __atomic_store_n(&unfinished, 1, __ATOMIC_RELAXED);
+                    // tan of the angle that makes the rows orthogonal: the smaller root of
+                    // t^2 + 2 zeta t - 1 = 0, zeta = delta / gamma, written without the quotient
+                    const double delta = 0.5 * (beta - alpha);
+                    const double h2 = fma(delta, delta, g2);
+                    const double hyp = h2 * rsq_newton(h2);
+                    const double t = (delta >= 0.0 ? gamma : -gamma) * rcp_newton(fabs(delta) + hyp);
+                    c = rsq_newton(fma(t, t, 1.0));
+                    s = c * t;
+#pragma unroll
+                    for (int j = 0; j < PER; ++j) {
+                        up[LANES * j] = make_double2(fma(c, a[j].x, -(s * b[j].x)), fma(c, a[j].y, -(s * b[j].y)));
+                        uq[LANES * j] = make_double2(fma(s, a[j].x, c * b[j].x), fma(s, a[j].y, c * b[j].y));
+                    }
+                }
+                if (sub == 0) rot[(size_t)round * half + pair] = make_double2(c, s);
+            }
+            __syncthreads();
+        }
+        const int more = __atomic_load_n(&unfinished, __ATOMIC_RELAXED);
+        __syncthreads();
+        if (tid == 0) unfinished = 0;
+        __syncthreads();
+        if (!more) break;  // the same in every thread
+    }
+    if (tid == 0) *n_rounds = round;
+    // unit columns of U; a zero column stays zero
+    for (int j = pair; j < n; j += 64) {
+        double s = 0.0;
+        for (int i = sub; i < n; i += LANES) s += ut[j * S + i] * ut[j * S + i];
+        s = sqrt(pair_sum<LANES>(s));
+        for (int i = sub; i < n; i += LANES) uhat[(size_t)j * n + i] = s > 0.0 ? ut[j * S + i] / s : ut[j * S + i];
+    }
+}
+
+constexpr int kJacobiRing = 16;
+
+// vt[l][i] = V[i][l]; grid = n workgroups of one wave, workgroup i makes row i of V
+static __global__ void __launch_bounds__(64) k_jacobi_accumulate(const double2 *__restrict__ rot,
+                                                                 const int *__restrict__ n_rounds, int n,
+                                                                 double *__restrict__ vt) {
+    const int i = blockIdx.x, g = threadIdx.x, half = n / 2;
+    const int rounds = *n_rounds;
+    const bool act = g < half;
+    const int gl = act ? g : 0;  // idle lanes follow lane 0's addresses and keep nothing
+    // seats of round 0: a = g, b = n - 1 - g (pair 0: n - 1)
+    double xa = (act && g == i) ? 1.0 : 0.0;
+    double xb = (act && (g == 0 ? n - 1 : n - 1 - g) == i) ? 1.0 : 0.0;
+    const int from_up = min(g + 1, 63), from_down = max(g - 1, 0);
+    double2 cs[kJacobiRing];
+#pragma unroll
+    for (int j = 0; j < kJacobiRing; ++j) {
+        cs[j] = rot[(size_t)min(j, rounds - 1) * half + gl];
+        asm volatile("" ::: "memory");
+    }
+    for (int t0 = 0; t0 < rounds; t0 += kJacobiRing) {
+#pragma unroll
+        for (int j = 0; j < kJacobiRing; ++j) {
+            const double c = cs[j].x, s = cs[j].y;
+            cs[j] = rot[(size_t)min(t0 + j + kJacobiRing, rounds - 1) * half + gl];
+            if (t0 + j < rounds) {  // the same in every lane
+                const double na = c * xa - s * xb, nb = s * xa + c * xb;
+                // the pairing of the next round: a moves down a lane, b up; the ends cross over
+                const double a_up = __shfl(na, from_up), b_down = __shfl(nb, from_down);
+                const double a0 = __shfl(na, 0);
+                xa = (g == half - 1 && half > 1) ? nb : (half > 1 ? a_up : na);  // n = 2: nothing moves
+                xb = g == 0 ? nb : (g == 1 ? a0 : b_down);
+            }
+        }
+    }
+    if (act) {
+        const int r = rounds % (n - 1);
+        const int ia = (r + g) % (n - 1), ib = g == 0 ? n - 1 : (r - g + (n - 1)) % (n - 1);
+        vt[(size_t)ia * n + i] = xa;
+        vt[(size_t)ib * n + i] = xb;
+    }
+}
+
+// out[i][j] = sum_l V[i][l] U[j][l], l ascending
+static __global__ void __launch_bounds__(256) k_jacobi_product(const double *__restrict__ vt,
+                                                               const double *__restrict__ uhat, int n,
+                                                               double *__restrict__ out) {
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= n * n) return;
+    const int i = e / n, j = e % n;
+    double acc = 0.0;
+    for (int l = 0; l < n; ++l) acc += vt[(size_t)l * n + i] * uhat[(size_t)l * n + j];
+    out[e] = acc;
+}
+
+}  // namespace vq

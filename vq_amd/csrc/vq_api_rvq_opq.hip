@@ -181,4 +181,39 @@ int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n,
     return VQ_OK;
 }
 
+int32_t vq_procrustes_rotation(vq_ctx *ctx, const double *h_A, int32_t dim, double *h_R) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (!h_A || !h_R || dim < 2) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    if (dim > vq::kJacobiMax || dim % 2 != 0)
+        return fail(ctx, VQ_ERR_UNSUPPORTED, "rotation update: dim %d is odd or above %d", dim, vq::kJacobiMax);
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    const size_t total = (size_t)dim * dim;
+    const int half = dim / 2;
+    VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(double) * total));
+    VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * total));
+    VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(double) * total));
+    VQ_TRY(ensure(ctx, ctx->tmp_d, sizeof(double) * total));
+    VQ_TRY(ensure(ctx, ctx->tmp_e, sizeof(double2) * (size_t)vq::kJacobiSweeps * (dim - 1) * half));
+    VQ_TRY(ensure(ctx, ctx->tmp_f, 256));
+    double *d_A = (double *)ctx->tmp_a.p, *d_vt = (double *)ctx->tmp_b.p, *d_uhat = (double *)ctx->tmp_c.p;
+    double *d_out = (double *)ctx->tmp_d.p;
+    double2 *d_rot = (double2 *)ctx->tmp_e.p;
+    int *d_rounds = (int *)ctx->tmp_f.p;
+    VQ_HIP(ctx, hipMemcpyAsync(d_A, h_A, sizeof(double) * total, hipMemcpyHostToDevice, ctx->stream));
+    constexpr int kLanes = 8;
+    const size_t lds = sizeof(double) * (size_t)dim * vq::kJacobiStride;
+    VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(vq::k_jacobi_sweeps<kLanes>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(vq::k_jacobi_sweeps<kLanes>, dim3(1), dim3(64 * kLanes), lds, ctx->stream, (const double *)d_A,
+                       dim, d_rot, d_rounds, d_uhat);
+    hipLaunchKernelGGL(vq::k_jacobi_accumulate, dim3(dim), dim3(64), 0, ctx->stream, (const double2 *)d_rot,
+                       (const int *)d_rounds, dim, d_vt);
+    hipLaunchKernelGGL(vq::k_jacobi_product, dim3((unsigned)cdiv(total, 256)), dim3(256), 0, ctx->stream,
+                       (const double *)d_vt, (const double *)d_uhat, dim, d_out);
+    VQ_HIP(ctx, hipGetLastError());
+    VQ_HIP(ctx, hipMemcpyAsync(h_R, d_out, sizeof(double) * total, hipMemcpyDeviceToHost, ctx->stream));
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return VQ_OK;
+}
+
 }  // extern "C"

@@ -492,7 +492,13 @@ public:
                                      q.codebooks_.get(), drec.get()));                            // 164-167
             dev->check(vq_cross_cov(c, drec.get(), drot.get(), (int64_t)n, (int32_t)dim, A.data())); // 172-179
             for (double &v : A) v = (double)(float)v;  // the reference's A is a DMatrix<f32>
-            procrustes_rotation(A, dim, Rd);           // 180-183, on the host
+            // 180-183: on the device while its kernel takes the size, else on the host
+            if (dim % 2 == 0 && dim >= 2 && dim <= 128) {
+                Rd.resize(dim * dim);
+                dev->check(vq_procrustes_rotation(c, A.data(), (int32_t)dim, Rd.data()));
+            } else {
+                procrustes_rotation(A, dim, Rd);
+            }
             for (size_t i = 0; i < dim * dim; ++i) q.rotation_[i] = (float)Rd[i];
             q.d_rotation_.upload(q.rotation_.data(), dim * dim);
             dev->check(vq_rotate(c, dx.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, q.d_rotation_.get(),
