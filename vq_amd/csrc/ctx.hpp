@@ -20,6 +20,9 @@ struct vq_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // second stream of the LBG update: the small clusters' gather path runs beside the streaming sums
+    hipStream_t side = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
     std::string err;
     // grow-only device workspace
     DevBuf flags, tables, hist, seg, part_sum, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;

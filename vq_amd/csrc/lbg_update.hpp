@@ -54,6 +54,10 @@ struct LbgState {
     int stream;            // 1: the large clusters are summed by k_lbg_stream8 / k_lbg_combine8
 };
 
+// The short kernels of the gather path run beside the streaming kernel, whose waves keep the
+// vector ALU busy: their waves are given the higher issue priority, or they would wait for it.
+__device__ __forceinline__ void side_chain_priority() { __builtin_amdgcn_s_setprio(3); }
+
 static __global__ void k_lbg_init(LbgState st, int m) {
     int s = blockIdx.x * blockDim.x + threadIdx.x;
     if (s < m) {
@@ -82,6 +86,7 @@ static __global__ void k_gather_rows(const float *__restrict__ x, int64_t ld, in
 
 // One wave per (part, column block): histogram of the codes of kPartRows rows.
 static __global__ void __launch_bounds__(64) k_lbg_hist(LbgState st, int64_t n) {
+    side_chain_priority();
     const int s = blockIdx.y, b = blockIdx.x;
     if (st.done[s]) return;
     __shared__ uint32_t cnt[kMaxK];
@@ -90,7 +95,24 @@ static __global__ void __launch_bounds__(64) k_lbg_hist(LbgState st, int64_t n) 
     const uint8_t *codes = st.codes + (size_t)s * n;
     int64_t lo = (int64_t)b * kPartRows;
     int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
-    for (int64_t i = lo + threadIdx.x; i < hi; i += 64) atomicAdd(&cnt[codes[i]], 1u);
+    if (hi - lo == kPartRows && ((uintptr_t)(codes + lo) & 15) == 0) {
+        // a full part: every lane takes 64 consecutive codes with four loads in flight together
+        // (a histogram does not care which lane counts which row)
+        const uint4 *cp = reinterpret_cast<const uint4 *>(codes + lo) + threadIdx.x * 4;
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = cp[u];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t w[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int sh = 0; sh < 32; sh += 8) atomicAdd(&cnt[(w[q] >> sh) & 255u], 1u);
+        }
+    } else {
+        for (int64_t i = lo + threadIdx.x; i < hi; i += 64) atomicAdd(&cnt[codes[i]], 1u);
+    }
     __syncthreads();
     uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
     for (int j = threadIdx.x; j < kMaxK; j += 64) h[j] = cnt[j];
@@ -98,6 +120,7 @@ static __global__ void __launch_bounds__(64) k_lbg_hist(LbgState st, int64_t n) 
 
 // Scan step 1: per (column block, segment of kScanSeg parts) sum of the histograms.
 static __global__ void __launch_bounds__(256) k_lbg_scan_seg(LbgState st) {
+    side_chain_priority();
     const int s = blockIdx.y, g = blockIdx.x, j = threadIdx.x;
     if (st.done[s]) return;
     const int b0 = g * kScanSeg, b1 = (b0 + kScanSeg < st.nparts) ? b0 + kScanSeg : st.nparts;
@@ -118,6 +141,7 @@ static __global__ void __launch_bounds__(256) k_lbg_scan_seg(LbgState st) {
 // Leaves: a small cluster (1..1024 members) is one leaf over its whole member list; a large
 // cluster has one leaf per part, unless the streaming kernel sums the large clusters.
 static __global__ void __launch_bounds__(256) k_lbg_plan(LbgState st, int k) {
+    side_chain_priority();
     const int s = blockIdx.x, j = threadIdx.x;
     if (st.done[s]) return;
     __shared__ uint32_t sh_cnt[kMaxK], sh_leaf[kMaxK], sh_empty[kMaxK], sh_small[kMaxK];
@@ -171,6 +195,7 @@ static __global__ void __launch_bounds__(256) k_lbg_plan(LbgState st, int k) {
 // of part b inside cluster j), in place; emits the per-part leaves of the large clusters when
 // they are summed by the gather path.
 static __global__ void __launch_bounds__(256) k_lbg_scan_blocks(LbgState st) {
+    side_chain_priority();
     const int s = blockIdx.y, g = blockIdx.x, j = threadIdx.x;
     if (st.done[s]) return;
     const int b0 = g * kScanSeg, b1 = (b0 + kScanSeg < st.nparts) ? b0 + kScanSeg : st.nparts;
@@ -198,12 +223,16 @@ static __global__ void __launch_bounds__(256) k_lbg_scan_blocks(LbgState st) {
 // One wave per (part, column block): stable ranked scatter of row ids into perm[s].  When the
 // streaming kernel sums the large clusters only the rows of small clusters are listed.
 static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t n) {
+    side_chain_priority();
     const int s = blockIdx.y, b = blockIdx.x;
     if (st.done[s]) return;
     if (st.stream && st.nsmall[s] == 0) return;
     __shared__ uint32_t base[kMaxK];
     __shared__ uint8_t listed[kMaxK];
-    __shared__ uint8_t pcodes[kPartRows];
+    // codes are staged a quarter of the part at a time (16 per lane, the next quarter's load in
+    // flight meanwhile): the workgroup keeps 2.3 KB of LDS and fits beside the streaming kernel
+    constexpr int kStage = kPartRows / 4;
+    __shared__ __attribute__((aligned(16))) uint8_t pcodes[kStage];
     const uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
     const uint32_t *start = st.start + (size_t)s * kMaxK;
     const uint32_t *count = st.count + (size_t)s * kMaxK;
@@ -217,43 +246,63 @@ static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t 
     const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     int64_t lo = (int64_t)b * kPartRows;
     int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
-    for (int64_t i = lo + lane; i < hi; i += 64) pcodes[i - lo] = codes[i];  // one round trip
-    __syncthreads();
-    for (int64_t i0 = lo; i0 < hi; i0 += 64) {
-        int64_t i = i0 + lane;
-        bool valid = i < hi;
-        uint32_t c = valid ? pcodes[i - lo] : 0u;
-        valid = valid && listed[c];
-        uint64_t mask = __ballot(valid);
-        if (mask == 0) continue;  // uniform
-        if (__popcll(mask) <= 4) {
-            // few listed rows (the small clusters beside the streaming kernel): one lane at a time,
-            // in lane = row order; LDS operations of one wave are performed in program order
-            for (uint64_t mm = mask; mm; mm &= mm - 1) {
-                if (lane == __ffsll((unsigned long long)mm) - 1) {
-                    const uint32_t pos = base[c];
-                    base[c] = pos + 1;
-                    perm[pos] = (uint32_t)i;
+    const bool vec = ((uintptr_t)(codes + lo) & 15) == 0;
+    auto fetch = [&](int64_t q0) {  // codes of rows q0 + 16 lane .. + 15; rows from hi on read as 0, never used
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        const int64_t r0 = q0 + 16 * lane;
+        if (vec && r0 + 16 <= hi) {
+            v = *reinterpret_cast<const uint4 *>(codes + r0);
+        } else {
+            uint32_t w[4] = {0u, 0u, 0u, 0u};
+            for (int u = 0; u < 16; ++u)
+                if (r0 + u < hi) w[u >> 2] |= (uint32_t)codes[r0 + u] << (8 * (u & 3));
+            v = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+        return v;
+    };
+    uint4 ahead = fetch(lo);
+    for (int64_t q0 = lo; q0 < hi; q0 += kStage) {
+        __syncthreads();  // the previous quarter has been consumed (and base / listed are written)
+        reinterpret_cast<uint4 *>(pcodes)[lane] = ahead;
+        if (q0 + kStage < hi) ahead = fetch(q0 + kStage);
+        __syncthreads();
+        const int64_t qhi = q0 + kStage < hi ? q0 + kStage : hi;
+        for (int64_t i0 = q0; i0 < qhi; i0 += 64) {
+            int64_t i = i0 + lane;
+            bool valid = i < hi;
+            uint32_t c = valid ? pcodes[i - q0] : 0u;
+            valid = valid && listed[c];
+            uint64_t mask = __ballot(valid);
+            if (mask == 0) continue;  // uniform
+            if (__popcll(mask) <= 4) {
+                // few listed rows (the small clusters beside the streaming kernel): one lane at a time,
+                // in lane = row order; LDS operations of one wave are performed in program order
+                for (uint64_t mm = mask; mm; mm &= mm - 1) {
+                    if (lane == __ffsll((unsigned long long)mm) - 1) {
+                        const uint32_t pos = base[c];
+                        base[c] = pos + 1;
+                        perm[pos] = (uint32_t)i;
+                    }
+                    __builtin_amdgcn_wave_barrier();
                 }
-                __builtin_amdgcn_wave_barrier();
+                continue;
             }
-            continue;
+    #pragma unroll
+            for (int bit = 0; bit < 8; ++bit) {
+                bool set = (c >> bit) & 1u;
+                uint64_t bal = __ballot(set);
+                mask &= set ? bal : ~bal;
+            }
+            // lanes with equal code and valid: mask (invalid lanes have a stale mask, unused)
+            uint32_t rank = (uint32_t)__popcll(mask & lt);
+            uint32_t tot = (uint32_t)__popcll(mask);
+            uint32_t pos = 0;
+            if (valid) pos = base[c] + rank;
+            __builtin_amdgcn_wave_barrier();  // one wave, LDS in program order: reads above, updates below
+            if (valid && rank == 0) base[c] += tot;
+            __builtin_amdgcn_wave_barrier();
+            if (valid) perm[pos] = (uint32_t)i;
         }
-#pragma unroll
-        for (int bit = 0; bit < 8; ++bit) {
-            bool set = (c >> bit) & 1u;
-            uint64_t bal = __ballot(set);
-            mask &= set ? bal : ~bal;
-        }
-        // lanes with equal code and valid: mask (invalid lanes have a stale mask, unused)
-        uint32_t rank = (uint32_t)__popcll(mask & lt);
-        uint32_t tot = (uint32_t)__popcll(mask);
-        uint32_t pos = 0;
-        if (valid) pos = base[c] + rank;
-        __builtin_amdgcn_wave_barrier();  // one wave, LDS in program order: reads above, updates below
-        if (valid && rank == 0) base[c] += tot;
-        __builtin_amdgcn_wave_barrier();
-        if (valid) perm[pos] = (uint32_t)i;
     }
 }
 
@@ -357,6 +406,7 @@ constexpr int kLeafWgFloats = 8192;  // floats staged per chunk
 
 static __global__ void __launch_bounds__(256) k_lbg_leafsum_wg(LbgState st, const float *__restrict__ x, int64_t n,
                                                                int64_t ld, int sd, int sd_shift) {
+    side_chain_priority();
     const int s = blockIdx.y;
     if (st.done[s]) return;
     const int64_t leaf = blockIdx.x;
@@ -477,7 +527,9 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const 
 // chunk are ranked inside their cluster with wave ballots and added to the cluster's
 // accumulator in LDS in rank order (round r: the lanes of rank r, all on different clusters) —
 // so every cluster receives its rows of this part in row order, one at a time, starting from
-// 0.0.  Emits the part's histogram and the per-part sums; no floating-point atomics.
+// 0.0.  Emits the per-part sums and, with HIST, the part's histogram (without it k_lbg_hist
+// counts, on another stream at the same time); no floating-point atomics.
+template <bool HIST>
 static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const float *__restrict__ x, int64_t n,
                                                             int64_t ld) {
     const int g = blockIdx.y, b = blockIdx.x;
@@ -564,7 +616,7 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
             const uint32_t same_lo = ~bad_lo, same_hi = ~bad_hi;
             const uint32_t rank =
                 pending ? (uint32_t)(__popc(same_lo & lt_lo) + __popc(same_hi & lt_hi)) : 0xFFFFFFFFu;
-            if (rank == 0) atomicAdd(&cnt[c], (uint32_t)(__popc(same_lo) + __popc(same_hi)));  // one lane per cluster
+            if (HIST && rank == 0) atomicAdd(&cnt[c], (uint32_t)(__popc(same_lo) + __popc(same_hi)));  // one lane per cluster
             // Round r: the lanes of rank r (all on different clusters) add their rows.  LDS
             // operations of one wave are performed in program order, so the next round sees these
             // writes; the wave barrier only pins the compiler's schedule (a fence or s_barrier
@@ -590,8 +642,10 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
     __builtin_amdgcn_wave_barrier();
     float4 *ps = reinterpret_cast<float4 *>(st.part_sum) + ((size_t)s * st.nparts + b) * kMaxK * 2;
     for (int i = lane; i < kMaxK * 2; i += 64) ps[i] = (i & 1) ? ahi[i >> 1] : alo[i >> 1];
-    uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
-    for (int j = lane; j < kMaxK; j += 64) h[j] = cnt[j];
+    if (HIST) {
+        uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
+        for (int j = lane; j < kMaxK; j += 64) h[j] = cnt[j];
+    }
 }
 
 // One lane per (cluster, component): sequential fold of the per-part sums of a large cluster.

@@ -345,7 +345,10 @@ int32_t vq_ctx_create(int32_t device, vq_ctx **out) {
     if ((e = hipSetDevice(device)) != hipSuccess ||
         (e = hipStreamCreate(&ctx->stream)) != hipSuccess ||
         (e = hipEventCreate(&ctx->ev0)) != hipSuccess ||
-        (e = hipEventCreate(&ctx->ev1)) != hipSuccess) {
+        (e = hipEventCreate(&ctx->ev1)) != hipSuccess ||
+        (e = hipStreamCreate(&ctx->side)) != hipSuccess ||
+        (e = hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming)) != hipSuccess ||
+        (e = hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming)) != hipSuccess) {
         int32_t rc = fail(nullptr, VQ_ERR_HIP, "context set-up failed: %s", hipGetErrorString(e));
         delete ctx;
         return rc;
@@ -358,6 +361,7 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     if (!ctx) return VQ_OK;
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->side) (void)hipStreamSynchronize(ctx->side);
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
                       &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
@@ -367,6 +371,9 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     for (hipEvent_t e : ctx->prof_pool) (void)hipEventDestroy(e);
     (void)hipEventDestroy(ctx->ev0);
     (void)hipEventDestroy(ctx->ev1);
+    if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
+    if (ctx->ev_join) (void)hipEventDestroy(ctx->ev_join);
+    if (ctx->side) (void)hipStreamDestroy(ctx->side);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return VQ_OK;
@@ -593,30 +600,40 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
             VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd));
         }
         ProfSpan sp(ctx, VQ_PROF_LBG_UPDATE);
-        if (stream)
-            hipLaunchKernelGGL(vq::k_lbg_stream8, dim3(nparts, m / 4), dim3(256), 0, st, S, d_x, n, ld);
-        else
-            hipLaunchKernelGGL(vq::k_lbg_hist, dim3(nparts, m), dim3(64), 0, st, S, n);
-        hipLaunchKernelGGL(vq::k_lbg_scan_seg, dim3(nseg, m), dim3(256), 0, st, S);
-        hipLaunchKernelGGL(vq::k_lbg_plan, dim3(m), dim3(256), 0, st, S, k);
-        hipLaunchKernelGGL(vq::k_lbg_scan_blocks, dim3(nseg, m), dim3(256), 0, st, S);
-        if (stream)
-            hipLaunchKernelGGL(vq::k_lbg_combine8, dim3(cdiv((int64_t)k * 8, 256), m), dim3(256), 0, st, S, k,
-                               d_codebooks);
-        hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nparts, m), dim3(64), 0, st, S, n);
         int shift = 0;
         while ((1 << shift) < sd) ++shift;
-        if (stream && sd >= 4 && sd <= 32 && (1 << shift) == sd && ld % 4 == 0 &&
-            (reinterpret_cast<uintptr_t>(d_x) & 15) == 0) {
+        const bool leaf_wg = stream && sd >= 4 && sd <= 32 && (1 << shift) == sd && ld % 4 == 0 &&
+                             (reinterpret_cast<uintptr_t>(d_x) & 15) == 0;
+        // The gather path of the small clusters needs only the new codes: with the streaming sums
+        // it runs on the second stream beside them (a chain of short, latency-bound kernels next to
+        // one long pass over the rows), and the two meet again before the large clusters' fold.
+        hipStream_t gs = stream ? ctx->side : st;
+        if (stream) {
+            VQ_HIP(ctx, hipEventRecord(ctx->ev_fork, st));
+            VQ_HIP(ctx, hipStreamWaitEvent(gs, ctx->ev_fork, 0));
+            hipLaunchKernelGGL(vq::k_lbg_stream8<false>, dim3(nparts, m / 4), dim3(256), 0, st, S, d_x, n, ld);
+        }
+        hipLaunchKernelGGL(vq::k_lbg_hist, dim3(nparts, m), dim3(64), 0, gs, S, n);
+        hipLaunchKernelGGL(vq::k_lbg_scan_seg, dim3(nseg, m), dim3(256), 0, gs, S);
+        hipLaunchKernelGGL(vq::k_lbg_plan, dim3(m), dim3(256), 0, gs, S, k);
+        hipLaunchKernelGGL(vq::k_lbg_scan_blocks, dim3(nseg, m), dim3(256), 0, gs, S);
+        hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nparts, m), dim3(64), 0, gs, S, n);
+        if (leaf_wg) {
             // leaves are the few clusters of up to 1024 members beside the streaming kernel
-            hipLaunchKernelGGL(vq::k_lbg_leafsum_wg, dim3(leaf_cap, m), dim3(256), 0, st, S, d_x, n, ld, sd,
+            hipLaunchKernelGGL(vq::k_lbg_leafsum_wg, dim3(leaf_cap, m), dim3(256), 0, gs, S, d_x, n, ld, sd,
                                shift);
         } else if (sd <= 32 && (1 << shift) == sd) {
-            hipLaunchKernelGGL(vq::k_lbg_leafsum_wave, dim3(cdiv(leaf_cap, 4), m), dim3(256), 0, st, S, d_x, n,
+            hipLaunchKernelGGL(vq::k_lbg_leafsum_wave, dim3(cdiv(leaf_cap, 4), m), dim3(256), 0, gs, S, d_x, n,
                                ld, sd, shift);
         } else {
-            hipLaunchKernelGGL(vq::k_lbg_leafsum, dim3(cdiv((int64_t)leaf_cap * sd, 256), m), dim3(256), 0, st,
+            hipLaunchKernelGGL(vq::k_lbg_leafsum, dim3(cdiv((int64_t)leaf_cap * sd, 256), m), dim3(256), 0, gs,
                                S, d_x, n, ld, sd);
+        }
+        if (stream) {
+            VQ_HIP(ctx, hipEventRecord(ctx->ev_join, gs));
+            VQ_HIP(ctx, hipStreamWaitEvent(st, ctx->ev_join, 0));
+            hipLaunchKernelGGL(vq::k_lbg_combine8, dim3(cdiv((int64_t)k * 8, 256), m), dim3(256), 0, st, S, k,
+                               d_codebooks);
         }
         hipLaunchKernelGGL(vq::k_lbg_finalize, dim3(cdiv((int64_t)k * sd, 256), m), dim3(256), 0, st, S,
                            d_x, ld, k, sd, (const uint32_t *)ctx->reseed.p, n_reseed, d_codebooks);
