@@ -132,18 +132,14 @@ __device__ __forceinline__ uint32_t bf16_pack2(float a, float b) {
 // (k <= 256).  Rows and centroids are scored relative to mu[s] = mean of the block's centroids
 // (distances do not change under a common shift, the bound on the score error, which is
 // proportional to ||x - mu||^2 + ||c - mu||^2, does); maxc2[s] = largest ||c - mu||^2 of the
-// block (NaN if any is NaN).
-static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__restrict__ cb, int m, int k, int nb,
-                                                             u32x4 *__restrict__ atab, float *__restrict__ c2perm,
-                                                             float *__restrict__ maxc2, float *__restrict__ mu,
-                                                             uint32_t *__restrict__ stat) {
-    const int s = blockIdx.x, j = threadIdx.x;
+// block (NaN if any is NaN).  mfma_bf_prep_block is the work of one workgroup, given centroid j
+// of the block in thread j's registers (zeros from k on); k_mfma_bf_prep reads the centroids from
+// the codebook, the LBG loop's last update kernel has just computed them.
+__device__ __forceinline__ void mfma_bf_prep_block(float (&c)[8], int s, int j, int k, int nb,
+                                                   u32x4 *__restrict__ atab, float *__restrict__ c2perm,
+                                                   float *__restrict__ maxc2, float *__restrict__ mu) {
     __shared__ float sh_max[4];
     __shared__ float sh_mu[4][8];
-    if (s == 0 && j < kStatSlots) stat[j * kStatStride] = 0u;
-    float c[8];
-#pragma unroll
-    for (int t = 0; t < 8; ++t) c[t] = (j < k) ? cb[((size_t)s * k + j) * 8 + t] : 0.0f;
     // centre: sum of c / 256 (no overflow for k <= 256), then * 256 / k
     float centre[8];
 #pragma unroll
@@ -209,6 +205,18 @@ static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__rest
         }
         maxc2[s] = r;
     }
+}
+
+static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__restrict__ cb, int m, int k, int nb,
+                                                             u32x4 *__restrict__ atab, float *__restrict__ c2perm,
+                                                             float *__restrict__ maxc2, float *__restrict__ mu,
+                                                             uint32_t *__restrict__ stat) {
+    const int s = blockIdx.x, j = threadIdx.x;
+    if (s == 0 && j < kStatSlots) stat[j * kStatStride] = 0u;
+    float c[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) c[t] = (j < k) ? cb[((size_t)s * k + j) * 8 + t] : 0.0f;
+    mfma_bf_prep_block(c, s, j, k, nb, atab, c2perm, maxc2, mu);
 }
 
 // The reference's argmin of one row's sub-vector (8 floats, the same in every lane) over the k

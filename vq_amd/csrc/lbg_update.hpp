@@ -18,6 +18,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "assign_mfma.hpp"
+
 namespace vq {
 
 constexpr int kPartRows = 4096;      // rows per part (histogram block and summation part)
@@ -674,6 +676,30 @@ static __global__ void __launch_bounds__(256) k_lbg_combine8(LbgState st, int k,
     cb[((size_t)s * k + j) * 8 + t] = sum / __uint2float_rn(cnt);
 }
 
+// The same fold for every cluster, sum only (big_sum[s][j][t]): it needs nothing from the gather
+// path, so it can follow the streaming kernel at once; k_lbg_finalize_prep8 picks the large
+// clusters' sums and divides.
+static __global__ void __launch_bounds__(256) k_lbg_fold8(LbgState st, int k, float *__restrict__ big_sum) {
+    const int s = blockIdx.y;
+    if (st.done[s]) return;
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    const int j = gid / 8, t = gid % 8;
+    if (j >= k) return;
+    const float *ps = st.part_sum + ((size_t)s * st.nparts * kMaxK + j) * 8 + t;
+    float sum = 0.0f;
+    constexpr int B = 64;  // four memory round trips for the 245 parts of a million rows
+    const int np = st.nparts;
+    for (int p = 0; p < np; p += B) {
+        float v[B];
+#pragma unroll
+        for (int u = 0; u < B; ++u) v[u] = ps[(size_t)(p + u < np ? p + u : np - 1) * kMaxK * 8];
+#pragma unroll
+        for (int u = 0; u < B; ++u)
+            if (p + u < np) sum = sum + v[u];
+    }
+    big_sum[((size_t)s * kMaxK + j) * 8 + t] = sum;
+}
+
 // Loop control of src/utils.rs:57,104-106, one thread per column block.
 static __global__ void k_lbg_advance(LbgState st, int m) {
     int s = blockIdx.x * blockDim.x + threadIdx.x;
@@ -681,6 +707,64 @@ static __global__ void k_lbg_advance(LbgState st, int m) {
     st.iters[s] += 1;
     if (!st.changed[s]) st.done[s] = 1;
     st.changed[s] = 0;
+}
+
+// The end of an update and the start of the next assignment pass, one workgroup per column block
+// (8-float blocks, streaming path, matrix-core assignment).  Thread j makes centroid j — the mean
+// of a small cluster from its leaf or of a large one from k_lbg_fold8's sum, the re-seed row of
+// an empty cluster (src/vector.rs:315-316, src/utils.rs:98-101) — thread 0 does the loop
+// control of src/utils.rs:57,104-106, and all of them the tables of k_assign_mfma_bf from the
+// centroids they hold.  Needs x 16-byte aligned, ld % 4 == 0 (as the streaming kernel does).
+static __global__ void __launch_bounds__(256) k_lbg_finalize_prep8(
+    LbgState st, const float *__restrict__ x, int64_t ld, int k, const uint32_t *__restrict__ reseed, int n_reseed,
+    float *__restrict__ cb, const float *__restrict__ big_sum, int nb, u32x4 *__restrict__ atab,
+    float *__restrict__ c2perm, float *__restrict__ maxc2, float *__restrict__ mu, uint32_t *__restrict__ stat) {
+    const int s = blockIdx.x, j = threadIdx.x;
+    if (s == 0 && j < kStatSlots) stat[j * kStatStride] = 0u;
+    if (st.done[s]) return;  // the same in the whole workgroup; a finished block is skipped by the assignment
+    float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (j < k) {
+        const size_t sj = (size_t)s * kMaxK + j;
+        const uint32_t cnt = st.count[sj];
+        float4 *out = reinterpret_cast<float4 *>(cb + ((size_t)s * k + j) * 8);
+        float4 lo4, hi4;
+        bool write = true;
+        if (cnt == 0) {
+            const int pos = st.ubase[s] + (int)st.empty_rank[sj];
+            if (pos >= n_reseed) {
+                st.err[0] = 1;
+                lo4 = out[0];  // the centroid stays
+                hi4 = out[1];
+                write = false;
+            } else {
+                const float4 *row =
+                    reinterpret_cast<const float4 *>(x + (int64_t)reseed[(size_t)s * n_reseed + pos] * ld + (int64_t)s * 8);
+                lo4 = row[0];
+                hi4 = row[1];
+            }
+        } else {
+            const float4 *ls = reinterpret_cast<const float4 *>(
+                cnt <= (uint32_t)kSeqMax ? st.leaf_sum + ((size_t)s * st.leaf_cap + st.leaf_start[sj]) * 8
+                                         : big_sum + ((size_t)s * kMaxK + j) * 8);
+            const float d = __uint2float_rn(cnt);
+            const float4 a = ls[0], b = ls[1];
+            lo4 = make_float4(a.x / d, a.y / d, a.z / d, a.w / d);
+            hi4 = make_float4(b.x / d, b.y / d, b.z / d, b.w / d);
+        }
+        if (write) {
+            out[0] = lo4;
+            out[1] = hi4;
+        }
+        c[0] = lo4.x, c[1] = lo4.y, c[2] = lo4.z, c[3] = lo4.w;
+        c[4] = hi4.x, c[5] = hi4.y, c[6] = hi4.z, c[7] = hi4.w;
+    }
+    __syncthreads();  // every thread has read done[s]
+    if (j == 0) {
+        st.iters[s] += 1;
+        if (!st.changed[s]) st.done[s] = 1;
+        st.changed[s] = 0;
+    }
+    mfma_bf_prep_block(c, s, j, k, nb, atab, c2perm, maxc2, mu);
 }
 
 }  // namespace vq

@@ -105,22 +105,39 @@ int32_t launch_assign_m(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
 
 // 8-float column blocks: bf16-split scores on the matrix cores, undecided rows resolved in the
 // same kernel by the reference-order argmin (assign_mfma.hpp).
-template <int METRIC, bool LBG>
-int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a) {
-    const int nb = 2 * ((a.k + 63) / 64);  // blocks of 32 centroids, an even number (the kernel scores them in pairs)
+// Where the tables of k_assign_mfma_bf live in the workspace.
+struct MfmaTabPtrs {
+    vq::u32x4 *atab;
+    float *c2perm, *maxc2, *mu;
+    uint32_t *stat;
+    int nb;
+};
+int32_t mfma_tab_ptrs(vq_ctx *ctx, int m, int k, MfmaTabPtrs &t) {
+    t.nb = 2 * ((k + 63) / 64);  // blocks of 32 centroids, an even number (the kernel scores them in pairs)
     // A operands: 2 x 64 lanes x 16 bytes per (s, block of 32 centroids)
-    const size_t n_atab = (size_t)a.m * nb * 512, n_c2 = (size_t)a.m * nb * 32;
-    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + 9 * (size_t)a.m) + 64));
+    const size_t n_atab = (size_t)m * t.nb * 512, n_c2 = (size_t)m * t.nb * 32;
+    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + 9 * (size_t)m) + 64));
     VQ_TRY(ensure(ctx, ctx->mfma_stat, sizeof(uint32_t) * vq::kStatSlots * vq::kStatStride));
     float *atab = (float *)ctx->mfma_tab.p;
-    float *c2perm = atab + n_atab;
-    float *maxc2 = c2perm + n_c2;
-    float *mu = maxc2 + a.m;
-    uint32_t *stat = (uint32_t *)ctx->mfma_stat.p;
+    t.atab = (vq::u32x4 *)atab;
+    t.c2perm = atab + n_atab;
+    t.maxc2 = t.c2perm + n_c2;
+    t.mu = t.maxc2 + m;
+    t.stat = (uint32_t *)ctx->mfma_stat.p;
+    return VQ_OK;
+}
+
+// tables_ready: the caller's last kernel has already written the tables of these centroids
+template <int METRIC, bool LBG>
+int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready) {
+    MfmaTabPtrs t;
+    VQ_TRY(mfma_tab_ptrs(ctx, a.m, a.k, t));
+    const int nb = t.nb;
     constexpr int TILES = VQ_MFMA_TILES;
-    hipLaunchKernelGGL(vq::k_mfma_bf_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb,
-                       (vq::u32x4 *)atab, c2perm, maxc2, mu, stat);
-    vq::MfmaBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, mu, stat, nb};
+    if (!tables_ready)
+        hipLaunchKernelGGL(vq::k_mfma_bf_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, t.atab,
+                           t.c2perm, t.maxc2, t.mu, t.stat);
+    vq::MfmaBfTables tb{(const vq::u32x4 *)t.atab, t.c2perm, t.maxc2, t.mu, t.stat, nb};
     // 4 column blocks of 8 floats = one 128-byte line per row
     constexpr int SG = VQ_MFMA_SG;
     const bool grouped = a.m % SG == 0;
@@ -225,11 +242,11 @@ bool mfma_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
 }
 
 template <bool LBG>
-int32_t launch_assign(vq_ctx *ctx, int metric, const vq::AssignArgs &a, int sd) {
+int32_t launch_assign(vq_ctx *ctx, int metric, const vq::AssignArgs &a, int sd, bool tables_ready = false) {
     if (metric == VQ_SQEUCLIDEAN && mfma_applicable<vq::M_SQ, LBG>(ctx, a, sd))
-        return launch_mfma<vq::M_SQ, LBG>(ctx, a);
+        return launch_mfma<vq::M_SQ, LBG>(ctx, a, tables_ready);
     if (metric == VQ_EUCLIDEAN && mfma_applicable<vq::M_EUCLID, LBG>(ctx, a, sd))
-        return launch_mfma<vq::M_EUCLID, LBG>(ctx, a);
+        return launch_mfma<vq::M_EUCLID, LBG>(ctx, a, tables_ready);
     if (metric == VQ_SQEUCLIDEAN && mfma_wide_applicable<vq::M_SQ, LBG>(ctx, a, sd))
         return launch_mfma_wide<vq::M_SQ, LBG>(ctx, a, sd);
     if (metric == VQ_EUCLIDEAN && mfma_wide_applicable<vq::M_EUCLID, LBG>(ctx, a, sd))
@@ -347,8 +364,8 @@ int32_t vq_ctx_create(int32_t device, vq_ctx **out) {
         (e = hipEventCreate(&ctx->ev0)) != hipSuccess ||
         (e = hipEventCreate(&ctx->ev1)) != hipSuccess ||
         (e = hipStreamCreate(&ctx->side)) != hipSuccess ||
-        (e = hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming)) != hipSuccess ||
-        (e = hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming)) != hipSuccess) {
+        (e = hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming | hipEventReleaseToDevice)) != hipSuccess ||
+        (e = hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming | hipEventReleaseToDevice)) != hipSuccess) {
         int32_t rc = fail(nullptr, VQ_ERR_HIP, "context set-up failed: %s", hipGetErrorString(e));
         delete ctx;
         return rc;
@@ -536,7 +553,8 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
     VQ_TRY(ensure(ctx, ctx->hist, sizeof(uint32_t) * (size_t)m * nparts * vq::kMaxK));
     VQ_TRY(ensure(ctx, ctx->seg, sizeof(uint32_t) * (size_t)m * nseg * vq::kMaxK));
     VQ_TRY(ensure(ctx, ctx->perm, sizeof(uint32_t) * (size_t)m * n));
-    if (stream) VQ_TRY(ensure(ctx, ctx->part_sum, sizeof(float) * (size_t)m * nparts * vq::kMaxK * 8));
+    // per-part sums of the streaming kernel, then one folded sum per cluster
+    if (stream) VQ_TRY(ensure(ctx, ctx->part_sum, sizeof(float) * (size_t)m * (nparts + 1) * vq::kMaxK * 8));
     VQ_TRY(ensure(ctx, ctx->leaf_desc, sizeof(uint2) * (size_t)m * leaf_cap));
     VQ_TRY(ensure(ctx, ctx->leaf_sum, sizeof(float) * (size_t)m * leaf_cap * sd));
     VQ_TRY(ensure(ctx, ctx->codes, (size_t)m * n));
@@ -594,10 +612,15 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
     a.changed = S.changed;
     a.done = S.done;
 
+    // With the streaming sums and the matrix-core assignment, one kernel ends the update: the new
+    // centroids, the loop control and the tables of the next assignment pass.
+    const bool fused_tail = stream && mfma_applicable<vq::M_SQ, true>(ctx, a, sd);
+    MfmaTabPtrs tabs{};
+    if (fused_tail) VQ_TRY(mfma_tab_ptrs(ctx, m, k, tabs));
     for (int it = 0; it < max_iters; ++it) {
         {
             ProfSpan sp(ctx, VQ_PROF_LBG_ASSIGN);
-            VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd));
+            VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd, fused_tail && it > 0));
         }
         ProfSpan sp(ctx, VQ_PROF_LBG_UPDATE);
         int shift = 0;
@@ -629,15 +652,25 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
             hipLaunchKernelGGL(vq::k_lbg_leafsum, dim3(cdiv((int64_t)leaf_cap * sd, 256), m), dim3(256), 0, gs,
                                S, d_x, n, ld, sd);
         }
+        float *big_sum = stream ? S.part_sum + (size_t)m * nparts * vq::kMaxK * 8 : nullptr;
+        if (fused_tail)  // needs the streaming kernel only: in flight while the gather path ends
+            hipLaunchKernelGGL(vq::k_lbg_fold8, dim3(cdiv((int64_t)k * 8, 256), m), dim3(256), 0, st, S, k, big_sum);
         if (stream) {
             VQ_HIP(ctx, hipEventRecord(ctx->ev_join, gs));
             VQ_HIP(ctx, hipStreamWaitEvent(st, ctx->ev_join, 0));
-            hipLaunchKernelGGL(vq::k_lbg_combine8, dim3(cdiv((int64_t)k * 8, 256), m), dim3(256), 0, st, S, k,
-                               d_codebooks);
+            if (!fused_tail)
+                hipLaunchKernelGGL(vq::k_lbg_combine8, dim3(cdiv((int64_t)k * 8, 256), m), dim3(256), 0, st, S, k,
+                                   d_codebooks);
         }
-        hipLaunchKernelGGL(vq::k_lbg_finalize, dim3(cdiv((int64_t)k * sd, 256), m), dim3(256), 0, st, S,
-                           d_x, ld, k, sd, (const uint32_t *)ctx->reseed.p, n_reseed, d_codebooks);
-        hipLaunchKernelGGL(vq::k_lbg_advance, dim3(cdiv(m, 64)), dim3(64), 0, st, S, m);
+        if (fused_tail) {
+            hipLaunchKernelGGL(vq::k_lbg_finalize_prep8, dim3(m), dim3(256), 0, st, S, d_x, ld, k,
+                               (const uint32_t *)ctx->reseed.p, n_reseed, d_codebooks, (const float *)big_sum,
+                               tabs.nb, tabs.atab, tabs.c2perm, tabs.maxc2, tabs.mu, tabs.stat);
+        } else {
+            hipLaunchKernelGGL(vq::k_lbg_finalize, dim3(cdiv((int64_t)k * sd, 256), m), dim3(256), 0, st, S,
+                               d_x, ld, k, sd, (const uint32_t *)ctx->reseed.p, n_reseed, d_codebooks);
+            hipLaunchKernelGGL(vq::k_lbg_advance, dim3(cdiv(m, 64)), dim3(64), 0, st, S, m);
+        }
         VQ_HIP(ctx, hipGetLastError());
     }
     std::vector<int> host(7 * (size_t)m + 1);
