@@ -529,23 +529,19 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const 
 // chunk are ranked inside their cluster with wave ballots and added to the cluster's
 // accumulator in LDS in rank order (round r: the lanes of rank r, all on different clusters) —
 // so every cluster receives its rows of this part in row order, one at a time, starting from
-// 0.0.  Emits the per-part sums and, with HIST, the part's histogram (without it k_lbg_hist
-// counts, on another stream at the same time); no floating-point atomics.
-template <bool HIST>
+// 0.0.  Emits the per-part sums (k_lbg_hist counts the members, on another stream at the same
+// time); no floating-point atomics.
 static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const float *__restrict__ x, int64_t n,
                                                             int64_t ld) {
     const int g = blockIdx.y, b = blockIdx.x;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int s = 4 * g + w;
     __shared__ float4 acc_lo[4][kMaxK], acc_hi[4][kMaxK];  // components 0-3 and 4-7 of every cluster
-    __shared__ uint32_t cnt_all[4][kMaxK];
     if (st.done[s]) return;  // uniform per wave; the waves never synchronise with each other
     float4 *alo = acc_lo[w], *ahi = acc_hi[w];
-    uint32_t *cnt = cnt_all[w];
     for (int i = lane; i < kMaxK; i += 64) {
         alo[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         ahi[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        cnt[i] = 0u;
     }
     __builtin_amdgcn_wave_barrier();
     const int64_t lo = (int64_t)b * kPartRows;
@@ -618,7 +614,6 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
             const uint32_t same_lo = ~bad_lo, same_hi = ~bad_hi;
             const uint32_t rank =
                 pending ? (uint32_t)(__popc(same_lo & lt_lo) + __popc(same_hi & lt_hi)) : 0xFFFFFFFFu;
-            if (HIST && rank == 0) atomicAdd(&cnt[c], (uint32_t)(__popc(same_lo) + __popc(same_hi)));  // one lane per cluster
             // Round r: the lanes of rank r (all on different clusters) add their rows.  LDS
             // operations of one wave are performed in program order, so the next round sees these
             // writes; the wave barrier only pins the compiler's schedule (a fence or s_barrier
@@ -644,10 +639,6 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
     __builtin_amdgcn_wave_barrier();
     float4 *ps = reinterpret_cast<float4 *>(st.part_sum) + ((size_t)s * st.nparts + b) * kMaxK * 2;
     for (int i = lane; i < kMaxK * 2; i += 64) ps[i] = (i & 1) ? ahi[i >> 1] : alo[i >> 1];
-    if (HIST) {
-        uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
-        for (int j = lane; j < kMaxK; j += 64) h[j] = cnt[j];
-    }
 }
 
 // One lane per (cluster, component): sequential fold of the per-part sums of a large cluster.

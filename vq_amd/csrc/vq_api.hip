@@ -634,7 +634,7 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
         if (stream) {
             VQ_HIP(ctx, hipEventRecord(ctx->ev_fork, st));
             VQ_HIP(ctx, hipStreamWaitEvent(gs, ctx->ev_fork, 0));
-            hipLaunchKernelGGL(vq::k_lbg_stream8<false>, dim3(nparts, m / 4), dim3(256), 0, st, S, d_x, n, ld);
+            hipLaunchKernelGGL(vq::k_lbg_stream8, dim3(nparts, m / 4), dim3(256), 0, st, S, d_x, n, ld);
         }
         hipLaunchKernelGGL(vq::k_lbg_hist, dim3(nparts, m), dim3(64), 0, gs, S, n);
         hipLaunchKernelGGL(vq::k_lbg_scan_seg, dim3(nseg, m), dim3(256), 0, gs, S);
