@@ -87,3 +87,37 @@ def test_random_shape_encode_and_fit(ctx, case):
     it, used = ctx.lbg_fit(dx, n, dim, m, sd, k, 2, init, reseed, dcb2)
     assert np.array_equal(it, w["iters"])
     assert np.array_equal(dcb2.download().view(np.uint32), w["codebooks"].view(np.uint32)), (n, dim, m, k, kind)
+
+
+@pytest.mark.parametrize("case", range(12))
+def test_random_fit_over_many_parts(ctx, case):
+    """Whole fits of 8-float blocks over up to 22 parts of 4096 rows: clusters on both sides of the
+    1024-member switch of mean_vector (src/vector.rs:298-313), empty clusters and re-seeds
+    (src/utils.rs:98-101), early stops; centroids, iteration and re-seed counts against the oracle,
+    and a second run that must give the same bits (the update runs on two streams)."""
+    rng = np.random.default_rng([case, 0x51])
+    m = int(rng.choice([4, 8, 16, 3]))
+    k = int(rng.choice([2, 8, 17, 64, 256]))
+    n = int(rng.integers(max(k, 5000), 90000))
+    iters = int(rng.integers(2, 6))
+    dim = 8 * m
+    kind = case % 4
+    if kind == 0:
+        x = rng.random((n, dim), dtype=F)
+    elif kind == 1:  # fewer centres than clusters: empty clusters and re-seeds
+        x = data.gaussian_mixture(n, dim, max(1, k // 4), 0.01, seed=case)
+    elif kind == 2:
+        x = data.gaussian_mixture(n, dim, 4 * k + 3, 0.05, seed=case)
+    else:            # many identical rows: ties
+        base = rng.random((max(2, k // 2), dim), dtype=F)
+        x = base[rng.integers(0, base.shape[0], n)]
+    init, reseed = data.index_streams(n, m, k, iters, seed=case)
+    want = O.pq_fit(x, m, k, iters, init, reseed)
+    dx = ctx.to_device(x)
+    dcb = ctx.empty((m, k, 8), F)
+    it, used = ctx.lbg_fit(dx, n, dim, m, 8, k, iters, init, reseed, dcb)
+    got = dcb.download()
+    assert np.array_equal(got.view(np.uint32), want["codebooks"].view(np.uint32))
+    assert np.array_equal(it, want["iters"]) and np.array_equal(used, want["reseeds"])
+    ctx.lbg_fit(dx, n, dim, m, 8, k, iters, init, reseed, dcb)
+    assert np.array_equal(dcb.download().view(np.uint32), got.view(np.uint32))
