@@ -17,6 +17,9 @@
  *   - all work is enqueued on the context's stream; functions that return host values
  *     synchronise that stream before returning, the others are asynchronous.
  *   - one context = one stream; a context is not re-entrant, distinct contexts are independent.
+ *     (vq_lbg_fit also runs part of its update on a second stream that the context owns; that
+ *     work is joined back into the context's stream inside the call, so callers order their own
+ *     work against the context's stream only.)
  *   - randomness never crosses the boundary as a seed: the host draws the index streams
  *     (initial rows, re-seed rows) with its own RNG and passes them as arrays.
  */
