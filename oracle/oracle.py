@@ -17,7 +17,11 @@ SQEUCLIDEAN, EUCLIDEAN, COSINE, MANHATTAN = 0, 1, 2, 3
 
 
 def build(force=False):
-    """Compile the oracle with the flags that keep the reference's rounding."""
+    """Compile the oracle with the flags that keep the reference's rounding.  VQ_ORACLE_LIB names
+    another build of the same source to load instead (the sanitizer build of the tests)."""
+    other = os.environ.get("VQ_ORACLE_LIB")
+    if other:
+        return other
     if force or not os.path.exists(_LIB_PATH):
         subprocess.check_call(["make", "-B", "-C", _HERE, "libvq_oracle.so"],
                               stdout=subprocess.DEVNULL)
@@ -36,8 +40,7 @@ _i64 = C.c_int64
 def lib():
     global _lib
     if _lib is None:
-        build()
-        L = C.CDLL(_LIB_PATH)
+        L = C.CDLL(build())
         L.vqo_dot.restype = C.c_float
         L.vqo_dot.argtypes = [_f32p, _f32p, _i64]
         L.vqo_distance2.restype = C.c_float
