@@ -192,3 +192,22 @@ def test_rows_as_vectors_and_as_one_array_agree(vq):
             q.quantize_batch_vectors(x, short_row=5, short_len=7)
         with pytest.raises(vq.VqError, match="Dimension mismatch: expected 12, got 3"):
             q.quantize_batch_vectors(x, short_row=0, short_len=3)
+
+
+def test_host_classes_under_ubsan():
+    """This file's tests once more in a child process that loads the host mirror built with
+    -fsanitize=undefined -fno-sanitize-recover (any finding aborts the child)."""
+    import os
+    import subprocess
+    import sys
+    if os.environ.get("VQ_HOST_LIB"):
+        pytest.skip("already the sanitizer run")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = os.path.join(root, "vq_amd", "libvqhost_ubsan.so")
+    assert os.path.exists(lib), "build it with `python -m vq_amd.build`"
+    env = dict(os.environ, VQ_HOST_LIB=lib, UBSAN_OPTIONS="halt_on_error=1:print_stacktrace=1")
+    res = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-p", "no:cacheprovider", "-m", "gpu",
+                          os.path.abspath(__file__)], cwd=root, env=env, capture_output=True, text=True,
+                         timeout=600)
+    assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
+    assert "runtime error" not in res.stderr

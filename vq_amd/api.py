@@ -12,7 +12,8 @@ from . import _ffi
 from ._ffi import VqError
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-HOST_LIB_PATH = os.path.join(_HERE, "libvqhost.so")
+# VQ_HOST_LIB names another build of the host mirror to load (the sanitizer build of the tests)
+HOST_LIB_PATH = os.environ.get("VQ_HOST_LIB") or os.path.join(_HERE, "libvqhost.so")
 
 if not os.path.exists(HOST_LIB_PATH):
     raise ImportError(f"{HOST_LIB_PATH} is missing: build it with `python -m vq_amd.build`")

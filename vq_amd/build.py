@@ -49,19 +49,28 @@ def build_lib(verbose=False, extra=()):
 HOST_LIB = os.path.join(HERE, "libvqhost.so")
 
 
-def build_host(verbose=False):
-    """Compiles the C++ host mirror (plain g++: it only needs the C ABI) and links it to libvqhip."""
-    cmd = ["g++", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-Wall",
-           os.path.join(HERE, "host", "vq_host_c.cpp"), "-o", HOST_LIB,
+HOST_LIB_UBSAN = os.path.join(HERE, "libvqhost_ubsan.so")
+
+
+def build_host(verbose=False, ubsan=False):
+    """Compiles the C++ host mirror (plain g++: it only needs the C ABI) and links it to libvqhip.
+    ubsan: a second build under the undefined-behaviour sanitizer (aborts at the first finding),
+    which the tests load through VQ_HOST_LIB."""
+    out = HOST_LIB_UBSAN if ubsan else HOST_LIB
+    opt = ["-O1", "-g", "-fsanitize=undefined", "-fno-sanitize-recover=undefined", "-static-libubsan"] \
+        if ubsan else ["-O3"]
+    cmd = ["g++", *opt, "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-Wall",
+           os.path.join(HERE, "host", "vq_host_c.cpp"), "-o", out,
            "-L" + HERE, "-lvqhip", "-Wl,-rpath,$ORIGIN"]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("g++ failed:\n" + res.stdout + res.stderr)
-    return HOST_LIB
+    return out
 
 
 if __name__ == "__main__":
     print(build_lib(verbose=True, extra=sys.argv[1:]))
     print(build_host(verbose=True))
+    print(build_host(verbose=True, ubsan=True))
