@@ -105,7 +105,6 @@ constexpr int kStatStride = 32;
 
 struct MfmaBfTables {
     const u32x4 *atab;     // [m][nb][2][64]  A operands of the two instructions, lane order
-    const float *c2perm;   // [m][nb][2][16]  ||c||^2 in accumulator order (kPadScore for padding)
     const float *maxc2;    // [m]  largest ||c - mu||^2 of the column block (NaN if any is NaN)
     const float *mu;       // [m][8]  the block's centre: mean of its centroids
     uint32_t *stat;        // [kStatSlots * kStatStride]  pairs decided by the exact path (measurement)
@@ -136,8 +135,8 @@ __device__ __forceinline__ uint32_t bf16_pack2(float a, float b) {
 // of the block in thread j's registers (zeros from k on); k_mfma_bf_prep reads the centroids from
 // the codebook, the LBG loop's last update kernel has just computed them.
 __device__ __forceinline__ void mfma_bf_prep_block(float (&c)[8], int s, int j, int k, int nb,
-                                                   u32x4 *__restrict__ atab, float *__restrict__ c2perm,
-                                                   float *__restrict__ maxc2, float *__restrict__ mu) {
+                                                   u32x4 *__restrict__ atab, float *__restrict__ maxc2,
+                                                   float *__restrict__ mu) {
     __shared__ float sh_max[4];
     __shared__ float sh_mu[4][8];
     // centre: sum of c / 256 (no overflow for k <= 256), then * 256 / k
@@ -175,18 +174,22 @@ __device__ __forceinline__ void mfma_bf_prep_block(float (&c)[8], int s, int j, 
             hb[t] = bf16_rne_bits(a);
             lb[t] = bf16_rne_bits(a - bf16_bits_to_float(hb[t]));
         }
-        // lane i + 32 h: instruction 1 {ah[4h..4h+3], ah[4h..4h+3]}, instruction 2 {al[4h..4h+3], 1, 1, 1, 0}
+        // ||c - mu||^2 rides in the spare slots of the second instruction as three bf16 parts
+        // (exact: 3 x 8 bits), against ones in the row operand
+        const uint32_t c2a = bf16_rne_bits(c2);
+        const float c2r = c2 - bf16_bits_to_float(c2a);
+        const uint32_t c2b = bf16_rne_bits(c2r);
+        const uint32_t c2c = bf16_rne_bits(c2r - bf16_bits_to_float(c2b));
+        // lane i + 32 h: instruction 1 {ah[4h..4h+3], ah[4h..4h+3]}, instruction 2
+        // {al[4h..4h+3], 1, 1, c2 parts: (1st, 2nd) in the lower half, (3rd, 0) in the upper}
         u32x4 *dst = atab + ((size_t)s * nb + b) * 128;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const uint32_t ah0 = hb[4 * h] | (hb[4 * h + 1] << 16), ah1 = hb[4 * h + 2] | (hb[4 * h + 3] << 16);
             const uint32_t al0 = lb[4 * h] | (lb[4 * h + 1] << 16), al1 = lb[4 * h + 2] | (lb[4 * h + 3] << 16);
             dst[32 * h + i] = u32x4{ah0, ah1, ah0, ah1};
-            dst[64 + 32 * h + i] = u32x4{al0, al1, 0x3f803f80u, 0x00003f80u};
+            dst[64 + 32 * h + i] = u32x4{al0, al1, 0x3f803f80u, h == 0 ? (c2a | (c2b << 16)) : c2c};
         }
-        // accumulator order: lane half h, register v <-> centroid 8*(v/4) + 4*h + v%4
-        const int hh = (i / 4) % 2, v = (i / 8) * 4 + i % 4;
-        c2perm[(((size_t)s * nb + b) * 2 + hh) * 16 + v] = c2;
     }
     // largest ||c||^2; a NaN poisons the bound on purpose
 #pragma unroll
@@ -208,15 +211,14 @@ __device__ __forceinline__ void mfma_bf_prep_block(float (&c)[8], int s, int j, 
 }
 
 static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__restrict__ cb, int m, int k, int nb,
-                                                             u32x4 *__restrict__ atab, float *__restrict__ c2perm,
-                                                             float *__restrict__ maxc2, float *__restrict__ mu,
-                                                             uint32_t *__restrict__ stat) {
+                                                             u32x4 *__restrict__ atab, float *__restrict__ maxc2,
+                                                             float *__restrict__ mu, uint32_t *__restrict__ stat) {
     const int s = blockIdx.x, j = threadIdx.x;
     if (s == 0 && j < kStatSlots) stat[j * kStatStride] = 0u;
     float c[8];
 #pragma unroll
     for (int t = 0; t < 8; ++t) c[t] = (j < k) ? cb[((size_t)s * k + j) * 8 + t] : 0.0f;
-    mfma_bf_prep_block(c, s, j, k, nb, atab, c2perm, maxc2, mu);
+    mfma_bf_prep_block(c, s, j, k, nb, atab, maxc2, mu);
 }
 
 // The reference's argmin of one row's sub-vector (8 floats, the same in every lane) over the k
@@ -272,7 +274,7 @@ __device__ __forceinline__ int exact_argmin8_wave(const float (&xs)[8], const fl
 template <int METRIC, bool LBG, int TILES, int SG>
 __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
     constexpr int SD = 8;
-    extern __shared__ __attribute__((aligned(16))) float lds_c2[];  // [SG][nb][2][16], the centres [SG][8], maxc2 [SG]
+    extern __shared__ __attribute__((aligned(16))) float lds_mu[];  // the centres [SG][8], maxc2 [SG]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int nb = tb.nb, m = a.m;
@@ -285,8 +287,6 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
     const unsigned chunk_id = blockIdx.x / per_chunk, rem = blockIdx.x % per_chunk;
     const int s0 = (int)(rem / 8u) * SG;
     const int64_t tile_id = (int64_t)chunk_id * 8 + (rem % 8u);
-    for (int i = threadIdx.x; i < SG * nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s0 * nb * 32 + i];
-    float *lds_mu = lds_c2 + SG * nb * 32;
     if (threadIdx.x < SG * 8) lds_mu[threadIdx.x] = tb.mu[(size_t)s0 * 8 + threadIdx.x];
     if (threadIdx.x < SG) lds_mu[SG * 8 + threadIdx.x] = tb.maxc2[s0 + threadIdx.x];
     // LBG: the blocks that have converged, read once (the same in every lane)
@@ -343,32 +343,28 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
             const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
             const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
             const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
-            // this half's share of ||x||^2 in three bf16 parts (exact to 2^-24)
+            // this half's share of ||x||^2 in two bf16 parts (it is the same in every score of the
+            // row, so its rounding cancels in their differences), then ones for the parts of ||c||^2
             const uint32_t p0 = bf16_pack2(p, 0.0f);
             const float r1 = p - __uint_as_float(p0 << 16);
             const uint32_t p1 = bf16_pack2(r1, 0.0f);
-            const float r2 = r1 - __uint_as_float(p1 << 16);
-            const uint32_t p2 = bf16_pack2(r2, 0.0f);
             b1[t] = u32x4{h01, h23, l01, l23};
-            b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu};
+            b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), 0x3f803f80u};
             int pa, pb;
             swap_halves(__float_as_int(p), pa, pb);
             x2[t] = __int_as_float(pa) + __int_as_float(pb);  // lower half's share + upper half's, in both
             m1[t] = 0x7f800000;  // +inf
             m2[t] = 0x7f800000;
         }
-        const float *cp = lds_c2 + ((size_t)q * nb * 2 + h) * 16;
         // One block of 32 centroids against the TILES row tiles.  The packed index leaves out the
         // lane half (bit 2), so it is the same in every lane and lives in scalar registers.
         const uint32_t keep = opaque_vgpr(0xFFFFFF00u);
         auto block = [&](int b, const u32x4 &a1c, const u32x4 &a2c) {
-            floatx16 c2v;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) c2v[v] = cp[b * 32 + v];
+            const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
                 floatx16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    __builtin_bit_cast(bf16x8, a1c), __builtin_bit_cast(bf16x8, b1[t]), c2v, 0, 0, 0);
+                    __builtin_bit_cast(bf16x8, a1c), __builtin_bit_cast(bf16x8, b1[t]), zero, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                     __builtin_bit_cast(bf16x8, a2c), __builtin_bit_cast(bf16x8, b2[t]), acc, 0, 0, 0);
                 int key[16];
@@ -417,7 +413,9 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
             const float bound = x2[t] + mc2;
             const float margin = 6.103515625e-05f * fabsf(s2) + 1.220703125e-04f * bound;
             bool sure = (s2 - s1) > margin;  // false for NaN / inf-inf
-            sure = sure && (bound < 1e29f) && (s1 < 1e29f);
+            // below 1e-31 the bf16 parts of ||c - mu||^2 may be subnormal, which the matrix cores may
+            // flush: up to 3 * 2^-126 lost, more than the margin allows for at such a bound
+            sure = sure && (bound < 1e29f) && (bound > 1e-31f) && (s1 < 1e29f);
             int code = (int)(__float_as_uint(s1) & 0xFFu);
             // undecided rows: the reference-order argmin, one row at a time by the whole wave
             unsigned long long todo = __ballot(mine && !sure);

@@ -709,7 +709,7 @@ static __global__ void k_lbg_advance(LbgState st, int m) {
 static __global__ void __launch_bounds__(256) k_lbg_finalize_prep8(
     LbgState st, const float *__restrict__ x, int64_t ld, int k, const uint32_t *__restrict__ reseed, int n_reseed,
     float *__restrict__ cb, const float *__restrict__ big_sum, int nb, u32x4 *__restrict__ atab,
-    float *__restrict__ c2perm, float *__restrict__ maxc2, float *__restrict__ mu, uint32_t *__restrict__ stat) {
+    float *__restrict__ maxc2, float *__restrict__ mu, uint32_t *__restrict__ stat) {
     const int s = blockIdx.x, j = threadIdx.x;
     if (s == 0 && j < kStatSlots) stat[j * kStatStride] = 0u;
     if (st.done[s]) return;  // the same in the whole workgroup; a finished block is skipped by the assignment
@@ -755,7 +755,7 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize_prep8(
         if (!st.changed[s]) st.done[s] = 1;
         st.changed[s] = 0;
     }
-    mfma_bf_prep_block(c, s, j, k, nb, atab, c2perm, maxc2, mu);
+    mfma_bf_prep_block(c, s, j, k, nb, atab, maxc2, mu);
 }
 
 }  // namespace vq

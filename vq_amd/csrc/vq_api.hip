@@ -108,20 +108,19 @@ int32_t launch_assign_m(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
 // Where the tables of k_assign_mfma_bf live in the workspace.
 struct MfmaTabPtrs {
     vq::u32x4 *atab;
-    float *c2perm, *maxc2, *mu;
+    float *maxc2, *mu;
     uint32_t *stat;
     int nb;
 };
 int32_t mfma_tab_ptrs(vq_ctx *ctx, int m, int k, MfmaTabPtrs &t) {
     t.nb = 2 * ((k + 63) / 64);  // blocks of 32 centroids, an even number (the kernel scores them in pairs)
     // A operands: 2 x 64 lanes x 16 bytes per (s, block of 32 centroids)
-    const size_t n_atab = (size_t)m * t.nb * 512, n_c2 = (size_t)m * t.nb * 32;
-    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + 9 * (size_t)m) + 64));
+    const size_t n_atab = (size_t)m * t.nb * 512;
+    VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + 9 * (size_t)m) + 64));
     VQ_TRY(ensure(ctx, ctx->mfma_stat, sizeof(uint32_t) * vq::kStatSlots * vq::kStatStride));
     float *atab = (float *)ctx->mfma_tab.p;
     t.atab = (vq::u32x4 *)atab;
-    t.c2perm = atab + n_atab;
-    t.maxc2 = t.c2perm + n_c2;
+    t.maxc2 = atab + n_atab;
     t.mu = t.maxc2 + m;
     t.stat = (uint32_t *)ctx->mfma_stat.p;
     return VQ_OK;
@@ -136,14 +135,14 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready) {
     constexpr int TILES = VQ_MFMA_TILES;
     if (!tables_ready)
         hipLaunchKernelGGL(vq::k_mfma_bf_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, t.atab,
-                           t.c2perm, t.maxc2, t.mu, t.stat);
-    vq::MfmaBfTables tb{(const vq::u32x4 *)t.atab, t.c2perm, t.maxc2, t.mu, t.stat, nb};
+                           t.maxc2, t.mu, t.stat);
+    vq::MfmaBfTables tb{(const vq::u32x4 *)t.atab, t.maxc2, t.mu, t.stat, nb};
     // 4 column blocks of 8 floats = one 128-byte line per row
     constexpr int SG = VQ_MFMA_SG;
     const bool grouped = a.m % SG == 0;
     auto kern = grouped ? vq::k_assign_mfma_bf<METRIC, LBG, TILES, SG> : vq::k_assign_mfma_bf<METRIC, LBG, TILES, 1>;
     const int sg = grouped ? SG : 1;
-    const size_t lds = sizeof(float) * sg * (nb * 32 + 9);
+    const size_t lds = sizeof(float) * sg * 9;
     const int64_t blocks = cdiv(cdiv(a.n, 4 * 32 * TILES), 8) * 8 * (a.m / sg);  // tiles in chunks of 8
     if (blocks >= (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * m too large for one launch");
     {
@@ -665,7 +664,7 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
         if (fused_tail) {
             hipLaunchKernelGGL(vq::k_lbg_finalize_prep8, dim3(m), dim3(256), 0, st, S, d_x, ld, k,
                                (const uint32_t *)ctx->reseed.p, n_reseed, d_codebooks, (const float *)big_sum,
-                               tabs.nb, tabs.atab, tabs.c2perm, tabs.maxc2, tabs.mu, tabs.stat);
+                               tabs.nb, tabs.atab, tabs.maxc2, tabs.mu, tabs.stat);
         } else {
             hipLaunchKernelGGL(vq::k_lbg_finalize, dim3(cdiv((int64_t)k * sd, 256), m), dim3(256), 0, st, S,
                                d_x, ld, k, sd, (const uint32_t *)ctx->reseed.p, n_reseed, d_codebooks);
