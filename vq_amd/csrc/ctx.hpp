@@ -37,6 +37,7 @@ struct vq_ctx {
     struct Span {
         int cls;
         hipEvent_t a, b;
+        bool own_a = true, own_b = true;  // false: the event belongs to another span (returned to the pool once)
     };
     std::vector<Span> prof_open;
     double prof_ms[VQ_PROF_CLASSES] = {0};
@@ -105,8 +106,8 @@ struct ProfSpan {
     vq_ctx *ctx;
     int cls;
     hipEvent_t a = nullptr;
-    ProfSpan(vq_ctx *c, int k) : ctx(c), cls(k) {
-        if (ctx->prof_on) {
+    ProfSpan(vq_ctx *c, int k) : ctx(c), cls(k) {  // k < 0: no span
+        if (ctx->prof_on && k >= 0) {
             a = prof_event(ctx);
             (void)hipEventRecord(a, ctx->stream);
         }
@@ -115,7 +116,7 @@ struct ProfSpan {
         if (a) {
             hipEvent_t b = prof_event(ctx);
             (void)hipEventRecord(b, ctx->stream);
-            ctx->prof_open.push_back({cls, a, b});
+            ctx->prof_open.push_back({cls, a, b, true, true});
         }
     }
 };
@@ -128,8 +129,10 @@ inline void prof_collect(vq_ctx *ctx) {
             ctx->prof_ms[sp.cls] += ms;
             ctx->prof_launches[sp.cls] += 1;
         }
-        ctx->prof_pool.push_back(sp.a);
-        ctx->prof_pool.push_back(sp.b);
+    }
+    for (auto &sp : ctx->prof_open) {
+        if (sp.own_a) ctx->prof_pool.push_back(sp.a);
+        if (sp.own_b) ctx->prof_pool.push_back(sp.b);
     }
     ctx->prof_open.clear();
 }

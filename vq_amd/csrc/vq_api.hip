@@ -2,6 +2,7 @@
 // Compile with: hipcc --offload-arch=gfx950 -O3 -ffp-contract=off
 //               -Xclang -target-feature -Xclang -packed-fp32-ops
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
@@ -126,9 +127,15 @@ int32_t mfma_tab_ptrs(vq_ctx *ctx, int m, int k, MfmaTabPtrs &t) {
     return VQ_OK;
 }
 
-// tables_ready: the caller's last kernel has already written the tables of these centroids
+// tables_ready: the caller's last kernel has already written the tables of these centroids.
+// Events ride on the kernel's own dispatch (hipExtLaunchKernelGGL) instead of being recorded
+// around it: a record is a packet of its own on the queue and delays the next kernel by several
+// microseconds.  With timing on, the kernel's start and stop events are a span of the kernel
+// class; started / done (if asked for) receive events that mark the kernel's start and end —
+// done is what another stream waits for — or stay null when the launch carries none.
 template <int METRIC, bool LBG>
-int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready) {
+int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready, hipEvent_t *started = nullptr,
+                    hipEvent_t *done = nullptr) {
     MfmaTabPtrs t;
     VQ_TRY(mfma_tab_ptrs(ctx, a.m, a.k, t));
     const int nb = t.nb;
@@ -145,11 +152,22 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready) {
     const size_t lds = sizeof(float) * sg * 9;
     const int64_t blocks = cdiv(cdiv(a.n, 4 * 32 * TILES), 8) * 8 * (a.m / sg);  // tiles in chunks of 8
     if (blocks >= (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * m too large for one launch");
-    {
-        ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
-        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, ctx->stream, a, tb);
+    hipEvent_t ev_a = nullptr, ev_b = nullptr;
+    if (ctx->prof_on) {
+        ev_a = prof_event(ctx);
+        ev_b = prof_event(ctx);
+        ctx->prof_open.push_back({VQ_PROF_ASSIGN_KERNEL, ev_a, ev_b, true, true});
+    } else if (done) {
+        ev_b = ctx->ev_fork;
     }
+    if (ev_a || ev_b)
+        hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), (uint32_t)lds, ctx->stream, ev_a, ev_b, 0u, a,
+                              tb);
+    else
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, ctx->stream, a, tb);
     VQ_HIP(ctx, hipGetLastError());
+    if (started) *started = ev_a;
+    if (done) *done = ev_b;
     ctx->recheck_src = 1;
     return VQ_OK;
 }
@@ -241,11 +259,14 @@ bool mfma_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
 }
 
 template <bool LBG>
-int32_t launch_assign(vq_ctx *ctx, int metric, const vq::AssignArgs &a, int sd, bool tables_ready = false) {
+int32_t launch_assign(vq_ctx *ctx, int metric, const vq::AssignArgs &a, int sd, bool tables_ready = false,
+                      hipEvent_t *started = nullptr, hipEvent_t *done = nullptr) {
+    if (started) *started = nullptr;
+    if (done) *done = nullptr;
     if (metric == VQ_SQEUCLIDEAN && mfma_applicable<vq::M_SQ, LBG>(ctx, a, sd))
-        return launch_mfma<vq::M_SQ, LBG>(ctx, a, tables_ready);
+        return launch_mfma<vq::M_SQ, LBG>(ctx, a, tables_ready, started, done);
     if (metric == VQ_EUCLIDEAN && mfma_applicable<vq::M_EUCLID, LBG>(ctx, a, sd))
-        return launch_mfma<vq::M_EUCLID, LBG>(ctx, a, tables_ready);
+        return launch_mfma<vq::M_EUCLID, LBG>(ctx, a, tables_ready, started, done);
     if (metric == VQ_SQEUCLIDEAN && mfma_wide_applicable<vq::M_SQ, LBG>(ctx, a, sd))
         return launch_mfma_wide<vq::M_SQ, LBG>(ctx, a, sd);
     if (metric == VQ_EUCLIDEAN && mfma_wide_applicable<vq::M_EUCLID, LBG>(ctx, a, sd))
@@ -363,7 +384,7 @@ int32_t vq_ctx_create(int32_t device, vq_ctx **out) {
         (e = hipEventCreate(&ctx->ev0)) != hipSuccess ||
         (e = hipEventCreate(&ctx->ev1)) != hipSuccess ||
         (e = hipStreamCreate(&ctx->side)) != hipSuccess ||
-        (e = hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming | hipEventReleaseToDevice)) != hipSuccess ||
+        (e = hipEventCreate(&ctx->ev_fork)) != hipSuccess ||  // rides on a kernel dispatch as its stop event
         (e = hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming | hipEventReleaseToDevice)) != hipSuccess) {
         int32_t rc = fail(nullptr, VQ_ERR_HIP, "context set-up failed: %s", hipGetErrorString(e));
         delete ctx;
@@ -616,12 +637,22 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
     const bool fused_tail = stream && mfma_applicable<vq::M_SQ, true>(ctx, a, sd);
     MfmaTabPtrs tabs{};
     if (fused_tail) VQ_TRY(mfma_tab_ptrs(ctx, m, k, tabs));
+    // Timing classes of the loop: where the assignment kernel carries its own events (started,
+    // done) the assignment span is the kernel's and an update span runs from one kernel's end to
+    // the next one's start, so nothing is recorded between the kernels of an iteration.
+    hipEvent_t prev_done = nullptr;
     for (int it = 0; it < max_iters; ++it) {
+        hipEvent_t started = nullptr, done = nullptr;
         {
-            ProfSpan sp(ctx, VQ_PROF_LBG_ASSIGN);
-            VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd, fused_tail && it > 0));
+            ProfSpan sp(ctx, fused_tail ? -1 : VQ_PROF_LBG_ASSIGN);
+            VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd, fused_tail && it > 0, &started, &done));
         }
-        ProfSpan sp(ctx, VQ_PROF_LBG_UPDATE);
+        if (ctx->prof_on && started && done) {
+            ctx->prof_open.push_back({VQ_PROF_LBG_ASSIGN, started, done, false, false});
+            if (prev_done) ctx->prof_open.push_back({VQ_PROF_LBG_UPDATE, prev_done, started, false, false});
+        }
+        prev_done = done;
+        ProfSpan sp(ctx, fused_tail ? -1 : VQ_PROF_LBG_UPDATE);
         int shift = 0;
         while ((1 << shift) < sd) ++shift;
         const bool leaf_wg = stream && sd >= 4 && sd <= 32 && (1 << shift) == sd && ld % 4 == 0 &&
@@ -631,8 +662,11 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
         // one long pass over the rows), and the two meet again before the large clusters' fold.
         hipStream_t gs = stream ? ctx->side : st;
         if (stream) {
-            VQ_HIP(ctx, hipEventRecord(ctx->ev_fork, st));
-            VQ_HIP(ctx, hipStreamWaitEvent(gs, ctx->ev_fork, 0));
+            if (!done) {  // the assignment kernel carried no event
+                VQ_HIP(ctx, hipEventRecord(ctx->ev_fork, st));
+                done = ctx->ev_fork;
+            }
+            VQ_HIP(ctx, hipStreamWaitEvent(gs, done, 0));
             hipLaunchKernelGGL(vq::k_lbg_stream8, dim3(nparts, m / 4), dim3(256), 0, st, S, d_x, n, ld);
         }
         hipLaunchKernelGGL(vq::k_lbg_hist, dim3(nparts, m), dim3(64), 0, gs, S, n);
@@ -671,6 +705,11 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
             hipLaunchKernelGGL(vq::k_lbg_advance, dim3(cdiv(m, 64)), dim3(64), 0, st, S, m);
         }
         VQ_HIP(ctx, hipGetLastError());
+    }
+    if (ctx->prof_on && fused_tail && prev_done) {  // the last update: up to an event recorded here
+        hipEvent_t end = prof_event(ctx);
+        VQ_HIP(ctx, hipEventRecord(end, st));
+        ctx->prof_open.push_back({VQ_PROF_LBG_UPDATE, prev_done, end, false, true});
     }
     std::vector<int> host(7 * (size_t)m + 1);
     VQ_HIP(ctx, hipMemcpyAsync(host.data(), f, sizeof(int) * host.size(), hipMemcpyDeviceToHost, st));
