@@ -678,7 +678,7 @@ static __global__ void __launch_bounds__(256) k_lbg_fold8(LbgState st, int k, fl
     if (j >= k) return;
     const float *ps = st.part_sum + ((size_t)s * st.nparts * kMaxK + j) * 8 + t;
     float sum = 0.0f;
-    constexpr int B = 64;  // four memory round trips for the 245 parts of a million rows
+    constexpr int B = 128;  // two memory round trips for the 245 parts of a million rows
     const int np = st.nparts;
     for (int p = 0; p < np; p += B) {
         float v[B];
