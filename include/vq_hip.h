@@ -97,13 +97,16 @@ int32_t vq_timer_start(vq_ctx *ctx);
 /* Records the stop event, synchronises, returns elapsed milliseconds since vq_timer_start. */
 int32_t vq_timer_stop(vq_ctx *ctx, float *h_ms);
 
-/* Per-kernel-class timing with HIP events recorded on the context's stream around the launches
- * the library makes (no counterpart in the reference; measurement only).  Enabling resets the
- * accumulators.  vq_prof_read synchronises the stream and returns the summed event time and
- * the number of timed spans of one class. */
+/* Per-kernel-class timing with HIP events on the context's stream around the launches the
+ * library makes (no counterpart in the reference; measurement only): recorded before and after
+ * the launches of a class, or, for the matrix-core assignment kernel, carried by the kernel's own
+ * dispatch as its start and stop events, which puts no extra packet on the queue.  Enabling
+ * resets the accumulators.  vq_prof_read synchronises the stream and returns the summed event
+ * time and the number of timed spans of one class. */
 enum vq_prof_class {
     VQ_PROF_LBG_ASSIGN = 0, /* the assignment kernels of one LBG iteration (utils.rs:59-73) */
-    VQ_PROF_LBG_UPDATE = 1, /* the update kernels of one LBG iteration (utils.rs:83-102) */
+    VQ_PROF_LBG_UPDATE = 1, /* the update kernels of one LBG iteration (utils.rs:83-102): from the end of
+                               its assignment kernel to the start of the next one */
     VQ_PROF_ENCODE = 2,     /* the kernels of one vq_assign call */
     VQ_PROF_ASSIGN_KERNEL = 3, /* the main assignment kernel alone (matrix-core pass or the
                                   vector-ALU kernel), in training and in vq_assign */
