@@ -308,3 +308,36 @@ def test_rows_with_leading_dimension_and_offset(ctx, sd, m, k, pad, shift):
     it, _ = ctx.lbg_fit(dbuf.ptr + 4 * shift, n, ld, m, sd, k, 3, init, reseed, dcb2)
     assert np.array_equal(it, w["iters"])
     assert np.array_equal(dcb2.download().view(np.uint32), w["codebooks"].view(np.uint32))
+
+
+@pytest.mark.parametrize("path", [0, 1])
+def test_timing_classes_count_every_pass(ctx, path):
+    """The per-class timers (measurement only): a fit of `iters` passes yields `iters` spans of the
+    assignment kernel, of the assignment class and of the update class, an encode one span more of
+    the kernel and one of the encode class — on the matrix-core path, where the events ride on the
+    kernel's dispatch, and on the vector path, where they are recorded around the launches — and
+    timing leaves the results as they are."""
+    import vq_amd
+    n, dim, m, k, iters = 20000, 64, 8, 64, 4
+    x = data.gaussian_mixture(n, dim, 4 * k, 0.05, seed=9)
+    init, reseed = data.index_streams(n, m, k, iters, seed=9)
+    ctx.set_assign_path(path)
+    try:
+        plain, _, _, dx, dcb = gpu_lbg(ctx, x, m, k, iters, init, reseed)
+        ctx.prof_enable(True)
+        for _ in range(2):  # twice: the events of the first fit are reused by the second
+            timed, it, _, dx, dcb = gpu_lbg(ctx, x, m, k, iters, init, reseed)
+        codes = gpu_encode(ctx, vq_amd.EUCLIDEAN, dx, n, dim, m, k, dcb)
+        spans = {c: ctx.prof_read(c) for c in (vq_amd._ffi.PROF_LBG_ASSIGN, vq_amd._ffi.PROF_LBG_UPDATE,
+                                              vq_amd._ffi.PROF_ENCODE, vq_amd._ffi.PROF_ASSIGN_KERNEL)}
+    finally:
+        ctx.prof_enable(False)
+        ctx.set_assign_path(0)
+    assert np.array_equal(plain.view(np.uint32), timed.view(np.uint32)) and int(it.max()) == iters
+    assert spans[vq_amd._ffi.PROF_LBG_ASSIGN][1] == 2 * iters
+    assert spans[vq_amd._ffi.PROF_LBG_UPDATE][1] == 2 * iters
+    assert spans[vq_amd._ffi.PROF_ASSIGN_KERNEL][1] == 2 * iters + 1
+    assert spans[vq_amd._ffi.PROF_ENCODE][1] == 1
+    assert all(ms > 0.0 for ms, _ in spans.values())
+    assert spans[vq_amd._ffi.PROF_ASSIGN_KERNEL][0] <= spans[vq_amd._ffi.PROF_LBG_ASSIGN][0] + spans[vq_amd._ffi.PROF_ENCODE][0] + 1e-3
+    assert codes.shape == (n, m)
