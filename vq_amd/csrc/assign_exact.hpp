@@ -584,6 +584,98 @@ __device__ __forceinline__ void wide_exact_groups(const AssignArgs &a, int sd, c
     }
 }
 
+// One listed pair by a whole workgroup: thread j walks centroid j (k <= 256) over the sub-vector in
+// the reference's order, 32 float4 loads in flight, so a handful of pairs costs a quarter of one
+// wave's walk over four centroids per lane.  Squared L2 and Euclidean only; sd % 4 == 0 and
+// 16-byte aligned centroids.  lds: the row (sd floats), then 16 floats of reduction space.
+template <int METRIC, bool LBG>
+__device__ __forceinline__ void wide_exact_pair_wg(const AssignArgs &a, int sd, uint32_t entry, float *lds) {
+    static_assert(METRIC == M_SQ || METRIC == M_EUCLID, "squared L2 / Euclidean");
+    const int j = threadIdx.x, lane = j & 63, wave = j >> 6, k = a.k;
+    const int64_t row = entry / (uint32_t)a.m;
+    const int s = (int)(entry % (uint32_t)a.m);
+    const float *xr = a.x + row * a.ld + (int64_t)s * sd;
+    for (int t = j; t < sd; t += 256) lds[t] = xr[t];
+    __syncthreads();
+    const float4 *cp = reinterpret_cast<const float4 *>(a.cb + ((size_t)s * k + (j < k ? j : 0)) * sd);
+    const int nv = sd / 4;
+    float acc = 0.0f;
+    for (int v0 = 0; v0 < nv; v0 += 32) {
+        float4 cv[32];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) cv[u] = cp[v0 + u < nv ? v0 + u : nv - 1];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) {
+            if (v0 + u < nv) {
+                const float4 xv = *reinterpret_cast<const float4 *>(lds + 4 * (v0 + u));
+                wide_step<METRIC>(acc, xv.x, cv[u].x);
+                wide_step<METRIC>(acc, xv.y, cv[u].y);
+                wide_step<METRIC>(acc, xv.z, cv[u].z);
+                wide_step<METRIC>(acc, xv.w, cv[u].w);
+            }
+        }
+    }
+    const float inf = __builtin_inff();
+    const float d = (j < k && acc == acc) ? acc : inf;  // a NaN distance never wins
+    float *red_d = lds + sd;
+    int *red_i = reinterpret_cast<int *>(lds + sd + 4);
+    int *red_f = reinterpret_cast<int *>(lds + sd + 8);
+    float bd = d;
+    int bi = j < k ? j : 0x7fffffff;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float od = __shfl_xor(bd, off);
+        const int oi = __shfl_xor(bi, off);
+        const bool take = (od < bd) || (od == bd && oi < bi);
+        bd = take ? od : bd;
+        bi = take ? oi : bi;
+    }
+    if (lane == 0) {
+        red_d[wave] = bd;
+        red_i[wave] = bi;
+    }
+    if (j == 0) lds[sd + 12] = acc;  // centroid 0's distance as computed
+    __syncthreads();
+    bd = red_d[0];
+    bi = red_i[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+        const float od = red_d[w];
+        const int oi = red_i[w];
+        const bool take = (od < bd) || (od == bd && oi < bi);
+        bd = take ? od : bd;
+        bi = take ? oi : bi;
+    }
+    if constexpr (METRIC == M_EUCLID) {
+        // the reference compares the roots: first index whose root equals the smallest root
+        const float sr = sqrtf(bd);
+        int fi = (j < k && sqrtf(d) == sr) ? j : 0x7fffffff;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const int oi = __shfl_xor(fi, off);
+            fi = oi < fi ? oi : fi;
+        }
+        if (lane == 0) red_f[wave] = fi;
+        __syncthreads();
+        bi = red_f[0];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) bi = red_f[w] < bi ? red_f[w] : bi;
+    }
+    const float d0 = lds[sd + 12];
+    if (!(d0 == d0)) bi = 0;  // NaN at index 0 is never displaced
+    if (j == 0) {
+        if constexpr (LBG) {
+            uint8_t *p = a.codes + (size_t)s * a.n + row;
+            if (*p != (uint8_t)bi) {
+                *p = (uint8_t)bi;
+                mark_changed(a.changed + s);
+            }
+        } else {
+            a.codes[row * a.m + s] = (uint8_t)bi;
+        }
+    }
+}
+
 template <int METRIC, bool LBG, bool LISTED, bool VEC>
 __global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd, const uint32_t *__restrict__ list,
                                                            const uint32_t *__restrict__ list_count) {
@@ -593,6 +685,13 @@ __global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd,
     const int64_t total = LISTED ? (int64_t)*list_count : a.n;
     if constexpr (LBG && !LISTED) {
         if (a.done[blockIdx.y]) return;
+    }
+    if constexpr (LISTED && VEC && (METRIC == M_SQ || METRIC == M_EUCLID)) {
+        // a handful of pairs: one per workgroup, one centroid per thread
+        if (total <= (int64_t)gridDim.x && a.k <= 256) {
+            if ((int64_t)blockIdx.x < total) wide_exact_pair_wg<METRIC, LBG>(a, sd, list[blockIdx.x], lds_wide);
+            return;
+        }
     }
     if constexpr (LISTED) {
         // a short list: one pair per wave, so that the pass is as long as one pair's scan, not eight
