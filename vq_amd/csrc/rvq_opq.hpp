@@ -368,38 +368,50 @@ static __global__ void __launch_bounds__(256) k_rotate_mfma(const float *__restr
     for (int b = 0; b < NBMAX; ++b)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[b][v] = 0.0f;
+    // The lane's pieces of its row are fetched kRotAhead chunks ahead (unconditional loads: a row
+    // past the end reads row 0 and is never stored); the barrier of a chunk waits for LDS only, so
+    // they stay in flight across it.  dim is a multiple of 32: the chunks come in fours.
+    constexpr int kRotAhead = 4;
     const float *xr = x + (valid ? row : 0) * ld + 4 * h;
-    for (int kc = 0; kc < nkc; ++kc) {
-        const int cur = kc & 1;
-        float4 pre[2];
-        const bool more = kc + 1 < nkc;
-        if (more) {
+    float4 xq[kRotAhead];
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                int i = threadIdx.x + 256 * q;
-                if (i < chunk4) pre[q] = ag[(size_t)(kc + 1) * chunk4 + i];
-            }
-        }
-        float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (valid) xv = *reinterpret_cast<const float4 *>(xr + kc * 8);
+    for (int u = 0; u < kRotAhead; ++u) xq[u] = *reinterpret_cast<const float4 *>(xr + (u < nkc ? u : nkc - 1) * 8);
+    for (int kc0 = 0; kc0 < nkc; kc0 += kRotAhead) {
 #pragma unroll
-        for (int b = 0; b < NBMAX; ++b) {
-            if (b < nb) {
-                const float4 av = lds_a[cur][b * 64 + lane];
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, xv.x, acc[b], 0, 0, 0);
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, xv.y, acc[b], 0, 0, 0);
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, xv.z, acc[b], 0, 0, 0);
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, xv.w, acc[b], 0, 0, 0);
-            }
-        }
-        if (more) {
+        for (int u = 0; u < kRotAhead; ++u) {
+            const int kc = kc0 + u;
+            const int cur = kc & 1;
+            float4 pre[2];
+            const bool more = kc + 1 < nkc;
+            if (more) {
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                int i = threadIdx.x + 256 * q;
-                if (i < chunk4) lds_a[cur ^ 1][i] = pre[q];
+                for (int q = 0; q < 2; ++q) {
+                    int i = threadIdx.x + 256 * q;
+                    if (i < chunk4) pre[q] = ag[(size_t)(kc + 1) * chunk4 + i];
+                }
             }
+            const float4 xv = xq[u];
+            const int nx = kc + kRotAhead < nkc ? kc + kRotAhead : nkc - 1;
+            xq[u] = *reinterpret_cast<const float4 *>(xr + nx * 8);
+#pragma unroll
+            for (int b = 0; b < NBMAX; ++b) {
+                if (b < nb) {
+                    const float4 av = lds_a[cur][b * 64 + lane];
+                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, xv.x, acc[b], 0, 0, 0);
+                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, xv.y, acc[b], 0, 0, 0);
+                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, xv.z, acc[b], 0, 0, 0);
+                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, xv.w, acc[b], 0, 0, 0);
+                }
+            }
+            if (more) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    int i = threadIdx.x + 256 * q;
+                    if (i < chunk4) lds_a[cur ^ 1][i] = pre[q];
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
-        __syncthreads();
     }
     if (!valid) return;
     // register v of block b holds output dimension 32 b + 8 (v / 4) + 4 h + v % 4 of this lane's row
