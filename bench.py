@@ -9,8 +9,10 @@ Prints ONE JSON line (see README of the bench contract):
   value        rows / second over fit + encode (whole job, one GPU)
   roofline     the dominant kernel (the matrix-core assignment pass) against the fp32 matrix
                peak, the path's arithmetic type (the bf16 issue rate is given beside it); its
-               time is measured with HIP events recorded on the library's stream around each
-               launch during the timed steps
+               time is measured with HIP events on the library's stream (the start and stop
+               events of each launch's own dispatch) during the timed steps; beside it the
+               floor set by the vector instructions of the selection at their measured rate
+  calibration  measured peaks of the box: plain-copy HBM rate, vector instruction issue rates
   cpu_baseline the C restatement of the reference (oracle/) timed on the host cores on a bounded
                sample of the same workload
 """
@@ -135,6 +137,24 @@ def main():
         "hbm_frac": round(bytes_per_launch / (avg_kern_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
         "assign_ms_incl_tables": round(assign_ms / max(assign_n, 1), 4),
     }
+    # Measured peaks of this box (vq_calibrate): the plain copy kernel's HBM rate and the issue
+    # rate of the vector instructions the selection is made of.  Per four scores the kernel issues
+    # 4 v_and_or_b32 (index tag), 3 v_min3_i32 and 2 v_med3_i32 (top-2 update); one wave64
+    # instruction handles 64 scores.  The floor is the time those instructions alone take with
+    # every SIMD full: the bound that actually binds the kernel (the matrix instructions hide
+    # behind them).
+    rate = {name: ctx.calibrate(kind) for kind, name in
+            ((1, "v_fma_f32"), (2, "v_min3_i32"), (3, "v_med3_i32"), (4, "v_and_or_b32"), (5, "v_add_u32"))}
+    scores = float(n) * M * K
+    floor_ms = scores / 64.0 * (1.0 / rate["v_and_or_b32"] + 0.75 / rate["v_min3_i32"]
+                                + 0.5 / rate["v_med3_i32"]) * 1e3
+    roofline["selection_floor_ms"] = round(floor_ms, 4)
+    roofline["frac_of_selection_floor"] = round(floor_ms / avg_kern_ms, 4)
+    calibration = {
+        "hbm_copy_GBs_read_plus_write": round(ctx.calibrate(0), 1),
+        "valu_wave64_Ginstr_per_s": {k_: round(v / 1e9, 1) for k_, v in rate.items()},
+        "valu_fma_TFLOPs": round(rate["v_fma_f32"] * 128.0 / 1e12, 1),
+    }
     breakdown = {
         "lbg_assign_ms_per_step": round(assign_ms / args.steps, 3),
         "lbg_update_ms_per_step": round(update_ms / args.steps, 3),
@@ -198,6 +218,7 @@ def main():
                    "rows": n, "dim": DIM, "m": M, "k": K, "lbg_iters": ITERS},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "calibration": calibration,
         "breakdown": breakdown,
         "parity": parity,
     }

@@ -72,6 +72,21 @@ void *vq_ctx_stream(vq_ctx *ctx);
  * Both give bit-identical codes; the switch exists for measurement and tests. */
 int32_t vq_ctx_set_assign_path(vq_ctx *ctx, int32_t path);
 
+/* Measured peaks of this GPU, for pricing the kernels (measurement only; no counterpart in the
+ * reference).  VQ_CALIB_HBM_COPY: GB/s of the plain copy kernel over 512 MB (bytes read + bytes
+ * written per second).  VQ_CALIB_VALU_*: wave64 instructions of that kind per second over the
+ * whole GPU with every SIMD kept full (v_fma_f32, v_min3_i32, v_med3_i32, v_and_or_b32, v_add_u32).
+ * Synchronises. */
+enum {
+    VQ_CALIB_HBM_COPY = 0,
+    VQ_CALIB_VALU_FMA = 1,
+    VQ_CALIB_VALU_MIN3 = 2,
+    VQ_CALIB_VALU_MED3 = 3,
+    VQ_CALIB_VALU_AND_OR = 4,
+    VQ_CALIB_VALU_ADD = 5
+};
+int32_t vq_calibrate(vq_ctx *ctx, int32_t what, double *h_rate);
+
 /* Number of (row, block) pairs the most recent matrix-core assignment pass left to the exact
  * re-check (0 if that path has not run).  Synchronises.  Measurement only. */
 int32_t vq_ctx_last_recheck_count(vq_ctx *ctx, uint32_t *h_count);

@@ -341,3 +341,19 @@ def test_timing_classes_count_every_pass(ctx, path):
     assert all(ms > 0.0 for ms, _ in spans.values())
     assert spans[vq_amd._ffi.PROF_ASSIGN_KERNEL][0] <= spans[vq_amd._ffi.PROF_LBG_ASSIGN][0] + spans[vq_amd._ffi.PROF_ENCODE][0] + 1e-3
     assert codes.shape == (n, m)
+
+
+def test_calibration_reports_plausible_peaks(ctx):
+    """vq_calibrate (measurement only): the plain copy kernel's rate lies between a tenth of and the
+    whole published HBM peak (read + write), a vector instruction costs between 1 and 16 cycles of a
+    2.4 GHz SIMD, and the three-input integer operations are not faster than a plain add."""
+    copy = ctx.calibrate(0)
+    assert 800.0 < copy < 8000.0, copy
+    simds = 256 * 4
+    rates = {kind: ctx.calibrate(kind) for kind in (1, 2, 3, 4, 5)}
+    for kind, r in rates.items():
+        cycles = 2.4e9 * simds / r
+        assert 1.0 < cycles < 16.0, (kind, cycles)
+    assert rates[2] <= 1.05 * rates[5] and rates[4] <= 1.05 * rates[5]
+    with pytest.raises(Exception):
+        ctx.calibrate(9)

@@ -27,6 +27,7 @@ SYMBOLS = {
     "vq_ctx_sync": (_i32, [_vp]),
     "vq_ctx_stream": (_vp, [_vp]),
     "vq_ctx_set_assign_path": (_i32, [_vp, _i32]),
+    "vq_calibrate": (_i32, [_vp, _i32, C.POINTER(C.c_double)]),
     "vq_ctx_last_recheck_count": (_i32, [_vp, C.POINTER(C.c_uint32)]),
     "vq_ctx_last_recheck_split": (_i32, [_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "vq_procrustes_rotation": (_i32, [_vp, _vp, _i32, _vp]),
@@ -192,6 +193,13 @@ class Context:
     def set_assign_path(self, path):
         """0 = matrix cores + exact re-check (default), 1 = vector ALU only."""
         self._check(_lib.vq_ctx_set_assign_path(self._h, path))
+
+    def calibrate(self, what):
+        """Measured peak: 0 copy GB/s (read + write); 1-5 wave64 instructions per second of
+        v_fma_f32, v_min3_i32, v_med3_i32, v_and_or_b32, v_add_u32 over the whole GPU."""
+        out = C.c_double(0)
+        self._check(_lib.vq_calibrate(self._h, what, C.byref(out)))
+        return out.value
 
     def last_recheck_count(self):
         c = C.c_uint32(0)

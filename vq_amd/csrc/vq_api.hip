@@ -24,6 +24,7 @@
 #define VQ_MFMA_SG 4     // column blocks of 8 floats per wave (4: one 128-byte line of each row)
 #endif
 #include "lbg_update.hpp"
+#include "calibrate.hpp"
 
 namespace vqh {
 std::string &create_error() {
@@ -467,6 +468,59 @@ int32_t vq_timer_stop(vq_ctx *ctx, float *h_ms) {
     VQ_HIP(ctx, hipEventRecord(ctx->ev1, ctx->stream));
     VQ_HIP(ctx, hipEventSynchronize(ctx->ev1));
     VQ_HIP(ctx, hipEventElapsedTime(h_ms, ctx->ev0, ctx->ev1));
+    return VQ_OK;
+}
+
+int32_t vq_calibrate(vq_ctx *ctx, int32_t what, double *h_rate) {
+    if (!ctx || !h_rate) return VQ_ERR_INVALID_ARG;
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    float ms = 0.f;
+    if (what == VQ_CALIB_HBM_COPY) {
+        // 512 MB read + 512 MB written by the plain copy kernel, best of five
+        const int64_t count = 128LL * 1000 * 1000;
+        VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(float) * count));
+        VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(float) * count));
+        VQ_HIP(ctx, hipMemsetAsync(ctx->tmp_a.p, 0, sizeof(float) * count, st));
+        float best = 1e30f;
+        for (int rep = 0; rep < 6; ++rep) {
+            VQ_HIP(ctx, hipEventRecord(ctx->ev0, st));
+            VQ_TRY(vq_copy_f32(ctx, (float *)ctx->tmp_b.p, (const float *)ctx->tmp_a.p, count));
+            VQ_HIP(ctx, hipEventRecord(ctx->ev1, st));
+            VQ_HIP(ctx, hipEventSynchronize(ctx->ev1));
+            VQ_HIP(ctx, hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1));
+            if (rep > 0 && ms < best) best = ms;
+        }
+        *h_rate = 2.0 * sizeof(float) * (double)count / (best * 1e-3) / 1e9;  // GB/s, read + write
+        return VQ_OK;
+    }
+    if (what < VQ_CALIB_VALU_FMA || what > VQ_CALIB_VALU_ADD)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: calibration kind %d", what);
+    hipDeviceProp_t prop;
+    VQ_HIP(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    const int iters = 2048;
+    const unsigned blocks = (unsigned)prop.multiProcessorCount * 8u;  // 8 waves on every SIMD
+    VQ_TRY(ensure(ctx, ctx->tmp_a, 256));
+    float best = 1e30f;
+    for (int rep = 0; rep < 4; ++rep) {
+        VQ_HIP(ctx, hipEventRecord(ctx->ev0, st));
+        uint32_t *sink = (uint32_t *)ctx->tmp_a.p;
+        switch (what) {
+        case VQ_CALIB_VALU_FMA: hipLaunchKernelGGL(vq::k_calib_valu<0>, dim3(blocks), dim3(256), 0, st, iters, 1u, sink); break;
+        case VQ_CALIB_VALU_MIN3: hipLaunchKernelGGL(vq::k_calib_valu<1>, dim3(blocks), dim3(256), 0, st, iters, 1u, sink); break;
+        case VQ_CALIB_VALU_MED3: hipLaunchKernelGGL(vq::k_calib_valu<2>, dim3(blocks), dim3(256), 0, st, iters, 1u, sink); break;
+        case VQ_CALIB_VALU_AND_OR: hipLaunchKernelGGL(vq::k_calib_valu<3>, dim3(blocks), dim3(256), 0, st, iters, 1u, sink); break;
+        default: hipLaunchKernelGGL(vq::k_calib_valu<4>, dim3(blocks), dim3(256), 0, st, iters, 1u, sink); break;
+        }
+        VQ_HIP(ctx, hipGetLastError());
+        VQ_HIP(ctx, hipEventRecord(ctx->ev1, st));
+        VQ_HIP(ctx, hipEventSynchronize(ctx->ev1));
+        VQ_HIP(ctx, hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1));
+        if (rep > 0 && ms < best) best = ms;
+    }
+    // wave64 instructions per second over the whole GPU
+    const double instr = (double)blocks * 4.0 * iters * vq::kCalibChains * vq::kCalibUnroll;
+    *h_rate = instr / (best * 1e-3);
     return VQ_OK;
 }
 
