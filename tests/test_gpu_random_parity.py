@@ -2,6 +2,8 @@
 blocks, encode and LBG mode) against the CPU oracle, bit for bit, over block widths, codebook sizes,
 metrics and data kinds drawn at random: far offsets, duplicate centroids (exact ties between
 candidates), tiny and huge magnitudes, non-finite values."""
+import os
+
 import numpy as np
 import pytest
 
@@ -10,6 +12,8 @@ from tests import data
 
 pytestmark = pytest.mark.gpu
 F = np.float32
+# VQ_PARITY_CASES widens the sweep (the same draws, more seeds)
+N_CASES = int(os.environ.get("VQ_PARITY_CASES", "72"))
 KINDS = ["normal", "uniform", "grid", "offset", "mixture", "dupcb", "tiny", "huge", "nonfinite"]
 
 
@@ -63,7 +67,7 @@ def draw(rng, case):
     return n, dim, m, k, sd, kind, x, cb
 
 
-@pytest.mark.parametrize("case", range(72))
+@pytest.mark.parametrize("case", range(N_CASES))
 def test_random_shape_encode_and_fit(ctx, case):
     import vq_amd
     rng = np.random.default_rng(1000 + case)
