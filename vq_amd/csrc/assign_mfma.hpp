@@ -498,10 +498,13 @@ namespace vq {
 // Error of a score: 3 * 2^-16 (split, as above) + (34 * sd/8 + 16) * 2^-24 (fp32 accumulation of
 // 2 x 17 addends per chunk) + 2^-22 (rounding of x - mu and c - mu), per unit of
 // ||x - mu||^2 + ||c - mu||^2; twice that for two candidates.
+#ifndef VQ_WIDE_STAGE_CHUNKS
+#define VQ_WIDE_STAGE_CHUNKS 2
+#endif
 constexpr int kWideCentreMax = 2048;  // widest column block whose centre is staged in LDS
 
 struct MfmaWideBfTables {
-    const u32x4 *atab;     // [m][sd/8][nb][2][64]
+    const u32x4 *atab;     // [m][sd/8][nb][64]  {ah, al} of the lane's four dimensions
     const float *c2perm;   // [m][nb][2][16]
     const float *blockmax; // [m][nb]  largest ||c - mu||^2 per block of 32 centroids (NaN if any is NaN)
     const float *mu;       // [m][sd]  centre of every column block: mean of its centroids
@@ -617,13 +620,12 @@ static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *_
             hw[w] = hb[0] | (hb[1] << 16);
             lw[w] = lb[0] | (lb[1] << 16);
         }
-        // lane i + 32 h: instruction 1 {ah[4h..4h+3], ah[4h..4h+3]}, instruction 2 {al[4h..4h+3], 1, 1, 1, 0}
-        u32x4 *dst = atab + (((size_t)s * nkc + kc) * nb + b) * 128;
+        // lane i + 32 h holds {ah[4h..4h+3], al[4h..4h+3]}: the kernel builds instruction 1's operand
+        // {ah, ah} and instruction 2's {al, 1, 1, 1, 0} from it, so that only the 16 bytes that differ
+        // between centroids go through LDS
+        u32x4 *dst = atab + (((size_t)s * nkc + kc) * nb + b) * 64;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            dst[32 * h + i] = u32x4{hw[2 * h], hw[2 * h + 1], hw[2 * h], hw[2 * h + 1]};
-            dst[64 + 32 * h + i] = u32x4{lw[2 * h], lw[2 * h + 1], 0x3f803f80u, 0x00003f80u};
-        }
+        for (int h = 0; h < 2; ++h) dst[32 * h + i] = u32x4{hw[2 * h], hw[2 * h + 1], lw[2 * h], lw[2 * h + 1]};
     }
     part[g][i] = p;
     __syncthreads();
@@ -656,7 +658,8 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 template <bool LBG>
 __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, MfmaWideBfTables tb) {
     constexpr int NBMAX = 8;
-    __shared__ u32x4 lds_a[2][NBMAX * 128];  // 2 x 16 KB
+    constexpr int SC = VQ_WIDE_STAGE_CHUNKS;  // chunks of 8 dimensions per stage (per barrier)
+    __shared__ u32x4 lds_a[2][SC * NBMAX * 64];  // 2 stages x SC chunks x 8 KB
     __shared__ float lds_c2[NBMAX * 32];
     __shared__ float lds_mu[kWideCentreMax];
     __shared__ int lds_top[2][2][3][32];     // [row pair][row tile][m1 | m2 | m3][row] of the upper centroid half
@@ -671,10 +674,10 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     const int r = lane & 31, h = lane >> 5;
     const int rp = wave & 1, ch = wave >> 1;
     const int nb = tb.nb, sd = tb.sd, nkc = sd / 8;
-    const u32x4 *ag = tb.atab + (size_t)s * nkc * nb * 128;
-    const int chunk16 = nb * 128;  // 16-byte pieces per chunk
+    const u32x4 *ag = tb.atab + (size_t)s * nkc * nb * 64;
+    const int chunk16 = nb * 64;  // 16-byte pieces per chunk
     for (int i = threadIdx.x; i < nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s * nb * 32 + i];
-    for (int i = threadIdx.x; i < chunk16; i += 256) lds_a[0][i] = ag[i];
+    for (int i = threadIdx.x; i < SC * chunk16; i += 256) lds_a[0][i] = ag[i < nkc * chunk16 ? i : nkc * chunk16 - 1];
     if (threadIdx.x == 0) {
         wg_count = 0;
         wg_pcount = 0;
@@ -711,81 +714,94 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
 #pragma unroll
     for (int t = 0; t < 2; ++t) xn[t] = *reinterpret_cast<const float4 *>(xr[t]);
     float x2[2] = {0.0f, 0.0f};
-    for (int kc = 0; kc < nkc; ++kc) {
-        const int cur = kc & 1;
-        const bool more = kc + 1 < nkc;
-        // operands of this chunk from the rows fetched one chunk ago
-        u32x4 b1[2], b2[2];
+    // A stage is SC chunks of 8 dimensions: one barrier per 16 SC matrix instructions of a wave.
+    // Chunks past the last one have zero row operands (they add nothing).
+    const int nst = (nkc + SC - 1) / SC;
+    const int total16 = nkc * chunk16;
+    for (int st = 0; st < nst; ++st) {
+        const int cur = st & 1;
+        const bool more = st + 1 < nst;
+        // the A operands of the next stage: into registers now, into LDS at the end of this stage
+        u32x4 pre[2 * SC];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            float xv[4] = {xn[t].x, xn[t].y, xn[t].z, xn[t].w};
-            if (shifted) {
-                const float4 mn = *reinterpret_cast<const float4 *>(lds_mu + kc * 8 + 4 * h);
-                xv[0] -= mn.x;
-                xv[1] -= mn.y;
-                xv[2] -= mn.z;
-                xv[3] -= mn.w;
+        for (int q = 0; q < 2 * SC; ++q) {
+            const int i = (st + 1) * SC * chunk16 + (int)threadIdx.x + 256 * q;
+            pre[q] = ag[i < total16 ? i : total16 - 1];
+        }
+#pragma unroll
+        for (int sub = 0; sub < SC; ++sub) {
+            const int kc = SC * st + sub;
+            const bool live = kc < nkc;  // uniform
+            const int kcc = live ? kc : nkc - 1;
+            // operands of this chunk from the rows fetched one chunk ago
+            u32x4 b1[2], b2[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                float xv[4] = {xn[t].x, xn[t].y, xn[t].z, xn[t].w};
+                if (shifted) {
+                    const float4 mn = *reinterpret_cast<const float4 *>(lds_mu + kcc * 8 + 4 * h);
+                    xv[0] -= mn.x;
+                    xv[1] -= mn.y;
+                    xv[2] -= mn.z;
+                    xv[3] -= mn.w;
+                }
+                if (!live) xv[0] = xv[1] = xv[2] = xv[3] = 0.0f;
+                float p = 0.0f;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
+                const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
+                const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
+                const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
+                x2[t] += p;
+                const uint32_t p0 = bf16_pack2(p, 0.0f);
+                const float r1 = p - __uint_as_float(p0 << 16);
+                const uint32_t p1 = bf16_pack2(r1, 0.0f);
+                const float r2 = r1 - __uint_as_float(p1 << 16);
+                const uint32_t p2 = bf16_pack2(r2, 0.0f);
+                b1[t] = u32x4{h01, h23, l01, l23};
+                b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu};
             }
-            float p = 0.0f;
+            // fetch the next chunk of the rows
+            const int nx = kc + 1 < nkc ? kc + 1 : nkc - 1;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
-            const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
-            const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
-            const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
-            x2[t] += p;
-            const uint32_t p0 = bf16_pack2(p, 0.0f);
-            const float r1 = p - __uint_as_float(p0 << 16);
-            const uint32_t p1 = bf16_pack2(r1, 0.0f);
-            const float r2 = r1 - __uint_as_float(p1 << 16);
-            const uint32_t p2 = bf16_pack2(r2, 0.0f);
-            b1[t] = u32x4{h01, h23, l01, l23};
-            b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu};
-        }
-        // fetch the next chunk: rows into registers, A operands into registers then LDS
-        u32x4 pre[4];
-        const int nx = more ? kc + 1 : kc;
+            for (int t = 0; t < 2; ++t) xn[t] = *reinterpret_cast<const float4 *>(xr[t] + nx * 8);
+            // the A operands of the wave's four centroid tiles are read from LDS together (a tile
+            // past the last block reads the last block and is not multiplied): one LDS round trip
+            // per chunk instead of one per tile
+            u32x4 a1[4], a2[4];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) xn[t] = *reinterpret_cast<const float4 *>(xr[t] + nx * 8);
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int i = threadIdx.x + 256 * q;
-            pre[q] = ag[(size_t)nx * chunk16 + (i < chunk16 ? i : chunk16 - 1)];
-        }
-        // the A operands of the wave's four centroid tiles are read from LDS together (a tile past
-        // the last block reads the last block and is not multiplied): one LDS round trip per
-        // chunk instead of one per tile
-        u32x4 a1[4], a2[4];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int b = 4 * ch + c < nb ? 4 * ch + c : nb - 1;
-            a1[c] = lds_a[cur][b * 128 + lane];
-            a2[c] = lds_a[cur][b * 128 + 64 + lane];
-        }
-        // first instruction of every accumulator tile, then the second: the two instructions of a
-        // tile depend on each other and are kept seven others apart
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if (4 * ch + c < nb) {
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8, a1[c]), __builtin_bit_cast(bf16x8, b1[t]), acc[t][c], 0, 0, 0);
+            for (int c = 0; c < 4; ++c) {
+                const int b = 4 * ch + c < nb ? 4 * ch + c : nb - 1;
+                const u32x4 v = lds_a[cur][sub * chunk16 + b * 64 + lane];
+                a1[c] = u32x4{v.x, v.y, v.x, v.y};
+                a2[c] = u32x4{v.z, v.w, 0x3f803f80u, 0x00003f80u};
             }
-        }
+            // first instruction of every accumulator tile, then the second: the two instructions
+            // of a tile depend on each other and are kept seven others apart
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if (4 * ch + c < nb) {
+            for (int c = 0; c < 4; ++c) {
+                if (4 * ch + c < nb) {
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-                    acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                        __builtin_bit_cast(bf16x8, a2[c]), __builtin_bit_cast(bf16x8, b2[t]), acc[t][c], 0, 0, 0);
+                    for (int t = 0; t < 2; ++t)
+                        acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(bf16x8, a1[c]), __builtin_bit_cast(bf16x8, b1[t]), acc[t][c], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (4 * ch + c < nb) {
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+                        acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(bf16x8, a2[c]), __builtin_bit_cast(bf16x8, b2[t]), acc[t][c], 0, 0, 0);
+                }
             }
         }
         if (more) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
+            for (int q = 0; q < 2 * SC; ++q) {
                 const int i = threadIdx.x + 256 * q;
-                if (i < chunk16) lds_a[cur ^ 1][i] = pre[q];
+                if (i < SC * chunk16) lds_a[cur ^ 1][i] = pre[q];
             }
         }
         lds_barrier();
