@@ -833,4 +833,20 @@ static __global__ void __launch_bounds__(256) k_tsvq_decode_f16(const int *__res
     out[i] = __half_as_ushort(__float2half_rn(cen[(size_t)leaf[row] * dim + t]));
 }
 
+// Four consecutive components per thread (dim a multiple of 4, 16-byte aligned centroids and output).
+static __global__ void __launch_bounds__(256) k_tsvq_decode4_f16(const int *__restrict__ leaf, int64_t n, int dim,
+                                                          const float *__restrict__ cen,
+                                                          uint2 *__restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int dim4 = dim / 4;
+    if (i >= n * dim4) return;
+    const int64_t row = i / dim4;
+    const int t = (int)(i % dim4) * 4;
+    const float4 v = *reinterpret_cast<const float4 *>(cen + (size_t)leaf[row] * dim + t);
+    uint2 o;
+    o.x = (uint32_t)__half_as_ushort(__float2half_rn(v.x)) | ((uint32_t)__half_as_ushort(__float2half_rn(v.y)) << 16);
+    o.y = (uint32_t)__half_as_ushort(__float2half_rn(v.z)) | ((uint32_t)__half_as_ushort(__float2half_rn(v.w)) << 16);
+    out[i] = o;
+}
+
 }  // namespace vq

@@ -293,6 +293,29 @@ __global__ void k_decode_f16(const uint8_t *__restrict__ codes, int64_t n, int m
     out[i] = __half_as_ushort(__float2half_rn(v));
 }
 
+// Four consecutive components per thread (sub_dim a multiple of 4, 16-byte aligned codebooks and
+// output rows): one 16-byte load of the centroid, one 8- or 16-byte store.  F16: binary16 bit
+// patterns (round to nearest even), else f32.
+template <bool F16>
+__global__ void __launch_bounds__(256) k_decode_vec4(const uint8_t *__restrict__ codes, int64_t n, int m, int sd,
+                                                     int k, const float *__restrict__ cb, void *__restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // group of four components
+    const int64_t dim4 = (int64_t)m * sd / 4;
+    if (i >= n * dim4) return;
+    const int64_t row = i / dim4;
+    const int c = (int)(i % dim4) * 4;
+    const int s = c / sd, t = c % sd;
+    const float4 v = *reinterpret_cast<const float4 *>(cb + ((size_t)s * k + codes[row * m + s]) * sd + t);
+    if constexpr (F16) {
+        uint2 o;
+        o.x = (uint32_t)__half_as_ushort(__float2half_rn(v.x)) | ((uint32_t)__half_as_ushort(__float2half_rn(v.y)) << 16);
+        o.y = (uint32_t)__half_as_ushort(__float2half_rn(v.z)) | ((uint32_t)__half_as_ushort(__float2half_rn(v.w)) << 16);
+        reinterpret_cast<uint2 *>(out)[i] = o;
+    } else {
+        reinterpret_cast<float4 *>(out)[i] = v;
+    }
+}
+
 __global__ void k_decode_f32(const uint8_t *__restrict__ codes, int64_t n, int m, int sd, int k,
                              const float *__restrict__ cb, float *__restrict__ out) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -789,8 +812,12 @@ int32_t vq_decode_f16(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m,
     if (!d_codes || !d_codebooks || !d_out || n < 0 || m <= 0 || sd <= 0 || k <= 0 || k > vq::kMaxK)
         return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
     VQ_HIP(ctx, hipSetDevice(ctx->device));
-    hipLaunchKernelGGL(k_decode_f16, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n,
-                       m, sd, k, d_codebooks, d_out);
+    if (sd % 4 == 0 && ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) == 0)
+        hipLaunchKernelGGL(k_decode_vec4<true>, dim3(cdiv(n * m * sd / 4, 256)), dim3(256), 0, ctx->stream, d_codes,
+                           n, m, sd, k, d_codebooks, (void *)d_out);
+    else
+        hipLaunchKernelGGL(k_decode_f16, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n,
+                           m, sd, k, d_codebooks, d_out);
     VQ_HIP(ctx, hipGetLastError());
     return VQ_OK;
 }
@@ -802,8 +829,12 @@ int32_t vq_decode_f32(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m,
     if (!d_codes || !d_codebooks || !d_out || n < 0 || m <= 0 || sd <= 0 || k <= 0 || k > vq::kMaxK)
         return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
     VQ_HIP(ctx, hipSetDevice(ctx->device));
-    hipLaunchKernelGGL(k_decode_f32, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n,
-                       m, sd, k, d_codebooks, d_out);
+    if (sd % 4 == 0 && ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) == 0)
+        hipLaunchKernelGGL(k_decode_vec4<false>, dim3(cdiv(n * m * sd / 4, 256)), dim3(256), 0, ctx->stream, d_codes,
+                           n, m, sd, k, d_codebooks, (void *)d_out);
+    else
+        hipLaunchKernelGGL(k_decode_f32, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n,
+                           m, sd, k, d_codebooks, d_out);
     VQ_HIP(ctx, hipGetLastError());
     return VQ_OK;
 }

@@ -468,8 +468,13 @@ int32_t vq_tsvq_decode_f16(vq_ctx *ctx, const vq_tree *tree, const int32_t *d_le
     if (n == 0) return VQ_OK;
     if (!d_leaf || !d_out || n < 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
     VQ_HIP(ctx, hipSetDevice(ctx->device));
-    hipLaunchKernelGGL(vq::k_tsvq_decode_f16, dim3(cdiv(n * tree->dim, 256)), dim3(256), 0, ctx->stream, d_leaf,
-                       n, tree->dim, tree->d_centroids, d_out);
+    if (tree->dim % 4 == 0 &&
+        ((reinterpret_cast<uintptr_t>(tree->d_centroids) | reinterpret_cast<uintptr_t>(d_out)) & 15) == 0)
+        hipLaunchKernelGGL(vq::k_tsvq_decode4_f16, dim3(cdiv(n * (tree->dim / 4), 256)), dim3(256), 0, ctx->stream,
+                           d_leaf, n, tree->dim, tree->d_centroids, reinterpret_cast<uint2 *>(d_out));
+    else
+        hipLaunchKernelGGL(vq::k_tsvq_decode_f16, dim3(cdiv(n * tree->dim, 256)), dim3(256), 0, ctx->stream, d_leaf,
+                           n, tree->dim, tree->d_centroids, d_out);
     VQ_HIP(ctx, hipGetLastError());
     return VQ_OK;
 }
