@@ -503,29 +503,45 @@ static __global__ void __launch_bounds__(256) k_seg_select_hist(const float *__r
     }
 }
 
-// One thread per (segment, target): the byte whose bin holds the rank; clears the bins.
-static __global__ void k_seg_select_pick(uint32_t *__restrict__ hist, SegSelect *__restrict__ sel, int nseg,
-                                         int pass) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+// One wave per (segment, target): the byte whose bin holds the rank; clears the bins.  A lane
+// takes four bins, a scan over the lanes finds the one whose bins hold the rank.
+static __global__ void __launch_bounds__(64) k_seg_select_pick(uint32_t *__restrict__ hist,
+                                                               SegSelect *__restrict__ sel, int nseg, int pass) {
+    const int i = blockIdx.x, lane = threadIdx.x;
     if (i >= 2 * nseg) return;
-    uint32_t *h = hist + (size_t)i * 256;
-    SegSelect s = sel[i];
-    uint32_t byte = 255u;
-    bool found = false;
-    for (uint32_t b = 0; b < 256u; ++b) {
-        const uint32_t c = h[b];
-        h[b] = 0u;
-        if (!found) {
-            if (s.rank < c) {
-                byte = b;
-                found = true;
-            } else {
-                s.rank -= c;
+    uint4 *h = reinterpret_cast<uint4 *>(hist + (size_t)i * 256);
+    const uint4 c = h[lane];
+    h[lane] = make_uint4(0u, 0u, 0u, 0u);
+    const SegSelect s = sel[i];
+    const uint32_t tot = c.x + c.y + c.z + c.w;
+    uint32_t inc = tot;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t v = __shfl_up(inc, off);
+        if (lane >= off) inc += v;
+    }
+    const uint32_t exc = inc - tot;
+    const bool mine = s.rank >= exc && s.rank < inc;
+    const int shift = 24 - 8 * pass;
+    if (mine) {
+        uint32_t r = s.rank - exc, byte = 4u * (uint32_t)lane;
+        if (r >= c.x) {
+            r -= c.x;
+            ++byte;
+            if (r >= c.y) {
+                r -= c.y;
+                ++byte;
+                if (r >= c.z) {
+                    r -= c.z;
+                    ++byte;
+                }
             }
         }
+        sel[i] = SegSelect{s.prefix | (byte << shift), r};
     }
-    s.prefix |= byte << (24 - 8 * pass);
-    sel[i] = s;
+    // a rank beyond the counted keys (never for a rank inside its segment): the last byte
+    const uint32_t all = __shfl(inc, 63);
+    if (lane == 0 && s.rank >= all) sel[i] = SegSelect{s.prefix | (255u << shift), s.rank - all};
 }
 
 static __global__ void k_seg_select_out(const SegSelect *__restrict__ sel, int nseg, float *__restrict__ mids) {

@@ -281,7 +281,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         for (int pass = 0; pass < 4; ++pass) {
             hipLaunchKernelGGL(vq::k_seg_select_hist, dim3(cdiv(n, 4096)), dim3(256), 0, st, (const float *)vals, n,
                                (const uint2 *)d_range, ns, (const vq::SegSelect *)d_sel, pass, (uint32_t *)d_hist);
-            hipLaunchKernelGGL(vq::k_seg_select_pick, dim3(cdiv(2 * ns, 64)), dim3(64), 0, st, (uint32_t *)d_hist,
+            hipLaunchKernelGGL(vq::k_seg_select_pick, dim3(2 * ns), dim3(64), 0, st, (uint32_t *)d_hist,
                                (vq::SegSelect *)d_sel, ns, pass);
         }
         hipLaunchKernelGGL(vq::k_seg_select_out, dim3(cdiv(2 * ns, 64)), dim3(64), 0, st,
