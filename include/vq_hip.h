@@ -72,6 +72,15 @@ void *vq_ctx_stream(vq_ctx *ctx);
  * Both give bit-identical codes; the switch exists for measurement and tests. */
 int32_t vq_ctx_set_assign_path(vq_ctx *ctx, int32_t path);
 
+/* How vq_tsvq_build sums a node's squared deviations per dimension in row order (src/tsvq.rs:88-99)
+ * when dim is a multiple of 8:
+ *   0 (default)  groups of 32 squares as integer maps on the running sum, composed by a scan, with
+ *                the groups in which the sum changes binade added one by one
+ *   1            one chain of dependent adds per column
+ * Both give the reference's sequential f32 sums bit for bit; the switch exists for measurement and
+ * tests.  No counterpart in the reference. */
+int32_t vq_ctx_set_tsvq_variance_path(vq_ctx *ctx, int32_t path);
+
 /* Measured peaks of this GPU, for pricing the kernels (measurement only; no counterpart in the
  * reference).  VQ_CALIB_HBM_COPY: GB/s of the plain copy kernel over 512 MB (bytes read + bytes
  * written per second).  VQ_CALIB_VALU_*: wave64 instructions of that kind per second over the

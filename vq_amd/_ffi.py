@@ -27,6 +27,7 @@ SYMBOLS = {
     "vq_ctx_sync": (_i32, [_vp]),
     "vq_ctx_stream": (_vp, [_vp]),
     "vq_ctx_set_assign_path": (_i32, [_vp, _i32]),
+    "vq_ctx_set_tsvq_variance_path": (_i32, [_vp, _i32]),
     "vq_calibrate": (_i32, [_vp, _i32, C.POINTER(C.c_double)]),
     "vq_ctx_last_recheck_count": (_i32, [_vp, C.POINTER(C.c_uint32)]),
     "vq_ctx_last_recheck_split": (_i32, [_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
@@ -200,6 +201,10 @@ class Context:
         out = C.c_double(0)
         self._check(_lib.vq_calibrate(self._h, what, C.byref(out)))
         return out.value
+
+    def set_tsvq_variance_path(self, path):
+        """0: composed integer maps (default); 1: one chain of adds per column."""
+        self._check(_lib.vq_ctx_set_tsvq_variance_path(self._h, path))
 
     def last_recheck_count(self):
         c = C.c_uint32(0)

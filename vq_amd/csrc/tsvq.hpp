@@ -100,11 +100,18 @@ static __global__ void __launch_bounds__(64) k_seg_variance(const uint32_t *__re
 // Grid (blocks of 64 positions, segments); one lane per (group of 32 positions, column).
 constexpr int kChainGroup = 32;  // positions per group
 
+// Index of a segment's first group in the per-group tables (group sums, binade guesses, maps):
+// segment g's squares start at row range.x + 32 g of sq32, and the groups of different segments
+// never share an index.
+__device__ __forceinline__ size_t seg_group0(const uint2 range, int g) {
+    return ((size_t)range.x + 32u * (size_t)g) / 32u;
+}
+
 static __global__ void __launch_bounds__(256) k_seg_sqdev32(const uint32_t *__restrict__ perm,
                                                             const uint2 *__restrict__ seg_range,
                                                             const float *__restrict__ means, int64_t first,
                                                             const float *__restrict__ x, int64_t ld, int dim,
-                                                            float *__restrict__ sq32) {
+                                                            float *__restrict__ sq32, float *__restrict__ gsum) {
     const int g = blockIdx.y;
     const uint2 range = seg_range[g];
     const uint32_t count = range.y - range.x;
@@ -119,6 +126,7 @@ static __global__ void __launch_bounds__(256) k_seg_sqdev32(const uint32_t *__re
         const uint32_t P = P0 + e / (uint32_t)dim, c = e % (uint32_t)dim;
         const float m = mrow[c];
         float4 *o = reinterpret_cast<float4 *>(out + (size_t)P * 32 * dim + (c / 8u) * 256u + (c % 8u) * 32u);
+        float gs = 0.0f;  // the group's sum, any order: only used to guess the running sum's binade
 #pragma unroll
         for (int h = 0; h < 2; ++h) {  // sixteen loads in flight at a time
             float q[16];
@@ -127,10 +135,12 @@ static __global__ void __launch_bounds__(256) k_seg_sqdev32(const uint32_t *__re
                 const uint32_t p = 32u * P + 16u * h + r;  // past the end: the last row again, never added
                 const float d = x[(int64_t)pm[p < count ? p : count - 1] * ld + c] - m;
                 q[r] = d * d;
+                gs += p < count ? q[r] : 0.0f;
             }
 #pragma unroll
             for (int r = 0; r < 4; ++r) o[4 * h + r] = make_float4(q[4 * r], q[4 * r + 1], q[4 * r + 2], q[4 * r + 3]);
         }
+        if (gsum) gsum[(seg_group0(range, g) + P) * dim + c] = gs;
     }
 }
 
@@ -215,6 +225,205 @@ static __global__ void __launch_bounds__(256) k_seg_chain32(const float *__restr
         }
     }
     if ((lane & 7) == 0) var[(size_t)g * dim + cb * 8 + (lane >> 3)] = acc;
+}
+
+// ---- the same sequential sums without the long chain -------------------------------------------
+// A sequential f32 sum of non-negative terms is, while the running sum S stays inside one binade
+// [2^e, 2^(e+1)], an integer accumulation: with u = 2^(e-23) and S = s u, fl(S + t) = (s + r) u where
+// r is t / u rounded to an integer, to nearest, a tie to the value that makes s + r even.  So a
+// group of 32 terms acts on s as s -> s + inc[parity of s], two integers per group that depend on e
+// only, and the maps of consecutive groups compose.  Three steps on top of k_seg_sqdev32 (which
+// also emits every group's approximate sum):
+//   k_seg_chain_guess    per column, a prefix over the group sums in f64 gives the binade the running
+//                        sum will be in at each group (two candidates near a boundary)
+//   k_seg_chain_maps     per (group, column), on the whole GPU: inc[0], inc[1] for the guessed binade(s)
+//   k_seg_chain_compose  per column, one wave: 64 groups at a time, the maps composed by a scan over
+//                        the lanes; it checks every assumption (S is in the guessed binade at the
+//                        group's start and does not leave it) and adds a group's 32 terms one by one
+//                        where one fails — the groups in which S crosses a binade, the first groups,
+//                        non-finite values.  The result is the sequential sum, bit for bit.
+constexpr uint32_t kMapInvalid = 0xFFFFFFFFu;
+// guess code: exponent field of the lower candidate | two candidates | all terms zero | usable
+constexpr uint16_t kGuessOk = 0x8000u, kGuessTwo = 0x0100u, kGuessZero = 0x0200u;
+
+// grid (segments, dim / 4); 256 threads = 4 waves, one column each.
+static __global__ void __launch_bounds__(256) k_seg_chain_guess(const float *__restrict__ gsum,
+                                                               const uint2 *__restrict__ seg_range, int dim,
+                                                               uint16_t *__restrict__ guess) {
+    const int g = blockIdx.x, lane = threadIdx.x & 63, c = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (c >= dim) return;
+    const uint2 range = seg_range[g];
+    const uint32_t count = range.y - range.x, nP = (count + 31u) / 32u;
+    const size_t g0 = seg_group0(range, g);
+    double carry = 0.0;
+    for (uint32_t P0 = 0; P0 < nP; P0 += 64) {
+        const uint32_t P = P0 + lane;
+        const double v = P < nP ? (double)gsum[(g0 + P) * dim + c] : 0.0;
+        double inc = v;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const double o = __shfl_up(inc, off);
+            if (lane >= off) inc += o;
+        }
+        const double before = carry + (inc - v), after = carry + inc;
+        carry = __shfl(after, 63);
+        if (P < nP) {
+            // the sequential f32 sum is within 2^-9 of the f64 one by a wide margin
+            const float lo = (float)(before * (1.0 - 0.001953125)), hi = (float)(after * (1.0 + 0.001953125));
+            const uint32_t elo = __float_as_uint(lo) >> 23, ehi = __float_as_uint(hi) >> 23;  // both >= +0
+            uint16_t code = 0;
+            if (v == 0.0)  // non-negative terms with a zero sum: every one is +0 and leaves any S as it is
+                code = (uint16_t)(kGuessOk | kGuessZero);
+            else if (before > 0.0 && elo >= 30u && ehi <= 250u && ehi - elo <= 1u)
+                code = (uint16_t)(kGuessOk | (ehi != elo ? kGuessTwo : 0u) | elo);
+            guess[(g0 + P) * dim + c] = code;
+        }
+    }
+}
+
+// inc[0], inc[1] of one group for a running sum in the binade of exponent field e.
+__device__ __forceinline__ void chain_group_map(const float (&t)[32], int valid, uint32_t e, uint32_t &inc0,
+                                                uint32_t &inc1) {
+    uint32_t a0 = 0, a1 = 0, par0 = 0, par1 = 1;
+    bool bad = false;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        if (i < valid) {
+            const uint32_t tb = __float_as_uint(t[i]);
+            uint32_t et = (tb >> 23) & 255u, m = tb & 0x7fffffu;
+            bad = bad || (tb >> 31) != 0u || et == 255u;
+            if (et == 0u) et = 1u; else m |= 0x800000u;
+            const int sh = (int)e - (int)et;
+            bad = bad || sh < 0;
+            uint32_t q = 0, up = 0, tie = 0;
+            if (sh >= 0 && sh < 25) {
+                q = m >> sh;
+                const uint32_t rem = m & ((1u << sh) - 1u), half = (1u << sh) >> 1;
+                up = rem > half ? 1u : 0u;
+                tie = (sh > 0 && rem == half) ? 1u : 0u;
+            }
+            const uint32_t d0 = q + up + (tie & (par0 + q)), d1 = q + up + (tie & (par1 + q));
+            a0 += d0;
+            a1 += d1;
+            par0 = (par0 + d0) & 1u;
+            par1 = (par1 + d1) & 1u;
+        }
+    }
+    inc0 = bad ? kMapInvalid : a0;
+    inc1 = bad ? kMapInvalid : a1;
+}
+
+// Grid (blocks of 64 positions, segments), as k_seg_sqdev32: one thread per (group, column).
+static __global__ void __launch_bounds__(256) k_seg_chain_maps(const float *__restrict__ sq32,
+                                                              const uint2 *__restrict__ seg_range, int dim,
+                                                              const uint16_t *__restrict__ guess,
+                                                              uint4 *__restrict__ maps) {
+    const int g = blockIdx.y;
+    const uint2 range = seg_range[g];
+    const uint32_t count = range.y - range.x;
+    const uint32_t P0 = blockIdx.x * 2u;
+    if (P0 * 32u >= count) return;
+    const uint32_t nP = (count + 31u) / 32u;
+    const uint32_t groups = nP - P0 < 2u ? nP - P0 : 2u;
+    const float *in = sq32 + ((size_t)range.x + 32u * (size_t)g) * dim;
+    const size_t g0 = seg_group0(range, g);
+    for (uint32_t e = threadIdx.x; e < groups * (uint32_t)dim; e += 256) {
+        const uint32_t P = P0 + e / (uint32_t)dim, c = e % (uint32_t)dim;
+        const uint16_t code = guess[(g0 + P) * dim + c];
+        uint4 out = make_uint4(kMapInvalid, kMapInvalid, kMapInvalid, kMapInvalid);
+        if (code & kGuessZero) {
+            out = make_uint4(0u, 0u, 0u, 0u);
+        } else if (code & kGuessOk) {
+            const float4 *q = reinterpret_cast<const float4 *>(in + (size_t)P * 32 * dim + (c / 8u) * 256u + (c % 8u) * 32u);
+            float t[32];
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const float4 v = q[r];
+                t[4 * r] = v.x, t[4 * r + 1] = v.y, t[4 * r + 2] = v.z, t[4 * r + 3] = v.w;
+            }
+            const int valid = (int)(count - 32u * P < 32u ? count - 32u * P : 32u);
+            const uint32_t elo = code & 255u;
+            chain_group_map(t, valid, elo, out.x, out.y);
+            if (code & kGuessTwo) chain_group_map(t, valid, elo + 1u, out.z, out.w);
+        }
+        maps[(g0 + P) * dim + c] = out;
+    }
+}
+
+// grid (segments, dim / 4); 256 threads = 4 waves, one column each.
+static __global__ void __launch_bounds__(256) k_seg_chain_compose(const float *__restrict__ sq32,
+                                                                 const uint2 *__restrict__ seg_range, int dim,
+                                                                 const uint16_t *__restrict__ guess,
+                                                                 const uint4 *__restrict__ maps,
+                                                                 float *__restrict__ var) {
+    const int g = blockIdx.x, lane = threadIdx.x & 63, c = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (c >= dim) return;
+    const uint2 range = seg_range[g];
+    const uint32_t count = range.y - range.x, nP = (count + 31u) / 32u;
+    const size_t g0 = seg_group0(range, g);
+    const float *q = sq32 + ((size_t)range.x + 32u * (size_t)g) * dim + (c / 8) * 256 + (c % 8) * 32;
+    float S = 0.0f;  // the same value in every lane
+    uint32_t P = 0;
+    while (P < nP) {
+        // S is +0, positive, +inf or a NaN; with the sign bit of a NaN eS is above every guess
+        const uint32_t Sb = __float_as_uint(S), eS = Sb >> 23;
+        bool seq = true;
+        uint32_t adv = 1;
+        {
+            const uint32_t s = (Sb & 0x7fffffu) | 0x800000u;  // S / u for a normal S
+            const uint32_t idx = P + lane;
+            const bool in = idx < nP;
+            const uint16_t code = in ? guess[(g0 + idx) * dim + c] : (uint16_t)0;
+            uint4 mp = make_uint4(kMapInvalid, kMapInvalid, kMapInvalid, kMapInvalid);
+            if (in) mp = maps[(g0 + idx) * dim + c];
+            const uint32_t elo = code & 255u;
+            const bool zero = (code & kGuessZero) != 0;
+            const bool is_lo = elo == eS, is_hi = (code & kGuessTwo) && elo + 1u == eS;
+            uint32_t a0 = is_lo ? mp.x : mp.z, a1 = is_lo ? mp.y : mp.w;
+            // a group of zeros keeps any finite S; another group needs S in the binade of its map
+            const bool ok = in && (code & kGuessOk) &&
+                            (zero ? eS < 255u : (eS >= 30u && eS <= 250u && (is_lo || is_hi) && a0 != kMapInvalid));
+            if (zero) a0 = a1 = 0u;
+            const unsigned long long okm = __ballot(ok);
+            const int first = okm == ~0ull ? 64 : __ffsll((long long)~okm) - 1;  // leading lanes that are ok
+            if (first > 0) {
+                const uint32_t cap = 1u << 25;
+                if (lane >= first) a0 = a1 = 0u;
+                a0 = a0 < cap ? a0 : cap;
+                a1 = a1 < cap ? a1 : cap;
+                // inclusive scan: the map of groups P .. P + lane, as increments for a start parity
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) {
+                    const uint32_t b0 = __shfl_up(a0, off), b1 = __shfl_up(a1, off);
+                    if (lane >= off) {
+                        const uint32_t n0 = b0 + ((b0 & 1u) ? a1 : a0);        // start even: after b0 the parity is b0 & 1
+                        const uint32_t n1 = b1 + (((b1 + 1u) & 1u) ? a1 : a0);  // start odd
+                        a0 = n0 < cap ? n0 : cap;
+                        a1 = n1 < cap ? n1 : cap;
+                    }
+                }
+                const uint32_t send = s + ((s & 1u) ? a1 : a0);
+                const bool fits = lane < first && send <= (1u << 24);
+                const int nv = __popcll(__ballot(fits));  // fits is monotone: the sums never decrease
+                if (nv > 0) {
+                    const uint32_t take = __shfl(send, nv - 1);
+                    // (a subnormal or zero S only passes groups of zeros: take == s and S stays)
+                    S = __uint_as_float(take == (1u << 24) ? (eS + 1u) << 23 : (eS << 23) | (take - (1u << 23)));
+                    seq = false;
+                    adv = (uint32_t)nv;
+                }
+            }
+        }
+        if (seq) {
+            // the group's terms one by one (positions past the end add +0.0, which changes nothing)
+            float t = 0.0f;
+            if (lane < 32 && P * 32u + (uint32_t)lane < count) t = q[(size_t)P * 32 * dim + lane];
+#pragma unroll
+            for (int i = 0; i < 32; ++i) S = S + __shfl(t, i);
+        }
+        P += adv;
+    }
+    if (lane == 0) var[(size_t)g * dim + c] = S;
 }
 
 // The same sums with everything but the adds taken off the chain of dependent adds.  One workgroup

@@ -425,7 +425,7 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     if (ctx->side) (void)hipStreamSynchronize(ctx->side);
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
-                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
+                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tsvq_gsum, &ctx->tsvq_guess, &ctx->tsvq_maps, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     prof_collect(ctx);
@@ -544,6 +544,12 @@ int32_t vq_calibrate(vq_ctx *ctx, int32_t what, double *h_rate) {
     // wave64 instructions per second over the whole GPU
     const double instr = (double)blocks * 4.0 * iters * vq::kCalibChains * vq::kCalibUnroll;
     *h_rate = instr / (best * 1e-3);
+    return VQ_OK;
+}
+
+int32_t vq_ctx_set_tsvq_variance_path(vq_ctx *ctx, int32_t path) {
+    if (!ctx || (path != 0 && path != 1)) return VQ_ERR_INVALID_ARG;
+    ctx->tsvq_var_path = path;
     return VQ_OK;
 }
 

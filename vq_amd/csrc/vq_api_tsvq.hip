@@ -99,6 +99,14 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     if (var_chain)
         VQ_TRY(ensure(ctx, ctx->tsvq_sq, sizeof(float) * ((size_t)n + vq::kChainGroup * (size_t)kChainSegs) * dim));
     float *d_sq = (float *)ctx->tsvq_sq.p;
+    // per group of 32 squares (composed-maps path): approximate sum, binade guess, integer maps
+    const bool var_maps = var_chain && ctx->tsvq_var_path == 0;
+    if (var_maps) {
+        const size_t ngroups = ((size_t)n + vq::kChainGroup * (size_t)kChainSegs) / vq::kChainGroup + 2;
+        VQ_TRY(ensure(ctx, ctx->tsvq_gsum, sizeof(float) * ngroups * dim));
+        VQ_TRY(ensure(ctx, ctx->tsvq_guess, sizeof(uint16_t) * ngroups * dim));
+        VQ_TRY(ensure(ctx, ctx->tsvq_maps, sizeof(uint4) * ngroups * dim));
+    }
     uint32_t *perm = (uint32_t *)ctx->tmp_a.p, *perm2 = (uint32_t *)ctx->tmp_b.p;
     float *vals = (float *)ctx->tmp_c.p;
     uint32_t *flags = (uint32_t *)ctx->tmp_e.p, *scan = (uint32_t *)ctx->tmp_f.p;
@@ -240,9 +248,22 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             for (int i = 0; i < ns; ++i) longest = std::max(longest, range[i].y - range[i].x);
             hipLaunchKernelGGL(vq::k_seg_sqdev32, dim3((unsigned)cdiv((int64_t)longest, 64), (unsigned)ns), dim3(256),
                                0, st, perm, (const uint2 *)d_range, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
-                               d_sq);
-            hipLaunchKernelGGL(vq::k_seg_chain32, dim3((unsigned)ns, (unsigned)cdiv(dim, 32)), dim3(256), 0, st,
-                               (const float *)d_sq, (const uint2 *)d_range, dim, (float *)d_var);
+                               d_sq, var_maps ? (float *)ctx->tsvq_gsum.p : (float *)nullptr);
+            if (var_maps) {
+                hipLaunchKernelGGL(vq::k_seg_chain_guess, dim3((unsigned)ns, (unsigned)cdiv(dim, 4)), dim3(256), 0, st,
+                                   (const float *)ctx->tsvq_gsum.p, (const uint2 *)d_range, dim,
+                                   (uint16_t *)ctx->tsvq_guess.p);
+                hipLaunchKernelGGL(vq::k_seg_chain_maps, dim3((unsigned)cdiv((int64_t)longest, 64), (unsigned)ns),
+                                   dim3(256), 0, st, (const float *)d_sq, (const uint2 *)d_range, dim,
+                                   (const uint16_t *)ctx->tsvq_guess.p, (uint4 *)ctx->tsvq_maps.p);
+                hipLaunchKernelGGL(vq::k_seg_chain_compose, dim3((unsigned)ns, (unsigned)cdiv(dim, 4)), dim3(256), 0,
+                                   st, (const float *)d_sq, (const uint2 *)d_range, dim,
+                                   (const uint16_t *)ctx->tsvq_guess.p, (const uint4 *)ctx->tsvq_maps.p,
+                                   (float *)d_var);
+            } else {
+                hipLaunchKernelGGL(vq::k_seg_chain32, dim3((unsigned)ns, (unsigned)cdiv(dim, 32)), dim3(256), 0, st,
+                                   (const float *)d_sq, (const uint2 *)d_range, dim, (float *)d_var);
+            }
         } else if (dim % 4 == 0 && dim <= 1024 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0) {
 #define VARIANCE_WG(D)                                                                                     \
     hipLaunchKernelGGL((vq::k_seg_variance_wg<D>), dim3(ns), dim3(1024), 0, st, perm, (const uint2 *)d_range, \
