@@ -256,27 +256,37 @@ static __global__ void __launch_bounds__(256) k_seg_chain_guess(const float *__r
     const uint32_t count = range.y - range.x, nP = (count + 31u) / 32u;
     const size_t g0 = seg_group0(range, g);
     double carry = 0.0;
-    for (uint32_t P0 = 0; P0 < nP; P0 += 64) {
-        const uint32_t P = P0 + lane;
-        const double v = P < nP ? (double)gsum[(g0 + P) * dim + c] : 0.0;
-        double inc = v;
+    constexpr int R = 16;  // batches of 64 groups per round of loads (one memory round trip per round)
+    for (uint32_t P0 = 0; P0 < nP; P0 += 64 * R) {
+        float vin[R];
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const double o = __shfl_up(inc, off);
-            if (lane >= off) inc += o;
+        for (int k = 0; k < R; ++k) {
+            const uint32_t P = P0 + 64 * k + lane;
+            vin[k] = gsum[(g0 + (P < nP ? P : nP - 1)) * dim + c];
         }
-        const double before = carry + (inc - v), after = carry + inc;
-        carry = __shfl(after, 63);
-        if (P < nP) {
-            // the sequential f32 sum is within 2^-9 of the f64 one by a wide margin
-            const float lo = (float)(before * (1.0 - 0.001953125)), hi = (float)(after * (1.0 + 0.001953125));
-            const uint32_t elo = __float_as_uint(lo) >> 23, ehi = __float_as_uint(hi) >> 23;  // both >= +0
-            uint16_t code = 0;
-            if (v == 0.0)  // non-negative terms with a zero sum: every one is +0 and leaves any S as it is
-                code = (uint16_t)(kGuessOk | kGuessZero);
-            else if (before > 0.0 && elo >= 30u && ehi <= 250u && ehi - elo <= 1u)
-                code = (uint16_t)(kGuessOk | (ehi != elo ? kGuessTwo : 0u) | elo);
-            guess[(g0 + P) * dim + c] = code;
+#pragma unroll
+        for (int k = 0; k < R; ++k) {
+            const uint32_t P = P0 + 64 * k + lane;
+            const double v = P < nP ? (double)vin[k] : 0.0;
+            double inc = v;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const double o = __shfl_up(inc, off);
+                if (lane >= off) inc += o;
+            }
+            const double before = carry + (inc - v), after = carry + inc;
+            carry = __shfl(after, 63);
+            if (P < nP) {
+                // the sequential f32 sum is within 2^-9 of the f64 one by a wide margin
+                const float lo = (float)(before * (1.0 - 0.001953125)), hi = (float)(after * (1.0 + 0.001953125));
+                const uint32_t elo = __float_as_uint(lo) >> 23, ehi = __float_as_uint(hi) >> 23;  // both >= +0
+                uint16_t code = 0;
+                if (v == 0.0)  // non-negative terms with a zero sum: every one is +0 and leaves any S as it is
+                    code = (uint16_t)(kGuessOk | kGuessZero);
+                else if (before > 0.0 && elo >= 30u && ehi <= 250u && ehi - elo <= 1u)
+                    code = (uint16_t)(kGuessOk | (ehi != elo ? kGuessTwo : 0u) | elo);
+                guess[(g0 + P) * dim + c] = code;
+            }
         }
     }
 }
@@ -363,65 +373,83 @@ static __global__ void __launch_bounds__(256) k_seg_chain_compose(const float *_
     const size_t g0 = seg_group0(range, g);
     const float *q = sq32 + ((size_t)range.x + 32u * (size_t)g) * dim + (c / 8) * 256 + (c % 8) * 32;
     float S = 0.0f;  // the same value in every lane
-    uint32_t P = 0;
-    while (P < nP) {
-        // S is +0, positive, +inf or a NaN; with the sign bit of a NaN eS is above every guess
-        const uint32_t Sb = __float_as_uint(S), eS = Sb >> 23;
-        bool seq = true;
-        uint32_t adv = 1;
-        {
-            const uint32_t s = (Sb & 0x7fffffu) | 0x800000u;  // S / u for a normal S
-            const uint32_t idx = P + lane;
-            const bool in = idx < nP;
-            const uint16_t code = in ? guess[(g0 + idx) * dim + c] : (uint16_t)0;
-            uint4 mp = make_uint4(kMapInvalid, kMapInvalid, kMapInvalid, kMapInvalid);
-            if (in) mp = maps[(g0 + idx) * dim + c];
+    // Batches of 64 groups at fixed positions (lane = group 64 b + lane), R batches per round of
+    // loads: one memory round trip per round instead of one per batch.
+    constexpr int R = 16;
+    const uint32_t nB = (nP + 63u) / 64u;
+    for (uint32_t b0 = 0; b0 < nB; b0 += R) {
+        uint16_t codeR[R];
+        uint4 mpR[R];
+#pragma unroll
+        for (int k = 0; k < R; ++k) {
+            const uint32_t idx = (b0 + k) * 64u + lane;
+            const size_t at = (g0 + (idx < nP ? idx : nP - 1u)) * dim + c;
+            codeR[k] = guess[at];
+            mpR[k] = maps[at];
+        }
+#pragma unroll
+        for (int k = 0; k < R; ++k) {
+            const uint32_t base = (b0 + k) * 64u;  // first group of the batch
+            // groups in the batch (none past the end: the loop below does not run; uniform)
+            const uint32_t left = base >= nP ? 0u : (nP - base < 64u ? nP - base : 64u);
+            const uint16_t code = codeR[k];
+            const uint4 mp = mpR[k];
             const uint32_t elo = code & 255u;
             const bool zero = (code & kGuessZero) != 0;
-            const bool is_lo = elo == eS, is_hi = (code & kGuessTwo) && elo + 1u == eS;
-            uint32_t a0 = is_lo ? mp.x : mp.z, a1 = is_lo ? mp.y : mp.w;
-            // a group of zeros keeps any finite S; another group needs S in the binade of its map
-            const bool ok = in && (code & kGuessOk) &&
-                            (zero ? eS < 255u : (eS >= 30u && eS <= 250u && (is_lo || is_hi) && a0 != kMapInvalid));
-            if (zero) a0 = a1 = 0u;
-            const unsigned long long okm = __ballot(ok);
-            const int first = okm == ~0ull ? 64 : __ffsll((long long)~okm) - 1;  // leading lanes that are ok
-            if (first > 0) {
-                const uint32_t cap = 1u << 25;
-                if (lane >= first) a0 = a1 = 0u;
-                a0 = a0 < cap ? a0 : cap;
-                a1 = a1 < cap ? a1 : cap;
-                // inclusive scan: the map of groups P .. P + lane, as increments for a start parity
+            uint32_t start = 0;  // groups of the batch already added
+            while (start < left) {
+                // S is +0, positive, +inf or a NaN; with the sign bit of a NaN eS is above every guess
+                const uint32_t Sb = __float_as_uint(S), eS = Sb >> 23;
+                const uint32_t s = (Sb & 0x7fffffu) | 0x800000u;  // S / u for a normal S
+                const bool is_lo = elo == eS, is_hi = (code & kGuessTwo) && elo + 1u == eS;
+                uint32_t a0 = is_lo ? mp.x : mp.z, a1 = is_lo ? mp.y : mp.w;
+                // a group of zeros keeps any finite S; another group needs S in the binade of its map
+                const bool mine = (uint32_t)lane >= start && (uint32_t)lane < left;
+                const bool ok = (code & kGuessOk) &&
+                                (zero ? eS < 255u : (eS >= 30u && eS <= 250u && (is_lo || is_hi) && a0 != kMapInvalid));
+                if (zero) a0 = a1 = 0u;
+                // the run of usable groups that starts at `start`
+                const unsigned long long stop = __ballot(mine && !ok) | (left < 64u ? ~0ull << left : 0ull);
+                const uint32_t end = stop ? (uint32_t)__ffsll((long long)stop) - 1u : 64u;
+                bool advanced = false;
+                if (end > start) {
+                    const uint32_t cap = 1u << 25;
+                    const bool part = (uint32_t)lane >= start && (uint32_t)lane < end;
+                    a0 = part ? (a0 < cap ? a0 : cap) : 0u;
+                    a1 = part ? (a1 < cap ? a1 : cap) : 0u;
+                    // inclusive scan: the map of groups start .. lane, as increments for a start parity
 #pragma unroll
-                for (int off = 1; off < 64; off <<= 1) {
-                    const uint32_t b0 = __shfl_up(a0, off), b1 = __shfl_up(a1, off);
-                    if (lane >= off) {
-                        const uint32_t n0 = b0 + ((b0 & 1u) ? a1 : a0);        // start even: after b0 the parity is b0 & 1
-                        const uint32_t n1 = b1 + (((b1 + 1u) & 1u) ? a1 : a0);  // start odd
-                        a0 = n0 < cap ? n0 : cap;
-                        a1 = n1 < cap ? n1 : cap;
+                    for (int off = 1; off < 64; off <<= 1) {
+                        const uint32_t l0 = __shfl_up(a0, off), l1 = __shfl_up(a1, off);
+                        if (lane >= off) {
+                            const uint32_t n0 = l0 + ((l0 & 1u) ? a1 : a0);        // start even: after l0 the parity is l0 & 1
+                            const uint32_t n1 = l1 + (((l1 + 1u) & 1u) ? a1 : a0);  // start odd
+                            a0 = n0 < cap ? n0 : cap;
+                            a1 = n1 < cap ? n1 : cap;
+                        }
+                    }
+                    const uint32_t send = s + ((s & 1u) ? a1 : a0);
+                    const bool fits = part && send <= (1u << 24);
+                    const int nv = __popcll(__ballot(fits));  // fits is monotone: the sums never decrease
+                    if (nv > 0) {
+                        const uint32_t take = __shfl(send, (int)start + nv - 1);
+                        // (a subnormal or zero S only passes groups of zeros: take == s and S stays)
+                        S = __uint_as_float(take == (1u << 24) ? (eS + 1u) << 23 : (eS << 23) | (take - (1u << 23)));
+                        start += (uint32_t)nv;
+                        advanced = true;
                     }
                 }
-                const uint32_t send = s + ((s & 1u) ? a1 : a0);
-                const bool fits = lane < first && send <= (1u << 24);
-                const int nv = __popcll(__ballot(fits));  // fits is monotone: the sums never decrease
-                if (nv > 0) {
-                    const uint32_t take = __shfl(send, nv - 1);
-                    // (a subnormal or zero S only passes groups of zeros: take == s and S stays)
-                    S = __uint_as_float(take == (1u << 24) ? (eS + 1u) << 23 : (eS << 23) | (take - (1u << 23)));
-                    seq = false;
-                    adv = (uint32_t)nv;
+                if (!advanced) {
+                    // the group's terms one by one (positions past the end add +0.0, which changes nothing)
+                    const uint32_t P = base + start;
+                    float t = 0.0f;
+                    if (lane < 32 && P * 32u + (uint32_t)lane < count) t = q[(size_t)P * 32 * dim + lane];
+#pragma unroll
+                    for (int i = 0; i < 32; ++i) S = S + __shfl(t, i);
+                    start += 1u;
                 }
             }
         }
-        if (seq) {
-            // the group's terms one by one (positions past the end add +0.0, which changes nothing)
-            float t = 0.0f;
-            if (lane < 32 && P * 32u + (uint32_t)lane < count) t = q[(size_t)P * 32 * dim + lane];
-#pragma unroll
-            for (int i = 0; i < 32; ++i) S = S + __shfl(t, i);
-        }
-        P += adv;
     }
     if (lane == 0) var[(size_t)g * dim + c] = S;
 }
