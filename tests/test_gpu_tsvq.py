@@ -134,3 +134,37 @@ def test_config5_shape_unit_rows_cosine_then_manhattan(ctx):
         ctx.tsvq_descend(metric, dx, n, dim, tree, dleaf)
         want = np.array([new_id[v] for v in O.tsvq_descend(metric, x, otree)], np.int32)
         assert np.array_equal(dleaf.download(), want)
+
+
+@pytest.mark.parametrize("kind", ["constant_columns", "all_zero", "tiny", "huge", "mixed", "integers", "wide_range"])
+@pytest.mark.parametrize("n,dim,depth", [(70000, 8, 3), (20000, 128, 5), (33, 16, 2), (4097, 24, 4)])
+def test_variance_paths_agree_with_the_oracle_on_edge_data(ctx, kind, n, dim, depth):
+    """The two ways of summing a node's squared deviations in row order (composed integer maps, one
+    chain of adds per column) against the oracle's sequential sums, through the tree they decide:
+    columns that never vary (every square is zero), values whose squares are subnormal or close to
+    the largest float, integers (every rounding a tie or exact), magnitudes spread over many binades."""
+    rng = np.random.default_rng([n, dim, len(kind)])
+    if kind == "constant_columns":
+        x = rng.standard_normal((n, dim)).astype(F)
+        x[:, ::3] = F(1.25)
+        x[:, 1] = 0.0
+    elif kind == "all_zero":
+        x = np.zeros((n, dim), F)
+    elif kind == "tiny":
+        x = (rng.standard_normal((n, dim)) * 1e-22).astype(F)
+    elif kind == "huge":
+        x = (rng.standard_normal((n, dim)) * 1e15).astype(F)
+    elif kind == "mixed":
+        x = (rng.standard_normal((n, dim)) * rng.choice([1e-6, 1.0, 1e4], (n, 1))).astype(F)
+    elif kind == "integers":
+        x = np.round(rng.standard_normal((n, dim)) * 3).astype(F)
+    else:
+        x = (rng.standard_normal((n, dim)) * np.exp2(rng.integers(-30, 30, (n, dim)))).astype(F)
+    want_tree, _ = bfs_order(O.tsvq_fit(x, depth))
+    dx = ctx.to_device(x)
+    try:
+        for path in (0, 1):
+            ctx.set_tsvq_variance_path(path)
+            assert_same_tree(ctx.tsvq_build(dx, n, dim, dim, depth).download(), want_tree)
+    finally:
+        ctx.set_tsvq_variance_path(0)
