@@ -206,19 +206,10 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         for (int i = 0; i < ns; ++i)
             std::copy_n(T->h_centroids.data() + (size_t)level[split[i]].node * dim, dim,
                         smeans.data() + (size_t)i * dim);
+        // the level's small tables: one grow-only arena of the context instead of nine allocations
         void *d_range = nullptr, *d_smeans = nullptr, *d_var = nullptr, *d_sdim = nullptr, *d_mids = nullptr,
              *d_median = nullptr, *d_nleft = nullptr, *d_sel = nullptr, *d_hist = nullptr;
-        auto free_split = [&]() {
-            (void)hipFree(d_range);
-            (void)hipFree(d_smeans);
-            (void)hipFree(d_var);
-            (void)hipFree(d_sdim);
-            (void)hipFree(d_mids);
-            (void)hipFree(d_median);
-            (void)hipFree(d_nleft);
-            (void)hipFree(d_sel);
-            (void)hipFree(d_hist);
-        };
+        auto free_split = [&]() {};
 #define SP_HIP(call)                                                                              \
     do {                                                                                          \
         hipError_t e__ = (call);                                                                  \
@@ -231,15 +222,27 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                                      __LINE__));                                                  \
         }                                                                                         \
     } while (0)
-        SP_HIP(hipMalloc(&d_range, sizeof(uint2) * ns));
-        SP_HIP(hipMalloc(&d_smeans, sizeof(float) * (size_t)ns * dim));
-        SP_HIP(hipMalloc(&d_var, sizeof(float) * (size_t)ns * dim));
-        SP_HIP(hipMalloc(&d_sdim, sizeof(int) * ns));
-        SP_HIP(hipMalloc(&d_mids, sizeof(float) * 2 * ns));
-        SP_HIP(hipMalloc(&d_median, sizeof(float) * ns));
-        SP_HIP(hipMalloc(&d_nleft, sizeof(uint32_t) * ns));
-        SP_HIP(hipMalloc(&d_sel, sizeof(vq::SegSelect) * 2 * ns));
-        SP_HIP(hipMalloc(&d_hist, sizeof(uint32_t) * 512 * (size_t)ns));
+        {
+            const size_t cap = (size_t)std::max(ns, 1024);  // sized once for the usual depths
+            const size_t sizes[9] = {sizeof(uint2) * cap, sizeof(float) * cap * dim, sizeof(float) * cap * dim,
+                                     sizeof(int) * cap, sizeof(float) * 2 * cap, sizeof(float) * cap,
+                                     sizeof(uint32_t) * cap, sizeof(vq::SegSelect) * 2 * cap,
+                                     sizeof(uint32_t) * 512 * cap};
+            void **ptrs[9] = {&d_range, &d_smeans, &d_var, &d_sdim, &d_mids, &d_median, &d_nleft, &d_sel, &d_hist};
+            size_t total = 0;
+            for (size_t z : sizes) total += (z + 255) & ~(size_t)255;
+            const int32_t rc = ensure(ctx, ctx->tsvq_split, total);
+            if (rc != VQ_OK) {
+                free_level();
+                (void)hipFree(rp_tmp);
+                return cleanup_fail(rc);
+            }
+            char *at = (char *)ctx->tsvq_split.p;
+            for (int z = 0; z < 9; ++z) {
+                *ptrs[z] = at;
+                at += (sizes[z] + 255) & ~(size_t)255;
+            }
+        }
         SP_HIP(hipMemcpyAsync(d_range, range.data(), sizeof(uint2) * ns, hipMemcpyHostToDevice, st));
         SP_HIP(hipMemcpyAsync(d_smeans, smeans.data(), sizeof(float) * (size_t)ns * dim, hipMemcpyHostToDevice, st));
         // per-dimension sums of squared deviations (src/tsvq.rs:88-99)
