@@ -242,6 +242,26 @@ static __global__ void __launch_bounds__(256) k_seg_chain32(const float *__restr
 //                        group's start and does not leave it) and adds a group's 32 terms one by one
 //                        where one fails — the groups in which S crosses a binade, the first groups,
 //                        non-finite values.  The result is the sequential sum, bit for bit.
+// The value of the lane K places down in its row of 16 lanes (DPP row shift), `fill` where that lane
+// is outside the row: scans over the wave take four of these steps and three broadcasts of a row's
+// last lane instead of six permutes through LDS.
+template <int K>
+__device__ __forceinline__ uint32_t row_shr(uint32_t v, uint32_t fill) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)fill, (int)v, 0x110 + K, 0xF, 0xF, false);
+}
+template <int K>
+__device__ __forceinline__ double row_shr_f64(double v) {  // 0.0 where the lane is outside the row
+    const unsigned long long b = (unsigned long long)__double_as_longlong(v);
+    const uint32_t lo = row_shr<K>((uint32_t)b, 0u), hi = row_shr<K>((uint32_t)(b >> 32), 0u);
+    return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+__device__ __forceinline__ double lane_f64(double v, int src) {  // src: a constant lane
+    const unsigned long long b = (unsigned long long)__double_as_longlong(v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, src);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), src);
+    return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
 constexpr uint32_t kMapInvalid = 0xFFFFFFFFu;
 // guess code: exponent field of the lower candidate | two candidates | all terms zero | usable
 constexpr uint16_t kGuessOk = 0x8000u, kGuessTwo = 0x0100u, kGuessZero = 0x0200u;
@@ -268,14 +288,22 @@ static __global__ void __launch_bounds__(256) k_seg_chain_guess(const float *__r
         for (int k = 0; k < R; ++k) {
             const uint32_t P = P0 + 64 * k + lane;
             const double v = P < nP ? (double)vin[k] : 0.0;
+            // inclusive prefix over the lanes: inside the rows of 16, then row by row
             double inc = v;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const double o = __shfl_up(inc, off);
-                if (lane >= off) inc += o;
+            inc += row_shr_f64<1>(inc);
+            inc += row_shr_f64<2>(inc);
+            inc += row_shr_f64<4>(inc);
+            inc += row_shr_f64<8>(inc);
+            {
+                const double r0 = lane_f64(inc, 15);
+                if ((lane >> 4) == 1) inc += r0;
+                const double r1 = lane_f64(inc, 31);
+                if ((lane >> 4) == 2) inc += r1;
+                const double r2 = lane_f64(inc, 47);
+                if ((lane >> 4) == 3) inc += r2;
             }
             const double before = carry + (inc - v), after = carry + inc;
-            carry = __shfl(after, 63);
+            carry = lane_f64(after, 63);
             if (P < nP) {
                 // the sequential f32 sum is within 2^-9 of the f64 one by a wide margin
                 const float lo = (float)(before * (1.0 - 0.001953125)), hi = (float)(after * (1.0 + 0.001953125));
@@ -418,21 +446,31 @@ static __global__ void __launch_bounds__(256) k_seg_chain_compose(const float *_
                     a0 = part ? (a0 < cap ? a0 : cap) : 0u;
                     a1 = part ? (a1 < cap ? a1 : cap) : 0u;
                     // inclusive scan: the map of groups start .. lane, as increments for a start parity
-#pragma unroll
-                    for (int off = 1; off < 64; off <<= 1) {
-                        const uint32_t l0 = __shfl_up(a0, off), l1 = __shfl_up(a1, off);
-                        if (lane >= off) {
-                            const uint32_t n0 = l0 + ((l0 & 1u) ? a1 : a0);        // start even: after l0 the parity is l0 & 1
-                            const uint32_t n1 = l1 + (((l1 + 1u) & 1u) ? a1 : a0);  // start odd
-                            a0 = n0 < cap ? n0 : cap;
-                            a1 = n1 < cap ? n1 : cap;
-                        }
+                    // (left, then this lane's map: c_p = l_p + a_[(p + l_p) mod 2]; (0, 0) is the identity, which
+                    // is what a lane outside the row supplies)
+                    auto after_left = [&](uint32_t l0, uint32_t l1) {
+                        const uint32_t n0 = l0 + ((l0 & 1u) ? a1 : a0);        // start even: after l0 the parity is l0 & 1
+                        const uint32_t n1 = l1 + (((l1 + 1u) & 1u) ? a1 : a0);  // start odd
+                        a0 = n0 < cap ? n0 : cap;
+                        a1 = n1 < cap ? n1 : cap;
+                    };
+                    after_left(row_shr<1>(a0, 0u), row_shr<1>(a1, 0u));
+                    after_left(row_shr<2>(a0, 0u), row_shr<2>(a1, 0u));
+                    after_left(row_shr<4>(a0, 0u), row_shr<4>(a1, 0u));
+                    after_left(row_shr<8>(a0, 0u), row_shr<8>(a1, 0u));
+                    {
+                        uint32_t t0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 15), t1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 15);
+                        if ((lane >> 4) == 1) after_left(t0, t1);
+                        t0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 31), t1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 31);
+                        if ((lane >> 4) == 2) after_left(t0, t1);
+                        t0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 47), t1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 47);
+                        if ((lane >> 4) == 3) after_left(t0, t1);
                     }
                     const uint32_t send = s + ((s & 1u) ? a1 : a0);
                     const bool fits = part && send <= (1u << 24);
                     const int nv = __popcll(__ballot(fits));  // fits is monotone: the sums never decrease
                     if (nv > 0) {
-                        const uint32_t take = __shfl(send, (int)start + nv - 1);
+                        const uint32_t take = (uint32_t)__builtin_amdgcn_readlane((int)send, __builtin_amdgcn_readfirstlane((int)start + nv - 1));
                         // (a subnormal or zero S only passes groups of zeros: take == s and S stays)
                         S = __uint_as_float(take == (1u << 24) ? (eS + 1u) << 23 : (eS << 23) | (take - (1u << 23)));
                         start += (uint32_t)nv;
