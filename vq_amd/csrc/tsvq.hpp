@@ -112,6 +112,7 @@ static __global__ void __launch_bounds__(256) k_seg_sqdev32(const uint32_t *__re
                                                             const float *__restrict__ means, int64_t first,
                                                             const float *__restrict__ x, int64_t ld, int dim,
                                                             float *__restrict__ sq32, float *__restrict__ gsum) {
+    // sq32 == nullptr: only the group sums are wanted (the squares are made again where they are used)
     const int g = blockIdx.y;
     const uint2 range = seg_range[g];
     const uint32_t count = range.y - range.x;
@@ -137,8 +138,9 @@ static __global__ void __launch_bounds__(256) k_seg_sqdev32(const uint32_t *__re
                 q[r] = d * d;
                 gs += p < count ? q[r] : 0.0f;
             }
+            if (sq32)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o[4 * h + r] = make_float4(q[4 * r], q[4 * r + 1], q[4 * r + 2], q[4 * r + 3]);
+                for (int r = 0; r < 4; ++r) o[4 * h + r] = make_float4(q[4 * r], q[4 * r + 1], q[4 * r + 2], q[4 * r + 3]);
         }
         if (gsum) gsum[(seg_group0(range, g) + P) * dim + c] = gs;
     }
@@ -352,8 +354,10 @@ __device__ __forceinline__ void chain_group_map(const float (&t)[32], int valid,
 }
 
 // Grid (blocks of 64 positions, segments), as k_seg_sqdev32: one thread per (group, column).
-static __global__ void __launch_bounds__(256) k_seg_chain_maps(const float *__restrict__ sq32,
-                                                              const uint2 *__restrict__ seg_range, int dim,
+static __global__ void __launch_bounds__(256) k_seg_chain_maps(const uint32_t *__restrict__ perm,
+                                                              const uint2 *__restrict__ seg_range,
+                                                              const float *__restrict__ means, int64_t first,
+                                                              const float *__restrict__ x, int64_t ld, int dim,
                                                               const uint16_t *__restrict__ guess,
                                                               uint4 *__restrict__ maps) {
     const int g = blockIdx.y;
@@ -363,7 +367,8 @@ static __global__ void __launch_bounds__(256) k_seg_chain_maps(const float *__re
     if (P0 * 32u >= count) return;
     const uint32_t nP = (count + 31u) / 32u;
     const uint32_t groups = nP - P0 < 2u ? nP - P0 : 2u;
-    const float *in = sq32 + ((size_t)range.x + 32u * (size_t)g) * dim;
+    const float *mrow = means + (first + g) * dim;
+    const uint32_t *pm = perm + range.x;
     const size_t g0 = seg_group0(range, g);
     for (uint32_t e = threadIdx.x; e < groups * (uint32_t)dim; e += 256) {
         const uint32_t P = P0 + e / (uint32_t)dim, c = e % (uint32_t)dim;
@@ -372,12 +377,14 @@ static __global__ void __launch_bounds__(256) k_seg_chain_maps(const float *__re
         if (code & kGuessZero) {
             out = make_uint4(0u, 0u, 0u, 0u);
         } else if (code & kGuessOk) {
-            const float4 *q = reinterpret_cast<const float4 *>(in + (size_t)P * 32 * dim + (c / 8u) * 256u + (c % 8u) * 32u);
+            // the squares again, with the same two roundings (past the end: the last row, not counted)
+            const float m = mrow[c];
             float t[32];
 #pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                const float4 v = q[r];
-                t[4 * r] = v.x, t[4 * r + 1] = v.y, t[4 * r + 2] = v.z, t[4 * r + 3] = v.w;
+            for (int r = 0; r < 32; ++r) {
+                const uint32_t p = 32u * P + r;
+                const float d = x[(int64_t)pm[p < count ? p : count - 1] * ld + c] - m;
+                t[r] = d * d;
             }
             const int valid = (int)(count - 32u * P < 32u ? count - 32u * P : 32u);
             const uint32_t elo = code & 255u;
@@ -389,8 +396,10 @@ static __global__ void __launch_bounds__(256) k_seg_chain_maps(const float *__re
 }
 
 // grid (segments, dim / 4); 256 threads = 4 waves, one column each.
-static __global__ void __launch_bounds__(256) k_seg_chain_compose(const float *__restrict__ sq32,
-                                                                 const uint2 *__restrict__ seg_range, int dim,
+static __global__ void __launch_bounds__(256) k_seg_chain_compose(const uint32_t *__restrict__ perm,
+                                                                 const uint2 *__restrict__ seg_range,
+                                                                 const float *__restrict__ means, int64_t first,
+                                                                 const float *__restrict__ x, int64_t ld, int dim,
                                                                  const uint16_t *__restrict__ guess,
                                                                  const uint4 *__restrict__ maps,
                                                                  float *__restrict__ var) {
@@ -399,7 +408,8 @@ static __global__ void __launch_bounds__(256) k_seg_chain_compose(const float *_
     const uint2 range = seg_range[g];
     const uint32_t count = range.y - range.x, nP = (count + 31u) / 32u;
     const size_t g0 = seg_group0(range, g);
-    const float *q = sq32 + ((size_t)range.x + 32u * (size_t)g) * dim + (c / 8) * 256 + (c % 8) * 32;
+    const float mean_c = means[(first + g) * dim + c];
+    const uint32_t *pm = perm + range.x;
     float S = 0.0f;  // the same value in every lane
     // Batches of 64 groups at fixed positions (lane = group 64 b + lane), R batches per round of
     // loads: one memory round trip per round instead of one per batch.
@@ -481,7 +491,10 @@ static __global__ void __launch_bounds__(256) k_seg_chain_compose(const float *_
                     // the group's terms one by one (positions past the end add +0.0, which changes nothing)
                     const uint32_t P = base + start;
                     float t = 0.0f;
-                    if (lane < 32 && P * 32u + (uint32_t)lane < count) t = q[(size_t)P * 32 * dim + lane];
+                    if (lane < 32 && P * 32u + (uint32_t)lane < count) {
+                        const float d = x[(int64_t)pm[P * 32u + lane] * ld + c] - mean_c;
+                        t = d * d;
+                    }
 #pragma unroll
                     for (int i = 0; i < 32; ++i) S = S + __shfl(t, i);
                     start += 1u;

@@ -96,11 +96,12 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     // for a level's squares with every node starting on its own group of 32 positions
     constexpr int kChainSegs = 2048;  // levels with more nodes than this take the other kernels
     const bool var_chain = dim % 8 == 0;
-    if (var_chain)
+    // per group of 32 squares (composed-maps path): approximate sum, binade guess, integer maps;
+    // the chain path keeps the squares themselves
+    const bool var_maps = var_chain && ctx->tsvq_var_path == 0;
+    if (var_chain && !var_maps)
         VQ_TRY(ensure(ctx, ctx->tsvq_sq, sizeof(float) * ((size_t)n + vq::kChainGroup * (size_t)kChainSegs) * dim));
     float *d_sq = (float *)ctx->tsvq_sq.p;
-    // per group of 32 squares (composed-maps path): approximate sum, binade guess, integer maps
-    const bool var_maps = var_chain && ctx->tsvq_var_path == 0;
     if (var_maps) {
         const size_t ngroups = ((size_t)n + vq::kChainGroup * (size_t)kChainSegs) / vq::kChainGroup + 2;
         VQ_TRY(ensure(ctx, ctx->tsvq_gsum, sizeof(float) * ngroups * dim));
@@ -251,16 +252,16 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             for (int i = 0; i < ns; ++i) longest = std::max(longest, range[i].y - range[i].x);
             hipLaunchKernelGGL(vq::k_seg_sqdev32, dim3((unsigned)cdiv((int64_t)longest, 64), (unsigned)ns), dim3(256),
                                0, st, perm, (const uint2 *)d_range, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
-                               d_sq, var_maps ? (float *)ctx->tsvq_gsum.p : (float *)nullptr);
+                               var_maps ? (float *)nullptr : d_sq, var_maps ? (float *)ctx->tsvq_gsum.p : (float *)nullptr);
             if (var_maps) {
                 hipLaunchKernelGGL(vq::k_seg_chain_guess, dim3((unsigned)ns, (unsigned)cdiv(dim, 4)), dim3(256), 0, st,
                                    (const float *)ctx->tsvq_gsum.p, (const uint2 *)d_range, dim,
                                    (uint16_t *)ctx->tsvq_guess.p);
                 hipLaunchKernelGGL(vq::k_seg_chain_maps, dim3((unsigned)cdiv((int64_t)longest, 64), (unsigned)ns),
-                                   dim3(256), 0, st, (const float *)d_sq, (const uint2 *)d_range, dim,
-                                   (const uint16_t *)ctx->tsvq_guess.p, (uint4 *)ctx->tsvq_maps.p);
+                                   dim3(256), 0, st, perm, (const uint2 *)d_range, (const float *)d_smeans, (int64_t)0,
+                                   d_x, ld, dim, (const uint16_t *)ctx->tsvq_guess.p, (uint4 *)ctx->tsvq_maps.p);
                 hipLaunchKernelGGL(vq::k_seg_chain_compose, dim3((unsigned)ns, (unsigned)cdiv(dim, 4)), dim3(256), 0,
-                                   st, (const float *)d_sq, (const uint2 *)d_range, dim,
+                                   st, perm, (const uint2 *)d_range, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
                                    (const uint16_t *)ctx->tsvq_guess.p, (const uint4 *)ctx->tsvq_maps.p,
                                    (float *)d_var);
             } else {
