@@ -837,6 +837,41 @@ static __global__ void k_seg_select_out(const SegSelect *__restrict__ sel, int n
     if (i < 2 * nseg) mids[i] = float_from_order_key(sel[i].prefix);
 }
 
+// The split dimension of every segment: argmax of its per-dimension sums with the LAST maximal
+// element winning (Iterator::max_by, src/tsvq.rs:102-106); one thread per segment.
+static __global__ void k_seg_argmax_last(const float *__restrict__ var, int nseg, int dim, int *__restrict__ sdim) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nseg) return;
+    const float *v = var + (size_t)i * dim;
+    int best = 0;
+    float vb = v[0];
+    for (int t0 = 1; t0 < dim; t0 += 16) {
+        float w[16];  // sixteen loads in flight
+#pragma unroll
+        for (int u = 0; u < 16; ++u) w[u] = v[t0 + u < dim ? t0 + u : dim - 1];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            if (t0 + u < dim && !(w[u] < vb)) {
+                best = t0 + u;
+                vb = w[u];
+            }
+        }
+    }
+    sdim[i] = best;
+}
+
+// The median of every segment from its two middle values (src/tsvq.rs:112-117): their f32 sum
+// divided by two for an even count, the middle value otherwise.
+static __global__ void k_seg_median(const float *__restrict__ mids, const uint2 *__restrict__ seg_range, int nseg,
+                                    float *__restrict__ median) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nseg) return;
+    const uint32_t cnt = seg_range[i].y - seg_range[i].x;
+    const float a = mids[2 * i], b = mids[2 * i + 1];
+    const float sum = a + b;
+    median[i] = (cnt % 2u == 0u) ? sum / 2.0f : a;
+}
+
 // ---- descent -------------------------------------------------------------------------------
 template <int METRIC>
 __device__ __forceinline__ float tsvq_dist(const float *__restrict__ xr, const float *__restrict__ c,

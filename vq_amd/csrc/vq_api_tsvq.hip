@@ -285,19 +285,9 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                                (const uint2 *)d_range, ns, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
                                (float *)d_var);
         SP_HIP(hipGetLastError());
-        std::vector<float> var((size_t)ns * dim);
-        SP_HIP(hipMemcpyAsync(var.data(), d_var, sizeof(float) * (size_t)ns * dim, hipMemcpyDeviceToHost, st));
-        SP_HIP(hipStreamSynchronize(st));
-        // argmax with the LAST maximal element winning (Iterator::max_by, src/tsvq.rs:102-106)
-        std::vector<int> sdim(ns);
-        for (int i = 0; i < ns; ++i) {
-            const float *v = var.data() + (size_t)i * dim;
-            int best = 0;
-            for (int t = 1; t < dim; ++t)
-                if (!(v[t] < v[best])) best = t;
-            sdim[i] = best;
-        }
-        SP_HIP(hipMemcpyAsync(d_sdim, sdim.data(), sizeof(int) * ns, hipMemcpyHostToDevice, st));
+        // split dimension on the device (src/tsvq.rs:102-106); read back with the left counts below
+        hipLaunchKernelGGL(vq::k_seg_argmax_last, dim3(cdiv(ns, 64)), dim3(64), 0, st, (const float *)d_var, ns, dim,
+                           (int *)d_sdim);
         // split column, middle values by radix select (src/tsvq.rs:109-117)
         hipLaunchKernelGGL(vq::k_seg_gather_col, dim3(cdiv(n, 256)), dim3(256), 0, st, perm, n,
                            (const uint2 *)d_range, ns, (const int *)d_sdim, d_x, ld, vals);
@@ -312,19 +302,8 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         hipLaunchKernelGGL(vq::k_seg_select_out, dim3(cdiv(2 * ns, 64)), dim3(64), 0, st,
                            (const vq::SegSelect *)d_sel, ns, (float *)d_mids);
         SP_HIP(hipGetLastError());
-        std::vector<float> mids(2 * (size_t)ns), median(ns);
-        SP_HIP(hipMemcpyAsync(mids.data(), d_mids, sizeof(float) * 2 * ns, hipMemcpyDeviceToHost, st));
-        SP_HIP(hipStreamSynchronize(st));
-        for (int i = 0; i < ns; ++i) {
-            uint32_t cnt = range[i].y - range[i].x;
-            if (cnt % 2 == 0) {
-                volatile float s = mids[2 * i] + mids[2 * i + 1];  // f32 add, then f32 divide
-                median[i] = s / 2.0f;
-            } else {
-                median[i] = mids[2 * i];
-            }
-        }
-        SP_HIP(hipMemcpyAsync(d_median, median.data(), sizeof(float) * ns, hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(vq::k_seg_median, dim3(cdiv(ns, 64)), dim3(64), 0, st, (const float *)d_mids,
+                           (const uint2 *)d_range, ns, (float *)d_median);
         // stable partition by `<= median` (src/tsvq.rs:120-123)
         hipLaunchKernelGGL(vq::k_seg_flags, dim3(cdiv(n, 256)), dim3(256), 0, st, vals, n, (const uint2 *)d_range,
                            ns, (const float *)d_median, flags);
@@ -341,7 +320,11 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                            (const uint2 *)d_range, ns, flags, scan, perm2, (uint32_t *)d_nleft);
         SP_HIP(hipGetLastError());
         std::vector<uint32_t> nleft(ns);
+        std::vector<int> sdim(ns);
+        std::vector<float> median(ns);
         SP_HIP(hipMemcpyAsync(nleft.data(), d_nleft, sizeof(uint32_t) * ns, hipMemcpyDeviceToHost, st));
+        SP_HIP(hipMemcpyAsync(sdim.data(), d_sdim, sizeof(int) * ns, hipMemcpyDeviceToHost, st));
+        SP_HIP(hipMemcpyAsync(median.data(), d_median, sizeof(float) * ns, hipMemcpyDeviceToHost, st));
         SP_HIP(hipStreamSynchronize(st));
         free_split();
         free_level();
