@@ -1008,50 +1008,37 @@ __global__ void __launch_bounds__(512) k_tsvq_descend_reg(const float *__restric
                                                          const int *__restrict__ left,
                                                          const int *__restrict__ right, int n_nodes,
                                                          int *__restrict__ leaf) {
-    constexpr int CH = 32;
     constexpr int TS = DIM + 4;
-    // one LDS area: first the eight waves' row tiles, then (the rows being in registers) the centroids
-    constexpr int kTileFloats = 64 * (CH + 4), kTopFloats = kTopNodes * TS;
-    __shared__ float lds[(8 * kTileFloats > kTopFloats) ? 8 * kTileFloats : kTopFloats];
+    // The centroids of the first nodes are staged once per workgroup; the workgroup then walks over
+    // batches of 8 x 64 rows (grid: one workgroup per compute unit), every lane fetching its own
+    // row with 16-byte loads, all of them in flight together.
+    constexpr int kTopFloats = kTopNodes * TS;
+    __shared__ float lds[kTopFloats];
     const int lane = threadIdx.x & 63;
-    float *tile = lds + (threadIdx.x >> 6) * kTileFloats;
     float *top = lds;
-    const int64_t row0 = ((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 64;  // one wave = 64 rows
     const int ntop = n_nodes < kTopNodes ? n_nodes : kTopNodes;
-    float xr[DIM];
-#pragma unroll
-    for (int c = 0; c < DIM / CH; ++c) {
-        float4 v[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int e = lane + 64 * i, r = e >> 3, pc = e & 7;
-            const int64_t row = row0 + r;
-            v[i] = (row < n) ? *reinterpret_cast<const float4 *>(x + row * ld + c * CH + pc * 4)
-                             : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-        __builtin_amdgcn_wave_barrier();  // one wave: LDS accesses are performed in program order
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int e = lane + 64 * i, r = e >> 3, pc = e & 7;
-            *reinterpret_cast<float4 *>(&tile[r * (CH + 4) + pc * 4]) = v[i];
-        }
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            const float4 t4 = *reinterpret_cast<const float4 *>(&tile[lane * (CH + 4) + q * 4]);
-            xr[c * CH + q * 4 + 0] = t4.x;
-            xr[c * CH + q * 4 + 1] = t4.y;
-            xr[c * CH + q * 4 + 2] = t4.z;
-            xr[c * CH + q * 4 + 3] = t4.w;
-        }
-    }
-    __syncthreads();  // every wave has its rows: the tiles make room for the centroids
     for (int e = threadIdx.x; e < ntop * (DIM / 4); e += 512) {
         const int nd = e / (DIM / 4), pc = e % (DIM / 4);
         *reinterpret_cast<float4 *>(&top[nd * TS + pc * 4]) =
             *reinterpret_cast<const float4 *>(cen + (size_t)nd * DIM + pc * 4);
     }
     __syncthreads();
+    const int64_t nbatch = (n + 63) / 64;
+    for (int64_t batch = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 6); batch < nbatch; batch += (int64_t)gridDim.x * 8) {
+    const int64_t row0 = batch * 64;  // one wave = 64 rows
+    float xr[DIM];
+    {
+        const int64_t row = row0 + lane < n ? row0 + lane : n - 1;  // past the end: the last row, not stored
+        const float4 *xp = reinterpret_cast<const float4 *>(x + row * ld);
+#pragma unroll
+        for (int q = 0; q < DIM / 4; ++q) {
+            const float4 v = xp[q];
+            xr[q * 4 + 0] = v.x;
+            xr[q * 4 + 1] = v.y;
+            xr[q * 4 + 2] = v.z;
+            xr[q * 4 + 3] = v.w;
+        }
+    }
     float na = 0.0f;
     if constexpr (METRIC == M_COS) {
         float sa = 0.0f;
@@ -1159,6 +1146,7 @@ __global__ void __launch_bounds__(512) k_tsvq_descend_reg(const float *__restric
         }
     }
     if (row0 + lane < n) leaf[row0 + lane] = node;
+    }  // batches
 }
 
 // out[i][t] = f16(centroid[leaf[i]][t])   (src/tsvq.rs:242-248)

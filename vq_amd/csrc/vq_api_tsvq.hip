@@ -431,7 +431,10 @@ int32_t vq_tsvq_descend(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n
     VQ_HIP(ctx, hipSetDevice(ctx->device));
     // rows in registers: dim a multiple of 32 up to 128, 16-byte aligned rows
     if (tree->dim % 32 == 0 && tree->dim <= 128 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0) {
-        dim3 g(cdiv(n, 512)), b(512);
+        // one workgroup per compute unit (the staged centroids fill its LDS), walking over the rows
+        int cus = 0;
+        VQ_HIP(ctx, hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device));
+        dim3 g(std::min<unsigned>(cdiv(n, 512), (unsigned)std::max(cus, 1))), b(512);
 #define DESC_REG(M, D)                                                                                \
     hipLaunchKernelGGL((vq::k_tsvq_descend_reg<M, D>), g, b, 0, ctx->stream, d_x, n, ld,              \
                        tree->d_centroids, tree->d_cnorm, tree->d_left, tree->d_right, (int)tree->h_left.size(),    \
