@@ -1014,9 +1014,14 @@ __global__ void __launch_bounds__(512) k_tsvq_descend_reg(const float *__restric
     // row with 16-byte loads, all of them in flight together.
     constexpr int kTopFloats = kTopNodes * TS;
     __shared__ float lds[kTopFloats];
+    __shared__ int lds_child[2 * kTopNodes];  // children of the staged nodes: the walk's dependent reads stay in LDS
     const int lane = threadIdx.x & 63;
     float *top = lds;
     const int ntop = n_nodes < kTopNodes ? n_nodes : kTopNodes;
+    for (int e = threadIdx.x; e < ntop; e += 512) {
+        lds_child[2 * e] = left[e];
+        lds_child[2 * e + 1] = right[e];
+    }
     for (int e = threadIdx.x; e < ntop * (DIM / 4); e += 512) {
         const int nd = e / (DIM / 4), pc = e % (DIM / 4);
         *reinterpret_cast<float4 *>(&top[nd * TS + pc * 4]) =
@@ -1054,8 +1059,13 @@ __global__ void __launch_bounds__(512) k_tsvq_descend_reg(const float *__restric
     while (__any(active)) {
         int l = -1, r = -1;
         if (active) {
-            l = left[node];
-            r = right[node];
+            if (node < ntop) {
+                l = lds_child[2 * node];
+                r = lds_child[2 * node + 1];
+            } else {
+                l = left[node];
+                r = right[node];
+            }
         }
         const bool both = l >= 0 && r >= 0;
         // every lane that compares two children finds them in LDS: the whole wave reads there
