@@ -1018,9 +1018,11 @@ __global__ void __launch_bounds__(512) k_tsvq_descend_reg(const float *__restric
     const int lane = threadIdx.x & 63;
     float *top = lds;
     const int ntop = n_nodes < kTopNodes ? n_nodes : kTopNodes;
+    __shared__ float lds_cn[kTopNodes];  // their norms (cosine)
     for (int e = threadIdx.x; e < ntop; e += 512) {
         lds_child[2 * e] = left[e];
         lds_child[2 * e + 1] = right[e];
+        if constexpr (METRIC == M_COS) lds_cn[e] = cnorm[e];
     }
     for (int e = threadIdx.x; e < ntop * (DIM / 4); e += 512) {
         const int nd = e / (DIM / 4), pc = e % (DIM / 4);
@@ -1084,7 +1086,7 @@ __global__ void __launch_bounds__(512) k_tsvq_descend_reg(const float *__restric
                 }
                 float dl, dr;
                 if constexpr (METRIC == M_COS) {
-                    float nl = cnorm[l], nr = cnorm[r];
+                    float nl = lds_cn[l], nr = lds_cn[r];
                     float ql = al / (na * nl), qr = ar / (na * nr);
                     dl = (na == 0.0f || nl == 0.0f) ? 1.0f : 1.0f - ql;
                     dr = (na == 0.0f || nr == 0.0f) ? 1.0f : 1.0f - qr;
