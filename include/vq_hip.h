@@ -170,6 +170,22 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
 int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                   int32_t sub_dim, int32_t k, const float *d_codebooks, uint8_t *d_codes);
 
+/* vq_assign for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, same codes, bit for bit; the call makes no hipMalloc / hipFree and never grows the
+ * context's workspace.  The tables of the matrix-core kernel (8-float column blocks under
+ * squared-L2 / Euclidean) and the centroid norms (cosine) live in one fixed array of 1.2 MB of
+ * device memory that the library holds on every GPU it runs on until the process ends.
+ *   limit: m <= 1024 and m * (k rounded up to a multiple of 64) <= 16384 (e.g. m = 64, k = 256);
+ *          beyond it VQ_ERR_UNSUPPORTED, and nothing is launched.
+ *   wider column blocks under squared-L2 / Euclidean take the vector-ALU kernel (the matrix-core
+ *   kernel for them keeps lists that grow with n).
+ * Every context on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
+ * contexts, two threads) race on it; a call leaves nothing the next one depends on.
+ * Asynchronous. */
+int32_t vq_assign_noalloc(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
+                          int32_t sub_dim, int32_t k, const float *d_codebooks, uint8_t *d_codes);
+
 /* d_out[i*(m*sub_dim) + s*sub_dim + t] = f16(codebook[s][code[i][s]][t]) — the value returned by
  * ProductQuantizer::quantize (src/pq.rs:176-186; f16::from_f32, round to nearest even).
  * d_out holds IEEE binary16 bit patterns.  Asynchronous. */

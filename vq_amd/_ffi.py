@@ -44,6 +44,7 @@ SYMBOLS = {
     "vq_lbg_fit": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp,
                           _vp]),
     "vq_assign": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
+    "vq_assign_noalloc": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_decode_f16": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_decode_f32": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_residual_sub": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp]),
@@ -254,6 +255,11 @@ class Context:
     def assign(self, metric, d_x, n, ld, m, sub_dim, k, d_codebooks, d_codes):
         self._check(_lib.vq_assign(self._h, metric, _ptr(d_x), n, ld, m, sub_dim, k,
                                    _ptr(d_codebooks), _ptr(d_codes)))
+
+    def assign_noalloc(self, metric, d_x, n, ld, m, sub_dim, k, d_codebooks, d_codes):
+        """vq_assign without any device allocation (fixed scratch; m * k padded <= 16384)."""
+        self._check(_lib.vq_assign_noalloc(self._h, metric, _ptr(d_x), n, ld, m, sub_dim, k,
+                                           _ptr(d_codebooks), _ptr(d_codes)))
 
     def decode_f16(self, d_codes, n, m, sub_dim, k, d_codebooks, d_out):
         self._check(_lib.vq_decode_f16(self._h, d_codes.ptr, n, m, sub_dim, k, d_codebooks.ptr,

@@ -31,8 +31,12 @@ struct vq_ctx {
     DevBuf tsvq_gsum, tsvq_guess, tsvq_maps;  // per group of 32 squares: sum, binade guess, integer maps
     int tsvq_var_path = 0;       // 0 = composed integer maps, 1 = one chain of adds per column
     DevBuf mfma_tab, mfma_list, mfma_stat;  // tables, re-check list and counters of the matrix-core assignment
-    int recheck_src = 0;         // where the last pass counted its undecided pairs: 1 mfma_stat, 2 mfma_list
+    int recheck_src = 0;         // where the last pass counted its undecided pairs: 1 mfma_stat, 2 mfma_list, 3 the fixed scratch
     int assign_path = 0;         // 0 = matrix cores where a kernel exists, 1 = vector ALU only
+    // vq_assign_noalloc: the device address of this GPU's file-scope scratch array, and whether a
+    // call that must not allocate is running (then `ensure` refuses to grow the workspace)
+    unsigned char *static_scratch = nullptr;
+    bool no_alloc = false;
     DevBuf tmp_a, tmp_b, tmp_c, tmp_d, tmp_e, tmp_f;  // scratch of the RVQ / OPQ / TSVQ entry points
     // optional per-kernel-class timing (HIP events on the stream)
     bool prof_on = false;
@@ -80,6 +84,8 @@ inline int32_t fail(vq_ctx *ctx, int32_t code, const char *fmt, ...) {
 
 inline int32_t ensure(vq_ctx *ctx, DevBuf &b, size_t bytes) {
     if (bytes <= b.cap) return VQ_OK;
+    if (ctx->no_alloc)
+        return fail(ctx, VQ_ERR_UNSUPPORTED, "this shape needs a workspace allocation, which this entry point may not make");
     if (b.p) {
         VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
         VQ_HIP(ctx, hipFree(b.p));

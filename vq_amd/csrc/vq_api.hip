@@ -37,6 +37,21 @@ using namespace vqh;
 
 namespace {
 
+// ---- the scratch of vq_assign_noalloc --------------------------------------------------------
+// One array per GPU, held from the moment the library is loaded on that GPU until the process
+// ends.  Host code never uses the array's name as an address: vq_ctx_create asks the runtime for
+// the device address once per context (hipGetSymbolAddress, with the context's device current)
+// and everything else goes through that pointer.
+constexpr size_t kNoAllocTabBytes = 1u << 20;       // A operands: 64 bytes per (column block, padded centroid)
+constexpr int kNoAllocMaxCells = 16384;             // column blocks x centroids (padded to 64) the tables hold
+constexpr int kNoAllocMaxM = 1024;
+constexpr size_t kNoAllocAuxOff = kNoAllocTabBytes;                                   // maxc2 [m], mu [m][8]
+constexpr size_t kNoAllocStatOff = kNoAllocAuxOff + 9 * sizeof(float) * kNoAllocMaxM + 256;  // counters
+constexpr size_t kNoAllocNormOff = kNoAllocStatOff + sizeof(uint32_t) * vq::kStatSlots * vq::kStatStride;
+constexpr size_t kNoAllocBytes = kNoAllocNormOff + sizeof(float) * kNoAllocMaxCells;  // centroid norms (cosine)
+static_assert(kNoAllocStatOff % 256 == 0 && kNoAllocNormOff % 256 == 0, "scratch areas stay 256-byte aligned");
+static __device__ __align__(256) unsigned char scratch[kNoAllocBytes];
+
 // ---- assignment dispatch -------------------------------------------------------------------
 
 template <int METRIC, bool LBG>
@@ -118,6 +133,13 @@ int32_t mfma_tab_ptrs(vq_ctx *ctx, int m, int k, MfmaTabPtrs &t) {
     t.nb = 2 * ((k + 63) / 64);  // blocks of 32 centroids, an even number (the kernel scores them in pairs)
     // A operands: 2 x 64 lanes x 16 bytes per (s, block of 32 centroids)
     const size_t n_atab = (size_t)m * t.nb * 512;
+    if (ctx->no_alloc) {  // the fixed scratch array; vq_assign_noalloc has checked that the shape fits
+        t.atab = (vq::u32x4 *)ctx->static_scratch;
+        t.maxc2 = (float *)(ctx->static_scratch + kNoAllocAuxOff);
+        t.mu = t.maxc2 + m;
+        t.stat = (uint32_t *)(ctx->static_scratch + kNoAllocStatOff);
+        return VQ_OK;
+    }
     VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + 9 * (size_t)m) + 64));
     VQ_TRY(ensure(ctx, ctx->mfma_stat, sizeof(uint32_t) * vq::kStatSlots * vq::kStatStride));
     float *atab = (float *)ctx->mfma_tab.p;
@@ -169,7 +191,7 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready, hip
     VQ_HIP(ctx, hipGetLastError());
     if (started) *started = ev_a;
     if (done) *done = ev_b;
-    ctx->recheck_src = 1;
+    ctx->recheck_src = ctx->no_alloc ? 3 : 1;
     return VQ_OK;
 }
 
@@ -242,7 +264,7 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
 
 template <int METRIC, bool LBG>
 bool mfma_wide_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
-    if (ctx->assign_path == 1) return false;
+    if (ctx->assign_path == 1 || ctx->no_alloc) return false;  // its lists grow with n: not for a fixed scratch
     if (METRIC != vq::M_SQ && METRIC != vq::M_EUCLID) return false;
     if (sd < 16 || sd % 8 != 0 || a.k > 256 || a.m > 65535) return false;
     // float4 row and centroid loads
@@ -377,10 +399,14 @@ int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, i
     a.changed = nullptr;
     a.done = nullptr;
     if (metric == VQ_COSINE) {
-        VQ_TRY(ensure(ctx, ctx->cnorm, sizeof(float) * (size_t)m * k));
+        float *cnorm = (float *)(ctx->static_scratch + kNoAllocNormOff);
+        if (!ctx->no_alloc) {
+            VQ_TRY(ensure(ctx, ctx->cnorm, sizeof(float) * (size_t)m * k));
+            cnorm = (float *)ctx->cnorm.p;
+        }
         hipLaunchKernelGGL(vq::k_centroid_norms, dim3(cdiv((int64_t)m * k, 256)), dim3(256), 0,
-                           ctx->stream, d_codebooks, (int64_t)m * k, sd, (float *)ctx->cnorm.p);
-        a.cnorm = (const float *)ctx->cnorm.p;
+                           ctx->stream, d_codebooks, (int64_t)m * k, sd, cnorm);
+        a.cnorm = cnorm;
     }
     ProfSpan sp(ctx, VQ_PROF_ENCODE);
     return launch_assign<false>(ctx, metric, a, sd);
@@ -414,6 +440,14 @@ int32_t vq_ctx_create(int32_t device, vq_ctx **out) {
         delete ctx;
         return rc;
     }
+    // this GPU's copy of the scratch array (every GPU holds its own, at its own address)
+    void *sp = nullptr;
+    if ((e = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch))) != hipSuccess || !sp) {
+        int32_t rc = fail(nullptr, VQ_ERR_HIP, "address of the scratch array: %s", hipGetErrorString(e));
+        vq_ctx_destroy(ctx);
+        return rc;
+    }
+    ctx->static_scratch = (unsigned char *)sp;
     *out = ctx;
     return VQ_OK;
 }
@@ -571,9 +605,10 @@ int32_t vq_ctx_last_recheck_split(vq_ctx *ctx, uint32_t *h_count, uint32_t *h_tw
     if (!ctx || !h_count || !h_two) return VQ_ERR_INVALID_ARG;
     *h_count = 0;
     *h_two = 0;
-    if (ctx->recheck_src == 1) {
+    if (ctx->recheck_src == 1 || ctx->recheck_src == 3) {
         uint32_t h[vq::kStatSlots * vq::kStatStride];
-        VQ_HIP(ctx, hipMemcpyAsync(h, ctx->mfma_stat.p, sizeof(h), hipMemcpyDeviceToHost, ctx->stream));
+        const void *src = ctx->recheck_src == 1 ? ctx->mfma_stat.p : ctx->static_scratch + kNoAllocStatOff;
+        VQ_HIP(ctx, hipMemcpyAsync(h, src, sizeof(h), hipMemcpyDeviceToHost, ctx->stream));
         VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
         for (int i = 0; i < vq::kStatSlots; ++i) *h_count += h[i * vq::kStatStride];
     } else if (ctx->recheck_src == 2) {
@@ -809,6 +844,27 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
 int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                   int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes) {
     return vqh::assign_codes(ctx, metric, d_x, n, ld, m, sd, k, d_codebooks, d_codes);
+}
+
+int32_t vq_assign_noalloc(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
+                          int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    // the tables of the call must fit the fixed scratch: column blocks x centroids padded to 64
+    if (m > 0 && k > 0 && k <= vq::kMaxK) {
+        const int64_t cells = (int64_t)m * 64 * ((k + 63) / 64);
+        if (m > kNoAllocMaxM || cells > kNoAllocMaxCells)
+            return fail(ctx, VQ_ERR_UNSUPPORTED,
+                        "vq_assign_noalloc: m * k (k padded to 64) = %lld exceeds the fixed scratch of %d "
+                        "(use vq_assign, which may allocate)", (long long)cells, kNoAllocMaxCells);
+    }
+    // no timing spans (their events are created on demand) and no workspace growth inside the call
+    const bool prof = ctx->prof_on;
+    ctx->prof_on = false;
+    ctx->no_alloc = true;
+    const int32_t rc = vqh::assign_codes(ctx, metric, d_x, n, ld, m, sd, k, d_codebooks, d_codes);
+    ctx->no_alloc = false;
+    ctx->prof_on = prof;
+    return rc;
 }
 
 int32_t vq_decode_f16(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sd, int32_t k,
