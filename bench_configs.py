@@ -10,7 +10,7 @@ the configurations that are otherwise parity-test cases:
 
     python bench_configs.py [c3] [c4] [c5]
 
-Prints one JSON object (milliseconds).  One GPU; inputs are the seeded generators of tests/data.py.
+Prints one JSON object (milliseconds).  One GPU; inputs are the seeded generators of vq_amd/synth.py.
 """
 import json
 import os
@@ -27,7 +27,7 @@ F = np.float32
 
 def main():
     import vq_amd
-    from tests import data
+    from vq_amd import synth as data
 
     which = sys.argv[1:] or ["c4", "c5", "c3"]
     ctx = vq_amd.Context(0)

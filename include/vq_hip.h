@@ -66,8 +66,9 @@ int32_t vq_ctx_sync(vq_ctx *ctx);
 void *vq_ctx_stream(vq_ctx *ctx);
 
 /* Which kernels decide the squared-L2 / Euclidean assignment where both exist:
- *   0 (default)  matrix-core scores (bf16-split operands for 8-float column blocks, fp32 operands
- *                for wider ones) with an exact re-check of every undecided (row, block) pair
+ *   0 (default)  matrix-core scores (bf16 matrix instructions on operands split into two bf16
+ *                parts, for 8-float column blocks and for wider ones whose width is a multiple
+ *                of 8) with an exact re-check of every undecided (row, block) pair
  *   1            the all-vector-ALU kernel in the reference's operation order
  * Both give bit-identical codes; the switch exists for measurement and tests. */
 int32_t vq_ctx_set_assign_path(vq_ctx *ctx, int32_t path);
@@ -105,6 +106,12 @@ int32_t vq_ctx_last_recheck_split(vq_ctx *ctx, uint32_t *h_all_centroids, uint32
 
 int32_t vq_malloc(vq_ctx *ctx, size_t bytes, void **d_ptr);
 int32_t vq_free(vq_ctx *ctx, void *d_ptr);
+/* Page-locked host memory for the packed rows and the returned codes: copies from and to it run at
+ * the link's rate (a pageable buffer is staged through a bounce buffer by the runtime, about half
+ * the rate).  The host packs `&[Vector<f32>]` (one heap allocation per row, src/vector.rs:150-152)
+ * straight into such a buffer.  No counterpart in the reference. */
+int32_t vq_host_alloc(vq_ctx *ctx, size_t bytes, void **h_ptr);
+int32_t vq_host_free(vq_ctx *ctx, void *h_ptr);
 /* Synchronous copies (they synchronise the context's stream). Replaces the per-vector heap
  * layout `&[Vector<f32>]` (src/vector.rs:150-152): the host packs rows into one buffer. */
 int32_t vq_h2d(vq_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
@@ -153,8 +160,10 @@ int32_t vq_prof_read(vq_ctx *ctx, int32_t cls, double *h_total_ms, int64_t *h_sp
  *   h_iters_run      out (nullable), m: loop bodies executed per problem (early break, 104-106)
  *   h_reseeds_used   out (nullable), m
  * Assignment is squared-L2, sequential f32 accumulation, strict '<' (utils.rs:62-70); the mean
- * follows mean_vector's order (src/vector.rs:282-318) for clusters of at most 1024 rows and a
- * fixed midpoint tree above that.
+ * follows mean_vector's order (src/vector.rs:282-318) for clusters of at most 1024 rows (row order
+ * from 0.0).  Above 1024 the reference's Rayon reduce has no fixed order; this library fixes one:
+ * the rows are cut into parts of 4096 consecutive rows, a cluster's members inside a part are added
+ * in row order from 0.0, and the part sums are added in part order from 0.0.
  * Errors: k == 0 or n < k -> VQ_ERR_INVALID_ARG (utils.rs:39-50); k > 256 -> VQ_ERR_UNSUPPORTED.
  * Synchronises the stream before returning. */
 int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t m,

@@ -672,13 +672,59 @@ void vqo_procrustes(const double *A, int64_t dim, double *R) {
         if (off < 1e-15) break;
     }
     /* normalise the columns of U (divide by singular values) */
+    double *sv = (double *)malloc(sizeof(double) * (size_t)n);
+    double top = 0.0;
     for (int64_t j = 0; j < n; ++j) {
         double s = 0;
         for (int64_t i = 0; i < n; ++i) s += U[i * n + j] * U[i * n + j];
         s = sqrt(s);
+        sv[j] = s;
+        if (s > top) top = s;
         if (s > 0)
             for (int64_t i = 0; i < n; ++i) U[i * n + j] /= s;
     }
+    /* A singular A does not determine the columns of U that belong to its zero singular values
+     * (an SVD library returns some orthonormal completion; nalgebra gives U = V = I for A = 0).
+     * Complete them, in ascending order: the matching column of V with the fixed columns
+     * projected out if more than half of it is left, else the unit vector of which the most is
+     * left.  U is then orthogonal and so is R. */
+    char *fixed = (char *)malloc((size_t)n);
+    double *w = (double *)malloc(sizeof(double) * (size_t)n);
+    double *best = (double *)malloc(sizeof(double) * (size_t)n);
+    for (int64_t j = 0; j < n; ++j) fixed[j] = top > 0.0 && sv[j] > 1e-12 * top;
+    for (int64_t j = 0; j < n; ++j) {
+        if (fixed[j]) continue;
+        double nrm = -1.0;
+        for (int64_t cand = -1; cand < n; ++cand) { /* -1: column j of V; then e_0 ... e_{n-1} */
+            for (int64_t i = 0; i < n; ++i) w[i] = cand < 0 ? V[i * n + j] : (i == cand ? 1.0 : 0.0);
+            for (int round = 0; round < 2; ++round)
+                for (int64_t l = 0; l < n; ++l) {
+                    if (!fixed[l]) continue;
+                    double d = 0.0;
+                    for (int64_t i = 0; i < n; ++i) d += U[i * n + l] * w[i];
+                    for (int64_t i = 0; i < n; ++i) w[i] -= d * U[i * n + l];
+                }
+            double r = 0.0;
+            for (int64_t i = 0; i < n; ++i) r += w[i] * w[i];
+            r = sqrt(r);
+            if (cand < 0) {
+                if (r > 0.5) {
+                    nrm = r;
+                    memcpy(best, w, sizeof(double) * (size_t)n);
+                    break;
+                }
+            } else if (r > nrm) {
+                nrm = r;
+                memcpy(best, w, sizeof(double) * (size_t)n);
+            }
+        }
+        for (int64_t i = 0; i < n; ++i) U[i * n + j] = best[i] / nrm;
+        fixed[j] = 1;
+    }
+    free(sv);
+    free(fixed);
+    free(w);
+    free(best);
     /* R = V U^T */
     for (int64_t i = 0; i < n; ++i)
         for (int64_t j = 0; j < n; ++j) {

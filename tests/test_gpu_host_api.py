@@ -128,6 +128,38 @@ def test_opq_first_outer_iteration_matches_oracle(vq):
     assert abs(e_got - e_want) <= 0.02 * e_want
 
 
+@pytest.mark.parametrize("dim,m", [(256, 16), (135, 3), (144, 2)])
+def test_opq_fit_above_dim_128_matches_oracle(vq, dim, m):
+    """The reference takes any dim divisible by m (src/opq.rs:103-115).  Above 128 the cross-
+    covariance runs in 128-wide output blocks and the rotation update on the host inside the
+    library; the first outer iteration is compared with the oracle as at dim 16."""
+    rng = np.random.default_rng(dim)
+    n, k, iters = 1500, 8, 4
+    x = (rng.standard_normal((n, dim)) @ (np.eye(dim) + 0.3 * rng.standard_normal((dim, dim)))).astype(F)
+    streams = data.index_streams(n, m, k, iters, seed=dim)
+    got = vq.OptimizedProductQuantizer.fit(x, m, k, iters, 1, vq.Distance.Euclidean, 0, streams=streams)
+    want = O.opq_fit(O.EUCLIDEAN, x, m, k, iters, 1, *streams)
+    assert np.array_equal(got.codebooks(), want["codebooks"])
+    R = got.rotation().astype(np.float64)
+    assert np.allclose(R.T @ R, np.eye(dim), atol=1e-5)
+    assert np.allclose(got.rotation(), want["rotation"], atol=5e-6)
+    qb = got.quantize_batch(x[:100])
+    assert qb.shape == (100, dim) and np.isfinite(qb.astype(F)).all()
+
+
+def test_opq_with_no_outer_iteration_has_no_codebooks(vq):
+    """opq_iters = 0: the reference returns an identity rotation and an empty codebook list, so
+    quantize pushes nothing and returns an empty vector (src/opq.rs:119-122, 244-263)."""
+    x = generate_test_data(100, 8)
+    opq = vq.OptimizedProductQuantizer.fit(x, 2, 4, 5, 0, vq.Distance.Euclidean, 1)
+    assert np.array_equal(opq.rotation(), np.eye(8, dtype=F))
+    assert len(opq.quantize(x[0])) == 0
+    assert opq.quantize_batch(x).shape == (100, 0)
+    assert opq.k == 0
+    with pytest.raises(vq.VqError, match="Dimension mismatch"):
+        opq.quantize(x[0][:5])
+
+
 # ---- tests/test_rvq.rs ---------------------------------------------------------------------------
 def test_rvq_on_random_vectors(vq):
     training = generate_test_data(1000, 10)
@@ -211,3 +243,24 @@ def test_host_classes_under_ubsan():
                          timeout=600)
     assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-3000:]
     assert "runtime error" not in res.stderr
+
+
+def test_host_classes_under_asan():
+    """The same once more against the host mirror built with -fsanitize=address,undefined (host
+    code only: the kernels are not instrumented).  The sanitizer's runtime is preloaded into the
+    child in front of whatever is preloaded already."""
+    import os
+    import subprocess
+    import sys
+    if os.environ.get("VQ_HOST_LIB"):
+        pytest.skip("already the sanitizer run")
+    from tests.test_oracle_sanitized import asan_env
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = os.path.join(root, "vq_amd", "libvqhost_asan.so")
+    assert os.path.exists(lib), "build it with `python -m vq_amd.build`"
+    res = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-p", "no:cacheprovider", "-m", "gpu",
+                          os.path.abspath(__file__)], cwd=root, env=asan_env(VQ_HOST_LIB=lib),
+                         capture_output=True, text=True, timeout=900)
+    at = max(res.stderr.find("AddressSanitizer"), 0)
+    assert res.returncode == 0, res.stdout[-1500:] + res.stderr[max(at - 200, 0):at + 4000]
+    assert "AddressSanitizer" not in res.stderr and "runtime error" not in res.stderr

@@ -357,3 +357,31 @@ def test_calibration_reports_plausible_peaks(ctx):
     assert rates[2] <= 1.05 * rates[5] and rates[4] <= 1.05 * rates[5]
     with pytest.raises(Exception):
         ctx.calibrate(9)
+
+
+def test_failures_forced_from_the_host_come_back_as_status_codes(ctx):
+    """Error paths of the ABI, forced from the host (no kernel faults): an allocation no GPU can
+    satisfy is VQ_ERR_OOM with the context still usable, and a re-seed stream that runs out is
+    VQ_ERR_RESEED_EXHAUSTED (the reference draws from an endless RNG, src/utils.rs:100; the ABI
+    takes a finite stream and must say when it was too short)."""
+    import vq_amd
+    with pytest.raises(vq_amd.VqError) as e:
+        ctx.empty((1 << 46,), np.uint8)  # 64 TiB
+    assert e.value.code == vq_amd._ffi.ERR_OOM
+    # all rows equal: every row lands in cluster 0, clusters 1..3 are empty in the first update
+    x = np.ones((64, 8), F)
+    dx = ctx.to_device(x)
+    dcb = ctx.empty((1, 4, 8), F)
+    init = np.arange(4, dtype=np.uint32)[None]
+    with pytest.raises(vq_amd.VqError) as e:
+        ctx.lbg_fit(dx, 64, 8, 1, 8, 4, 3, init, np.zeros((1, 2), np.uint32), dcb)
+    assert e.value.code == vq_amd._ffi.ERR_RESEED_EXHAUSTED
+    with pytest.raises(vq_amd.VqError) as e:   # the generic update path (sub_dim 3) reports it too
+        ctx.lbg_fit(ctx.to_device(np.ones((64, 3), F)), 64, 3, 1, 3, 4, 3, init, np.zeros((1, 1), np.uint32),
+                    ctx.empty((1, 4, 3), F))
+    assert e.value.code == vq_amd._ffi.ERR_RESEED_EXHAUSTED
+    # the context survives both: the same fit with a stream that is long enough matches the oracle
+    reseed = np.arange(12, dtype=np.uint32)[None] % 64
+    ctx.lbg_fit(dx, 64, 8, 1, 8, 4, 3, init, reseed, dcb)
+    want = O.lbg(x, 4, 3, init[0], reseed[0])
+    assert np.array_equal(dcb.download()[0].view(np.uint32), want["centroids"].view(np.uint32))

@@ -126,7 +126,8 @@ def test_rotate_matches_matrix_product(ctx, n, dim):
     assert np.array_equal(dy.download(), x)  # identity is exact (opq.rs:119-121)
 
 
-@pytest.mark.parametrize("n,dim", [(1000, 10), (5000, 128), (2049, 32), (4099, 16), (2050, 80), (777, 20)])
+@pytest.mark.parametrize("n,dim", [(1000, 10), (5000, 128), (2049, 32), (4099, 16), (2050, 80), (777, 20),
+                                   (9000, 256), (5000, 144), (3000, 200), (2100, 135), (10000, 384)])
 def test_cross_cov_matches_f64_product(ctx, n, dim):
     rng = np.random.default_rng(n)
     x = rng.standard_normal((n, dim)).astype(F)
@@ -155,15 +156,33 @@ def test_procrustes_rotation_is_the_polar_factor(ctx, dim):
     assert np.allclose(R, O.procrustes(A), atol=1e-9)
     Q, _ = np.linalg.qr(rng.standard_normal((dim, dim)))
     assert np.allclose(ctx.procrustes_rotation(Q), Q.T, atol=1e-12)
-    # a zero matrix has no unit singular vectors: zero comes back, as from the host routine
-    assert np.array_equal(ctx.procrustes_rotation(np.zeros((dim, dim))), O.procrustes(np.zeros((dim, dim))))
+    # a zero matrix determines no singular vector: the completion gives the identity (U = V = I,
+    # as an SVD library returns), not a rank-deficient R
+    assert np.array_equal(ctx.procrustes_rotation(np.zeros((dim, dim))), np.eye(dim))
 
 
-def test_procrustes_rotation_rejects_sizes_outside_the_kernel(ctx):
-    import vq_amd
-    for dim in (3, 130):
-        with pytest.raises(vq_amd.VqError):
-            ctx.procrustes_rotation(np.eye(dim))
+@pytest.mark.parametrize("dim,rank", [(4, 2), (16, 10), (64, 63), (128, 100), (7, 3), (130, 60)])
+def test_procrustes_rotation_of_a_singular_matrix_is_orthogonal(ctx, dim, rank):
+    """Directions that A leaves open (zero singular values; an all-zero column such as a padded
+    dimension) are completed to an orthonormal basis: R stays orthogonal and optimal.  Even sizes
+    up to 128 run the device SVD, the others the host routine inside the library."""
+    rng = np.random.default_rng(dim + rank)
+    A = rng.standard_normal((dim, rank)) @ rng.standard_normal((rank, dim))
+    for M in (A, np.where(np.arange(dim) == dim - 1, 0.0, rng.standard_normal((dim, dim)))):
+        R = ctx.procrustes_rotation(M)
+        assert np.allclose(R.T @ R, np.eye(dim), atol=1e-10)
+        P = R @ M
+        assert np.allclose(P, P.T, atol=1e-8 * np.abs(M).max())
+        assert abs(np.trace(P) - np.linalg.svd(M, compute_uv=False).sum()) <= 1e-9 * np.abs(P).sum()
+
+
+@pytest.mark.parametrize("dim", [3, 9, 130, 200])
+def test_procrustes_rotation_sizes_outside_the_device_kernel(ctx, dim):
+    rng = np.random.default_rng(dim)
+    A = rng.standard_normal((dim, dim))
+    R = ctx.procrustes_rotation(A)
+    assert np.allclose(R.T @ R, np.eye(dim), atol=1e-10)
+    assert np.allclose(R, O.procrustes(A), atol=1e-9)
 
 
 def test_opq_outer_iteration_stepwise(ctx):

@@ -311,6 +311,29 @@ def test_procrustes_is_the_polar_factor():
     assert np.allclose(O.procrustes(Q), Q.T, atol=1e-12)  # orthogonal A -> R = A^T
 
 
+@pytest.mark.parametrize("dim,rank", [(4, 0), (6, 3), (8, 7), (5, 1), (16, 10)])
+def test_procrustes_of_a_singular_matrix_is_still_orthogonal(dim, rank):
+    """A of rank < dim leaves directions of U open; whatever completion is chosen, R = V U^T must
+    be orthogonal, R A symmetric positive semi-definite with trace = nuclear norm of A (that is
+    what makes it a Procrustes solution), and A = 0 gives the identity, as an SVD library's
+    U = V = I does."""
+    rng = np.random.default_rng(dim * 31 + rank)
+    A = (rng.standard_normal((dim, rank)) @ rng.standard_normal((rank, dim))) if rank else np.zeros((dim, dim))
+    R = O.procrustes(A)
+    assert np.allclose(R.T @ R, np.eye(dim), atol=1e-10)
+    P = R @ A
+    assert np.allclose(P, P.T, atol=1e-9 * max(1.0, np.abs(A).max()))
+    assert abs(np.trace(P) - np.linalg.svd(A, compute_uv=False).sum()) <= 1e-9 * max(1.0, np.abs(P).sum())
+    if rank == 0:
+        assert np.array_equal(R, np.eye(dim))
+    # an all-zero column (a padded dimension) must not cost the rotation its rank
+    B = rng.standard_normal((dim, dim))
+    B[:, dim - 1] = 0.0
+    Rb = O.procrustes(B)
+    assert np.allclose(Rb.T @ Rb, np.eye(dim), atol=1e-10)
+    assert abs(np.trace(Rb @ B) - np.linalg.svd(B, compute_uv=False).sum()) <= 1e-9 * np.abs(B).sum()
+
+
 def test_rotate_is_matrix_vector_product():
     rng = np.random.default_rng(42)
     x = rng.standard_normal((20, 8)).astype(F)

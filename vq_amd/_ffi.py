@@ -34,6 +34,8 @@ SYMBOLS = {
     "vq_procrustes_rotation": (_i32, [_vp, _vp, _i32, _vp]),
     "vq_malloc": (_i32, [_vp, _sz, C.POINTER(_vp)]),
     "vq_free": (_i32, [_vp, _vp]),
+    "vq_host_alloc": (_i32, [_vp, _sz, C.POINTER(_vp)]),
+    "vq_host_free": (_i32, [_vp, _vp]),
     "vq_h2d": (_i32, [_vp, _vp, _vp, _sz]),
     "vq_d2h": (_i32, [_vp, _vp, _vp, _sz]),
     "vq_copy_f32": (_i32, [_vp, _vp, _vp, _i64]),
@@ -165,9 +167,13 @@ class Context:
         if rc != VQ_OK:
             raise VqError(rc, (_lib.vq_last_error(None) or b"").decode())
         self._h = h
+        self._pinned = {}
 
     def close(self):
         if self._h:
+            for p in list(self._pinned.values()):
+                _lib.vq_host_free(self._h, p)
+            self._pinned.clear()
             _lib.vq_ctx_destroy(self._h)
             self._h = None
 
@@ -188,6 +194,24 @@ class Context:
     def to_device(self, host, dtype=None):
         host = np.ascontiguousarray(host, dtype=dtype)
         return DeviceArray(self, host.shape, host.dtype).upload(host)
+
+    def host_empty(self, shape, dtype):
+        """A numpy array over page-locked host memory (vq_host_alloc); release it with
+        host_free(array) once no view of it is in use."""
+        dtype = np.dtype(dtype)
+        shape = tuple(int(s) for s in np.atleast_1d(shape))
+        nbytes = int(np.prod(shape)) * dtype.itemsize
+        p = _vp()
+        self._check(_lib.vq_host_alloc(self._h, nbytes, C.byref(p)))
+        buf = (C.c_char * max(nbytes, 1)).from_address(p.value)
+        arr = np.frombuffer(buf, dtype=dtype, count=int(np.prod(shape))).reshape(shape)
+        self._pinned[arr.ctypes.data] = p.value
+        return arr
+
+    def host_free(self, arr):
+        p = self._pinned.pop(arr.ctypes.data, None)
+        if p:
+            self._check(_lib.vq_host_free(self._h, p))
 
     def copy_f32(self, d_dst, d_src, count):
         self._check(_lib.vq_copy_f32(self._h, d_dst.ptr, d_src.ptr, count))

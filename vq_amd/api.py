@@ -93,8 +93,9 @@ class _Quantizer:
         """quantize(&self, &Vector<f32>) -> Vector<f16>"""
         v = np.ascontiguousarray(vector, np.float32).reshape(-1)
         out = np.zeros(max(self.dim, v.size), np.uint16)
-        _check(_h.vqh_quantize(_vp(self._o), _p(v), _i64(v.size), _p(out)))
-        return out[:self.dim].view(np.float16)
+        got = _i64(0)
+        _check(_h.vqh_quantize(_vp(self._o), _p(v), _i64(v.size), _p(out), C.byref(got)))
+        return out[:got.value].view(np.float16)
 
     def quantize_batch(self, data):
         x = _rows(data)
@@ -149,9 +150,14 @@ class OptimizedProductQuantizer(_Quantizer):
         _check(_h.vqh_opq_fit(_p(x), _i64(n), _i64(dim), _i64(m), _i64(k), _i64(max_iters),
                               _i64(opq_iters), kind, C.c_double(p), _u64(seed), _p(init), _p(reseed),
                               _i32(nr), C.byref(h)))
-        q = cls(h.value)
-        q.m, q.k, q.sub_dim = m, k, dim // m
-        return q
+        return cls(h.value)  # m, k, sub_dim from vqh_info; k = 0 when opq_iters == 0 left no codebooks
+
+    def quantize_batch(self, data):
+        if self.k == 0:  # the reference returns an empty vector per row (src/opq.rs:122,244-263)
+            x = _rows(data)
+            _check(_h.vqh_quantize_batch(_vp(self._o), _p(x), _i64(x.shape[0]), _i64(x.shape[1]), None))
+            return np.zeros((x.shape[0], 0), np.float16)
+        return super().quantize_batch(data)
 
     def encode(self, data):
         x = _rows(data)

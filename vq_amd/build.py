@@ -50,14 +50,18 @@ HOST_LIB = os.path.join(HERE, "libvqhost.so")
 
 
 HOST_LIB_UBSAN = os.path.join(HERE, "libvqhost_ubsan.so")
+HOST_LIB_ASAN = os.path.join(HERE, "libvqhost_asan.so")
 
 
-def build_host(verbose=False, ubsan=False):
+def build_host(verbose=False, ubsan=False, asan=False):
     """Compiles the C++ host mirror (plain g++: it only needs the C ABI) and links it to libvqhip.
     ubsan: a second build under the undefined-behaviour sanitizer (aborts at the first finding),
-    which the tests load through VQ_HOST_LIB."""
-    out = HOST_LIB_UBSAN if ubsan else HOST_LIB
-    opt = ["-O1", "-g", "-fsanitize=undefined", "-fno-sanitize-recover=undefined", "-static-libubsan"] \
+    which the tests load through VQ_HOST_LIB.  asan: a third one under the address and the
+    undefined-behaviour sanitizers (the process that loads it preloads libasan.so)."""
+    out = HOST_LIB_ASAN if asan else HOST_LIB_UBSAN if ubsan else HOST_LIB
+    opt = ["-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined", "-fno-sanitize-recover=all"] \
+        if asan else \
+        ["-O1", "-g", "-fsanitize=undefined", "-fno-sanitize-recover=undefined", "-static-libubsan"] \
         if ubsan else ["-O3"]
     cmd = ["g++", *opt, "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-Wall",
            os.path.join(HERE, "host", "vq_host_c.cpp"), "-o", out,
@@ -74,3 +78,4 @@ if __name__ == "__main__":
     print(build_lib(verbose=True, extra=sys.argv[1:]))
     print(build_host(verbose=True))
     print(build_host(verbose=True, ubsan=True))
+    print(build_host(verbose=True, asan=True))

@@ -71,9 +71,12 @@ inline int32_t fail(vq_ctx *ctx, int32_t code, const char *fmt, ...) {
 #define VQ_HIP(ctx, call)                                                                          \
     do {                                                                                           \
         hipError_t e__ = (call);                                                                   \
-        if (e__ != hipSuccess)                                                                     \
+        if (e__ != hipSuccess) {                                                                   \
+            (void)hipGetLastError(); /* the runtime keeps the error until it is read: a later   */ \
+                                     /* check of a good launch would report this one again      */ \
             return vqh::fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,            \
                              "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__, __LINE__); \
+        }                                                                                          \
     } while (0)
 
 #define VQ_TRY(expr)                    \

@@ -228,49 +228,52 @@ static __global__ void __launch_bounds__(256) k_rotate_generic(const float *__re
 
 // ---- cross-covariance ----------------------------------------------------------------------
 // part[c][a][b] = sum over the rows of chunk c of yr[i][a] * x[i][b], accumulated in f64 in row
-// order; chunks are combined in chunk order by k_crosscov_reduce.  Generic dimension.
+// order; chunks are combined in chunk order by k_crosscov_reduce.  Generic dimension: a workgroup
+// takes one tile of up to 128 x 128 outputs of one chunk (grid.y walks the tiles row by row).
 static __global__ void __launch_bounds__(256) k_crosscov_partial(const float *__restrict__ yr,
                                                           const float *__restrict__ x, int64_t n,
                                                           int dim, int64_t rows_per_chunk,
                                                           double *__restrict__ part) {
-    extern __shared__ float lds[];  // 2 * 32 * dim floats
-    float *ly = lds, *lx = lds + 32 * dim;
+    __shared__ float ly[32 * 128], lx[32 * 128];
+    const int tiles = (dim + 127) / 128;
+    const int a0 = (int)(blockIdx.y / tiles) * 128, b0 = (int)(blockIdx.y % tiles) * 128;
+    const int da = dim - a0 < 128 ? dim - a0 : 128, db = dim - b0 < 128 ? dim - b0 : 128;
     const int64_t lo = (int64_t)blockIdx.x * rows_per_chunk;
     const int64_t hi = lo + rows_per_chunk < n ? lo + rows_per_chunk : n;
-    const int total = dim * dim;
-    // each thread owns outputs e = tid, tid+256, ... (at most 64 per thread: dim <= 128)
+    const int total = da * db;
+    // each thread owns outputs e = tid, tid+256, ... of the tile (at most 64 per thread)
     double acc[64];
 #pragma unroll
     for (int u = 0; u < 64; ++u) acc[u] = 0.0;
     for (int64_t r0 = lo; r0 < hi; r0 += 32) {
         int rows = (int)((hi - r0) < 32 ? (hi - r0) : 32);
         __syncthreads();
-        for (int i = threadIdx.x; i < rows * dim; i += 256) {
-            ly[i] = yr[r0 * dim + i];
-            lx[i] = x[r0 * dim + i];
-        }
+        for (int i = threadIdx.x; i < rows * da; i += 256) ly[i] = yr[(r0 + i / da) * dim + a0 + i % da];
+        for (int i = threadIdx.x; i < rows * db; i += 256) lx[i] = x[(r0 + i / db) * dim + b0 + i % db];
         __syncthreads();
 #pragma unroll
         for (int u = 0; u < 64; ++u) {
             int e = threadIdx.x + u * 256;
             if (e < total) {
-                int a = e / dim, b = e % dim;
+                int a = e / db, b = e % db;
                 double s = acc[u];
-                for (int r = 0; r < rows; ++r) s += (double)ly[r * dim + a] * (double)lx[r * dim + b];
+                for (int r = 0; r < rows; ++r) s += (double)ly[r * da + a] * (double)lx[r * db + b];
                 acc[u] = s;
             }
         }
     }
-    double *out = part + (size_t)blockIdx.x * total;
+    double *out = part + (size_t)blockIdx.x * dim * dim;
 #pragma unroll
     for (int u = 0; u < 64; ++u) {
         int e = threadIdx.x + u * 256;
-        if (e < total) out[e] = acc[u];
+        if (e < total) out[(size_t)(a0 + e / db) * dim + b0 + e % db] = acc[u];
     }
 }
 
-// The same partial sums on the f64 matrix cores (v_mfma_f64_16x16x4_f64) for dim = 16 * NT <= 128.
-// One wave owns the 16 output rows [16 ti, 16 ti + 16) of a chunk and all NT column tiles; a
+// The same partial sums on the f64 matrix cores (v_mfma_f64_16x16x4_f64) for dim a multiple of 16:
+// a launch covers the output columns [b0 + 128 z, b0 + 128 z + 16 NT) for z = blockIdx.z and every
+// output row.
+// One wave owns the 16 output rows [16 ti, 16 ti + 16) of a chunk and NT column tiles; a
 // contraction step takes 4 rows: lane l supplies y[row + l/16][16 ti + l%16] and, per column
 // tile, x[row + l/16][16 tj + l%16], converted to f64 (the products are then exact).  The result
 // register v of lane l is A[16 ti + 4 v + l/16][16 tj + l%16].  Fixed order: deterministic.
@@ -278,12 +281,12 @@ typedef double doublex4 __attribute__((ext_vector_type(4)));
 
 template <int NT>
 __global__ void __launch_bounds__(256) k_crosscov_mfma(const float *__restrict__ yr, const float *__restrict__ x,
-                                                       int64_t n, int64_t rows_per_chunk,
+                                                       int64_t n, int DIM, int b0, int64_t rows_per_chunk,
                                                        double *__restrict__ part) {
-    constexpr int DIM = 16 * NT;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int ti = blockIdx.y * 4 + w;
-    if (ti >= NT) return;
+    if (ti >= DIM / 16) return;
+    b0 += 128 * blockIdx.z;
     const int kk = lane >> 4, jj = lane & 15;
     const int64_t lo = (int64_t)blockIdx.x * rows_per_chunk;
     const int64_t hi = lo + rows_per_chunk < n ? lo + rows_per_chunk : n;
@@ -291,7 +294,7 @@ __global__ void __launch_bounds__(256) k_crosscov_mfma(const float *__restrict__
 #pragma unroll
     for (int tj = 0; tj < NT; ++tj) acc[tj] = doublex4{0.0, 0.0, 0.0, 0.0};
     const float *yp = yr + (lo + kk) * DIM + 16 * ti + jj;
-    const float *xp = x + (lo + kk) * DIM + jj;
+    const float *xp = x + (lo + kk) * DIM + b0 + jj;
     float a = 0.0f, b[NT];
     bool valid = lo + kk < hi;
     a = valid ? *yp : 0.0f;
@@ -316,7 +319,7 @@ __global__ void __launch_bounds__(256) k_crosscov_mfma(const float *__restrict__
 #pragma unroll
     for (int tj = 0; tj < NT; ++tj)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) out[(size_t)(16 * ti + 4 * v + kk) * DIM + 16 * tj + jj] = acc[tj][v];
+        for (int v = 0; v < 4; ++v) out[(size_t)(16 * ti + 4 * v + kk) * DIM + b0 + 16 * tj + jj] = acc[tj][v];
 }
 
 static __global__ void __launch_bounds__(256) k_crosscov_reduce(const double *__restrict__ part, int chunks,
@@ -484,7 +487,8 @@ template <int LANES>
 static __global__ void __launch_bounds__(64 * LANES) k_jacobi_sweeps(const double *__restrict__ A, int n,
                                                                       double2 *__restrict__ rot,
                                                                       int *__restrict__ n_rounds,
-                                                                      double *__restrict__ uhat) {
+                                                                      double *__restrict__ uhat,
+                                                                      double *__restrict__ sv) {
     extern __shared__ __attribute__((aligned(16))) double ut[];  // n rows of stride kJacobiStride
     __shared__ int unfinished;
     constexpr int S = kJacobiStride, NT = 64 * LANES, PER = kJacobiMax / (2 * LANES);
@@ -554,11 +558,13 @@ static __global__ void __launch_bounds__(64 * LANES) k_jacobi_sweeps(const doubl
         if (!more) break;  // the same in every thread
     }
     if (tid == 0) *n_rounds = round;
-    // unit columns of U; a zero column stays zero
+    // unit columns of U and their lengths, the singular values; a zero column stays zero (the
+    // host completes the directions that A does not determine)
     for (int j = pair; j < n; j += 64) {
         double s = 0.0;
         for (int i = sub; i < n; i += LANES) s += ut[j * S + i] * ut[j * S + i];
         s = sqrt(pair_sum<LANES>(s));
+        if (sub == 0) sv[j] = s;
         for (int i = sub; i < n; i += LANES) uhat[(size_t)j * n + i] = s > 0.0 ? ut[j * S + i] / s : ut[j * S + i];
     }
 }

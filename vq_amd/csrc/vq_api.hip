@@ -500,6 +500,22 @@ int32_t vq_free(vq_ctx *ctx, void *d_ptr) {
     return VQ_OK;
 }
 
+int32_t vq_host_alloc(vq_ctx *ctx, size_t bytes, void **h_ptr) {
+    if (!ctx || !h_ptr) return VQ_ERR_INVALID_ARG;
+    *h_ptr = nullptr;
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    VQ_HIP(ctx, hipHostMalloc(h_ptr, bytes ? bytes : 1, hipHostMallocDefault));
+    return VQ_OK;
+}
+
+int32_t vq_host_free(vq_ctx *ctx, void *h_ptr) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (!h_ptr) return VQ_OK;
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    VQ_HIP(ctx, hipHostFree(h_ptr));
+    return VQ_OK;
+}
+
 int32_t vq_h2d(vq_ctx *ctx, void *d_dst, const void *h_src, size_t bytes) {
     if (!ctx || (bytes && (!d_dst || !h_src))) return VQ_ERR_INVALID_ARG;
     VQ_HIP(ctx, hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->stream));

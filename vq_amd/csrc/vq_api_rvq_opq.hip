@@ -8,6 +8,7 @@
 
 #include "ctx.hpp"
 #include "rvq_opq.hpp"
+#include "procrustes_host.hpp"
 
 using namespace vqh;
 
@@ -143,35 +144,38 @@ int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n,
     if (!ctx) return VQ_ERR_INVALID_ARG;
     if (n == 0) return fail(ctx, VQ_ERR_EMPTY_INPUT, "Empty input: at least one vector is required.");
     if (!d_y || !d_x || !h_A || n < 0 || dim <= 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
-    if (dim > 128) return fail(ctx, VQ_ERR_UNSUPPORTED, "cross-covariance: dim %d > 128", dim);
+    if (dim > 4096) return fail(ctx, VQ_ERR_UNSUPPORTED, "cross-covariance: dim %d > 4096", dim);
     VQ_HIP(ctx, hipSetDevice(ctx->device));
-    const int64_t rows_per_chunk = 2048;
+    // chunks of 2048 rows up to dim 128; longer chunks for larger matrices, so that the partial
+    // sums (one dim x dim matrix per chunk) stay at about 64 B per row
+    const int64_t scale = ((int64_t)dim + 127) / 128;
+    const int64_t rows_per_chunk = 2048 * scale * scale;
     const int chunks = (int)cdiv(n, rows_per_chunk);
     const int total = dim * dim;
     VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(double) * (size_t)chunks * total));
     VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * (size_t)total));
     if (dim % 16 == 0) {
-        const int nt = dim / 16;
-        const dim3 grid(chunks, (nt + 3) / 4);
+        const int nt_all = dim / 16, full = dim / 128, rest = nt_all % 8;
         double *part = (double *)ctx->tmp_a.p;
-#define CROSSCOV(NT)                                                                                 \
-    hipLaunchKernelGGL((vq::k_crosscov_mfma<NT>), grid, dim3(256), 0, ctx->stream, d_y, d_x, n,     \
-                       rows_per_chunk, part)
-        switch (nt) {
-        case 1: CROSSCOV(1); break;
-        case 2: CROSSCOV(2); break;
-        case 3: CROSSCOV(3); break;
-        case 4: CROSSCOV(4); break;
-        case 5: CROSSCOV(5); break;
-        case 6: CROSSCOV(6); break;
-        case 7: CROSSCOV(7); break;
-        default: CROSSCOV(8); break;
+#define CROSSCOV(NT, B0, Z)                                                                                 \
+    hipLaunchKernelGGL((vq::k_crosscov_mfma<NT>), dim3(chunks, (nt_all + 3) / 4, Z), dim3(256), 0, ctx->stream, \
+                       d_y, d_x, n, dim, B0, rows_per_chunk, part)
+        if (full) CROSSCOV(8, 0, full);
+        switch (rest) {
+        case 1: CROSSCOV(1, 128 * full, 1); break;
+        case 2: CROSSCOV(2, 128 * full, 1); break;
+        case 3: CROSSCOV(3, 128 * full, 1); break;
+        case 4: CROSSCOV(4, 128 * full, 1); break;
+        case 5: CROSSCOV(5, 128 * full, 1); break;
+        case 6: CROSSCOV(6, 128 * full, 1); break;
+        case 7: CROSSCOV(7, 128 * full, 1); break;
+        default: break;
         }
 #undef CROSSCOV
     } else {
-        size_t lds = sizeof(float) * 2 * 32 * (size_t)dim;
-        hipLaunchKernelGGL(vq::k_crosscov_partial, dim3(chunks), dim3(256), lds, ctx->stream, d_y, d_x, n, dim,
-                           rows_per_chunk, (double *)ctx->tmp_a.p);
+        const int tiles = (dim + 127) / 128;
+        hipLaunchKernelGGL(vq::k_crosscov_partial, dim3(chunks, tiles * tiles), dim3(256), 0, ctx->stream, d_y, d_x,
+                           n, dim, rows_per_chunk, (double *)ctx->tmp_a.p);
     }
     hipLaunchKernelGGL(vq::k_crosscov_reduce, dim3(cdiv(total, 256)), dim3(256), 0, ctx->stream,
                        (const double *)ctx->tmp_a.p, chunks, total, (double *)ctx->tmp_b.p);
@@ -183,19 +187,25 @@ int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n,
 
 int32_t vq_procrustes_rotation(vq_ctx *ctx, const double *h_A, int32_t dim, double *h_R) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
-    if (!h_A || !h_R || dim < 2) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
-    if (dim > vq::kJacobiMax || dim % 2 != 0)
-        return fail(ctx, VQ_ERR_UNSUPPORTED, "rotation update: dim %d is odd or above %d", dim, vq::kJacobiMax);
-    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    if (!h_A || !h_R || dim < 1) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    if (dim > 4096) return fail(ctx, VQ_ERR_UNSUPPORTED, "rotation update: dim %d above 4096", dim);
     const size_t total = (size_t)dim * dim;
+    // sizes the device kernel does not take: the same Jacobi SVD on the host (the reference runs
+    // its SVD on the host as well, src/opq.rs:180)
+    if (dim > vq::kJacobiMax || dim % 2 != 0) {
+        vqh::procrustes_host(h_A, (size_t)dim, h_R);
+        return VQ_OK;
+    }
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
     const int half = dim / 2;
     VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(double) * total));
     VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * total));
-    VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(double) * total));
+    VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(double) * (total + dim)));
     VQ_TRY(ensure(ctx, ctx->tmp_d, sizeof(double) * total));
     VQ_TRY(ensure(ctx, ctx->tmp_e, sizeof(double2) * (size_t)vq::kJacobiSweeps * (dim - 1) * half));
     VQ_TRY(ensure(ctx, ctx->tmp_f, 256));
     double *d_A = (double *)ctx->tmp_a.p, *d_vt = (double *)ctx->tmp_b.p, *d_uhat = (double *)ctx->tmp_c.p;
+    double *d_sv = d_uhat + total;
     double *d_out = (double *)ctx->tmp_d.p;
     double2 *d_rot = (double2 *)ctx->tmp_e.p;
     int *d_rounds = (int *)ctx->tmp_f.p;
@@ -205,14 +215,30 @@ int32_t vq_procrustes_rotation(vq_ctx *ctx, const double *h_A, int32_t dim, doub
     VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(vq::k_jacobi_sweeps<kLanes>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(vq::k_jacobi_sweeps<kLanes>, dim3(1), dim3(64 * kLanes), lds, ctx->stream, (const double *)d_A,
-                       dim, d_rot, d_rounds, d_uhat);
+                       dim, d_rot, d_rounds, d_uhat, d_sv);
     hipLaunchKernelGGL(vq::k_jacobi_accumulate, dim3(dim), dim3(64), 0, ctx->stream, (const double2 *)d_rot,
                        (const int *)d_rounds, dim, d_vt);
     hipLaunchKernelGGL(vq::k_jacobi_product, dim3((unsigned)cdiv(total, 256)), dim3(256), 0, ctx->stream,
                        (const double *)d_vt, (const double *)d_uhat, dim, d_out);
     VQ_HIP(ctx, hipGetLastError());
+    std::vector<double> sv((size_t)dim);
     VQ_HIP(ctx, hipMemcpyAsync(h_R, d_out, sizeof(double) * total, hipMemcpyDeviceToHost, ctx->stream));
+    VQ_HIP(ctx, hipMemcpyAsync(sv.data(), d_sv, sizeof(double) * dim, hipMemcpyDeviceToHost, ctx->stream));
     VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    // A singular A leaves directions of U open (their columns came back as zero or as rounding
+    // noise): complete them on the host and form the product again.  Rare; a full-rank A ends here.
+    double top = 0.0;
+    for (double v : sv) top = std::max(top, v);
+    bool open = false;
+    for (double v : sv) open = open || !(top > 0.0 && v > vqh::kNullRel * top);
+    if (open) {
+        std::vector<double> Ut(total), Vt(total);
+        VQ_HIP(ctx, hipMemcpyAsync(Ut.data(), d_uhat, sizeof(double) * total, hipMemcpyDeviceToHost, ctx->stream));
+        VQ_HIP(ctx, hipMemcpyAsync(Vt.data(), d_vt, sizeof(double) * total, hipMemcpyDeviceToHost, ctx->stream));
+        VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        vqh::complete_null_columns(Ut, Vt, sv, (size_t)dim);
+        vqh::product_v_ut(Vt, Ut, (size_t)dim, h_R);
+    }
     return VQ_OK;
 }
 

@@ -388,60 +388,6 @@ private:
     Distance distance_;
 };
 
-// ---- orthogonal Procrustes on the host (src/opq.rs:180-183) -------------------------------------
-// R = V U^T for A = U S V^T, by a cyclic one-sided Jacobi SVD in f64; row-major dim x dim.
-inline void procrustes_rotation(const std::vector<double> &A, size_t dim, std::vector<double> &R) {
-    const size_t n = dim;
-    // columns of U and V are kept as contiguous rows (Ut, Vt): every inner loop is unit-stride
-    std::vector<double> Ut(n * n), Vt(n * n, 0.0);
-    for (size_t i = 0; i < n; ++i) {
-        Vt[i * n + i] = 1.0;
-        for (size_t j = 0; j < n; ++j) Ut[j * n + i] = A[i * n + j];
-    }
-    for (int sweep = 0; sweep < 60; ++sweep) {
-        double off = 0.0;
-        for (size_t p = 0; p + 1 < n; ++p)
-            for (size_t q = p + 1; q < n; ++q) {
-                double *up = &Ut[p * n], *uq = &Ut[q * n];
-                double alpha = 0, beta = 0, gamma = 0;
-                for (size_t i = 0; i < n; ++i) {
-                    alpha += up[i] * up[i];
-                    beta += uq[i] * uq[i];
-                    gamma += up[i] * uq[i];
-                }
-                if (gamma == 0.0) continue;
-                off = std::max(off, std::fabs(gamma) / std::sqrt(alpha * beta + 1e-300));
-                double zeta = (beta - alpha) / (2.0 * gamma);
-                double t = (zeta >= 0 ? 1.0 : -1.0) / (std::fabs(zeta) + std::sqrt(1.0 + zeta * zeta));
-                double c = 1.0 / std::sqrt(1.0 + t * t), s = c * t;
-                double *vp = &Vt[p * n], *vq = &Vt[q * n];
-                for (size_t i = 0; i < n; ++i) {
-                    double a = up[i], b = uq[i];
-                    up[i] = c * a - s * b;
-                    uq[i] = s * a + c * b;
-                    double d = vp[i], e = vq[i];
-                    vp[i] = c * d - s * e;
-                    vq[i] = s * d + c * e;
-                }
-            }
-        if (off < 1e-15) break;
-    }
-    for (size_t j = 0; j < n; ++j) {
-        double s = 0;
-        for (size_t i = 0; i < n; ++i) s += Ut[j * n + i] * Ut[j * n + i];
-        s = std::sqrt(s);
-        if (s > 0)
-            for (size_t i = 0; i < n; ++i) Ut[j * n + i] /= s;
-    }
-    // R[i][j] = sum_l V[i][l] U[j][l], l ascending
-    R.assign(n * n, 0.0);
-    for (size_t l = 0; l < n; ++l)
-        for (size_t i = 0; i < n; ++i) {
-            const double v = Vt[l * n + i];
-            for (size_t j = 0; j < n; ++j) R[i * n + j] += v * Ut[l * n + j];
-        }
-}
-
 // ---- OptimizedProductQuantizer (src/opq.rs) -----------------------------------------------------
 class OptimizedProductQuantizer {
 public:
@@ -492,35 +438,48 @@ public:
                                      q.codebooks_.get(), drec.get()));                            // 164-167
             dev->check(vq_cross_cov(c, drec.get(), drot.get(), (int64_t)n, (int32_t)dim, A.data())); // 172-179
             for (double &v : A) v = (double)(float)v;  // the reference's A is a DMatrix<f32>
-            // 180-183: on the device while its kernel takes the size, else on the host
-            if (dim % 2 == 0 && dim >= 2 && dim <= 128) {
-                Rd.resize(dim * dim);
-                dev->check(vq_procrustes_rotation(c, A.data(), (int32_t)dim, Rd.data()));
-            } else {
-                procrustes_rotation(A, dim, Rd);
-            }
+            // 180-183 (the library runs the SVD on the device while its kernel takes the size,
+            // else on the host, and completes the directions a singular A leaves open)
+            Rd.resize(dim * dim);
+            dev->check(vq_procrustes_rotation(c, A.data(), (int32_t)dim, Rd.data()));
             for (size_t i = 0; i < dim * dim; ++i) q.rotation_[i] = (float)Rd[i];
             q.d_rotation_.upload(q.rotation_.data(), dim * dim);
             dev->check(vq_rotate(c, dx.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, q.d_rotation_.get(),
                                  drot.get()));                                                    // 186-194
         }
-        if (opq_iters == 0) q.d_rotation_.upload(q.rotation_.data(), dim * dim);
+        if (opq_iters == 0) {
+            // no outer iteration: the reference keeps an identity rotation and NO codebooks
+            // (src/opq.rs:122), so quantize returns an empty vector
+            q.d_rotation_.upload(q.rotation_.data(), dim * dim);
+            q.codebooks_ = DeviceBuffer<float>();
+            q.trained_ = false;
+        }
         return q;
     }
 
     // src/opq.rs:222-264
     Vector<f16> quantize(const Vector<float> &vector) const {
         if (vector.len() != dim_) throw VqError::DimensionMismatch(dim_, vector.len());
+        if (!trained_) return Vector<f16>();  // the loop over no codebooks pushes nothing (opq.rs:244-263)
         return quantize_batch(std::vector<Vector<float>>{vector})[0];
     }
 
     std::vector<Vector<f16>> quantize_batch(const Rows &vectors) const {
+        if (!trained_) {
+            vectors.expect_dim(dim_);
+            return std::vector<Vector<f16>>(vectors.size());
+        }
         return unpack_f16(quantize_batch_flat(vectors), vectors.size(), dim_);
     }
 
+    // n x dim f16 bit patterns; empty (n rows of length 0) when fit ran no outer iteration
     std::vector<uint16_t> quantize_batch_flat(const Rows &vectors) const {
         size_t n = vectors.size();
         if (n == 0) return {};
+        if (!trained_) {
+            vectors.expect_dim(dim_);
+            return {};
+        }
         DeviceBuffer<uint8_t> dcodes = encode_device(vectors);
         DeviceBuffer<uint16_t> dout(dev_, n * dim_);
         dev_->check(vq_decode_f16(dev_->ctx(), dcodes.get(), (int64_t)n, (int32_t)m_, (int32_t)sub_dim_,
@@ -529,12 +488,16 @@ public:
     }
 
     std::vector<uint8_t> encode(const Rows &vectors) const {
-        if (vectors.empty()) return {};
+        if (vectors.empty() || !trained_) return {};
         return encode_device(vectors).to_host();
     }
 
-    std::vector<float> codebooks() const { return codebooks_.to_host(); }
+    std::vector<float> codebooks() const { return trained_ ? codebooks_.to_host() : std::vector<float>(); }
     const std::vector<float> &rotation() const { return rotation_; }  // row-major dim x dim
+    bool trained() const { return trained_; }  // false: fit ran with opq_iters == 0
+    size_t m() const { return m_; }
+    size_t k() const { return k_; }
+    size_t sub_dim() const { return sub_dim_; }
 
 private:
     DeviceBuffer<uint8_t> encode_device(const Rows &vectors) const {
@@ -554,6 +517,7 @@ private:
     std::shared_ptr<Device> dev_;
     DeviceBuffer<float> codebooks_, d_rotation_;
     std::vector<float> rotation_;
+    bool trained_ = true;
     size_t sub_dim_ = 0, m_ = 0, k_ = 0, dim_ = 0;
     Distance distance_;
 };

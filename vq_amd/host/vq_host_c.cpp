@@ -132,7 +132,8 @@ int vqh_tsvq_new(const float *x, int64_t n, int64_t dim, int64_t max_depth, int 
 }
 
 // quantize(&Vector<f32>) of whichever quantizer obj holds; len is the vector's own length
-int vqh_quantize(void *obj, const float *v, int64_t len, uint16_t *out) {
+// *out_len (nullable) receives the length of the returned vector
+int vqh_quantize(void *obj, const float *v, int64_t len, uint16_t *out, int64_t *out_len) {
     return guarded([&] {
         Obj *o = (Obj *)obj;
         vq::Vector<float> vec(std::vector<float>(v, v + len));
@@ -144,6 +145,7 @@ int vqh_quantize(void *obj, const float *v, int64_t len, uint16_t *out) {
         default: q = o->tsvq->quantize(vec); break;
         }
         for (size_t t = 0; t < q.len(); ++t) out[t] = q.data[t].bits;
+        if (out_len) *out_len = (int64_t)q.len();
     });
 }
 
@@ -219,6 +221,10 @@ int vqh_info(void *obj, int64_t *info) {
             info[1] = (int64_t)o->pq->m();
             info[2] = (int64_t)o->pq->k();
             info[3] = (int64_t)o->pq->sub_dim();
+        } else if (o->kind == 2) {
+            info[1] = (int64_t)o->opq->m();
+            info[2] = o->opq->trained() ? (int64_t)o->opq->k() : 0;  // no codebooks after opq_iters == 0
+            info[3] = (int64_t)o->opq->sub_dim();
         } else if (o->kind == 3) {
             info[5] = (int64_t)o->rvq->stages();
         } else if (o->kind == 4) {
