@@ -109,7 +109,8 @@ def test_rvq_k1_and_early_training_stop(ctx):
 
 
 # ---- OPQ pieces -------------------------------------------------------------------------------
-@pytest.mark.parametrize("n,dim", [(1000, 10), (4097, 128), (300, 64), (70, 33), (129, 256), (5000, 32)])
+@pytest.mark.parametrize("n,dim", [(1000, 10), (4097, 128), (300, 64), (70, 33), (129, 256), (5000, 32), (2500, 96),
+                                   (3001, 160), (1111, 224), (300001, 64)])
 def test_rotate_matches_matrix_product(ctx, n, dim):
     rng = np.random.default_rng(dim)
     x = rng.standard_normal((n, dim)).astype(F)

@@ -221,51 +221,102 @@ static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__rest
     mfma_bf_prep_block(c, s, j, k, nb, atab, maxc2, mu);
 }
 
-// The reference's argmin of one row's sub-vector (8 floats, the same in every lane) over the k
-// centroids of a block, by the whole wave: lane l takes centroids l, l + 64, ...; the smallest
-// (distance, index) pair wins, which is the reference's strict '<' scan (src/utils.rs:63-70,
-// src/pq.rs:166-174).  A NaN distance is never chosen unless it is centroid 0's, which is never
-// replaced.  Euclidean compares the roots, as the reference does.
+// ---- the exact path of k_assign_mfma_bf ---------------------------------------------------------
+// Undecided rows of one (tile of 32 rows, column block) are decided by the whole wave in the
+// reference's order (src/utils.rs:63-70, src/pq.rs:166-174): lane l owns centroids l, l + 64,
+// l + 128, l + 192 (loaded once per wave and column block, when its first undecided row turns
+// up), computes their distances to the row in sequential f32 order, keeps the first smallest
+// (strict '<' over ascending indices), and the smallest (distance, index) pair over the lanes wins.
+// A NaN distance is never chosen unless it is centroid 0's, which is never replaced.  Euclidean
+// compares the roots, as the reference does.  No LDS and, per batch of up to eight rows, one
+// memory round trip: lane L fetches float L % 8 of the batch's row L / 8, and the row's floats
+// reach every lane as scalars (v_readlane).
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+// (d, i) <- the lexicographically smaller of (d, i) and (od, oi); d holds non-negative float bits
+__device__ __forceinline__ void lexmin(uint32_t &d, uint32_t &i, uint32_t od, uint32_t oi) {
+    const bool take = od < d || (od == d && oi < i);
+    d = take ? od : d;
+    i = take ? oi : i;
+}
+
+struct ExactCentroids {  // this lane's four centroids of the column block
+    float4 c0[4], c1[4];
+};
+__device__ __forceinline__ void exact_load_centroids(ExactCentroids &ec, const float *__restrict__ cb, int k,
+                                                     int lane) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int j = lane + 64 * q;
+        const float4 *cp = reinterpret_cast<const float4 *>(cb + (size_t)(j < k ? j : 0) * 8);
+        ec.c0[q] = cp[0];
+        ec.c1[q] = cp[1];
+    }
+}
+
+// todo: ballot of the lanes (below 32) whose row is undecided; rows = first row of the tile.
+// Returns the codes of those rows in their lanes (other lanes keep `code`).
 template <int METRIC>
-__device__ __forceinline__ int exact_argmin8_wave(const float (&xs)[8], const float *__restrict__ cb, int k,
-                                                  int lane) {
+__device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, const ExactCentroids &ec,
+                                           const float *__restrict__ xblk, int64_t ld, int k, int lane) {
     const float inf = __builtin_inff();
-    float bd = inf, d0 = 0.0f;
-    int bi = 0x7fffffff;
-    for (int j0 = 0; j0 < k; j0 += 256) {
-        // the four loads of a lane are issued together: one memory round trip per 256 centroids
-        float4 c0[4], c1[4];
+    while (todo) {
+        // the batch: up to eight undecided rows; lane L reads float L % 8 of batch row L / 8
+        int src[8];
+        int cnt = 0;
+        int mine = __builtin_amdgcn_readfirstlane(__ffsll(todo) - 1);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int j = j0 + lane + 64 * q;
-            const float4 *cp = reinterpret_cast<const float4 *>(cb + (size_t)(j < k ? j : 0) * 8);
-            c0[q] = cp[0];
-            c1[q] = cp[1];
+        for (int i = 0; i < 8; ++i) {
+            src[i] = todo ? __builtin_amdgcn_readfirstlane(__ffsll(todo) - 1) : src[0];
+            if (todo) ++cnt;
+            todo &= todo - 1;
+            if ((lane >> 3) == i) mine = src[i];
         }
+        const float val = xblk[(int64_t)mine * ld + (lane & 7)];
+        for (int i = 0; i < cnt; ++i) {  // a loop, not unrolled: the path is rare and code size is not free
+            float xs[8];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int j = j0 + lane + 64 * q;
-            const float c[8] = {c0[q].x, c0[q].y, c0[q].z, c0[q].w, c1[q].x, c1[q].y, c1[q].z, c1[q].w};
-            float d = d_sq<8>(xs, c);
-            if constexpr (METRIC == M_EUCLID) d = sqrtf(d);
-            if (j == 0) d0 = d;
-            d = (d == d) ? d : inf;
-            if (j < k && (d < bd || bi == 0x7fffffff)) {  // ascending j inside the lane: strict '<' keeps the first
-                bd = d;
-                bi = j;
+            for (int d = 0; d < 8; ++d)
+                xs[d] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(val), 8 * i + d));
+            float bd = inf, dfirst = 0.0f;
+            uint32_t bi = 0x7fffffffu;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int j = lane + 64 * q;
+                const float c[8] = {ec.c0[q].x, ec.c0[q].y, ec.c0[q].z, ec.c0[q].w,
+                                    ec.c1[q].x, ec.c1[q].y, ec.c1[q].z, ec.c1[q].w};
+                float d = d_sq<8>(xs, c);
+                if constexpr (METRIC == M_EUCLID) d = sqrtf(d);
+                if (q == 0) dfirst = d;
+                d = (d == d) ? d : inf;
+                if (j < k && (d < bd || bi == 0x7fffffffu)) {  // ascending j: strict '<' keeps the first
+                    bd = d;
+                    bi = (uint32_t)j;
+                }
             }
+            // smallest (distance, index) of the wave: four steps inside the rows of 16 lanes, then
+            // the four rows as scalars
+            uint32_t kd = __float_as_uint(bd), ki = bi;
+            lexmin(kd, ki, dpp_u32<0xB1>(kd), dpp_u32<0xB1>(ki));    // quad_perm [1,0,3,2]
+            lexmin(kd, ki, dpp_u32<0x4E>(kd), dpp_u32<0x4E>(ki));    // quad_perm [2,3,0,1]
+            lexmin(kd, ki, dpp_u32<0x141>(kd), dpp_u32<0x141>(ki));  // row_half_mirror
+            lexmin(kd, ki, dpp_u32<0x140>(kd), dpp_u32<0x140>(ki));  // row_mirror
+            uint32_t rd = (uint32_t)__builtin_amdgcn_readlane((int)kd, 0), ri = (uint32_t)__builtin_amdgcn_readlane((int)ki, 0);
+#pragma unroll
+            for (int row = 1; row < 4; ++row)
+                lexmin(rd, ri, (uint32_t)__builtin_amdgcn_readlane((int)kd, 16 * row),
+                       (uint32_t)__builtin_amdgcn_readlane((int)ki, 16 * row));
+            const float d0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(dfirst), 0));
+            const int best = (d0 == d0) ? (int)ri : 0;
+            // src[i] with a loop index: a chain of selects over the eight scalars
+            int who = src[0];
+#pragma unroll
+            for (int u = 1; u < 8; ++u) who = (i == u) ? src[u] : who;
+            if (lane == who) code = best;
         }
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const float od = __shfl_xor(bd, off);
-        const int oi = __shfl_xor(bi, off);
-        const bool take = (od < bd) || (od == bd && oi < bi);
-        bd = take ? od : bd;
-        bi = take ? oi : bi;
-    }
-    d0 = __shfl(d0, 0);
-    return (d0 == d0) ? bi : 0;
+    return code;
 }
 
 // One wave = TILES tiles of 32 rows and SG consecutive column blocks of 8 floats (SG = 4: one
@@ -334,25 +385,27 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
                 const int64_t row = row_base + 32 * t + r;
                 old[t] = a.codes[(size_t)s * a.n + (row < a.n ? row : 0)];
             }
-            float xv[4];  // relative to the block's centre
+            {
+                float xv[4];  // relative to the block's centre
 #pragma unroll
-            for (int u = 0; u < 4; ++u) xv[u] = xall[t][q][u] - lds_mu[q * 8 + 4 * h + u];
-            float p = 0.0f;
+                for (int u = 0; u < 4; ++u) xv[u] = xall[t][q][u] - lds_mu[q * 8 + 4 * h + u];
+                float p = 0.0f;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
-            const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
-            const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
-            const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
-            // this half's share of ||x||^2 in two bf16 parts (it is the same in every score of the
-            // row, so its rounding cancels in their differences), then ones for the parts of ||c||^2
-            const uint32_t p0 = bf16_pack2(p, 0.0f);
-            const float r1 = p - __uint_as_float(p0 << 16);
-            const uint32_t p1 = bf16_pack2(r1, 0.0f);
-            b1[t] = u32x4{h01, h23, l01, l23};
-            b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), 0x3f803f80u};
-            int pa, pb;
-            swap_halves(__float_as_int(p), pa, pb);
-            x2[t] = __int_as_float(pa) + __int_as_float(pb);  // lower half's share + upper half's, in both
+                for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
+                const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
+                const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
+                const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
+                // this half's share of ||x||^2 in two bf16 parts (it is the same in every score of the
+                // row, so its rounding cancels in their differences), then ones for the parts of ||c||^2
+                const uint32_t p0 = bf16_pack2(p, 0.0f);
+                const float r1 = p - __uint_as_float(p0 << 16);
+                const uint32_t p1 = bf16_pack2(r1, 0.0f);
+                b1[t] = u32x4{h01, h23, l01, l23};
+                b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), 0x3f803f80u};
+                int pa, pb;
+                swap_halves(__float_as_int(p), pa, pb);
+                x2[t] = __int_as_float(pa) + __int_as_float(pb);  // lower half's share + upper half's, in both
+            }
             m1[t] = 0x7f800000;  // +inf
             m2[t] = 0x7f800000;
         }
@@ -397,7 +450,8 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
             qa2 = ap[(size_t)(f2 + 1) * 128 + 64];
         }
         const float mc2 = lds_mu[SG * 8 + q];
-        const float *cb_s = a.cb + (size_t)s * a.k * SD;
+        int code[TILES];
+        unsigned long long todo[TILES], any_todo = 0;
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
             // the partner lane (other half) saw the other 16 centroids of every block
@@ -416,31 +470,35 @@ __global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_
             // below 1e-31 the bf16 parts of ||c - mu||^2 may be subnormal, which the matrix cores may
             // flush: up to 3 * 2^-126 lost, more than the margin allows for at such a bound
             sure = sure && (bound < 1e29f) && (bound > 1e-31f) && (s1 < 1e29f);
-            int code = (int)(__float_as_uint(s1) & 0xFFu);
-            // undecided rows: the reference-order argmin, one row at a time by the whole wave
-            unsigned long long todo = __ballot(mine && !sure);
-            n_exact += (uint32_t)__popcll(todo);
-            while (todo) {
-                const int src = __builtin_amdgcn_readfirstlane(__ffsll(todo) - 1);
-                // the row's 8 floats, read again (same address in every lane) rather than kept in
-                // registers through the scoring of every block for this rare path
-                const float4 *xp = reinterpret_cast<const float4 *>(a.x + (row_base + 32 * t + src) * a.ld + (int64_t)s * SD);
-                const float4 xa = xp[0], xb = xp[1];
-                const float xs[SD] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
-                const int best = exact_argmin8_wave<METRIC>(xs, cb_s, a.k, lane);
-                if (lane == src) code = best;
-                todo &= todo - 1;
+            code[t] = (int)(__float_as_uint(s1) & 0xFFu);
+            todo[t] = __ballot(mine && !sure);
+            any_todo |= todo[t];
+        }
+        if (any_todo) {  // the same in every lane: the reference-order argmin of the undecided rows
+            ExactCentroids ec;
+            exact_load_centroids(ec, a.cb + (size_t)s * a.k * SD, a.k, lane);
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) {
+                n_exact += (uint32_t)__popcll(todo[t]);
+                if (todo[t])
+                    code[t] = exact_rows8<METRIC>(todo[t], code[t], ec, a.x + (row_base + 32 * t) * a.ld + (int64_t)s * SD,
+                                                  a.ld, a.k, lane);
             }
+        }
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int64_t row = row_base + 32 * t + r;
+            const bool mine = h == 0 && row < a.n;
             if (mine) {
                 if constexpr (LBG) {
-                    if (old[t] != (uint8_t)code) {
-                        a.codes[(size_t)s * a.n + row] = (uint8_t)code;
+                    if (old[t] != (uint8_t)code[t]) {
+                        a.codes[(size_t)s * a.n + row] = (uint8_t)code[t];
                         chg |= 1u << q;
                     }
                 } else if (SG == 4 || SG == 2) {
-                    cw[t] |= (uint32_t)code << (8 * q);
+                    cw[t] |= (uint32_t)code[t] << (8 * q);
                 } else {
-                    a.codes[row * m + s] = (uint8_t)code;
+                    a.codes[row * m + s] = (uint8_t)code[t];
                 }
             }
         }

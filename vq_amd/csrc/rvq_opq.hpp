@@ -335,97 +335,257 @@ static __global__ void __launch_bounds__(256) k_crosscov_reduce(const double *__
 
 // ---- rotation on the matrix cores ------------------------------------------------------------
 // y[i][a] = sum_b R[a][b] * x[i][b] for dim a multiple of 32, at most 256: D = R * X^T in tiles of
-// 32 output dimensions x 32 rows with v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate).
+// 32 output dimensions x 32 rows on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16, 16x the rate
+// of the fp32 instruction).  Every fp32 number is the exact sum of three bf16 numbers
+// (v = h + m + l, round to nearest even three times: 3 x 8 significant bits), and the six
+// products hh, hm, mh, mm, hl, lh are accumulated in fp32; the three left out (ml, lm, ll) are
+// below 2^-23 of |R||x| each, so the result is as good as an fp32 fused-multiply-add chain, and a
+// rotation by the identity returns the rows bit for bit.  With the matrix time at 0.08 ms for
+// 1M x 128 the kernel is bound by the 1 GB it moves.
 namespace vq {
 
 typedef float rot_floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 rot_bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t rot_u32x4 __attribute__((ext_vector_type(4)));
 
-// rtab[kc][b][lane][u] = R[32 b + lane % 32][8 kc + 4 (lane / 32) + u]   (MFMA A-operand order)
+// v -> (h, m, l) bf16 bit patterns, h + m + l == v
+__device__ __forceinline__ void rot_split3(float v, uint32_t &h, uint32_t &m, uint32_t &l) {
+    auto rne = [](float f) -> uint32_t {
+        uint32_t u = __float_as_uint(f);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return u >> 16;
+    };
+    h = rne(v);
+    const float r1 = v - __uint_as_float(h << 16);
+    m = rne(r1);
+    const float r2 = r1 - __uint_as_float(m << 16);
+    l = rne(r2);
+}
+
+// two floats -> their (h, m, l) parts as packed bf16 pairs (low half = first), by the hardware's
+// round-to-nearest-even conversion
+typedef float rot_floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 rot_bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t rot_pack2(float a, float b) {
+    rot_floatx2 f = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, rot_bf16x2));
+}
+__device__ __forceinline__ void rot_split3_pair(float a, float b, uint32_t &h, uint32_t &m, uint32_t &l) {
+    h = rot_pack2(a, b);
+    const float ra = a - __uint_as_float(h << 16), rb = b - __uint_as_float(h & 0xffff0000u);
+    m = rot_pack2(ra, rb);
+    l = rot_pack2(ra - __uint_as_float(m << 16), rb - __uint_as_float(m & 0xffff0000u));
+}
+
+// rtab[kc][b][e][lane] (16 bytes each), lane = 32 hh + o: the parts of R[32 b + o][8 kc + 4 hh + u],
+// u = 0..3:  e = 0: {h01, h23, m01, m23}   e = 1: {h01, h23, l01, l23}
 static __global__ void __launch_bounds__(256) k_rotate_prep(const float *__restrict__ R, int dim,
-                                                            float *__restrict__ rtab) {
+                                                            rot_u32x4 *__restrict__ rtab) {
     const int nb = dim / 32, nkc = dim / 8;
-    const int total = nkc * nb * 64 * 4;
+    const int total = nkc * nb * 64;
     for (int e = blockIdx.x * 256 + threadIdx.x; e < total; e += gridDim.x * 256) {
-        const int u = e % 4, lane = (e / 4) % 64, b = (e / 256) % nb, kc = e / (256 * nb);
-        rtab[e] = R[(size_t)(32 * b + lane % 32) * dim + 8 * kc + 4 * (lane / 32) + u];
+        const int lane = e % 64, b = (e / 64) % nb, kc = e / (64 * nb);
+        const float *src = R + (size_t)(32 * b + lane % 32) * dim + 8 * kc + 4 * (lane / 32);
+        uint32_t h[4], m[4], l[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) rot_split3(src[u], h[u], m[u], l[u]);
+        const uint32_t h01 = h[0] | (h[1] << 16), h23 = h[2] | (h[3] << 16);
+        rot_u32x4 *dst = rtab + ((size_t)kc * nb + b) * 128;
+        dst[lane] = rot_u32x4{h01, h23, m[0] | (m[1] << 16), m[2] | (m[3] << 16)};
+        dst[64 + lane] = rot_u32x4{h01, h23, l[0] | (l[1] << 16), l[2] | (l[3] << 16)};
     }
 }
 
-// grid ceil(n/128); 256 threads = 4 waves, one tile of 32 rows per wave.
+// grid ceil(n / (128 TILES)); 256 threads = 4 waves, TILES tiles of 32 rows per wave, NB = dim / 32.
+// The operands of R for a chunk of 8 dimensions (NB x 2 KB) are staged in LDS by the workgroup,
+// double-buffered behind a barrier that waits for LDS only; a lane's 16 bytes of a row and chunk
+// are fetched kRotAhead chunks ahead and stay in flight across the barriers.
+template <int NB, int TILES>
 static __global__ void __launch_bounds__(256) k_rotate_mfma(const float *__restrict__ x, int64_t n, int64_t ld,
-                                                            int dim, const float *__restrict__ rtab,
+                                                            const rot_u32x4 *__restrict__ rtab,
                                                             float *__restrict__ y) {
-    constexpr int NBMAX = 8;
-    __shared__ float4 lds_a[2][NBMAX * 64];
+    constexpr int DIM = 32 * NB, NKC = DIM / 8, CHUNK = NB * 128;  // u32x4 entries per chunk
+    __shared__ rot_u32x4 lds_a[2][CHUNK];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int nb = dim / 32, nkc = dim / 8;
-    const int64_t row = ((int64_t)blockIdx.x * 4 + wave) * 32 + r;
-    const bool valid = row < n;
-    const float4 *ag = reinterpret_cast<const float4 *>(rtab);
-    const int chunk4 = nb * 64;
-    for (int i = threadIdx.x; i < chunk4; i += 256) lds_a[0][i] = ag[i];
+    int64_t row[TILES];
+    const float *xr[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        row[t] = (((int64_t)blockIdx.x * 4 + wave) * TILES + t) * 32 + r;
+        xr[t] = x + (row[t] < n ? row[t] : 0) * ld + 4 * h;  // a row past the end reads row 0, never stored
+    }
+    for (int i = threadIdx.x; i < CHUNK; i += 256) lds_a[0][i] = rtab[i];
     __syncthreads();
-    rot_floatx16 acc[NBMAX];
+    rot_floatx16 acc[TILES][NB];
 #pragma unroll
-    for (int b = 0; b < NBMAX; ++b)
+    for (int t = 0; t < TILES; ++t)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[b][v] = 0.0f;
-    // The lane's pieces of its row are fetched kRotAhead chunks ahead (unconditional loads: a row
-    // past the end reads row 0 and is never stored); the barrier of a chunk waits for LDS only, so
-    // they stay in flight across it.  dim is a multiple of 32: the chunks come in fours.
-    constexpr int kRotAhead = 4;
-    const float *xr = x + (valid ? row : 0) * ld + 4 * h;
-    float4 xq[kRotAhead];
+        for (int b = 0; b < NB; ++b)
 #pragma unroll
-    for (int u = 0; u < kRotAhead; ++u) xq[u] = *reinterpret_cast<const float4 *>(xr + (u < nkc ? u : nkc - 1) * 8);
-    for (int kc0 = 0; kc0 < nkc; kc0 += kRotAhead) {
+            for (int v = 0; v < 16; ++v) acc[t][b][v] = 0.0f;
+    constexpr int kRotAhead = 4;  // NKC is a multiple of 4
+    float4 xq[TILES][kRotAhead];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t)
+#pragma unroll
+        for (int u = 0; u < kRotAhead; ++u) xq[t][u] = *reinterpret_cast<const float4 *>(xr[t] + u * 8);
+    for (int kc0 = 0; kc0 < NKC; kc0 += kRotAhead) {
 #pragma unroll
         for (int u = 0; u < kRotAhead; ++u) {
             const int kc = kc0 + u;
             const int cur = kc & 1;
-            float4 pre[2];
-            const bool more = kc + 1 < nkc;
+            constexpr int PER = (CHUNK + 255) / 256;
+            rot_u32x4 pre[PER];
+            const bool more = kc + 1 < NKC;
             if (more) {
 #pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    int i = threadIdx.x + 256 * q;
-                    if (i < chunk4) pre[q] = ag[(size_t)(kc + 1) * chunk4 + i];
+                for (int q = 0; q < PER; ++q) {
+                    const int i = threadIdx.x + 256 * q;
+                    if (i < CHUNK) pre[q] = rtab[(size_t)(kc + 1) * CHUNK + i];
                 }
             }
-            const float4 xv = xq[u];
-            const int nx = kc + kRotAhead < nkc ? kc + kRotAhead : nkc - 1;
-            xq[u] = *reinterpret_cast<const float4 *>(xr + nx * 8);
+            rot_u32x4 b1[TILES], b2[TILES], b3[TILES];
 #pragma unroll
-            for (int b = 0; b < NBMAX; ++b) {
-                if (b < nb) {
-                    const float4 av = lds_a[cur][b * 64 + lane];
-                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.x, xv.x, acc[b], 0, 0, 0);
-                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.y, xv.y, acc[b], 0, 0, 0);
-                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.z, xv.z, acc[b], 0, 0, 0);
-                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(av.w, xv.w, acc[b], 0, 0, 0);
+            for (int t = 0; t < TILES; ++t) {
+                const float4 xv = xq[t][u];
+                const int nx = kc + kRotAhead < NKC ? kc + kRotAhead : NKC - 1;
+                xq[t][u] = *reinterpret_cast<const float4 *>(xr[t] + nx * 8);
+                uint32_t h01, m01, l01, h23, m23, l23;
+                rot_split3_pair(xv.x, xv.y, h01, m01, l01);
+                rot_split3_pair(xv.z, xv.w, h23, m23, l23);
+                b1[t] = rot_u32x4{h01, h23, h01, h23};
+                b2[t] = rot_u32x4{m01, m23, m01, m23};
+                b3[t] = rot_u32x4{l01, l23, h01, h23};
+            }
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const rot_u32x4 a12 = lds_a[cur][b * 128 + lane];       // {Rh, Rm}
+                const rot_u32x4 a3 = lds_a[cur][b * 128 + 64 + lane];   // {Rh, Rl}
+#pragma unroll
+                for (int t = 0; t < TILES; ++t) {
+                    acc[t][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(rot_bf16x8, a12), __builtin_bit_cast(rot_bf16x8, b1[t]), acc[t][b], 0, 0, 0);
+                    acc[t][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(rot_bf16x8, a12), __builtin_bit_cast(rot_bf16x8, b2[t]), acc[t][b], 0, 0, 0);
+                    acc[t][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(rot_bf16x8, a3), __builtin_bit_cast(rot_bf16x8, b3[t]), acc[t][b], 0, 0, 0);
                 }
             }
             if (more) {
 #pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    int i = threadIdx.x + 256 * q;
-                    if (i < chunk4) lds_a[cur ^ 1][i] = pre[q];
+                for (int q = 0; q < PER; ++q) {
+                    const int i = threadIdx.x + 256 * q;
+                    if (i < CHUNK) lds_a[cur ^ 1][i] = pre[q];
                 }
             }
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
     }
-    if (!valid) return;
     // register v of block b holds output dimension 32 b + 8 (v / 4) + 4 h + v % 4 of this lane's row
-    float *yr = y + row * dim + 4 * h;
 #pragma unroll
-    for (int b = 0; b < NBMAX; ++b) {
-        if (b < nb) {
+    for (int t = 0; t < TILES; ++t) {
+        if (row[t] >= n) continue;
+        float *yr = y + row[t] * DIM + 4 * h;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int g = 0; g < 4; ++g)
                 *reinterpret_cast<float4 *>(yr + 32 * b + 8 * g) =
-                    make_float4(acc[b][4 * g], acc[b][4 * g + 1], acc[b][4 * g + 2], acc[b][4 * g + 3]);
+                    make_float4(acc[t][b][4 * g], acc[t][b][4 * g + 1], acc[t][b][4 * g + 2], acc[t][b][4 * g + 3]);
+    }
+}
+
+// The same product for dim <= 128 with the whole operand table of R resident in LDS (NB * 32 KB):
+// one workgroup of 8 waves per compute unit stages it once and then walks over the row tiles, so
+// the steady state has no barrier, and a wave's row fetches run kRotAhead chunks ahead straight
+// across tile boundaries while the finished tile's 32 KB of output is still being written.
+template <int NB, int TILES>
+static __global__ void __launch_bounds__(512) k_rotate_mfma_resident(const float *__restrict__ x, int64_t n,
+                                                                     int64_t ld, const rot_u32x4 *__restrict__ rtab,
+                                                                     float *__restrict__ y) {
+    constexpr int DIM = 32 * NB, NKC = DIM / 8, CHUNK = NB * 128;
+    extern __shared__ __attribute__((aligned(16))) rot_u32x4 lds_r[];  // [NKC][NB][2][64]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    for (int i = threadIdx.x; i < NKC * CHUNK; i += 512) lds_r[i] = rtab[i];
+    __syncthreads();
+    const int64_t groups = (n + 32 * TILES - 1) / (32 * TILES);  // groups of TILES row tiles
+    const int64_t stride = (int64_t)gridDim.x * 8;
+    int64_t g = (int64_t)blockIdx.x * 8 + wave;
+    if (g >= groups) return;
+    auto row_ptr = [&](int64_t grp, int t) {
+        const int64_t row = (grp * TILES + t) * 32 + r;
+        return x + (row < n ? row : 0) * ld + 4 * h;  // a row past the end reads row 0, never stored
+    };
+    constexpr int kRotAhead = 4;  // NKC is a multiple of 4
+    const float *xr[TILES];
+    float4 xq[TILES][kRotAhead];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        xr[t] = row_ptr(g, t);
+#pragma unroll
+        for (int u = 0; u < kRotAhead; ++u) xq[t][u] = *reinterpret_cast<const float4 *>(xr[t] + u * 8);
+    }
+    for (; g < groups; g += stride) {
+        const int64_t gn = g + stride < groups ? g + stride : g;  // the next group (or this one again: unused loads)
+        const float *xn[TILES];
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) xn[t] = row_ptr(gn, t);
+        rot_floatx16 acc[TILES][NB];
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[t][b][v] = 0.0f;
+        for (int kc0 = 0; kc0 < NKC; kc0 += kRotAhead) {
+#pragma unroll
+            for (int u = 0; u < kRotAhead; ++u) {
+                const int kc = kc0 + u;
+                rot_u32x4 b1[TILES], b2[TILES], b3[TILES];
+#pragma unroll
+                for (int t = 0; t < TILES; ++t) {
+                    const float4 xv = xq[t][u];
+                    const float *src = kc + kRotAhead < NKC ? xr[t] + (kc + kRotAhead) * 8 : xn[t] + (kc + kRotAhead - NKC) * 8;
+                    xq[t][u] = *reinterpret_cast<const float4 *>(src);
+                    uint32_t h01, m01, l01, h23, m23, l23;
+                    rot_split3_pair(xv.x, xv.y, h01, m01, l01);
+                    rot_split3_pair(xv.z, xv.w, h23, m23, l23);
+                    b1[t] = rot_u32x4{h01, h23, h01, h23};
+                    b2[t] = rot_u32x4{m01, m23, m01, m23};
+                    b3[t] = rot_u32x4{l01, l23, h01, h23};
+                }
+#pragma unroll
+                for (int b = 0; b < NB; ++b) {
+                    const rot_u32x4 a12 = lds_r[(size_t)kc * CHUNK + b * 128 + lane];      // {Rh, Rm}
+                    const rot_u32x4 a3 = lds_r[(size_t)kc * CHUNK + b * 128 + 64 + lane];  // {Rh, Rl}
+#pragma unroll
+                    for (int t = 0; t < TILES; ++t) {
+                        acc[t][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(rot_bf16x8, a12), __builtin_bit_cast(rot_bf16x8, b1[t]), acc[t][b], 0, 0, 0);
+                        acc[t][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(rot_bf16x8, a12), __builtin_bit_cast(rot_bf16x8, b2[t]), acc[t][b], 0, 0, 0);
+                        acc[t][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(rot_bf16x8, a3), __builtin_bit_cast(rot_bf16x8, b3[t]), acc[t][b], 0, 0, 0);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int64_t row = (g * TILES + t) * 32 + r;
+            if (row < n) {
+                float *yr = y + row * DIM + 4 * h;
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq)
+                        *reinterpret_cast<float4 *>(yr + 32 * b + 8 * gq) = make_float4(
+                            acc[t][b][4 * gq], acc[t][b][4 * gq + 1], acc[t][b][4 * gq + 2], acc[t][b][4 * gq + 3]);
+            }
+            xr[t] = xn[t];
         }
     }
 }

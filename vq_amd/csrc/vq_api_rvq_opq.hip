@@ -121,11 +121,40 @@ int32_t vq_rotate(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t 
     // matrix-core kernel: dim a multiple of 32 up to 256, rows and output 16-byte aligned
     if (dim % 32 == 0 && dim <= 256 && ld % 4 == 0 &&
         ((reinterpret_cast<uintptr_t>(d_x) | reinterpret_cast<uintptr_t>(d_y)) & 15) == 0) {
-        VQ_TRY(ensure(ctx, ctx->tmp_f, sizeof(float) * (size_t)dim * dim));
-        hipLaunchKernelGGL(vq::k_rotate_prep, dim3(cdiv((int64_t)dim * dim, 256)), dim3(256), 0, ctx->stream,
-                           d_R, dim, (float *)ctx->tmp_f.p);
-        hipLaunchKernelGGL(vq::k_rotate_mfma, dim3(cdiv(n, 128)), dim3(256), 0, ctx->stream, d_x, n, ld, dim,
-                           (const float *)ctx->tmp_f.p, d_y);
+        // operand table: 32 bytes per (output dimension, 4 input dimensions)
+        VQ_TRY(ensure(ctx, ctx->tmp_f, 8 * (size_t)dim * dim));
+        vq::rot_u32x4 *rtab = (vq::rot_u32x4 *)ctx->tmp_f.p;
+        hipLaunchKernelGGL(vq::k_rotate_prep, dim3(cdiv((int64_t)dim * dim / 4, 256)), dim3(256), 0, ctx->stream,
+                           d_R, dim, rtab);
+        // dim <= 128: the table (dim / 32 x 32 KB) stays in LDS, one workgroup per compute unit
+#define ROTATE_RESIDENT(NB, TILES)                                                                              \
+    do {                                                                                                        \
+        const size_t lds = (size_t)NB * 32 * 1024;                                                              \
+        auto kern = vq::k_rotate_mfma_resident<NB, TILES>;                                                      \
+        VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                   \
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                 \
+        hipDeviceProp_t prop;                                                                                   \
+        VQ_HIP(ctx, hipGetDeviceProperties(&prop, ctx->device));                                                \
+        const int64_t groups = cdiv(n, 32 * TILES);                                                             \
+        const unsigned wgs = (unsigned)std::min<int64_t>(prop.multiProcessorCount, cdiv(groups, 8));            \
+        hipLaunchKernelGGL(kern, dim3(wgs), dim3(512), lds, ctx->stream, d_x, n, ld,                            \
+                           (const vq::rot_u32x4 *)rtab, d_y);                                                   \
+    } while (0)
+#define ROTATE(NB, TILES)                                                                                    \
+    hipLaunchKernelGGL((vq::k_rotate_mfma<NB, TILES>), dim3(cdiv(n, 128 * TILES)), dim3(256), 0, ctx->stream, \
+                       d_x, n, ld, (const vq::rot_u32x4 *)rtab, d_y)
+        switch (dim / 32) {
+        case 1: ROTATE_RESIDENT(1, 2); break;
+        case 2: ROTATE_RESIDENT(2, 2); break;
+        case 3: ROTATE_RESIDENT(3, 2); break;
+        case 4: ROTATE_RESIDENT(4, 2); break;
+        case 5: ROTATE(5, 1); break;
+        case 6: ROTATE(6, 1); break;
+        case 7: ROTATE(7, 1); break;
+        default: ROTATE(8, 1); break;
+        }
+#undef ROTATE
+#undef ROTATE_RESIDENT
         VQ_HIP(ctx, hipGetLastError());
         return VQ_OK;
     }
