@@ -273,7 +273,7 @@ static __global__ void __launch_bounds__(256) k_crosscov_partial(const float *__
 // The same partial sums on the f64 matrix cores (v_mfma_f64_16x16x4_f64) for dim a multiple of 16:
 // a launch covers the output columns [b0 + 128 z, b0 + 128 z + 16 NT) for z = blockIdx.z and every
 // output row.
-// One wave owns the 16 output rows [16 ti, 16 ti + 16) of a chunk and NT column tiles; a
+// One wave owns the 32 output rows [16 ti, 16 ti + 32) of a chunk and NT column tiles; a
 // contraction step takes 4 rows: lane l supplies y[row + l/16][16 ti + l%16] and, per column
 // tile, x[row + l/16][16 tj + l%16], converted to f64 (the products are then exact).  The result
 // register v of lane l is A[16 ti + 4 v + l/16][16 tj + l%16].  Fixed order: deterministic.
@@ -283,52 +283,93 @@ template <int NT>
 __global__ void __launch_bounds__(256) k_crosscov_mfma(const float *__restrict__ yr, const float *__restrict__ x,
                                                        int64_t n, int DIM, int b0, int64_t rows_per_chunk,
                                                        double *__restrict__ part) {
+    // a wave owns TWO tiles of 16 output rows (32 dimensions of y), so every operand of x it
+    // fetches feeds two matrix instructions
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int ti = blockIdx.y * 4 + w;
-    if (ti >= DIM / 16) return;
+    const int ti = 2 * (blockIdx.y * 4 + w), nti = DIM / 16;
+    if (ti >= nti) return;
+    const bool two = ti + 1 < nti;
     b0 += 128 * blockIdx.z;
     const int kk = lane >> 4, jj = lane & 15;
     const int64_t lo = (int64_t)blockIdx.x * rows_per_chunk;
     const int64_t hi = lo + rows_per_chunk < n ? lo + rows_per_chunk : n;
-    doublex4 acc[NT];
+    doublex4 acc0[NT], acc1[NT];
 #pragma unroll
-    for (int tj = 0; tj < NT; ++tj) acc[tj] = doublex4{0.0, 0.0, 0.0, 0.0};
-    const float *yp = yr + (lo + kk) * DIM + 16 * ti + jj;
-    const float *xp = x + (lo + kk) * DIM + b0 + jj;
-    float a = 0.0f, b[NT];
-    bool valid = lo + kk < hi;
-    a = valid ? *yp : 0.0f;
+    for (int tj = 0; tj < NT; ++tj) {
+        acc0[tj] = doublex4{0.0, 0.0, 0.0, 0.0};
+        acc1[tj] = doublex4{0.0, 0.0, 0.0, 0.0};
+    }
+    // Operands are fetched kAhead steps (of 4 rows) ahead.  The loads are unconditional — an
+    // address past the chunk is clamped to the lane's first row and the value zeroed afterwards —
+    // because a load under a branch makes the compiler wait for every load in flight at its use.
+    constexpr int kAhead = 4;
+    const int64_t base_row = lo + (lo + kk < hi ? kk : 0);  // the chunk is not empty: lo < hi
+    const float *yp = yr + base_row * (int64_t)DIM + 16 * ti + jj;
+    const float *yp1 = two ? yp + 16 : yp;
+    const float *xp = x + base_row * (int64_t)DIM + b0 + jj;
+    float a0[kAhead], a1[kAhead], b[kAhead][NT];
+    bool ok[kAhead];
 #pragma unroll
-    for (int tj = 0; tj < NT; ++tj) b[tj] = valid ? xp[16 * tj] : 0.0f;
-    for (int64_t r = lo; r < hi; r += 4) {
-        const float ac = a;
-        float bc[NT];
+    for (int u = 0; u < kAhead; ++u) {
+        ok[u] = lo + 4 * u + kk < hi;
+        const int64_t off = ok[u] ? (int64_t)(4 * u) * DIM : 0;
+        a0[u] = yp[off];
+        a1[u] = yp1[off];
 #pragma unroll
-        for (int tj = 0; tj < NT; ++tj) bc[tj] = b[tj];
-        yp += 4 * DIM;
-        xp += 4 * DIM;
-        valid = r + 4 + kk < hi;  // the next step's operands are fetched while this one is multiplied
-        a = valid ? *yp : 0.0f;
+        for (int tj = 0; tj < NT; ++tj) b[u][tj] = xp[off + 16 * tj];
+    }
+    for (int64_t r = lo; r < hi; r += 4 * kAhead) {
 #pragma unroll
-        for (int tj = 0; tj < NT; ++tj) b[tj] = valid ? xp[16 * tj] : 0.0f;
+        for (int u = 0; u < kAhead; ++u) {
+            const double ac0 = ok[u] ? (double)a0[u] : 0.0, ac1 = (ok[u] && two) ? (double)a1[u] : 0.0;
+            double bc[NT];
 #pragma unroll
-        for (int tj = 0; tj < NT; ++tj)
-            acc[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64((double)ac, (double)bc[tj], acc[tj], 0, 0, 0);
+            for (int tj = 0; tj < NT; ++tj) bc[tj] = ok[u] ? (double)b[u][tj] : 0.0;
+            const int64_t rn = r + 4 * (u + kAhead);  // first row of the step this slot holds next
+            ok[u] = rn + kk < hi;
+            const int64_t off = ok[u] ? (rn - lo) * (int64_t)DIM : 0;
+            a0[u] = yp[off];
+            a1[u] = yp1[off];
+#pragma unroll
+            for (int tj = 0; tj < NT; ++tj) b[u][tj] = xp[off + 16 * tj];
+            if (r + 4 * u < hi) {  // the same in every lane
+#pragma unroll
+                for (int tj = 0; tj < NT; ++tj) {
+                    acc0[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(ac0, bc[tj], acc0[tj], 0, 0, 0);
+                    acc1[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(ac1, bc[tj], acc1[tj], 0, 0, 0);
+                }
+            }
+        }
     }
     double *out = part + (size_t)blockIdx.x * DIM * DIM;
 #pragma unroll
     for (int tj = 0; tj < NT; ++tj)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) out[(size_t)(16 * ti + 4 * v + kk) * DIM + b0 + 16 * tj + jj] = acc[tj][v];
+        for (int v = 0; v < 4; ++v) {
+            out[(size_t)(16 * ti + 4 * v + kk) * DIM + b0 + 16 * tj + jj] = acc0[tj][v];
+            if (two) out[(size_t)(16 * ti + 16 + 4 * v + kk) * DIM + b0 + 16 * tj + jj] = acc1[tj][v];
+        }
 }
 
+// out[e] = sum over the chunks [g * per_group, (g + 1) * per_group) of part[c][e], c ascending, for
+// group g = blockIdx.y: called once over the chunks (out = one sum per group) and once more over
+// those sums, so the order of the additions is fixed (groups of chunks in chunk order, then the
+// groups in group order) whatever the GPU does.  Sixteen loads in flight per thread.
 static __global__ void __launch_bounds__(256) k_crosscov_reduce(const double *__restrict__ part, int chunks,
-                                                         int total, double *__restrict__ out) {
-    int e = blockIdx.x * 256 + threadIdx.x;
+                                                         int per_group, int total, double *__restrict__ out) {
+    const int e = blockIdx.x * 256 + threadIdx.x;
     if (e >= total) return;
+    const int c0 = blockIdx.y * per_group, c1 = min(chunks, c0 + per_group);
     double s = 0.0;
-    for (int c = 0; c < chunks; ++c) s += part[(size_t)c * total + e];
-    out[e] = s;
+    for (int c = c0; c < c1; c += 16) {
+        double v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = part[(size_t)min(c + u, c1 - 1) * total + e];
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            if (c + u < c1) s += v[u];
+    }
+    out[(size_t)blockIdx.y * total + e] = s;
 }
 
 }  // namespace vq

@@ -338,6 +338,59 @@ __global__ void __launch_bounds__(256) k_decode_vec4(const uint8_t *__restrict__
     }
 }
 
+// The same gather with the whole codebook table resident in LDS (up to 128 KB, one workgroup of
+// 1024 threads per compute unit walking over the output): a thread makes one 16-byte piece of the
+// output per step — eight f16 values (F16; sub_dim a multiple of 8) or four f32 values (sub_dim a
+// multiple of 4) — so a wave's stores are 1 KB of consecutive bytes, its code reads consecutive
+// bytes, and the centroid comes from LDS instead of a scattered read of the 128 KB table through
+// the vector cache.  Four pieces per thread are in flight.
+template <bool F16>
+__global__ void __launch_bounds__(1024) k_decode_resident(const uint8_t *__restrict__ codes, int64_t n, int m, int sd,
+                                                          int k, const float *__restrict__ cb,
+                                                          vq::u32x4 *__restrict__ out) {
+    extern __shared__ __attribute__((aligned(16))) vq::u32x4 tab[];  // [m * k][pieces of a centroid]
+    const int pieces = F16 ? sd / 8 : sd / 4;                        // 16-byte output pieces per centroid
+    const int entries = m * k * pieces;
+    for (int e = threadIdx.x; e < entries; e += 1024) {
+        if constexpr (F16) {
+            const float4 a = reinterpret_cast<const float4 *>(cb)[2 * (size_t)e];
+            const float4 b = reinterpret_cast<const float4 *>(cb)[2 * (size_t)e + 1];
+            auto two = [](float lo, float hi) {
+                return (uint32_t)__half_as_ushort(__float2half_rn(lo)) | ((uint32_t)__half_as_ushort(__float2half_rn(hi)) << 16);
+            };
+            tab[e] = vq::u32x4{two(a.x, a.y), two(a.z, a.w), two(b.x, b.y), two(b.z, b.w)};
+        } else {
+            tab[e] = reinterpret_cast<const vq::u32x4 *>(cb)[e];
+        }
+    }
+    __syncthreads();
+    const int64_t total = n * m * pieces;
+    const int64_t stride = (int64_t)gridDim.x * 1024;
+    const int per_row = m * pieces;
+    constexpr int U = F16 ? 4 : 8;  // pieces in flight per thread
+    for (int64_t i0 = (int64_t)blockIdx.x * 1024 + threadIdx.x; i0 < total; i0 += U * stride) {
+        uint32_t code[U];
+        int64_t idx[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            idx[u] = i0 + u * stride;
+            const int64_t ic = idx[u] < total ? idx[u] : i0;
+            code[u] = codes[ic / pieces];  // codes are n x m row-major: piece ic belongs to (row, block) ic / pieces
+        }
+        vq::u32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t ic = idx[u] < total ? idx[u] : i0;
+            const int within = (int)(ic % per_row);  // (block, piece) of the row
+            const int s = within / pieces, pc = within % pieces;
+            v[u] = tab[(s * k + (int)code[u]) * pieces + pc];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (idx[u] < total) out[idx[u]] = v[u];
+    }
+}
+
 __global__ void k_decode_f32(const uint8_t *__restrict__ codes, int64_t n, int m, int sd, int k,
                              const float *__restrict__ cb, float *__restrict__ out) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -357,6 +410,29 @@ __global__ void __launch_bounds__(256) k_copy_f32(const float4 *__restrict__ src
     int64_t stride = (int64_t)gridDim.x * 256;
     for (; i < n4; i += stride) dst[i] = src[i];
     if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x];
+}
+
+// LDS-resident decode where the table fits and the output is large enough to pay for staging it.
+template <bool F16>
+int32_t launch_decode_resident(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int m, int sd, int k,
+                               const float *d_codebooks, void *d_out, bool *done) {
+    *done = false;
+    const size_t lds = (size_t)m * k * sd * (F16 ? 2 : 4);
+    if (sd % (F16 ? 8 : 4) != 0 || lds > 128 * 1024 || n * m < (1 << 16)) return VQ_OK;
+    if ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) return VQ_OK;
+    auto kern = k_decode_resident<F16>;
+    VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds));
+    hipDeviceProp_t prop;
+    VQ_HIP(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    const int64_t pieces = (int64_t)n * m * (F16 ? sd / 8 : sd / 4);
+    const unsigned per_cu = lds <= 64 * 1024 ? 2u : 1u;
+    const unsigned wgs = (unsigned)std::min<int64_t>((int64_t)prop.multiProcessorCount * per_cu, cdiv(pieces, 4096));
+    hipLaunchKernelGGL(kern, dim3(wgs), dim3(1024), lds, ctx->stream, d_codes, n, m, sd, k, d_codebooks,
+                       (vq::u32x4 *)d_out);
+    VQ_HIP(ctx, hipGetLastError());
+    *done = true;
+    return VQ_OK;
 }
 
 }  // namespace
@@ -890,6 +966,9 @@ int32_t vq_decode_f16(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m,
     if (!d_codes || !d_codebooks || !d_out || n < 0 || m <= 0 || sd <= 0 || k <= 0 || k > vq::kMaxK)
         return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
     VQ_HIP(ctx, hipSetDevice(ctx->device));
+    bool done = false;
+    VQ_TRY(launch_decode_resident<true>(ctx, d_codes, n, m, sd, k, d_codebooks, d_out, &done));
+    if (done) return VQ_OK;
     if (sd % 4 == 0 && ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) == 0)
         hipLaunchKernelGGL(k_decode_vec4<true>, dim3(cdiv(n * m * sd / 4, 256)), dim3(256), 0, ctx->stream, d_codes,
                            n, m, sd, k, d_codebooks, (void *)d_out);
@@ -907,6 +986,9 @@ int32_t vq_decode_f32(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m,
     if (!d_codes || !d_codebooks || !d_out || n < 0 || m <= 0 || sd <= 0 || k <= 0 || k > vq::kMaxK)
         return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
     VQ_HIP(ctx, hipSetDevice(ctx->device));
+    bool done = false;
+    VQ_TRY(launch_decode_resident<false>(ctx, d_codes, n, m, sd, k, d_codebooks, d_out, &done));
+    if (done) return VQ_OK;
     if (sd % 4 == 0 && ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) == 0)
         hipLaunchKernelGGL(k_decode_vec4<false>, dim3(cdiv(n * m * sd / 4, 256)), dim3(256), 0, ctx->stream, d_codes,
                            n, m, sd, k, d_codebooks, (void *)d_out);

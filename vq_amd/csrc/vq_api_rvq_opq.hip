@@ -183,11 +183,12 @@ int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n,
     const int total = dim * dim;
     VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(double) * (size_t)chunks * total));
     VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * (size_t)total));
+    VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(double) * (size_t)total * ((chunks + 31) / 32)));
     if (dim % 16 == 0) {
         const int nt_all = dim / 16, full = dim / 128, rest = nt_all % 8;
         double *part = (double *)ctx->tmp_a.p;
 #define CROSSCOV(NT, B0, Z)                                                                                 \
-    hipLaunchKernelGGL((vq::k_crosscov_mfma<NT>), dim3(chunks, (nt_all + 3) / 4, Z), dim3(256), 0, ctx->stream, \
+    hipLaunchKernelGGL((vq::k_crosscov_mfma<NT>), dim3(chunks, (nt_all + 7) / 8, Z), dim3(256), 0, ctx->stream, \
                        d_y, d_x, n, dim, B0, rows_per_chunk, part)
         if (full) CROSSCOV(8, 0, full);
         switch (rest) {
@@ -206,8 +207,12 @@ int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n,
         hipLaunchKernelGGL(vq::k_crosscov_partial, dim3(chunks, tiles * tiles), dim3(256), 0, ctx->stream, d_y, d_x,
                            n, dim, rows_per_chunk, (double *)ctx->tmp_a.p);
     }
-    hipLaunchKernelGGL(vq::k_crosscov_reduce, dim3(cdiv(total, 256)), dim3(256), 0, ctx->stream,
-                       (const double *)ctx->tmp_a.p, chunks, total, (double *)ctx->tmp_b.p);
+    // chunk sums in groups of 32 chunks, then the groups
+    const int per_group = 32, groups = (chunks + per_group - 1) / per_group;
+    hipLaunchKernelGGL(vq::k_crosscov_reduce, dim3(cdiv(total, 256), groups), dim3(256), 0, ctx->stream,
+                       (const double *)ctx->tmp_a.p, chunks, per_group, total, (double *)ctx->tmp_c.p);
+    hipLaunchKernelGGL(vq::k_crosscov_reduce, dim3(cdiv(total, 256), 1), dim3(256), 0, ctx->stream,
+                       (const double *)ctx->tmp_c.p, groups, groups, total, (double *)ctx->tmp_b.p);
     VQ_HIP(ctx, hipGetLastError());
     VQ_HIP(ctx, hipMemcpyAsync(h_A, ctx->tmp_b.p, sizeof(double) * total, hipMemcpyDeviceToHost, ctx->stream));
     VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
