@@ -27,15 +27,24 @@ static __global__ void __launch_bounds__(256) k_seg_leafsum(const uint32_t *__re
     uint2 d = desc[leaf];
     const float *__restrict__ xc = x + t;
     float acc = 0.0f;
+    // a leaf has up to 1024 rows and the lane adds them one after the other: 32 loads are in
+    // flight per memory round trip (unconditional, clamped to the leaf's last row), the adds keep
+    // their order
     uint32_t p = d.x;
-    for (; p + 8 <= d.y; p += 8) {
-        float v[8];
+    if (d.y > d.x) {
+        const uint32_t last = d.y - 1;
+        for (; p < d.y; p += 32) {
+            uint32_t id[32];
+            float v[32];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = xc[(int64_t)perm[p + u] * ld];
+            for (int u = 0; u < 32; ++u) id[u] = perm[p + u <= last ? p + u : last];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) acc = acc + v[u];
+            for (int u = 0; u < 32; ++u) v[u] = xc[(int64_t)id[u] * ld];
+#pragma unroll
+            for (int u = 0; u < 32; ++u)
+                if (p + u <= last) acc = acc + v[u];
+        }
     }
-    for (; p < d.y; ++p) acc = acc + xc[(int64_t)perm[p] * ld];
     leaf_sum[leaf * sd + t] = acc;
 }
 
@@ -51,9 +60,23 @@ static __global__ void __launch_bounds__(256) k_seg_mean(float *__restrict__ lea
     uint4 info = seg_info[g];
     uint32_t nl = 1u << info.y;
     float *ls = leaf_sum + (size_t)info.x * sd + t;
-    for (uint32_t h = 1; h < nl; h <<= 1)
-        for (uint32_t i = 0; i < nl; i += 2 * h)
-            ls[(size_t)i * sd] = ls[(size_t)i * sd] + ls[(size_t)(i + h) * sd];
+    // the pairs of one level of the tree are independent: eight of them per memory round trip
+    // (clamped to the level's last pair); a lane only reads what it wrote itself
+    for (uint32_t h = 1; h < nl; h <<= 1) {
+        const uint32_t npairs = nl / (2 * h);
+        for (uint32_t q0 = 0; q0 < npairs; q0 += 8) {
+            float a[8], b[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u) {
+                const uint32_t qi = q0 + u < npairs ? q0 + u : npairs - 1;
+                a[u] = ls[(size_t)(2 * h * qi) * sd];
+                b[u] = ls[(size_t)(2 * h * qi + h) * sd];
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u)
+                if (q0 + u < npairs) ls[(size_t)(2 * h * (q0 + u)) * sd] = a[u] + b[u];
+        }
+    }
     out[(out_first + g) * sd + t] = ls[0] / __uint2float_rn(info.z);
 }
 
@@ -870,6 +893,15 @@ static __global__ void k_seg_median(const float *__restrict__ mids, const uint2 
     const float a = mids[2 * i], b = mids[2 * i + 1];
     const float sum = a + b;
     median[i] = (cnt % 2u == 0u) ? sum / 2.0f : a;
+}
+
+// out[i][t] = means[idx[i]][t]: the means of the nodes that split, side by side
+static __global__ void __launch_bounds__(256) k_gather_means(const float *__restrict__ means,
+                                                             const int *__restrict__ idx, int ns, int dim,
+                                                             float *__restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= (int64_t)ns * dim) return;
+    out[e] = means[(size_t)idx[e / dim] * dim + e % dim];
 }
 
 // ---- descent -------------------------------------------------------------------------------

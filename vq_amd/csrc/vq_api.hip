@@ -535,7 +535,7 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     if (ctx->side) (void)hipStreamSynchronize(ctx->side);
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
-                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tsvq_split, &ctx->tsvq_gsum, &ctx->tsvq_guess, &ctx->tsvq_maps, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
+                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tsvq_split, &ctx->tsvq_level, &ctx->tsvq_gsum, &ctx->tsvq_guess, &ctx->tsvq_maps, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     prof_collect(ctx);

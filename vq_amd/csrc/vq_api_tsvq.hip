@@ -132,12 +132,24 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     void *rp_tmp = nullptr;
     size_t rp_cap = 0;
     int32_t rc = VQ_OK;
+    struct LevelMeans {
+        void *d;
+        int32_t first_node;
+        int nseg;
+    };
+    std::vector<LevelMeans> level_means;  // device means of every level, read back after the last one
+    std::vector<uint2> desc;
+    std::vector<uint4> info;
+    auto free_means = [&]() {
+        for (auto &lm : level_means) (void)hipFree(lm.d);
+        level_means.clear();
+    };
 
     while (!level.empty()) {
         const int nseg = (int)level.size();
         // ---- means of every node of the level ------------------------------------------------
-        std::vector<uint2> desc;
-        std::vector<uint4> info(nseg);
+        desc.clear();  // (both outlive the level: their uploads are enqueued, not waited for)
+        info.assign(nseg, make_uint4(0u, 0u, 0u, 0u));
         for (int g = 0; g < nseg; ++g) {
             uint32_t cnt = level[g].hi - level[g].lo;
             int dep = tree_depth(cnt);
@@ -155,28 +167,43 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             }
         }
         const size_t nleaves = desc.size();
+        // The level's leaf tables live in a grow-only arena of the context; its node means stay in
+        // an allocation of their own until the end of the build, when all means are read back at
+        // once — nothing here waits for the GPU: which nodes split depends on their sizes only.
         void *d_desc = nullptr, *d_info = nullptr, *d_lsum = nullptr, *d_means = nullptr;
-        auto free_level = [&]() {
-            (void)hipFree(d_desc);
-            (void)hipFree(d_info);
-            (void)hipFree(d_lsum);
-            (void)hipFree(d_means);
-        };
+        auto free_level = [&]() {};
 #define LV_HIP(call)                                                                              \
     do {                                                                                          \
         hipError_t e__ = (call);                                                                  \
         if (e__ != hipSuccess) {                                                                  \
-            free_level();                                                                         \
+            (void)hipGetLastError();                                                              \
+            free_means();                                                                         \
             (void)hipFree(rp_tmp);                                                                \
             return cleanup_fail(fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,   \
                                      "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__,   \
                                      __LINE__));                                                  \
         }                                                                                         \
     } while (0)
-        LV_HIP(hipMalloc(&d_desc, sizeof(uint2) * nleaves));
-        LV_HIP(hipMalloc(&d_info, sizeof(uint4) * nseg));
-        LV_HIP(hipMalloc(&d_lsum, sizeof(float) * nleaves * dim));
+        {
+            const size_t sizes[3] = {sizeof(uint2) * nleaves, sizeof(uint4) * (size_t)nseg, sizeof(float) * nleaves * dim};
+            void **ptrs[3] = {&d_desc, &d_info, &d_lsum};
+            size_t total = 0;
+            for (size_t z : sizes) total += (z + 255) & ~(size_t)255;
+            const int32_t rc = ensure(ctx, ctx->tsvq_level, total);
+            if (rc != VQ_OK) {
+                free_means();
+                (void)hipFree(rp_tmp);
+                return cleanup_fail(rc);
+            }
+            char *at = (char *)ctx->tsvq_level.p;
+            for (int z = 0; z < 3; ++z) {
+                *ptrs[z] = at;
+                at += (sizes[z] + 255) & ~(size_t)255;
+            }
+        }
         LV_HIP(hipMalloc(&d_means, sizeof(float) * (size_t)nseg * dim));
+        const int32_t first_node = level[0].node;
+        level_means.push_back({d_means, first_node, nseg});
         LV_HIP(hipMemcpyAsync(d_desc, desc.data(), sizeof(uint2) * nleaves, hipMemcpyHostToDevice, st));
         LV_HIP(hipMemcpyAsync(d_info, info.data(), sizeof(uint4) * nseg, hipMemcpyHostToDevice, st));
         hipLaunchKernelGGL(vq::k_seg_leafsum, dim3(cdiv((int64_t)nleaves * dim, 256)), dim3(256), 0, st, perm,
@@ -184,39 +211,26 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         hipLaunchKernelGGL(vq::k_seg_mean, dim3(cdiv((int64_t)nseg * dim, 256)), dim3(256), 0, st,
                            (float *)d_lsum, (const uint4 *)d_info, nseg, dim, (float *)d_means, (int64_t)0);
         LV_HIP(hipGetLastError());
-        const int32_t first_node = level[0].node;
-        T->h_centroids.resize((size_t)(first_node + nseg) * dim);
-        LV_HIP(hipMemcpyAsync(T->h_centroids.data() + (size_t)first_node * dim, d_means,
-                              sizeof(float) * (size_t)nseg * dim, hipMemcpyDeviceToHost, st));
-        LV_HIP(hipStreamSynchronize(st));
 
         // ---- which nodes split (src/tsvq.rs:78) ---------------------------------------------
         std::vector<int> split;  // indices into level
         if (depth_left > 0)
             for (int g = 0; g < nseg; ++g)
                 if (level[g].hi - level[g].lo > 1) split.push_back(g);
-        if (split.empty()) {
-            free_level();
-            break;
-        }
+        if (split.empty()) break;
         const int ns = (int)split.size();
         std::vector<uint2> range(ns);
         for (int i = 0; i < ns; ++i) range[i] = make_uint2(level[split[i]].lo, level[split[i]].hi);
-        // means of the splitting nodes, compacted
-        std::vector<float> smeans((size_t)ns * dim);
-        for (int i = 0; i < ns; ++i)
-            std::copy_n(T->h_centroids.data() + (size_t)level[split[i]].node * dim, dim,
-                        smeans.data() + (size_t)i * dim);
         // the level's small tables: one grow-only arena of the context instead of nine allocations
         void *d_range = nullptr, *d_smeans = nullptr, *d_var = nullptr, *d_sdim = nullptr, *d_mids = nullptr,
-             *d_median = nullptr, *d_nleft = nullptr, *d_sel = nullptr, *d_hist = nullptr;
+             *d_median = nullptr, *d_nleft = nullptr, *d_sel = nullptr, *d_hist = nullptr, *d_split = nullptr;
         auto free_split = [&]() {};
 #define SP_HIP(call)                                                                              \
     do {                                                                                          \
         hipError_t e__ = (call);                                                                  \
         if (e__ != hipSuccess) {                                                                  \
-            free_split();                                                                         \
-            free_level();                                                                         \
+            (void)hipGetLastError();                                                              \
+            free_means();                                                                         \
             (void)hipFree(rp_tmp);                                                                \
             return cleanup_fail(fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,   \
                                      "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__,   \
@@ -225,27 +239,31 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     } while (0)
         {
             const size_t cap = (size_t)std::max(ns, 1024);  // sized once for the usual depths
-            const size_t sizes[9] = {sizeof(uint2) * cap, sizeof(float) * cap * dim, sizeof(float) * cap * dim,
-                                     sizeof(int) * cap, sizeof(float) * 2 * cap, sizeof(float) * cap,
-                                     sizeof(uint32_t) * cap, sizeof(vq::SegSelect) * 2 * cap,
-                                     sizeof(uint32_t) * 512 * cap};
-            void **ptrs[9] = {&d_range, &d_smeans, &d_var, &d_sdim, &d_mids, &d_median, &d_nleft, &d_sel, &d_hist};
+            const size_t sizes[10] = {sizeof(uint2) * cap, sizeof(float) * cap * dim, sizeof(float) * cap * dim,
+                                      sizeof(int) * cap, sizeof(float) * 2 * cap, sizeof(float) * cap,
+                                      sizeof(uint32_t) * cap, sizeof(vq::SegSelect) * 2 * cap,
+                                      sizeof(uint32_t) * 512 * cap, sizeof(int) * cap};
+            void **ptrs[10] = {&d_range, &d_smeans, &d_var, &d_sdim, &d_mids, &d_median, &d_nleft, &d_sel, &d_hist,
+                               &d_split};
             size_t total = 0;
             for (size_t z : sizes) total += (z + 255) & ~(size_t)255;
             const int32_t rc = ensure(ctx, ctx->tsvq_split, total);
             if (rc != VQ_OK) {
-                free_level();
+                free_means();
                 (void)hipFree(rp_tmp);
                 return cleanup_fail(rc);
             }
             char *at = (char *)ctx->tsvq_split.p;
-            for (int z = 0; z < 9; ++z) {
+            for (int z = 0; z < 10; ++z) {
                 *ptrs[z] = at;
                 at += (sizes[z] + 255) & ~(size_t)255;
             }
         }
         SP_HIP(hipMemcpyAsync(d_range, range.data(), sizeof(uint2) * ns, hipMemcpyHostToDevice, st));
-        SP_HIP(hipMemcpyAsync(d_smeans, smeans.data(), sizeof(float) * (size_t)ns * dim, hipMemcpyHostToDevice, st));
+        // the means of the splitting nodes, compacted on the device
+        SP_HIP(hipMemcpyAsync(d_split, split.data(), sizeof(int) * ns, hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(vq::k_gather_means, dim3(cdiv((int64_t)ns * dim, 256)), dim3(256), 0, st,
+                           (const float *)d_means, (const int *)d_split, ns, dim, (float *)d_smeans);
         // per-dimension sums of squared deviations (src/tsvq.rs:88-99)
         if (var_chain && ns <= kChainSegs) {
             uint32_t longest = 0;
@@ -326,8 +344,6 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         SP_HIP(hipMemcpyAsync(sdim.data(), d_sdim, sizeof(int) * ns, hipMemcpyDeviceToHost, st));
         SP_HIP(hipMemcpyAsync(median.data(), d_median, sizeof(float) * ns, hipMemcpyDeviceToHost, st));
         SP_HIP(hipStreamSynchronize(st));
-        free_split();
-        free_level();
         std::swap(perm, perm2);
 
         // ---- children (src/tsvq.rs:126-141) ---------------------------------------------------
@@ -353,10 +369,17 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         level.swap(next);
         --depth_left;
     }
+    (void)hipFree(rp_tmp);
+    rp_tmp = nullptr;
+    T->n_nodes = (int32_t)T->h_left.size();
+    T->h_centroids.resize((size_t)T->n_nodes * dim);
+    for (auto &lm : level_means)
+        LV_HIP(hipMemcpyAsync(T->h_centroids.data() + (size_t)lm.first_node * dim, lm.d,
+                              sizeof(float) * (size_t)lm.nseg * dim, hipMemcpyDeviceToHost, st));
+    LV_HIP(hipStreamSynchronize(st));
+    free_means();
 #undef LV_HIP
 #undef SP_HIP
-    (void)hipFree(rp_tmp);
-    T->n_nodes = (int32_t)T->h_left.size();
     rc = tree_to_device(ctx, T);
     if (rc != VQ_OK) return cleanup_fail(rc);
     *out = T;
