@@ -548,14 +548,21 @@ namespace vq {
 // every chunk of 8 dimensions (two instructions per chunk and tile of 32 centroids; each lane half
 // owns 4 of the 8 dimensions, the three bf16 parts of its share of ||x||^2 ride in the spare slots
 // of the second instruction).
-// A workgroup = 128 rows; wave w takes the row tiles {2 (w&1), 2 (w&1) + 1} and the centroid tiles
-// [4 (w>>1), 4 (w>>1) + 4): 8 accumulator tiles (128 registers), every A operand read from LDS
-// feeds two matrix instructions.  The A operands of a chunk (16 KB for 256 centroids) are staged
-// in LDS once per workgroup, double-buffered; the rows and the next A chunk are fetched one chunk
-// ahead.  The two waves that share rows merge their (smallest, second smallest) through LDS.
-// Error of a score: 3 * 2^-16 (split, as above) + (34 * sd/8 + 16) * 2^-24 (fp32 accumulation of
-// 2 x 17 addends per chunk) + 2^-22 (rounding of x - mu and c - mu), per unit of
-// ||x - mu||^2 + ||c - mu||^2; twice that for two candidates.
+// A workgroup = 128 rows; a wave takes one tile of 32 rows against every tile of 32 centroids: 8
+// accumulator tiles (128 registers) that start at ||c - mu||^2.  The centroid operand of a tile and
+// chunk is the 16 bytes {ah, al} as they lie in LDS, used by both instructions:
+//     A . {xh, xh} = ah.xh + al.xh        A . {xl, 0} = ah.xl
+// so the row is split once per chunk for 16 matrix instructions and no operand is assembled in
+// registers (vector and matrix instructions mostly take turns on a SIMD: an earlier shape — two
+// row tiles x four centroid tiles per wave, operands {ah, ah} and {al, 1, ...} built from the LDS
+// word, ||x||^2 fed through spare slots — spent as many cycles on vector work as on the matrix
+// instructions: 0.55 ms per pass at 1M x 256 against 0.39 ms now).  ||x - mu||^2 is summed on the
+// vector ALU and added to the scores before the selection.  The A operands of a chunk (16 KB for
+// 256 centroids) are staged in LDS once per workgroup, double-buffered; the row and the next A
+// chunk are fetched one chunk ahead.
+// Error of a score: 3 * 2^-16 (split, as above) + (34 * sd/8 + 16) * 2^-24 (fp32 accumulation, an
+// upper bound: 12 non-zero addends per chunk and the final sum) + 2^-22 (rounding of x - mu and
+// c - mu), per unit of ||x - mu||^2 + ||c - mu||^2; twice that for two candidates.
 #ifndef VQ_WIDE_STAGE_CHUNKS
 #define VQ_WIDE_STAGE_CHUNKS 2
 #endif
@@ -712,15 +719,16 @@ static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *_
 // (__syncthreads would wait for the prefetches as well).
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// grid (ceil(n/128), m); 256 threads = 4 waves.
-template <bool LBG>
+// grid (ceil(n/128), m); 256 threads = 4 waves, one tile of 32 rows each against every centroid.
+// NB = tiles of 32 centroids (tb.nb), a template parameter so that the chains of matrix
+// instructions are straight-line code.
+template <bool LBG, int NB>
 __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, MfmaWideBfTables tb) {
     constexpr int NBMAX = 8;
     constexpr int SC = VQ_WIDE_STAGE_CHUNKS;  // chunks of 8 dimensions per stage (per barrier)
     __shared__ u32x4 lds_a[2][SC * NBMAX * 64];  // 2 stages x SC chunks x 8 KB
     __shared__ float lds_c2[NBMAX * 32];
     __shared__ float lds_mu[kWideCentreMax];
-    __shared__ int lds_top[2][2][3][32];     // [row pair][row tile][m1 | m2 | m3][row] of the upper centroid half
     __shared__ uint32_t wg_list[128];
     __shared__ uint2 wg_pairs[128];
     __shared__ uint32_t wg_count, wg_base, wg_pcount, wg_pbase;
@@ -730,8 +738,8 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int rp = wave & 1, ch = wave >> 1;
-    const int nb = tb.nb, sd = tb.sd, nkc = sd / 8;
+    constexpr int nb = NB;
+    const int sd = tb.sd, nkc = sd / 8;
     const u32x4 *ag = tb.atab + (size_t)s * nkc * nb * 64;
     const int chunk16 = nb * 64;  // 16-byte pieces per chunk
     for (int i = threadIdx.x; i < nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s * nb * 32 + i];
@@ -744,34 +752,22 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         for (int i = threadIdx.x; i < sd; i += 256) lds_mu[i] = tb.mu[(size_t)s * sd + i];
     __syncthreads();
 
-    int64_t row[2];
-    bool valid[2];
-    const float *xr[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        row[t] = (int64_t)blockIdx.x * 128 + (2 * rp + t) * 32 + r;
-        valid[t] = row[t] < a.n;
-        xr[t] = a.x + (valid[t] ? row[t] : 0) * a.ld + (int64_t)s * sd + 4 * h;  // this half's 4 dimensions
-    }
+    const int64_t row = (int64_t)blockIdx.x * 128 + wave * 32 + r;
+    const bool valid = row < a.n;
+    const float *xr = a.x + (valid ? row : 0) * a.ld + (int64_t)s * sd + 4 * h;  // this half's 4 dimensions
     const bool shifted = tb.shifted[s] != 0;  // uniform
-    floatx16 acc[2][4];
+    // the accumulators start at ||c - mu||^2; ||x - mu||^2, the same in every score of a row, is
+    // summed on the side and added before the selection
+    floatx16 acc[NB];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const int b = 4 * ch + c;
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const float c2 = (b < nb) ? lds_c2[(b * 2 + h) * 16 + v] : kPadScore;
-            acc[0][c][v] = c2;
-            acc[1][c][v] = c2;
-        }
-    }
+        for (int v = 0; v < 16; ++v) acc[b][v] = lds_c2[(b * 2 + h) * 16 + v];
     // Loads are unconditional (a row past the end reads row 0 and is never stored; A pieces past
     // the chunk are clamped): loads under a branch make the compiler wait for every outstanding
     // load at each use instead of counting them.
-    float4 xn[2];  // the next chunk of the rows
-#pragma unroll
-    for (int t = 0; t < 2; ++t) xn[t] = *reinterpret_cast<const float4 *>(xr[t]);
-    float x2[2] = {0.0f, 0.0f};
+    float4 xn = *reinterpret_cast<const float4 *>(xr);  // the next chunk of the row
+    float x2 = 0.0f;
     // A stage is SC chunks of 8 dimensions: one barrier per 16 SC matrix instructions of a wave.
     // Chunks past the last one have zero row operands (they add nothing).
     const int nst = (nkc + SC - 1) / SC;
@@ -786,72 +782,59 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
             const int i = (st + 1) * SC * chunk16 + (int)threadIdx.x + 256 * q;
             pre[q] = ag[i < total16 ? i : total16 - 1];
         }
+        // The stage's centroid operands are read from LDS four tiles (one group) at a time (reading a
+        // group ahead of its use measured the same and costs 16 registers).
+        constexpr int NG = (NB + 3) / 4;  // groups of four centroid tiles per chunk
+        auto read_group = [&](int sub, int g, u32x4 (&av)[4]) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int b = 4 * g + c < nb ? 4 * g + c : nb - 1;  // past the last block: read it, not multiplied
+                av[c] = lds_a[cur][sub * chunk16 + b * 64 + lane];
+            }
+        };
 #pragma unroll
         for (int sub = 0; sub < SC; ++sub) {
             const int kc = SC * st + sub;
             const bool live = kc < nkc;  // uniform
             const int kcc = live ? kc : nkc - 1;
-            // operands of this chunk from the rows fetched one chunk ago
-            u32x4 b1[2], b2[2];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                float xv[4] = {xn[t].x, xn[t].y, xn[t].z, xn[t].w};
-                if (shifted) {
-                    const float4 mn = *reinterpret_cast<const float4 *>(lds_mu + kcc * 8 + 4 * h);
-                    xv[0] -= mn.x;
-                    xv[1] -= mn.y;
-                    xv[2] -= mn.z;
-                    xv[3] -= mn.w;
-                }
-                if (!live) xv[0] = xv[1] = xv[2] = xv[3] = 0.0f;
-                float p = 0.0f;
-#pragma unroll
-                for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
-                const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
-                const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
-                const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
-                x2[t] += p;
-                const uint32_t p0 = bf16_pack2(p, 0.0f);
-                const float r1 = p - __uint_as_float(p0 << 16);
-                const uint32_t p1 = bf16_pack2(r1, 0.0f);
-                const float r2 = r1 - __uint_as_float(p1 << 16);
-                const uint32_t p2 = bf16_pack2(r2, 0.0f);
-                b1[t] = u32x4{h01, h23, l01, l23};
-                b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), p2 & 0xffffu};
+            // operands of this chunk from the row piece fetched one chunk ago.  With the centroid
+            // operand A = {ah, al} (as it lies in LDS, no register shuffling):
+            //   A . {xh, xh} = ah.xh + al.xh      A . {xl, 0} = ah.xl
+            float xv[4] = {xn.x, xn.y, xn.z, xn.w};
+            if (shifted) {
+                const float4 mn = *reinterpret_cast<const float4 *>(lds_mu + kcc * 8 + 4 * h);
+                xv[0] -= mn.x;
+                xv[1] -= mn.y;
+                xv[2] -= mn.z;
+                xv[3] -= mn.w;
             }
-            // fetch the next chunk of the rows
+            if (!live) xv[0] = xv[1] = xv[2] = xv[3] = 0.0f;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x2 = __builtin_fmaf(xv[u], xv[u], x2);
+            const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
+            const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
+            const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
+            const u32x4 b1 = u32x4{h01, h23, h01, h23}, b2 = u32x4{l01, l23, 0u, 0u};
+            // fetch the next chunk of the row
             const int nx = kc + 1 < nkc ? kc + 1 : nkc - 1;
+            xn = *reinterpret_cast<const float4 *>(xr + nx * 8);
 #pragma unroll
-            for (int t = 0; t < 2; ++t) xn[t] = *reinterpret_cast<const float4 *>(xr[t] + nx * 8);
-            // the A operands of the wave's four centroid tiles are read from LDS together (a tile
-            // past the last block reads the last block and is not multiplied): one LDS round trip
-            // per chunk instead of one per tile
-            u32x4 a1[4], a2[4];
+            for (int g = 0; g < NG; ++g) {
+                u32x4 av[4];
+                read_group(sub, g, av);
+                {
+                    // the first instruction of every tile, then the second: the two dependent
+                    // instructions of a tile are three others apart
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int b = 4 * ch + c < nb ? 4 * ch + c : nb - 1;
-                const u32x4 v = lds_a[cur][sub * chunk16 + b * 64 + lane];
-                a1[c] = u32x4{v.x, v.y, v.x, v.y};
-                a2[c] = u32x4{v.z, v.w, 0x3f803f80u, 0x00003f80u};
-            }
-            // first instruction of every accumulator tile, then the second: the two instructions
-            // of a tile depend on each other and are kept seven others apart
+                    for (int c = 0; c < 4; ++c)
+                        if (4 * g + c < nb)
+                            acc[4 * g + c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                __builtin_bit_cast(bf16x8, av[c]), __builtin_bit_cast(bf16x8, b1), acc[4 * g + c], 0, 0, 0);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if (4 * ch + c < nb) {
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-                        acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8, a1[c]), __builtin_bit_cast(bf16x8, b1[t]), acc[t][c], 0, 0, 0);
-                }
-            }
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if (4 * ch + c < nb) {
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-                        acc[t][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8, a2[c]), __builtin_bit_cast(bf16x8, b2[t]), acc[t][c], 0, 0, 0);
+                    for (int c = 0; c < 4; ++c)
+                        if (4 * g + c < nb)
+                            acc[4 * g + c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                __builtin_bit_cast(bf16x8, av[c]), __builtin_bit_cast(bf16x8, b2), acc[4 * g + c], 0, 0, 0);
                 }
             }
         }
@@ -864,83 +847,59 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         }
         lds_barrier();
     }
-    x2[0] += __shfl_xor(x2[0], 32);  // both halves' shares of ||x||^2
-    x2[1] += __shfl_xor(x2[1], 32);
-    // the three smallest scores of this wave's centroid tiles (index in the low 8 bits)
+    x2 += __shfl_xor(x2, 32);  // both halves' shares of ||x - mu||^2
+    // the three smallest scores of the row (index in the low 8 bits, one v_and_or per score)
     auto push = [](int &m1, int &m2, int &m3, int key) {
         m3 = imed3(m2, m3, key);
         m2 = imed3(m1, m2, key);
         m1 = imin(m1, key);
     };
-    int m1[2], m2[2], m3[2];
+    int m1 = 0x7f800000, m2 = 0x7f800000, m3 = 0x7f800000;
+    const uint32_t keep = opaque_vgpr(0xFFFFFF00u);
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        m1[t] = 0x7f800000;
-        m2[t] = 0x7f800000;
-        m3[t] = 0x7f800000;
+    for (int b = 0; b < NB; ++b) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int b = 4 * ch + c;
-            if (b < nb) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const uint32_t idx = (uint32_t)(32 * b + 8 * (v / 4) + 4 * h + v % 4);
-                    push(m1[t], m2[t], m3[t], (int)((__float_as_uint(acc[t][c][v]) & 0xFFFFFF00u) | idx));
-                }
-            }
-        }
-        const int o1 = __shfl_xor(m1[t], 32), o2 = __shfl_xor(m2[t], 32), o3 = __shfl_xor(m3[t], 32);
-        push(m1[t], m2[t], m3[t], o1);
-        push(m1[t], m2[t], m3[t], o2);
-        push(m1[t], m2[t], m3[t], o3);
+        for (int v = 0; v < 16; ++v)
+            push(m1, m2, m3, pack_tag(acc[b][v] + x2, keep, (uint32_t)(32 * b + 8 * (v / 4) + v % 4) | (uint32_t)(4 * h)));
     }
-    if (ch == 1 && h == 0) {
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            lds_top[rp][t][0][r] = m1[t];
-            lds_top[rp][t][1][r] = m2[t];
-            lds_top[rp][t][2][r] = m3[t];
-        }
+    {
+        const int o1 = __shfl_xor(m1, 32), o2 = __shfl_xor(m2, 32), o3 = __shfl_xor(m3, 32);
+        push(m1, m2, m3, o1);
+        push(m1, m2, m3, o2);
+        push(m1, m2, m3, o3);
     }
-    __syncthreads();
-    if (ch == 0 && h == 0) {
+    const uint32_t i1 = (uint32_t)m1 & 0xFFu, i2 = (uint32_t)m2 & 0xFFu;
+    if (h == 0) {
         float mc2 = 0.0f;  // largest ||c||^2 of the column block; a NaN stays
         for (int b = 0; b < nb; ++b) {
             const float o = tb.blockmax[(size_t)s * nb + b];
             mc2 = (mc2 == mc2 && o == o) ? fmaxf(mc2, o) : __builtin_nanf("");
         }
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            push(m1[t], m2[t], m3[t], lds_top[rp][t][0][r]);
-            push(m1[t], m2[t], m3[t], lds_top[rp][t][1][r]);
-            push(m1[t], m2[t], m3[t], lds_top[rp][t][2][r]);
-            const float s1 = __int_as_float(m1[t]), s2 = __int_as_float(m2[t]), s3 = __int_as_float(m3[t]);
-            if (valid[t]) {
-                const float bound = x2[t] + mc2;
-                const bool finite = (bound < 1e29f) && (s1 < 1e29f);  // false for NaN
-                const float slack = tb.kappa * bound;
-                // the smallest exact distance is the best-scored centroid's when the second score is
-                // further away than the error bound ...
-                const bool sure = finite && (s2 - s1) > 6.103515625e-05f * fabsf(s2) + slack;
-                // ... and one of the two best-scored centroids' when the third score is
-                const bool two = finite && (s2 < 1e29f) && (s3 - s1) > 6.103515625e-05f * fabsf(s3) + slack;
-                if (sure) {
-                    const uint8_t code = (uint8_t)(__float_as_uint(s1) & 0xFFu);
-                    if constexpr (LBG) {
-                        uint8_t *pc = a.codes + (size_t)s * a.n + row[t];
-                        if (*pc != code) {
-                            *pc = code;
-                            mark_changed(a.changed + s);
-                        }
-                    } else {
-                        a.codes[row[t] * a.m + s] = code;
+        const float s1 = __int_as_float(m1), s2 = __int_as_float(m2), s3 = __int_as_float(m3);
+        if (valid) {
+            const float bound = x2 + mc2;
+            const bool finite = (bound < 1e29f) && (s1 < 1e29f);  // false for NaN
+            const float slack = tb.kappa * bound;
+            // the smallest exact distance is the best-scored centroid's when the second score is
+            // further away than the error bound ...
+            const bool sure = finite && (s2 - s1) > 6.103515625e-05f * fabsf(s2) + slack;
+            // ... and one of the two best-scored centroids' when the third score is
+            const bool two = finite && (s2 < 1e29f) && (s3 - s1) > 6.103515625e-05f * fabsf(s3) + slack;
+            if (sure) {
+                const uint8_t code = (uint8_t)i1;
+                if constexpr (LBG) {
+                    uint8_t *pc = a.codes + (size_t)s * a.n + row;
+                    if (*pc != code) {
+                        *pc = code;
+                        mark_changed(a.changed + s);
                     }
-                } else if (two) {
-                    wg_pairs[atomicAdd(&wg_pcount, 1u)] = make_uint2(
-                        (uint32_t)(row[t] * a.m + s), (__float_as_uint(s1) & 0xFFu) | ((__float_as_uint(s2) & 0xFFu) << 8));
                 } else {
-                    wg_list[atomicAdd(&wg_count, 1u)] = (uint32_t)(row[t] * a.m + s);
+                    a.codes[row * a.m + s] = code;
                 }
+            } else if (two) {
+                wg_pairs[atomicAdd(&wg_pcount, 1u)] = make_uint2((uint32_t)(row * a.m + s), i1 | (i2 << 8));
+            } else {
+                wg_list[atomicAdd(&wg_count, 1u)] = (uint32_t)(row * a.m + s);
             }
         }
     }

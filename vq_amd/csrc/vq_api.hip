@@ -250,8 +250,20 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     vq::MfmaWideBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, mu, shifted, list, count, pairs, nb, sd, kappa};
     {
         ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
-        hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0,
-                           ctx->stream, a, tb);
+#define WIDE(NB)                                                                                             \
+    hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG, NB>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0, \
+                       ctx->stream, a, tb)
+        switch (nb) {
+        case 1: WIDE(1); break;
+        case 2: WIDE(2); break;
+        case 3: WIDE(3); break;
+        case 4: WIDE(4); break;
+        case 5: WIDE(5); break;
+        case 6: WIDE(6); break;
+        case 7: WIDE(7); break;
+        default: WIDE(8); break;
+        }
+#undef WIDE
     }
     VQ_HIP(ctx, hipGetLastError());
     ctx->recheck_src = 2;
