@@ -13,7 +13,9 @@
  *     context's device); pointers named h_* are host pointers.
  *   - matrices are row-major f32, `ld` = row stride in elements; a "column block" s of width
  *     sub_dim covers columns [s*sub_dim, (s+1)*sub_dim).
- *   - codes are uint8 (k <= 256), row-major n x m unless stated otherwise.
+ *   - codes are uint8 (k <= 256) or, in the entry points named *_u16, uint16 (k <= 65536: the
+ *     reference's k is a usize, src/utils.rs:32-37, and its codes are usize indices); row-major
+ *     n x m unless stated otherwise.
  *   - all work is enqueued on the context's stream; functions that return host values
  *     synchronise that stream before returning, the others are asynchronous.
  *   - one context = one stream; a context is not re-entrant, distinct contexts are independent.
@@ -164,7 +166,10 @@ int32_t vq_prof_read(vq_ctx *ctx, int32_t cls, double *h_total_ms, int64_t *h_sp
  * from 0.0).  Above 1024 the reference's Rayon reduce has no fixed order; this library fixes one:
  * the rows are cut into parts of 4096 consecutive rows, a cluster's members inside a part are added
  * in row order from 0.0, and the part sums are added in part order from 0.0.
- * Errors: k == 0 or n < k -> VQ_ERR_INVALID_ARG (utils.rs:39-50); k > 256 -> VQ_ERR_UNSUPPORTED.
+ * k up to 65536: above 256 the assignment runs chunk by chunk (see vq_assign_u16) and the update
+ * lists the clusters' members with a sort of (column block, code, row) keys, same orders of
+ * summation; that path needs n * m < 2^32.
+ * Errors: k == 0 or n < k -> VQ_ERR_INVALID_ARG (utils.rs:39-50); k > 65536 -> VQ_ERR_UNSUPPORTED.
  * Synchronises the stream before returning. */
 int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t m,
                    int32_t sub_dim, int32_t k, int32_t max_iters, const uint32_t *h_init_idx,
@@ -178,6 +183,16 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
  * src/rvq.rs:116-124,189-197 (m = 1 there).  Asynchronous. */
 int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                   int32_t sub_dim, int32_t k, const float *d_codebooks, uint8_t *d_codes);
+
+/* vq_assign with 16-bit codes, for any k up to 65536 (`k: usize` at src/utils.rs:32-37 and
+ * src/pq.rs:79-86; the reference's codes are usize indices).  Same rule, same metrics.  Above 256
+ * centroids every column block's codebook is cut into chunks of 256 consecutive centroids; each
+ * chunk goes through the kernels of vq_assign and its winner's distance, evaluated in the
+ * reference's operation order, replaces the running minimum only when strictly below it, chunks
+ * in ascending order — the lowest index of the overall minimum, as one loop over all k gives.
+ * d_codes 2-byte aligned.  Asynchronous. */
+int32_t vq_assign_u16(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
+                      int32_t sub_dim, int32_t k, const float *d_codebooks, uint16_t *d_codes);
 
 /* vq_assign for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
@@ -205,12 +220,21 @@ int32_t vq_decode_f16(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m,
 int32_t vq_decode_f32(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sub_dim,
                       int32_t k, const float *d_codebooks, float *d_out);
 
+/* The two decodes for the 16-bit codes of vq_assign_u16 (k <= 65536). */
+int32_t vq_decode_f16_u16(vq_ctx *ctx, const uint16_t *d_codes, int64_t n, int32_t m, int32_t sub_dim,
+                          int32_t k, const float *d_codebooks, uint16_t *d_out);
+int32_t vq_decode_f32_u16(vq_ctx *ctx, const uint16_t *d_codes, int64_t n, int32_t m, int32_t sub_dim,
+                          int32_t k, const float *d_codebooks, float *d_out);
+
 /* ---- residual quantizer (src/rvq.rs) -------------------------------------------------------- */
 
 /* d_res[i] -= d_codebook[d_codes[i]] for every row (the residual update of src/rvq.rs:127).
  * d_codes: n uint8 (the output of vq_assign with m = 1).  Asynchronous. */
 int32_t vq_residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
                         const float *d_codebook, const uint8_t *d_codes);
+/* The same for the 16-bit codes of vq_assign_u16 (k <= 65536; `k: usize` at src/rvq.rs:87-95). */
+int32_t vq_residual_sub_u16(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
+                            const float *d_codebook, const uint16_t *d_codes);
 
 /* *h_out = (sum_i sqrt(sum_t x[i][t]^2)) / n — the early-stop statistic of src/rvq.rs:131-138.
  * Row norms follow the reference's sequential f32 order; the sum over rows (a Rayon sum of
@@ -224,10 +248,14 @@ int32_t vq_mean_l2norm(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int
  *   d_codes        out, n*stages uint8 (0 for stages a row did not reach)
  *   d_stages_used  out (nullable), n uint8: stages applied to the row
  *   d_recon_f16    out (nullable), n*dim binary16 bit patterns of the f32 sum (rvq.rs:209-214)
- * Asynchronous. */
+ * stages <= 255 (the count of a row's stages is a byte).  Asynchronous. */
 int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t dim,
                       int32_t stages, int32_t k, const float *d_codebooks, float epsilon,
                       uint8_t *d_codes, uint8_t *d_stages_used, uint16_t *d_recon_f16);
+/* The same with n*stages uint16 codes, k <= 65536 (`k: usize` at src/rvq.rs:87-95). */
+int32_t vq_rvq_encode_u16(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t dim,
+                          int32_t stages, int32_t k, const float *d_codebooks, float epsilon,
+                          uint16_t *d_codes, uint8_t *d_stages_used, uint16_t *d_recon_f16);
 
 /* ---- optimized product quantizer (src/opq.rs) ---------------------------------------------- */
 

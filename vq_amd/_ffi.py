@@ -47,9 +47,15 @@ SYMBOLS = {
                           _vp]),
     "vq_assign": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_assign_noalloc": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
+    "vq_assign_u16": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_decode_f16": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_decode_f32": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
+    "vq_decode_f16_u16": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
+    "vq_decode_f32_u16": (_i32, [_vp, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_residual_sub": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp]),
+    "vq_residual_sub_u16": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _vp, _vp]),
+    "vq_rvq_encode_u16": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, C.c_float, _vp, _vp,
+                                 _vp]),
     "vq_mean_l2norm": (_i32, [_vp, _vp, _i64, _i64, _i32, C.POINTER(C.c_float)]),
     "vq_rvq_encode": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, C.c_float, _vp, _vp,
                              _vp]),
@@ -285,6 +291,19 @@ class Context:
         self._check(_lib.vq_assign_noalloc(self._h, metric, _ptr(d_x), n, ld, m, sub_dim, k,
                                            _ptr(d_codebooks), _ptr(d_codes)))
 
+    def assign_u16(self, metric, d_x, n, ld, m, sub_dim, k, d_codebooks, d_codes):
+        """vq_assign with uint16 codes (k <= 65536)."""
+        self._check(_lib.vq_assign_u16(self._h, metric, _ptr(d_x), n, ld, m, sub_dim, k,
+                                       _ptr(d_codebooks), _ptr(d_codes)))
+
+    def decode_f16_u16(self, d_codes, n, m, sub_dim, k, d_codebooks, d_out):
+        self._check(_lib.vq_decode_f16_u16(self._h, d_codes.ptr, n, m, sub_dim, k, d_codebooks.ptr,
+                                           d_out.ptr))
+
+    def decode_f32_u16(self, d_codes, n, m, sub_dim, k, d_codebooks, d_out):
+        self._check(_lib.vq_decode_f32_u16(self._h, d_codes.ptr, n, m, sub_dim, k, d_codebooks.ptr,
+                                           d_out.ptr))
+
     def decode_f16(self, d_codes, n, m, sub_dim, k, d_codebooks, d_out):
         self._check(_lib.vq_decode_f16(self._h, d_codes.ptr, n, m, sub_dim, k, d_codebooks.ptr,
                                        d_out.ptr))
@@ -298,6 +317,10 @@ class Context:
         self._check(_lib.vq_residual_sub(self._h, d_res.ptr, n, ld, dim, k, _ptr(d_codebook),
                                          d_codes.ptr))
 
+    def residual_sub_u16(self, d_res, n, ld, dim, k, d_codebook, d_codes):
+        self._check(_lib.vq_residual_sub_u16(self._h, d_res.ptr, n, ld, dim, k, _ptr(d_codebook),
+                                             d_codes.ptr))
+
     def mean_l2norm(self, d_x, n, ld, dim):
         out = C.c_float(0)
         self._check(_lib.vq_mean_l2norm(self._h, d_x.ptr, n, ld, dim, C.byref(out)))
@@ -309,6 +332,13 @@ class Context:
                                        d_codebooks.ptr, epsilon, d_codes.ptr,
                                        d_used.ptr if d_used else None,
                                        d_recon.ptr if d_recon else None))
+
+    def rvq_encode_u16(self, metric, d_x, n, ld, dim, stages, k, d_codebooks, epsilon, d_codes,
+                       d_used=None, d_recon=None):
+        self._check(_lib.vq_rvq_encode_u16(self._h, metric, d_x.ptr, n, ld, dim, stages, k,
+                                           d_codebooks.ptr, epsilon, d_codes.ptr,
+                                           d_used.ptr if d_used else None,
+                                           d_recon.ptr if d_recon else None))
 
     # -- optimized product quantizer -----------------------------------------------------------
     def rotate(self, d_x, n, ld, dim, d_R, d_y):

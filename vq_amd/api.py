@@ -103,6 +103,16 @@ class _Quantizer:
         _check(_h.vqh_quantize_batch(_vp(self._o), _p(x), _i64(x.shape[0]), _i64(x.shape[1]), _p(out)))
         return out.view(np.float16)
 
+    def _encode(self, x, width):
+        """n x width codes: bytes up to 256 centroids, uint16 above."""
+        if self.k > 256:
+            codes = np.zeros((x.shape[0], width), np.uint16)
+            _check(_h.vqh_encode16(_vp(self._o), _p(x), _i64(x.shape[0]), _i64(x.shape[1]), _p(codes)))
+        else:
+            codes = np.zeros((x.shape[0], width), np.uint8)
+            _check(_h.vqh_encode(_vp(self._o), _p(x), _i64(x.shape[0]), _i64(x.shape[1]), _p(codes)))
+        return codes
+
     def quantize_batch_vectors(self, data, short_row=-1, short_len=0):
         """quantize_batch through the reference's shape, one heap-allocated vector per row; row
         `short_row` (if >= 0) is passed with only `short_len` floats."""
@@ -128,9 +138,7 @@ class ProductQuantizer(_Quantizer):
 
     def encode(self, data):
         x = _rows(data)
-        codes = np.zeros((x.shape[0], self.m), np.uint8)
-        _check(_h.vqh_encode(_vp(self._o), _p(x), _i64(x.shape[0]), _i64(x.shape[1]), _p(codes)))
-        return codes
+        return self._encode(x, self.m)
 
     def codebooks(self):
         out = np.zeros((self.m, self.k, self.sub_dim), np.float32)
@@ -161,9 +169,7 @@ class OptimizedProductQuantizer(_Quantizer):
 
     def encode(self, data):
         x = _rows(data)
-        codes = np.zeros((x.shape[0], self.m), np.uint8)
-        _check(_h.vqh_encode(_vp(self._o), _p(x), _i64(x.shape[0]), _i64(x.shape[1]), _p(codes)))
-        return codes
+        return self._encode(x, self.m)
 
     def codebooks(self):
         out = np.zeros((self.m, self.k, self.sub_dim), np.float32)
@@ -194,9 +200,7 @@ class ResidualQuantizer(_Quantizer):
 
     def encode(self, data):
         x = _rows(data)
-        codes = np.zeros((x.shape[0], self.stages), np.uint8)
-        _check(_h.vqh_encode(_vp(self._o), _p(x), _i64(x.shape[0]), _i64(x.shape[1]), _p(codes)))
-        return codes
+        return self._encode(x, self.stages)
 
     def codebooks(self):
         out = np.zeros((self.stages, self.k, self.dim), np.float32)

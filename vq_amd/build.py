@@ -6,7 +6,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libvqhip.so")
 SRC = [os.path.join(HERE, "csrc", f) for f in
-       ("vq_api.hip", "vq_api_rvq_opq.hip", "vq_api_tsvq.hip")]
+       ("vq_api.hip", "vq_api_rvq_opq.hip", "vq_api_tsvq.hip", "vq_api_bigk.hip")]
 
 # -ffp-contract=off: the exact kernels must round multiply and add separately, as the
 #   reference's Rust code does.  Fused operations are written explicitly where wanted.

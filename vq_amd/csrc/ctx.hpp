@@ -39,6 +39,10 @@ struct vq_ctx {
     unsigned char *static_scratch = nullptr;
     bool no_alloc = false;
     DevBuf tmp_a, tmp_b, tmp_c, tmp_d, tmp_e, tmp_f;  // scratch of the RVQ / OPQ / TSVQ entry points
+    // codebooks above 256 centroids: chunk tables, chunk winners, running minimum, merged codes,
+    // the LBG's assignment, sort keys in and out, the sort's workspace, per-cluster tables, flags
+    DevBuf big_chunk, big_win, big_best, big_fresh, big_codes, big_keys, big_sorted, big_sort_tmp, big_tables,
+        big_flags;
     // optional per-kernel-class timing (HIP events on the stream)
     bool prof_on = false;
     std::vector<hipEvent_t> prof_pool;
@@ -151,10 +155,20 @@ inline void prof_collect(vq_ctx *ctx) {
 }
 
 // Argument checks shared by the entry points that take a row matrix and codebooks.
-int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t m, int32_t sd, int32_t k);
+// k_max: 256 where the codes are bytes, 65536 where they are 16 bits wide.
+int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t m, int32_t sd, int32_t k,
+                     int32_t k_max = 256);
 
 // Launchers defined in vq_api.hip, used by the RVQ / OPQ entry points.
 int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                      int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes);
+
+// Defined in vq_api_bigk.hip: the same for any k up to 65536 with 16-bit codes, and the LBG above
+// 256 centroids (arguments as vq_lbg_fit, already validated).
+int32_t assign_codes_u16(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
+                         int32_t sd, int32_t k, const float *d_codebooks, uint16_t *d_codes);
+int32_t lbg_fit_big(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t m, int32_t sd, int32_t k,
+                    int32_t max_iters, const uint32_t *h_init_idx, const uint32_t *h_reseed_stream,
+                    int32_t n_reseed, float *d_codebooks, int32_t *h_iters_run, int32_t *h_reseeds_used);
 
 }  // namespace vqh

@@ -8,9 +8,10 @@
 namespace vq {
 
 // res[i] -= codebook[code[i]]   (src/rvq.rs:127).  One lane per element.
+template <typename CodeT>
 static __global__ void __launch_bounds__(256) k_residual_sub(float *__restrict__ res, int64_t n, int64_t ld,
                                                       int dim, const float *__restrict__ cb,
-                                                      const uint8_t *__restrict__ codes,
+                                                      const CodeT *__restrict__ codes,
                                                       int code_stride) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n * dim) return;
@@ -24,11 +25,12 @@ static __global__ void __launch_bounds__(256) k_residual_sub(float *__restrict__
 // workgroup covers 1024 consecutive float4 of the n x dim/4 grid.  active == nullptr: every row.
 // codes_out / used (both or neither): RVQ encode bookkeeping of the stage, written by the lane
 // that holds a row's first components (src/rvq.rs:196-202).
+template <typename CodeT>
 static __global__ void __launch_bounds__(256) k_residual_sub4(float *__restrict__ res, int64_t n, int64_t ld,
                                                        int dim4, const float *__restrict__ cb,
-                                                       const uint8_t *__restrict__ codes,
+                                                       const CodeT *__restrict__ codes,
                                                        const uint8_t *__restrict__ active,
-                                                       uint8_t *__restrict__ codes_out, int stages, int stage,
+                                                       CodeT *__restrict__ codes_out, int stages, int stage,
                                                        uint8_t *__restrict__ used) {
     const int64_t first = (int64_t)blockIdx.x * 1024;
     const int64_t row0 = first / dim4;            // uniform
@@ -42,7 +44,7 @@ static __global__ void __launch_bounds__(256) k_residual_sub4(float *__restrict_
         const bool on = active ? active[row] != 0 : true;
         const uint32_t code = on ? codes[row] : 0u;
         if (codes_out && t4 == 0) {
-            codes_out[row * stages + stage] = (uint8_t)code;
+            codes_out[row * stages + stage] = (CodeT)code;
             if (on) used[row] = (uint8_t)(stage + 1);
         }
         if (!on) continue;
@@ -115,10 +117,11 @@ static __global__ void __launch_bounds__(256) k_sum_f64(const float *__restrict_
 // One stage of ResidualQuantizer::quantize for every row still active (src/rvq.rs:200-202), the
 // residual's half: residual -= c; the stage's code and the number of stages used are recorded.
 // The other half (sum += c) is replayed from the codes by k_rvq_recon_f16.  One lane per element.
+template <typename CodeT>
 static __global__ void __launch_bounds__(256) k_rvq_stage_apply(float *__restrict__ res, int64_t n, int dim,
                                                          const float *__restrict__ cb,
-                                                         const uint8_t *__restrict__ stage_codes,
-                                                         uint8_t *__restrict__ codes_out, int stages,
+                                                         const CodeT *__restrict__ stage_codes,
+                                                         CodeT *__restrict__ codes_out, int stages,
                                                          int stage, const uint8_t *__restrict__ active,
                                                          uint8_t *__restrict__ used) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -128,7 +131,7 @@ static __global__ void __launch_bounds__(256) k_rvq_stage_apply(float *__restric
     const bool on = active[row] != 0;
     const int code = on ? stage_codes[row] : 0;
     if (t == 0) {
-        codes_out[row * stages + stage] = (uint8_t)code;
+        codes_out[row * stages + stage] = (CodeT)code;
         if (on) used[row] = (uint8_t)(stage + 1);
     }
     if (!on) return;
@@ -138,9 +141,10 @@ static __global__ void __launch_bounds__(256) k_rvq_stage_apply(float *__restric
 // The reconstruction of ResidualQuantizer::quantize from the codes: sum = 0; for every stage the
 // row used, in order, sum = sum + c (src/rvq.rs:183,201); then f16 (src/rvq.rs:212).  One lane
 // per element; the codebooks (stages x k x dim) stay in L2.
+template <typename CodeT>
 static __global__ void __launch_bounds__(256) k_rvq_recon_f16(int64_t n, int dim, int k,
                                                        const float *__restrict__ codebooks,
-                                                       const uint8_t *__restrict__ codes, int stages,
+                                                       const CodeT *__restrict__ codes, int stages,
                                                        const uint8_t *__restrict__ used,
                                                        uint16_t *__restrict__ out) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -156,9 +160,10 @@ static __global__ void __launch_bounds__(256) k_rvq_recon_f16(int64_t n, int dim
 
 // The same, four components per lane (dim a multiple of 4, 16-byte aligned codebooks, 8-byte
 // aligned output).
+template <typename CodeT>
 static __global__ void __launch_bounds__(256) k_rvq_recon4_f16(int64_t n, int dim4, int k,
                                                         const float *__restrict__ codebooks,
-                                                        const uint8_t *__restrict__ codes, int stages,
+                                                        const CodeT *__restrict__ codes, int stages,
                                                         const uint8_t *__restrict__ used,
                                                         uint16_t *__restrict__ out) {
     const int64_t first = (int64_t)blockIdx.x * 1024;
@@ -194,7 +199,8 @@ static __global__ void __launch_bounds__(256) k_rvq_stage_stop(const float *__re
     if (row < n && active[row] && norms[row] < epsilon) active[row] = 0;
 }
 
-static __global__ void __launch_bounds__(256) k_fill_u8(uint8_t *__restrict__ p, int64_t count, uint8_t v) {
+template <typename T>
+static __global__ void __launch_bounds__(256) k_fill(T *__restrict__ p, int64_t count, T v) {
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < count) p[i] = v;
 }

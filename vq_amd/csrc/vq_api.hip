@@ -315,7 +315,8 @@ int32_t launch_assign(vq_ctx *ctx, int metric, const vq::AssignArgs &a, int sd, 
     }
 }
 
-__global__ void k_decode_f16(const uint8_t *__restrict__ codes, int64_t n, int m, int sd, int k,
+template <typename CodeT>
+__global__ void k_decode_f16(const CodeT *__restrict__ codes, int64_t n, int m, int sd, int k,
                              const float *__restrict__ cb, uint16_t *__restrict__ out) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     int64_t dim = (int64_t)m * sd;
@@ -330,8 +331,8 @@ __global__ void k_decode_f16(const uint8_t *__restrict__ codes, int64_t n, int m
 // Four consecutive components per thread (sub_dim a multiple of 4, 16-byte aligned codebooks and
 // output rows): one 16-byte load of the centroid, one 8- or 16-byte store.  F16: binary16 bit
 // patterns (round to nearest even), else f32.
-template <bool F16>
-__global__ void __launch_bounds__(256) k_decode_vec4(const uint8_t *__restrict__ codes, int64_t n, int m, int sd,
+template <bool F16, typename CodeT>
+__global__ void __launch_bounds__(256) k_decode_vec4(const CodeT *__restrict__ codes, int64_t n, int m, int sd,
                                                      int k, const float *__restrict__ cb, void *__restrict__ out) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // group of four components
     const int64_t dim4 = (int64_t)m * sd / 4;
@@ -356,8 +357,8 @@ __global__ void __launch_bounds__(256) k_decode_vec4(const uint8_t *__restrict__
 // multiple of 4) — so a wave's stores are 1 KB of consecutive bytes, its code reads consecutive
 // bytes, and the centroid comes from LDS instead of a scattered read of the 128 KB table through
 // the vector cache.  Four pieces per thread are in flight.
-template <bool F16>
-__global__ void __launch_bounds__(1024) k_decode_resident(const uint8_t *__restrict__ codes, int64_t n, int m, int sd,
+template <bool F16, typename CodeT>
+__global__ void __launch_bounds__(1024) k_decode_resident(const CodeT *__restrict__ codes, int64_t n, int m, int sd,
                                                           int k, const float *__restrict__ cb,
                                                           vq::u32x4 *__restrict__ out) {
     extern __shared__ __attribute__((aligned(16))) vq::u32x4 tab[];  // [m * k][pieces of a centroid]
@@ -403,7 +404,8 @@ __global__ void __launch_bounds__(1024) k_decode_resident(const uint8_t *__restr
     }
 }
 
-__global__ void k_decode_f32(const uint8_t *__restrict__ codes, int64_t n, int m, int sd, int k,
+template <typename CodeT>
+__global__ void k_decode_f32(const CodeT *__restrict__ codes, int64_t n, int m, int sd, int k,
                              const float *__restrict__ cb, float *__restrict__ out) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     int64_t dim = (int64_t)m * sd;
@@ -425,14 +427,14 @@ __global__ void __launch_bounds__(256) k_copy_f32(const float4 *__restrict__ src
 }
 
 // LDS-resident decode where the table fits and the output is large enough to pay for staging it.
-template <bool F16>
-int32_t launch_decode_resident(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int m, int sd, int k,
+template <bool F16, typename CodeT>
+int32_t launch_decode_resident(vq_ctx *ctx, const CodeT *d_codes, int64_t n, int m, int sd, int k,
                                const float *d_codebooks, void *d_out, bool *done) {
     *done = false;
     const size_t lds = (size_t)m * k * sd * (F16 ? 2 : 4);
     if (sd % (F16 ? 8 : 4) != 0 || lds > 128 * 1024 || n * m < (1 << 16)) return VQ_OK;
     if ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) return VQ_OK;
-    auto kern = k_decode_resident<F16>;
+    auto kern = k_decode_resident<F16, CodeT>;
     VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)lds));
     hipDeviceProp_t prop;
@@ -447,11 +449,36 @@ int32_t launch_decode_resident(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, i
     return VQ_OK;
 }
 
+// Decode of 8- or 16-bit codes to binary16 bit patterns (F16) or f32.
+template <bool F16, typename CodeT>
+int32_t decode_codes(vq_ctx *ctx, const CodeT *d_codes, int64_t n, int32_t m, int32_t sd, int32_t k, int32_t k_max,
+                     const float *d_codebooks, void *d_out) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return VQ_OK;
+    if (!d_codes || !d_codebooks || !d_out || n < 0 || m <= 0 || sd <= 0 || k <= 0 || k > k_max)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    bool done = false;
+    VQ_TRY((launch_decode_resident<F16, CodeT>(ctx, d_codes, n, m, sd, k, d_codebooks, d_out, &done)));
+    if (done) return VQ_OK;
+    if (sd % 4 == 0 && ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) == 0)
+        hipLaunchKernelGGL((k_decode_vec4<F16, CodeT>), dim3(cdiv(n * m * sd / 4, 256)), dim3(256), 0, ctx->stream,
+                           d_codes, n, m, sd, k, d_codebooks, d_out);
+    else if constexpr (F16)
+        hipLaunchKernelGGL(k_decode_f16<CodeT>, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n, m,
+                           sd, k, d_codebooks, (uint16_t *)d_out);
+    else
+        hipLaunchKernelGGL(k_decode_f32<CodeT>, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n, m,
+                           sd, k, d_codebooks, (float *)d_out);
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
 }  // namespace
 
 namespace vqh {
 int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t m, int32_t sd,
-                     int32_t k) {
+                     int32_t k, int32_t k_max) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
     if (n == 0) return fail(ctx, VQ_ERR_EMPTY_INPUT, "Empty input: at least one vector is required.");
     if (!x || n < 0 || m <= 0 || sd <= 0)
@@ -460,8 +487,10 @@ int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t 
         return fail(ctx, VQ_ERR_DIM_MISMATCH, "Dimension mismatch: expected %lld, got %lld",
                     (long long)m * sd, (long long)ld);
     if (k <= 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: k must be greater than 0");
-    if (k > vq::kMaxK)
-        return fail(ctx, VQ_ERR_UNSUPPORTED, "k = %d: codes are uint8, k must be <= 256", k);
+    if (k > k_max)
+        return fail(ctx, VQ_ERR_UNSUPPORTED,
+                    k_max <= vq::kMaxK ? "k = %d: the codes of this entry point are uint8, k must be <= 256"
+                                       : "k = %d: codes are at most 16 bits wide, k must be <= 65536", k);
     if (n >= (1LL << 32)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n must be below 2^32");
     return VQ_OK;
 }
@@ -547,7 +576,9 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     if (ctx->side) (void)hipStreamSynchronize(ctx->side);
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
-                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tsvq_split, &ctx->tsvq_level, &ctx->tsvq_gsum, &ctx->tsvq_guess, &ctx->tsvq_maps, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f};
+                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tsvq_split, &ctx->tsvq_level, &ctx->tsvq_gsum, &ctx->tsvq_guess, &ctx->tsvq_maps, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f,
+                      &ctx->big_chunk, &ctx->big_win, &ctx->big_best, &ctx->big_fresh, &ctx->big_codes, &ctx->big_keys,
+                      &ctx->big_sorted, &ctx->big_sort_tmp, &ctx->big_tables, &ctx->big_flags};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     prof_collect(ctx);
@@ -768,7 +799,7 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
                    int32_t *h_iters_run, int32_t *h_reseeds_used) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
     if (k == 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: k must be greater than 0");
-    VQ_TRY(check_common(ctx, d_x, n, ld, m, sd, k));
+    VQ_TRY(check_common(ctx, d_x, n, ld, m, sd, k, 65536));
     if (n < k)
         return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: Not enough data points for k clusters");
     if (m > 65535) return fail(ctx, VQ_ERR_UNSUPPORTED, "m must be at most 65535");
@@ -781,6 +812,9 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
         if (h_reseed_stream[i] >= (uint64_t)n)
             return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: reseed index %u out of range", h_reseed_stream[i]);
     VQ_HIP(ctx, hipSetDevice(ctx->device));
+    if (k > vq::kMaxK)
+        return vqh::lbg_fit_big(ctx, d_x, n, ld, m, sd, k, max_iters, h_init_idx, h_reseed_stream, n_reseed,
+                                d_codebooks, h_iters_run, h_reseeds_used);
     hipStream_t st = ctx->stream;
 
     const int nparts = (int)((n + vq::kPartRows - 1) / vq::kPartRows);
@@ -973,42 +1007,22 @@ int32_t vq_assign_noalloc(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t
 
 int32_t vq_decode_f16(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sd, int32_t k,
                       const float *d_codebooks, uint16_t *d_out) {
-    if (!ctx) return VQ_ERR_INVALID_ARG;
-    if (n == 0) return VQ_OK;
-    if (!d_codes || !d_codebooks || !d_out || n < 0 || m <= 0 || sd <= 0 || k <= 0 || k > vq::kMaxK)
-        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
-    VQ_HIP(ctx, hipSetDevice(ctx->device));
-    bool done = false;
-    VQ_TRY(launch_decode_resident<true>(ctx, d_codes, n, m, sd, k, d_codebooks, d_out, &done));
-    if (done) return VQ_OK;
-    if (sd % 4 == 0 && ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) == 0)
-        hipLaunchKernelGGL(k_decode_vec4<true>, dim3(cdiv(n * m * sd / 4, 256)), dim3(256), 0, ctx->stream, d_codes,
-                           n, m, sd, k, d_codebooks, (void *)d_out);
-    else
-        hipLaunchKernelGGL(k_decode_f16, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n,
-                           m, sd, k, d_codebooks, d_out);
-    VQ_HIP(ctx, hipGetLastError());
-    return VQ_OK;
+    return decode_codes<true>(ctx, d_codes, n, m, sd, k, vq::kMaxK, d_codebooks, (void *)d_out);
 }
 
 int32_t vq_decode_f32(vq_ctx *ctx, const uint8_t *d_codes, int64_t n, int32_t m, int32_t sd, int32_t k,
                       const float *d_codebooks, float *d_out) {
-    if (!ctx) return VQ_ERR_INVALID_ARG;
-    if (n == 0) return VQ_OK;
-    if (!d_codes || !d_codebooks || !d_out || n < 0 || m <= 0 || sd <= 0 || k <= 0 || k > vq::kMaxK)
-        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
-    VQ_HIP(ctx, hipSetDevice(ctx->device));
-    bool done = false;
-    VQ_TRY(launch_decode_resident<false>(ctx, d_codes, n, m, sd, k, d_codebooks, d_out, &done));
-    if (done) return VQ_OK;
-    if (sd % 4 == 0 && ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) == 0)
-        hipLaunchKernelGGL(k_decode_vec4<false>, dim3(cdiv(n * m * sd / 4, 256)), dim3(256), 0, ctx->stream, d_codes,
-                           n, m, sd, k, d_codebooks, (void *)d_out);
-    else
-        hipLaunchKernelGGL(k_decode_f32, dim3(cdiv(n * m * sd, 256)), dim3(256), 0, ctx->stream, d_codes, n,
-                           m, sd, k, d_codebooks, d_out);
-    VQ_HIP(ctx, hipGetLastError());
-    return VQ_OK;
+    return decode_codes<false>(ctx, d_codes, n, m, sd, k, vq::kMaxK, d_codebooks, (void *)d_out);
+}
+
+int32_t vq_decode_f16_u16(vq_ctx *ctx, const uint16_t *d_codes, int64_t n, int32_t m, int32_t sd, int32_t k,
+                          const float *d_codebooks, uint16_t *d_out) {
+    return decode_codes<true>(ctx, d_codes, n, m, sd, k, 65536, d_codebooks, (void *)d_out);
+}
+
+int32_t vq_decode_f32_u16(vq_ctx *ctx, const uint16_t *d_codes, int64_t n, int32_t m, int32_t sd, int32_t k,
+                          const float *d_codebooks, float *d_out) {
+    return decode_codes<false>(ctx, d_codes, n, m, sd, k, 65536, d_codebooks, (void *)d_out);
 }
 
 }  // extern "C"

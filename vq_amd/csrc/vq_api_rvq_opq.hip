@@ -12,25 +12,122 @@
 
 using namespace vqh;
 
-extern "C" {
+namespace {
 
-int32_t vq_residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
-                        const float *d_codebook, const uint8_t *d_codes) {
+template <typename CodeT>
+int32_t residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k, int32_t k_max,
+                     const float *d_codebook, const CodeT *d_codes) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
     if (n == 0) return VQ_OK;
-    if (!d_res || !d_codebook || !d_codes || n < 0 || dim <= 0 || ld < dim || k <= 0 || k > 256)
+    if (!d_res || !d_codebook || !d_codes || n < 0 || dim <= 0 || ld < dim || k <= 0 || k > k_max)
         return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
     VQ_HIP(ctx, hipSetDevice(ctx->device));
     if (dim % 4 == 0 && ld % 4 == 0 &&
         ((reinterpret_cast<uintptr_t>(d_res) | reinterpret_cast<uintptr_t>(d_codebook)) & 15) == 0)
-        hipLaunchKernelGGL(vq::k_residual_sub4, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, ctx->stream, d_res,
-                           n, ld, dim / 4, d_codebook, d_codes, (const uint8_t *)nullptr, (uint8_t *)nullptr, 0, 0,
+        hipLaunchKernelGGL(vq::k_residual_sub4<CodeT>, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, ctx->stream,
+                           d_res, n, ld, dim / 4, d_codebook, d_codes, (const uint8_t *)nullptr, (CodeT *)nullptr, 0, 0,
                            (uint8_t *)nullptr);
     else
-        hipLaunchKernelGGL(vq::k_residual_sub, dim3(cdiv(n * dim, 256)), dim3(256), 0, ctx->stream, d_res, n,
+        hipLaunchKernelGGL(vq::k_residual_sub<CodeT>, dim3(cdiv(n * dim, 256)), dim3(256), 0, ctx->stream, d_res, n,
                            ld, dim, d_codebook, d_codes, 1);
     VQ_HIP(ctx, hipGetLastError());
     return VQ_OK;
+}
+
+inline int32_t assign_any(vq_ctx *ctx, int32_t metric, const float *x, int64_t n, int32_t dim, int32_t k,
+                          const float *cb, uint8_t *codes) {
+    return assign_codes(ctx, metric, x, n, dim, 1, dim, k, cb, codes);
+}
+inline int32_t assign_any(vq_ctx *ctx, int32_t metric, const float *x, int64_t n, int32_t dim, int32_t k,
+                          const float *cb, uint16_t *codes) {
+    return assign_codes_u16(ctx, metric, x, n, dim, 1, dim, k, cb, codes);
+}
+
+template <typename CodeT>
+int32_t rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t dim, int32_t stages,
+                   int32_t k, int32_t k_max, const float *d_codebooks, float epsilon, CodeT *d_codes,
+                   uint8_t *d_stages_used, uint16_t *d_recon_f16) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (n == 0) return VQ_OK;
+    if (!d_x || !d_codebooks || !d_codes || n < 0 || dim <= 0 || ld < dim || stages < 0 || k <= 0 || k > k_max ||
+        stages > 255)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(float) * (size_t)n * dim));   // residual
+    VQ_TRY(ensure(ctx, ctx->tmp_e, (size_t)n * (2 + sizeof(CodeT)) + 16));  // stage codes, active, used
+    VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(float) * (size_t)n));         // row norms
+    float *norms = (float *)ctx->tmp_a.p;
+    float *res = (float *)ctx->tmp_c.p;
+    CodeT *stage_codes = (CodeT *)ctx->tmp_e.p;
+    uint8_t *active = (uint8_t *)ctx->tmp_e.p + (((size_t)n * sizeof(CodeT) + 3) & ~(size_t)3);
+    uint8_t *used = active + n;
+    VQ_HIP(ctx, hipMemcpy2DAsync(res, sizeof(float) * dim, d_x, sizeof(float) * ld, sizeof(float) * dim,
+                                 (size_t)n, hipMemcpyDeviceToDevice, st));
+    const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(d_codebooks) & 15) == 0;
+    hipLaunchKernelGGL(vq::k_fill<uint8_t>, dim3(cdiv(n, 256)), dim3(256), 0, st, active, n, (uint8_t)1);
+    hipLaunchKernelGGL(vq::k_fill<uint8_t>, dim3(cdiv(n, 256)), dim3(256), 0, st, used, n, (uint8_t)0);
+    for (int s = 0; s < stages; ++s) {
+        const float *cb = d_codebooks + (size_t)s * k * dim;
+        if (k < 2)  // src/rvq.rs:186-187
+            hipLaunchKernelGGL(vq::k_fill<CodeT>, dim3(cdiv(n, 256)), dim3(256), 0, st, stage_codes, n, (CodeT)0);
+        else
+            VQ_TRY(assign_any(ctx, metric, res, n, dim, k, cb, stage_codes));
+        if (vec4)
+            hipLaunchKernelGGL(vq::k_residual_sub4<CodeT>, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, st, res, n,
+                               (int64_t)dim, dim / 4, cb, (const CodeT *)stage_codes, (const uint8_t *)active, d_codes,
+                               stages, s, used);
+        else
+            hipLaunchKernelGGL(vq::k_rvq_stage_apply<CodeT>, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, res, n, dim,
+                               cb, (const CodeT *)stage_codes, d_codes, stages, s, (const uint8_t *)active, used);
+        if (epsilon > 0.0f) {  // a norm is never below a non-positive threshold
+            hipLaunchKernelGGL(vq::k_row_norms, dim3(cdiv(n, 64)), dim3(64), 0, st, res, n, (int64_t)dim, dim,
+                               norms);
+            hipLaunchKernelGGL(vq::k_rvq_stage_stop, dim3(cdiv(n, 256)), dim3(256), 0, st, norms, n, epsilon,
+                               active);
+        }
+    }
+    if (d_stages_used)
+        VQ_HIP(ctx, hipMemcpyAsync(d_stages_used, used, (size_t)n, hipMemcpyDeviceToDevice, st));
+    if (d_recon_f16) {
+        if (vec4 && (reinterpret_cast<uintptr_t>(d_recon_f16) & 7) == 0)
+            hipLaunchKernelGGL(vq::k_rvq_recon4_f16<CodeT>, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, st, n,
+                               dim / 4, k, d_codebooks, (const CodeT *)d_codes, stages, (const uint8_t *)used,
+                               d_recon_f16);
+        else
+            hipLaunchKernelGGL(vq::k_rvq_recon_f16<CodeT>, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, n, dim, k,
+                               d_codebooks, (const CodeT *)d_codes, stages, (const uint8_t *)used, d_recon_f16);
+    }
+    VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t vq_residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
+                        const float *d_codebook, const uint8_t *d_codes) {
+    return residual_sub<uint8_t>(ctx, d_res, n, ld, dim, k, 256, d_codebook, d_codes);
+}
+
+int32_t vq_residual_sub_u16(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
+                            const float *d_codebook, const uint16_t *d_codes) {
+    return residual_sub<uint16_t>(ctx, d_res, n, ld, dim, k, 65536, d_codebook, d_codes);
+}
+
+int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t dim,
+                      int32_t stages, int32_t k, const float *d_codebooks, float epsilon, uint8_t *d_codes,
+                      uint8_t *d_stages_used, uint16_t *d_recon_f16) {
+    return rvq_encode<uint8_t>(ctx, metric, d_x, n, ld, dim, stages, k, 256, d_codebooks, epsilon, d_codes,
+                               d_stages_used, d_recon_f16);
+}
+
+int32_t vq_rvq_encode_u16(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t dim,
+                          int32_t stages, int32_t k, const float *d_codebooks, float epsilon, uint16_t *d_codes,
+                          uint8_t *d_stages_used, uint16_t *d_recon_f16) {
+    return rvq_encode<uint16_t>(ctx, metric, d_x, n, ld, dim, stages, k, 65536, d_codebooks, epsilon, d_codes,
+                                d_stages_used, d_recon_f16);
 }
 
 int32_t vq_mean_l2norm(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, float *h_out) {
@@ -54,61 +151,6 @@ int32_t vq_mean_l2norm(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int
     VQ_HIP(ctx, hipMemcpyAsync(&total, part + blocks, sizeof(double), hipMemcpyDeviceToHost, ctx->stream));
     VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
     *h_out = (float)total / (float)n;  // src/rvq.rs:137-138
-    return VQ_OK;
-}
-
-int32_t vq_rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t dim,
-                      int32_t stages, int32_t k, const float *d_codebooks, float epsilon, uint8_t *d_codes,
-                      uint8_t *d_stages_used, uint16_t *d_recon_f16) {
-    if (!ctx) return VQ_ERR_INVALID_ARG;
-    if (n == 0) return VQ_OK;
-    if (!d_x || !d_codebooks || !d_codes || n < 0 || dim <= 0 || ld < dim || stages < 0 || k <= 0 || k > 256)
-        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
-    VQ_HIP(ctx, hipSetDevice(ctx->device));
-    hipStream_t st = ctx->stream;
-    VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(float) * (size_t)n * dim));   // residual
-    VQ_TRY(ensure(ctx, ctx->tmp_e, (size_t)n * 3 + 16));                // stage codes, active, used
-    VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(float) * (size_t)n));         // row norms
-    float *norms = (float *)ctx->tmp_a.p;
-    float *res = (float *)ctx->tmp_c.p;
-    uint8_t *stage_codes = (uint8_t *)ctx->tmp_e.p;
-    uint8_t *active = stage_codes + ((n + 3) & ~(int64_t)3);
-    uint8_t *used = active + n;
-    VQ_HIP(ctx, hipMemcpy2DAsync(res, sizeof(float) * dim, d_x, sizeof(float) * ld, sizeof(float) * dim,
-                                 (size_t)n, hipMemcpyDeviceToDevice, st));
-    const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(d_codebooks) & 15) == 0;
-    hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, active, n, (uint8_t)1);
-    hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, used, n, (uint8_t)0);
-    for (int s = 0; s < stages; ++s) {
-        const float *cb = d_codebooks + (size_t)s * k * dim;
-        if (k < 2)  // src/rvq.rs:186-187
-            hipLaunchKernelGGL(vq::k_fill_u8, dim3(cdiv(n, 256)), dim3(256), 0, st, stage_codes, n, (uint8_t)0);
-        else
-            VQ_TRY(assign_codes(ctx, metric, res, n, dim, 1, dim, k, cb, stage_codes));
-        if (vec4)
-            hipLaunchKernelGGL(vq::k_residual_sub4, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, st, res, n,
-                               (int64_t)dim, dim / 4, cb, stage_codes, active, d_codes, stages, s, used);
-        else
-            hipLaunchKernelGGL(vq::k_rvq_stage_apply, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, res, n, dim, cb,
-                               stage_codes, d_codes, stages, s, active, used);
-        if (epsilon > 0.0f) {  // a norm is never below a non-positive threshold
-            hipLaunchKernelGGL(vq::k_row_norms, dim3(cdiv(n, 64)), dim3(64), 0, st, res, n, (int64_t)dim, dim,
-                               norms);
-            hipLaunchKernelGGL(vq::k_rvq_stage_stop, dim3(cdiv(n, 256)), dim3(256), 0, st, norms, n, epsilon,
-                               active);
-        }
-    }
-    if (d_stages_used)
-        VQ_HIP(ctx, hipMemcpyAsync(d_stages_used, used, (size_t)n, hipMemcpyDeviceToDevice, st));
-    if (d_recon_f16) {
-        if (vec4 && (reinterpret_cast<uintptr_t>(d_recon_f16) & 7) == 0)
-            hipLaunchKernelGGL(vq::k_rvq_recon4_f16, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, st, n, dim / 4, k,
-                               d_codebooks, d_codes, stages, used, d_recon_f16);
-        else
-            hipLaunchKernelGGL(vq::k_rvq_recon_f16, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, n, dim, k,
-                               d_codebooks, d_codes, stages, used, d_recon_f16);
-    }
-    VQ_HIP(ctx, hipGetLastError());
     return VQ_OK;
 }
 

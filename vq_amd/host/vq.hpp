@@ -218,6 +218,55 @@ private:
     size_t count_ = 0;
 };
 
+// Device codes of either width: bytes up to 256 centroids, 16 bits above (`k: usize` in the
+// reference, src/utils.rs:32-37; the library's *_u16 entry points).
+class DeviceCodes {
+public:
+    DeviceCodes() = default;
+    DeviceCodes(std::shared_ptr<Device> dev, size_t count, size_t k) : wide_(k > 256) {
+        if (wide_)
+            b16_ = DeviceBuffer<uint16_t>(std::move(dev), count);
+        else
+            b8_ = DeviceBuffer<uint8_t>(std::move(dev), count);
+    }
+    bool wide() const { return wide_; }
+    DeviceBuffer<uint8_t> &narrow() { return b8_; }
+    uint8_t *p8() const { return b8_.get(); }
+    uint16_t *p16() const { return b16_.get(); }
+    std::vector<uint8_t> to_host8() const {
+        if (wide_) throw VqError::InvalidParameter("codes above 256 centroids are 16 bits wide");
+        return b8_.to_host();
+    }
+    std::vector<uint16_t> to_host16() const {
+        if (wide_) return b16_.to_host();
+        const std::vector<uint8_t> v = b8_.to_host();
+        return std::vector<uint16_t>(v.begin(), v.end());
+    }
+
+private:
+    bool wide_ = false;
+    DeviceBuffer<uint8_t> b8_;
+    DeviceBuffer<uint16_t> b16_;
+};
+
+inline int32_t abi_assign(vq_ctx *c, int32_t metric, const float *x, size_t n, size_t ld, size_t m, size_t sd,
+                          size_t k, const float *cb, const DeviceCodes &codes) {
+    return codes.wide() ? vq_assign_u16(c, metric, x, (int64_t)n, (int64_t)ld, (int32_t)m, (int32_t)sd, (int32_t)k,
+                                        cb, codes.p16())
+                        : vq_assign(c, metric, x, (int64_t)n, (int64_t)ld, (int32_t)m, (int32_t)sd, (int32_t)k, cb,
+                                    codes.p8());
+}
+inline int32_t abi_decode_f16(vq_ctx *c, const DeviceCodes &codes, size_t n, size_t m, size_t sd, size_t k,
+                              const float *cb, uint16_t *out) {
+    return codes.wide() ? vq_decode_f16_u16(c, codes.p16(), (int64_t)n, (int32_t)m, (int32_t)sd, (int32_t)k, cb, out)
+                        : vq_decode_f16(c, codes.p8(), (int64_t)n, (int32_t)m, (int32_t)sd, (int32_t)k, cb, out);
+}
+inline int32_t abi_decode_f32(vq_ctx *c, const DeviceCodes &codes, size_t n, size_t m, size_t sd, size_t k,
+                              const float *cb, float *out) {
+    return codes.wide() ? vq_decode_f32_u16(c, codes.p16(), (int64_t)n, (int32_t)m, (int32_t)sd, (int32_t)k, cb, out)
+                        : vq_decode_f32(c, codes.p8(), (int64_t)n, (int32_t)m, (int32_t)sd, (int32_t)k, cb, out);
+}
+
 // `&[Vector<f32>]` as the device wants it: one row-major buffer.  The reference's shape — one
 // heap allocation per vector (src/vector.rs:150-152) — converts implicitly: packed once, lengths
 // checked.  Rows that are contiguous already (a matrix of another library, a memory-mapped file)
@@ -353,28 +402,18 @@ public:
         const float *flat = vectors.data();
         DeviceBuffer<float> dx(dev_, n * dim);
         dx.upload(flat, dx.size());
-        DeviceBuffer<uint8_t> dcodes(dev_, n * m_);
+        DeviceCodes dcodes(dev_, n * m_, k_);
         DeviceBuffer<uint16_t> dout(dev_, n * dim);
-        dev_->check(vq_assign(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim, (int32_t)m_,
-                              (int32_t)sub_dim_, (int32_t)k_, codebooks_.get(), dcodes.get()));
-        dev_->check(vq_decode_f16(dev_->ctx(), dcodes.get(), (int64_t)n, (int32_t)m_, (int32_t)sub_dim_,
-                                  (int32_t)k_, codebooks_.get(), dout.get()));
+        dev_->check(abi_assign(dev_->ctx(), distance_.abi_metric(), dx.get(), n, dim, m_, sub_dim_, k_,
+                               codebooks_.get(), dcodes));
+        dev_->check(abi_decode_f16(dev_->ctx(), dcodes, n, m_, sub_dim_, k_, codebooks_.get(), dout.get()));
         return dout.to_host();
     }
 
-    // The integer codes the reference keeps only as `best_index` (src/pq.rs:166-174): n x m bytes.
-    std::vector<uint8_t> encode(const Rows &vectors) const {
-        size_t dim = sub_dim_ * m_, n = vectors.size();
-        if (n == 0) return {};
-        vectors.expect_dim(dim);
-        const float *flat = vectors.data();
-        DeviceBuffer<float> dx(dev_, n * dim);
-        dx.upload(flat, dx.size());
-        DeviceBuffer<uint8_t> dcodes(dev_, n * m_);
-        dev_->check(vq_assign(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim, (int32_t)m_,
-                              (int32_t)sub_dim_, (int32_t)k_, codebooks_.get(), dcodes.get()));
-        return dcodes.to_host();
-    }
+    // The integer codes the reference keeps only as `best_index` (src/pq.rs:166-174): n x m bytes
+    // (k <= 256), or 16 bits each for any k.
+    std::vector<uint8_t> encode(const Rows &vectors) const { return encode_device(vectors).to_host8(); }
+    std::vector<uint16_t> encode16(const Rows &vectors) const { return encode_device(vectors).to_host16(); }
 
     std::vector<float> codebooks() const { return codebooks_.to_host(); }  // m*k*sub_dim
     size_t m() const { return m_; }
@@ -382,6 +421,19 @@ public:
     size_t sub_dim() const { return sub_dim_; }
 
 private:
+    DeviceCodes encode_device(const Rows &vectors) const {
+        size_t dim = sub_dim_ * m_, n = vectors.size();
+        if (n == 0) return DeviceCodes();
+        vectors.expect_dim(dim);
+        const float *flat = vectors.data();
+        DeviceBuffer<float> dx(dev_, n * dim);
+        dx.upload(flat, dx.size());
+        DeviceCodes dcodes(dev_, n * m_, k_);
+        dev_->check(abi_assign(dev_->ctx(), distance_.abi_metric(), dx.get(), n, dim, m_, sub_dim_, k_,
+                               codebooks_.get(), dcodes));
+        dev_->check(vq_ctx_sync(dev_->ctx()));
+        return dcodes;
+    }
     std::shared_ptr<Device> dev_;
     DeviceBuffer<float> codebooks_;
     size_t sub_dim_ = 0, m_ = 0, k_ = 0;
@@ -420,7 +472,7 @@ public:
         }
         vq_ctx *c = dev->ctx();
         DeviceBuffer<float> dx(dev, n * dim), drot(dev, n * dim), drec(dev, n * dim);
-        DeviceBuffer<uint8_t> dcodes(dev, n * m);
+        DeviceCodes dcodes(dev, n * m, k);
         dx.upload(flat, dx.size());
         dev->check(vq_copy_f32(c, drot.get(), dx.get(), (int64_t)(n * dim)));  // opq.rs:121
         q.codebooks_ = DeviceBuffer<float>(dev, m * k * sd);
@@ -432,10 +484,8 @@ public:
             dev->check(vq_lbg_fit(c, drot.get(), (int64_t)n, (int64_t)dim, (int32_t)m, (int32_t)sd, (int32_t)k,
                                   (int32_t)max_iters, streams->init.data(), streams->reseed.data(),
                                   streams->n_reseed, q.codebooks_.get(), nullptr, nullptr));  // 127-142
-            dev->check(vq_assign(c, metric, drot.get(), (int64_t)n, (int64_t)dim, (int32_t)m, (int32_t)sd,
-                                 (int32_t)k, q.codebooks_.get(), dcodes.get()));                // 146-163
-            dev->check(vq_decode_f32(c, dcodes.get(), (int64_t)n, (int32_t)m, (int32_t)sd, (int32_t)k,
-                                     q.codebooks_.get(), drec.get()));                            // 164-167
+            dev->check(abi_assign(c, metric, drot.get(), n, dim, m, sd, k, q.codebooks_.get(), dcodes));  // 146-163
+            dev->check(abi_decode_f32(c, dcodes, n, m, sd, k, q.codebooks_.get(), drec.get()));         // 164-167
             dev->check(vq_cross_cov(c, drec.get(), drot.get(), (int64_t)n, (int32_t)dim, A.data())); // 172-179
             for (double &v : A) v = (double)(float)v;  // the reference's A is a DMatrix<f32>
             // 180-183 (the library runs the SVD on the device while its kernel takes the size,
@@ -480,16 +530,19 @@ public:
             vectors.expect_dim(dim_);
             return {};
         }
-        DeviceBuffer<uint8_t> dcodes = encode_device(vectors);
+        DeviceCodes dcodes = encode_device(vectors);
         DeviceBuffer<uint16_t> dout(dev_, n * dim_);
-        dev_->check(vq_decode_f16(dev_->ctx(), dcodes.get(), (int64_t)n, (int32_t)m_, (int32_t)sub_dim_,
-                                  (int32_t)k_, codebooks_.get(), dout.get()));
+        dev_->check(abi_decode_f16(dev_->ctx(), dcodes, n, m_, sub_dim_, k_, codebooks_.get(), dout.get()));
         return dout.to_host();
     }
 
     std::vector<uint8_t> encode(const Rows &vectors) const {
         if (vectors.empty() || !trained_) return {};
-        return encode_device(vectors).to_host();
+        return encode_device(vectors).to_host8();
+    }
+    std::vector<uint16_t> encode16(const Rows &vectors) const {  // any k
+        if (vectors.empty() || !trained_) return {};
+        return encode_device(vectors).to_host16();
     }
 
     std::vector<float> codebooks() const { return trained_ ? codebooks_.to_host() : std::vector<float>(); }
@@ -500,17 +553,17 @@ public:
     size_t sub_dim() const { return sub_dim_; }
 
 private:
-    DeviceBuffer<uint8_t> encode_device(const Rows &vectors) const {
+    DeviceCodes encode_device(const Rows &vectors) const {
         size_t n = vectors.size();
         vectors.expect_dim(dim_);
         const float *flat = vectors.data();
         DeviceBuffer<float> dx(dev_, n * dim_), dy(dev_, n * dim_);
         dx.upload(flat, dx.size());
-        DeviceBuffer<uint8_t> dcodes(dev_, n * m_);
+        DeviceCodes dcodes(dev_, n * m_, k_);
         vq_ctx *c = dev_->ctx();
         dev_->check(vq_rotate(c, dx.get(), (int64_t)n, (int64_t)dim_, (int32_t)dim_, d_rotation_.get(), dy.get()));
-        dev_->check(vq_assign(c, distance_.abi_metric(), dy.get(), (int64_t)n, (int64_t)dim_, (int32_t)m_,
-                              (int32_t)sub_dim_, (int32_t)k_, codebooks_.get(), dcodes.get()));
+        dev_->check(abi_assign(c, distance_.abi_metric(), dy.get(), n, dim_, m_, sub_dim_, k_, codebooks_.get(),
+                               dcodes));
         dev_->check(vq_ctx_sync(c));
         return dcodes;
     }
@@ -552,7 +605,7 @@ public:
         }
         vq_ctx *c = dev->ctx();
         DeviceBuffer<float> dx(dev, n * dim), dres(dev, n * dim);
-        DeviceBuffer<uint8_t> dcodes(dev, n + 16);
+        DeviceCodes dcodes(dev, n + 16, k);
         dx.upload(flat, dx.size());
         dev->check(vq_copy_f32(c, dres.get(), dx.get(), (int64_t)(n * dim)));  // rvq.rs:103
         q.codebooks_ = DeviceBuffer<float>(dev, std::max<size_t>(stages * k * dim, 1));
@@ -566,12 +619,14 @@ public:
                                   nullptr, nullptr));  // rvq.rs:107
             ++produced;
             if (k < 2)  // rvq.rs:113-115
-                dcodes.upload(zeros.data(), n);
+                dcodes.narrow().upload(zeros.data(), n);
             else
-                dev->check(vq_assign(c, metric, dres.get(), (int64_t)n, (int64_t)dim, 1, (int32_t)dim, (int32_t)k,
-                                     cb, dcodes.get()));  // rvq.rs:116-125
-            dev->check(vq_residual_sub(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)k, cb,
-                                       dcodes.get()));  // rvq.rs:127
+                dev->check(abi_assign(c, metric, dres.get(), n, dim, 1, dim, k, cb, dcodes));  // rvq.rs:116-125
+            dev->check(dcodes.wide()
+                           ? vq_residual_sub_u16(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)k, cb,
+                                                 dcodes.p16())
+                           : vq_residual_sub(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)k, cb,
+                                             dcodes.p8()));  // rvq.rs:127
             if (epsilon > 0.f) {  // a mean norm is never below a non-positive (or NaN) threshold
                 float avg = 0.f;
                 dev->check(vq_mean_l2norm(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, &avg));  // 131-138
@@ -592,19 +647,27 @@ public:
         return unpack_f16(quantize_batch_flat(vectors, codes), vectors.size(), dim_);
     }
 
-    std::vector<uint16_t> quantize_batch_flat(const Rows &vectors, std::vector<uint8_t> *codes = nullptr) const {
+    // codes: n x stages bytes (k <= 256 only); codes16: the same 16 bits wide, any k
+    std::vector<uint16_t> quantize_batch_flat(const Rows &vectors, std::vector<uint8_t> *codes = nullptr,
+                                              std::vector<uint16_t> *codes16 = nullptr) const {
         size_t n = vectors.size();
         if (n == 0) return {};
         vectors.expect_dim(dim_);
         const float *flat = vectors.data();
         DeviceBuffer<float> dx(dev_, n * dim_);
         dx.upload(flat, dx.size());
-        DeviceBuffer<uint8_t> dcodes(dev_, std::max<size_t>(n * stages_, 1));
+        DeviceCodes dcodes(dev_, std::max<size_t>(n * stages_, 1), k_);
         DeviceBuffer<uint16_t> dout(dev_, n * dim_);
-        dev_->check(vq_rvq_encode(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim_,
-                                  (int32_t)dim_, (int32_t)stages_, (int32_t)std::max<size_t>(k_, 1),
-                                  codebooks_.get(), epsilon_, dcodes.get(), nullptr, dout.get()));
-        if (codes) *codes = dcodes.to_host();
+        const int32_t k = (int32_t)std::max<size_t>(k_, 1);
+        dev_->check(dcodes.wide()
+                        ? vq_rvq_encode_u16(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim_,
+                                            (int32_t)dim_, (int32_t)stages_, k, codebooks_.get(), epsilon_,
+                                            dcodes.p16(), nullptr, dout.get())
+                        : vq_rvq_encode(dev_->ctx(), distance_.abi_metric(), dx.get(), (int64_t)n, (int64_t)dim_,
+                                        (int32_t)dim_, (int32_t)stages_, k, codebooks_.get(), epsilon_, dcodes.p8(),
+                                        nullptr, dout.get()));
+        if (codes) *codes = dcodes.to_host8();
+        if (codes16) *codes16 = dcodes.to_host16();
         return dout.to_host();
     }
 

@@ -200,6 +200,22 @@ int vqh_encode(void *obj, const float *x, int64_t n, int64_t dim, uint8_t *codes
     });
 }
 
+// the same 16 bits wide: any k up to 65536
+int vqh_encode16(void *obj, const float *x, int64_t n, int64_t dim, uint16_t *codes) {
+    return guarded([&] {
+        Obj *o = (Obj *)obj;
+        auto rows = rows_of(x, n, dim);
+        std::vector<uint16_t> c;
+        switch (o->kind) {
+        case 1: c = o->pq->encode16(rows); break;
+        case 2: c = o->opq->encode16(rows); break;
+        case 3: o->rvq->quantize_batch_flat(rows, nullptr, &c); break;
+        default: throw vq::VqError::InvalidParameter("TSVQ has leaves, not codes");
+        }
+        std::memcpy(codes, c.data(), c.size() * sizeof(uint16_t));
+    });
+}
+
 int vqh_leaves(void *obj, const float *x, int64_t n, int64_t dim, int32_t *leaves) {
     return guarded([&] {
         Obj *o = (Obj *)obj;
