@@ -36,7 +36,7 @@ PEAK_HBM_GBS = 8000.0
 PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X published dense bf16 matrix peak
 # rocprofv3 FETCH_SIZE / WRITE_SIZE of one LBG launch of k_assign_mfma_bf (KiB per dispatch), scaled by
 # the plain copy kernel (FETCH x 2.000, WRITE x 1.000): profiles/pq_fit_encode_1Mx128.md
-MEASURED_ASSIGN_TRAFFIC_BYTES = int((262981.0 * 2.000 + 12193.8 * 1.000) * 1024)
+MEASURED_ASSIGN_TRAFFIC_BYTES = int((263610.0 * 2.000 + 12207.0 * 1.000) * 1024)
 
 
 def log(*a):
@@ -46,8 +46,8 @@ def log(*a):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--rows", type=int, default=N_ROWS, help="rows of the workload (default 1M)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run the plain copy kernel on the workload's rows (3 launches): the "
