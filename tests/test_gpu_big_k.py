@@ -219,3 +219,37 @@ def test_opq_class_above_256_first_iteration_matches_oracle(vq):
     rec = np.concatenate([got.codebooks()[s][codes[:, s]] for s in range(m)], 1)
     assert np.array_equal(got.quantize_batch(x).view(np.uint16), rec.astype(np.float16).view(np.uint16))
     assert ((y - rec) ** 2).mean() < ((y - y.mean(0)) ** 2).mean()
+
+
+# ---- seeded random shapes ------------------------------------------------------------------------
+@pytest.mark.parametrize("seed", range(32))
+def test_random_shapes_above_256(ctx, seed):
+    """Encode under a random metric and two LBG iterations on a random shape with 257..1500
+    centroids, against the oracle bit for bit."""
+    rng = np.random.default_rng(9000 + seed)
+    sd = int(rng.choice([1, 2, 3, 5, 8, 8, 8, 16, 24, 32]))
+    m = int(rng.choice([1, 2, 3, 4, 8]))
+    k = int(rng.integers(257, 1501))
+    n = int(rng.integers(k, k + 4000))
+    kind = ["normal", "grid", "uniform", "blobs", "offset", "dup"][seed % 6]
+    dim = m * sd
+    if kind == "offset":      # far from the origin: cancellation in the matrix-core scores
+        x = (1000.0 + rng.standard_normal((n, dim))).astype(F)
+    elif kind == "dup":       # duplicate rows -> duplicate centroids, exact ties
+        base = rng.standard_normal((max(n // 7, 1), dim)).astype(F)
+        x = base[rng.integers(0, base.shape[0], n)]
+    else:
+        x = make_rows(rng, n, dim, kind)
+    metric = int(rng.integers(0, 4))
+    ctx.set_assign_path(seed % 2)
+    init, reseed = data.index_streams(n, m, k, 2, seed=seed)
+    want = O.pq_fit(x, m, k, 2, init, reseed)
+    assert want["rc"] == 0
+    dx = ctx.to_device(x)
+    dcb = ctx.empty((m, k, sd), F)
+    it, used = ctx.lbg_fit(dx, n, dim, m, sd, k, 2, init, reseed, dcb)
+    assert np.array_equal(it, want["iters"]) and np.array_equal(used, want["reseeds"])
+    assert np.array_equal(dcb.download().view(np.uint32), want["codebooks"].view(np.uint32))
+    dcodes = ctx.empty((n, m), np.uint16)
+    ctx.assign_u16(metric, dx, n, dim, m, sd, k, dcb, dcodes)
+    assert np.array_equal(dcodes.download(), O.pq_encode(metric, x, want["codebooks"]).astype(np.uint16))
