@@ -28,7 +28,10 @@ struct vq_ctx {
     DevBuf flags, tables, hist, seg, part_sum, perm, leaf_desc, leaf_sum, codes, idx, reseed, cnorm;
     DevBuf tsvq_sq;              // TSVQ build: squared deviations of a level
     DevBuf tsvq_split;           // TSVQ build: the small per-level tables of the nodes being split
-    DevBuf tsvq_level;           // TSVQ build: leaf descriptors and leaf sums of the level's node means
+    DevBuf tsvq_level;           // TSVQ build: the level's uploaded tables and the leaf sums of its node means
+    DevBuf tsvq_means;           // TSVQ build: the means of all nodes, read back once at the end
+    void *tsvq_pin = nullptr;    // TSVQ build: page-locked staging of a level's tables and decisions
+    size_t tsvq_pin_cap = 0;
     DevBuf tsvq_gsum, tsvq_guess, tsvq_maps;  // per group of 32 squares: sum, binade guess, integer maps
     int tsvq_var_path = 0;       // 0 = composed integer maps, 1 = one chain of adds per column
     DevBuf mfma_tab, mfma_list, mfma_stat;  // tables, re-check list and counters of the matrix-core assignment

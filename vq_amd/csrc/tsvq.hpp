@@ -80,6 +80,29 @@ static __global__ void __launch_bounds__(256) k_seg_mean(float *__restrict__ lea
     out[(out_first + g) * sd + t] = ls[0] / __uint2float_rn(info.z);
 }
 
+// The same tree for the levels near the root, where a segment has hundreds of leaves and there are
+// few segments: one workgroup per (segment, 8 components), the leaf sums in LDS, the pairs of a tree
+// level side by side — the same additions as k_seg_mean, which walks them in one thread.
+constexpr int kMeanWgLeaves = 1024;
+static __global__ void __launch_bounds__(256) k_seg_mean_wg(const float *__restrict__ leaf_sum,
+                                                            const uint4 *__restrict__ seg_info, int sd,
+                                                            float *__restrict__ out, int64_t out_first) {
+    __shared__ float tree[kMeanWgLeaves][8];
+    const int g = blockIdx.x, t = threadIdx.x & 7, q = threadIdx.x >> 3;
+    const int c = blockIdx.y * 8 + t;
+    const uint4 info = seg_info[g];
+    const uint32_t nl = 1u << info.y;  // <= kMeanWgLeaves (the host checks)
+    const float *ls = leaf_sum + (size_t)info.x * sd + (c < sd ? c : 0);
+    for (uint32_t leaf = q; leaf < nl; leaf += 32) tree[leaf][t] = ls[(size_t)leaf * sd];
+    __syncthreads();
+    for (uint32_t h = 1; h < nl; h <<= 1) {
+        const uint32_t npairs = nl / (2 * h);
+        for (uint32_t qi = q; qi < npairs; qi += 32) tree[2 * h * qi][t] = tree[2 * h * qi][t] + tree[2 * h * qi + h][t];
+        __syncthreads();
+    }
+    if (q == 0 && c < sd) out[(out_first + g) * sd + c] = tree[0][t] / __uint2float_rn(info.z);
+}
+
 // One lane per (segment, dimension): sequential sum of squared deviations in row order.
 // seg_range[g] = {lo, hi} positions in perm; mean of segment g at means[(first + g) * dim].
 static __global__ void __launch_bounds__(64) k_seg_variance(const uint32_t *__restrict__ perm,

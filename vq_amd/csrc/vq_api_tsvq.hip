@@ -140,10 +140,29 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     std::vector<LevelMeans> level_means;  // device means of every level, read back after the last one
     std::vector<uint2> desc;
     std::vector<uint4> info;
+    // The means of all nodes in one workspace buffer when the deepest possible tree stays small (nodes
+    // are numbered level by level, so a level's means are one run of it); else an allocation per level.
+    const uint64_t max_nodes = std::min<uint64_t>(2 * (uint64_t)n - 1, (2ull << std::min(max_depth, 40)) - 1);
+    const bool means_arena = max_nodes * (uint64_t)dim * sizeof(float) <= (256ull << 20);
+    if (means_arena) VQ_TRY(ensure(ctx, ctx->tsvq_means, sizeof(float) * (size_t)max_nodes * dim));
     auto free_means = [&]() {
-        for (auto &lm : level_means) (void)hipFree(lm.d);
+        if (!means_arena)
+            for (auto &lm : level_means) (void)hipFree(lm.d);
         level_means.clear();
     };
+    // A level's small tables go up in ONE copy from page-locked memory and its decisions come back in
+    // one: the host waits for the GPU once per level, so the staging area is free again by then.
+    auto pinned = [&](size_t bytes) -> int32_t {
+        if (bytes <= ctx->tsvq_pin_cap) return VQ_OK;
+        if (ctx->tsvq_pin) (void)hipHostFree(ctx->tsvq_pin);
+        ctx->tsvq_pin = nullptr;
+        ctx->tsvq_pin_cap = 0;
+        const size_t want = bytes + bytes / 2 + 4096;
+        VQ_HIP(ctx, hipHostMalloc(&ctx->tsvq_pin, want, hipHostMallocDefault));
+        ctx->tsvq_pin_cap = want;
+        return VQ_OK;
+    };
+    auto pad = [](size_t z) { return (z + 255) & ~(size_t)255; };
 
     while (!level.empty()) {
         const int nseg = (int)level.size();
@@ -167,11 +186,18 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             }
         }
         const size_t nleaves = desc.size();
-        // The level's leaf tables live in a grow-only arena of the context; its node means stay in
-        // an allocation of their own until the end of the build, when all means are read back at
-        // once — nothing here waits for the GPU: which nodes split depends on their sizes only.
-        void *d_desc = nullptr, *d_info = nullptr, *d_lsum = nullptr, *d_means = nullptr;
-        auto free_level = [&]() {};
+        // ---- which nodes split (src/tsvq.rs:78): their sizes decide, nothing waits for the GPU ----
+        std::vector<int> split;  // indices into level
+        if (depth_left > 0)
+            for (int g = 0; g < nseg; ++g)
+                if (level[g].hi - level[g].lo > 1) split.push_back(g);
+        const int ns = (int)split.size();
+        std::vector<uint2> range(ns);
+        for (int i = 0; i < ns; ++i) range[i] = make_uint2(level[split[i]].lo, level[split[i]].hi);
+        // The level's tables live in a grow-only arena of the context; its node means stay on the
+        // device until the end of the build, when all means are read back at once.
+        void *d_desc = nullptr, *d_info = nullptr, *d_range = nullptr, *d_split = nullptr, *d_lsum = nullptr,
+             *d_means = nullptr;
 #define LV_HIP(call)                                                                              \
     do {                                                                                          \
         hipError_t e__ = (call);                                                                  \
@@ -184,47 +210,56 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                                      __LINE__));                                                  \
         }                                                                                         \
     } while (0)
+        // uploaded tables first (one contiguous run: descriptors, node info, ranges, split indices)
+        const size_t up_sizes[4] = {sizeof(uint2) * nleaves, sizeof(uint4) * (size_t)nseg, sizeof(uint2) * (size_t)ns,
+                                    sizeof(int) * (size_t)ns};
+        const void *up_src[4] = {desc.data(), info.data(), range.data(), split.data()};
+        size_t up_bytes = 0;
+        for (size_t z : up_sizes) up_bytes += pad(z);
+        const size_t down_bytes = 3 * sizeof(uint32_t) * (size_t)ns;
         {
-            const size_t sizes[3] = {sizeof(uint2) * nleaves, sizeof(uint4) * (size_t)nseg, sizeof(float) * nleaves * dim};
-            void **ptrs[3] = {&d_desc, &d_info, &d_lsum};
-            size_t total = 0;
-            for (size_t z : sizes) total += (z + 255) & ~(size_t)255;
-            const int32_t rc = ensure(ctx, ctx->tsvq_level, total);
+            void **ptrs[5] = {&d_desc, &d_info, &d_range, &d_split, &d_lsum};
+            const size_t total = up_bytes + pad(sizeof(float) * nleaves * dim);
+            int32_t rc = ensure(ctx, ctx->tsvq_level, total);
+            if (rc == VQ_OK) rc = pinned(up_bytes + pad(down_bytes));
             if (rc != VQ_OK) {
                 free_means();
                 (void)hipFree(rp_tmp);
                 return cleanup_fail(rc);
             }
-            char *at = (char *)ctx->tsvq_level.p;
-            for (int z = 0; z < 3; ++z) {
+            char *at = (char *)ctx->tsvq_level.p, *h = (char *)ctx->tsvq_pin;
+            for (int z = 0; z < 4; ++z) {
                 *ptrs[z] = at;
-                at += (sizes[z] + 255) & ~(size_t)255;
+                if (up_sizes[z]) memcpy(h, up_src[z], up_sizes[z]);
+                at += pad(up_sizes[z]);
+                h += pad(up_sizes[z]);
             }
+            d_lsum = at;
         }
-        LV_HIP(hipMalloc(&d_means, sizeof(float) * (size_t)nseg * dim));
         const int32_t first_node = level[0].node;
+        if (means_arena)
+            d_means = (float *)ctx->tsvq_means.p + (size_t)first_node * dim;
+        else
+            LV_HIP(hipMalloc(&d_means, sizeof(float) * (size_t)nseg * dim));
         level_means.push_back({d_means, first_node, nseg});
-        LV_HIP(hipMemcpyAsync(d_desc, desc.data(), sizeof(uint2) * nleaves, hipMemcpyHostToDevice, st));
-        LV_HIP(hipMemcpyAsync(d_info, info.data(), sizeof(uint4) * nseg, hipMemcpyHostToDevice, st));
+        LV_HIP(hipMemcpyAsync(ctx->tsvq_level.p, ctx->tsvq_pin, up_bytes, hipMemcpyHostToDevice, st));
         hipLaunchKernelGGL(vq::k_seg_leafsum, dim3(cdiv((int64_t)nleaves * dim, 256)), dim3(256), 0, st, perm,
                            (const uint2 *)d_desc, (int64_t)nleaves, d_x, ld, dim, (float *)d_lsum);
-        hipLaunchKernelGGL(vq::k_seg_mean, dim3(cdiv((int64_t)nseg * dim, 256)), dim3(256), 0, st,
-                           (float *)d_lsum, (const uint4 *)d_info, nseg, dim, (float *)d_means, (int64_t)0);
+        int max_dep = 0;
+        for (int g = 0; g < nseg; ++g) max_dep = std::max(max_dep, (int)info[g].y);
+        if (max_dep >= 5 && (1 << max_dep) <= vq::kMeanWgLeaves && nseg <= 64)  // few segments of many leaves
+            hipLaunchKernelGGL(vq::k_seg_mean_wg, dim3((unsigned)nseg, cdiv(dim, 8)), dim3(256), 0, st,
+                               (const float *)d_lsum, (const uint4 *)d_info, dim, (float *)d_means, (int64_t)0);
+        else
+            hipLaunchKernelGGL(vq::k_seg_mean, dim3(cdiv((int64_t)nseg * dim, 256)), dim3(256), 0, st,
+                               (float *)d_lsum, (const uint4 *)d_info, nseg, dim, (float *)d_means, (int64_t)0);
         LV_HIP(hipGetLastError());
 
-        // ---- which nodes split (src/tsvq.rs:78) ---------------------------------------------
-        std::vector<int> split;  // indices into level
-        if (depth_left > 0)
-            for (int g = 0; g < nseg; ++g)
-                if (level[g].hi - level[g].lo > 1) split.push_back(g);
         if (split.empty()) break;
-        const int ns = (int)split.size();
-        std::vector<uint2> range(ns);
-        for (int i = 0; i < ns; ++i) range[i] = make_uint2(level[split[i]].lo, level[split[i]].hi);
-        // the level's small tables: one grow-only arena of the context instead of nine allocations
-        void *d_range = nullptr, *d_smeans = nullptr, *d_var = nullptr, *d_sdim = nullptr, *d_mids = nullptr,
-             *d_median = nullptr, *d_nleft = nullptr, *d_sel = nullptr, *d_hist = nullptr, *d_split = nullptr;
-        auto free_split = [&]() {};
+        // the level's small tables: one grow-only arena of the context instead of nine allocations;
+        // split dimension, median and left count of every node side by side, so that one copy returns them
+        void *d_smeans = nullptr, *d_var = nullptr, *d_down = nullptr, *d_mids = nullptr, *d_sel = nullptr,
+             *d_hist = nullptr;
 #define SP_HIP(call)                                                                              \
     do {                                                                                          \
         hipError_t e__ = (call);                                                                  \
@@ -239,12 +274,10 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     } while (0)
         {
             const size_t cap = (size_t)std::max(ns, 1024);  // sized once for the usual depths
-            const size_t sizes[10] = {sizeof(uint2) * cap, sizeof(float) * cap * dim, sizeof(float) * cap * dim,
-                                      sizeof(int) * cap, sizeof(float) * 2 * cap, sizeof(float) * cap,
-                                      sizeof(uint32_t) * cap, sizeof(vq::SegSelect) * 2 * cap,
-                                      sizeof(uint32_t) * 512 * cap, sizeof(int) * cap};
-            void **ptrs[10] = {&d_range, &d_smeans, &d_var, &d_sdim, &d_mids, &d_median, &d_nleft, &d_sel, &d_hist,
-                               &d_split};
+            const size_t sizes[6] = {sizeof(float) * cap * dim, sizeof(float) * cap * dim, 3 * sizeof(uint32_t) * cap,
+                                     sizeof(float) * 2 * cap, sizeof(vq::SegSelect) * 2 * cap,
+                                     sizeof(uint32_t) * 512 * cap};
+            void **ptrs[6] = {&d_smeans, &d_var, &d_down, &d_mids, &d_sel, &d_hist};
             size_t total = 0;
             for (size_t z : sizes) total += (z + 255) & ~(size_t)255;
             const int32_t rc = ensure(ctx, ctx->tsvq_split, total);
@@ -254,14 +287,15 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                 return cleanup_fail(rc);
             }
             char *at = (char *)ctx->tsvq_split.p;
-            for (int z = 0; z < 10; ++z) {
+            for (int z = 0; z < 6; ++z) {
                 *ptrs[z] = at;
                 at += (sizes[z] + 255) & ~(size_t)255;
             }
         }
-        SP_HIP(hipMemcpyAsync(d_range, range.data(), sizeof(uint2) * ns, hipMemcpyHostToDevice, st));
+        int *d_sdim = (int *)d_down;
+        float *d_median = (float *)d_down + ns;
+        uint32_t *d_nleft = (uint32_t *)d_down + 2 * (size_t)ns;
         // the means of the splitting nodes, compacted on the device
-        SP_HIP(hipMemcpyAsync(d_split, split.data(), sizeof(int) * ns, hipMemcpyHostToDevice, st));
         hipLaunchKernelGGL(vq::k_gather_means, dim3(cdiv((int64_t)ns * dim, 256)), dim3(256), 0, st,
                            (const float *)d_means, (const int *)d_split, ns, dim, (float *)d_smeans);
         // per-dimension sums of squared deviations (src/tsvq.rs:88-99)
@@ -337,13 +371,12 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         hipLaunchKernelGGL(vq::k_seg_partition, dim3(cdiv(n, 256)), dim3(256), 0, st, perm, n,
                            (const uint2 *)d_range, ns, flags, scan, perm2, (uint32_t *)d_nleft);
         SP_HIP(hipGetLastError());
-        std::vector<uint32_t> nleft(ns);
-        std::vector<int> sdim(ns);
-        std::vector<float> median(ns);
-        SP_HIP(hipMemcpyAsync(nleft.data(), d_nleft, sizeof(uint32_t) * ns, hipMemcpyDeviceToHost, st));
-        SP_HIP(hipMemcpyAsync(sdim.data(), d_sdim, sizeof(int) * ns, hipMemcpyDeviceToHost, st));
-        SP_HIP(hipMemcpyAsync(median.data(), d_median, sizeof(float) * ns, hipMemcpyDeviceToHost, st));
+        char *h_down = (char *)ctx->tsvq_pin + up_bytes;
+        SP_HIP(hipMemcpyAsync(h_down, d_down, down_bytes, hipMemcpyDeviceToHost, st));
         SP_HIP(hipStreamSynchronize(st));
+        const int *sdim = (const int *)h_down;
+        const float *median = (const float *)h_down + ns;
+        const uint32_t *nleft = (const uint32_t *)h_down + 2 * (size_t)ns;
         std::swap(perm, perm2);
 
         // ---- children (src/tsvq.rs:126-141) ---------------------------------------------------
@@ -373,9 +406,13 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     rp_tmp = nullptr;
     T->n_nodes = (int32_t)T->h_left.size();
     T->h_centroids.resize((size_t)T->n_nodes * dim);
-    for (auto &lm : level_means)
-        LV_HIP(hipMemcpyAsync(T->h_centroids.data() + (size_t)lm.first_node * dim, lm.d,
-                              sizeof(float) * (size_t)lm.nseg * dim, hipMemcpyDeviceToHost, st));
+    if (means_arena)
+        LV_HIP(hipMemcpyAsync(T->h_centroids.data(), ctx->tsvq_means.p, sizeof(float) * (size_t)T->n_nodes * dim,
+                              hipMemcpyDeviceToHost, st));
+    else
+        for (auto &lm : level_means)
+            LV_HIP(hipMemcpyAsync(T->h_centroids.data() + (size_t)lm.first_node * dim, lm.d,
+                                  sizeof(float) * (size_t)lm.nseg * dim, hipMemcpyDeviceToHost, st));
     LV_HIP(hipStreamSynchronize(st));
     free_means();
 #undef LV_HIP
