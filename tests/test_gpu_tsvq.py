@@ -58,6 +58,8 @@ def assert_same_tree(got, want):
     (30000, 32, 9, "normal"),  # dim a multiple of 8: squares on the whole GPU, then the chains
     (12345, 128, 7, "normal"), # node sizes that are no multiples of 32
     (9000, 64, 13, "normal"),  # deep: levels with more than 2048 nodes take the lane-per-sum kernel
+    (400000, 16, 2, "normal"), # columns above 4096 groups: block sums before the guesses, runs of composed maps
+    (270001, 8, 4, "grid"),
     (5000, 24, 5, "grid"),     # dim 24, tied variances and medians
 ])
 def test_build_matches_oracle(ctx, n, dim, depth, kind):
@@ -137,7 +139,8 @@ def test_config5_shape_unit_rows_cosine_then_manhattan(ctx):
 
 
 @pytest.mark.parametrize("kind", ["constant_columns", "all_zero", "tiny", "huge", "mixed", "integers", "wide_range"])
-@pytest.mark.parametrize("n,dim,depth", [(70000, 8, 3), (20000, 128, 5), (33, 16, 2), (4097, 24, 4)])
+@pytest.mark.parametrize("n,dim,depth", [(70000, 8, 3), (20000, 128, 5), (33, 16, 2), (4097, 24, 4),
+                                         (300000, 8, 3)])  # the last: columns long enough for blocks and runs
 def test_variance_paths_agree_with_the_oracle_on_edge_data(ctx, kind, n, dim, depth):
     """The two ways of summing a node's squared deviations in row order (composed integer maps, one
     chain of adds per column) against the oracle's sequential sums, through the tree they decide:

@@ -33,6 +33,7 @@ struct vq_ctx {
     void *tsvq_pin = nullptr;    // TSVQ build: page-locked staging of a level's tables and decisions
     size_t tsvq_pin_cap = 0;
     DevBuf tsvq_gsum, tsvq_guess, tsvq_maps;  // per group of 32 squares: sum, binade guess, integer maps
+    DevBuf tsvq_bsum, tsvq_segmaps;           // per block of groups: f64 sum; per run of groups: composed map
     int tsvq_var_path = 0;       // 0 = composed integer maps, 1 = one chain of adds per column
     DevBuf mfma_tab, mfma_list, mfma_stat;  // tables, re-check list and counters of the matrix-core assignment
     int recheck_src = 0;         // where the last pass counted its undecided pairs: 1 mfma_stat, 2 mfma_list, 3 the fixed scratch

@@ -314,18 +314,57 @@ constexpr uint32_t kMapInvalid = 0xFFFFFFFFu;
 // guess code: exponent field of the lower candidate | two candidates | all terms zero | usable
 constexpr uint16_t kGuessOk = 0x8000u, kGuessTwo = 0x0100u, kGuessZero = 0x0200u;
 
-// grid (segments, dim / 4); 256 threads = 4 waves, one column each.
-static __global__ void __launch_bounds__(256) k_seg_chain_guess(const float *__restrict__ gsum,
-                                                               const uint2 *__restrict__ seg_range, int dim,
-                                                               uint16_t *__restrict__ guess) {
+// Long columns are cut into blocks of kGuessBlock groups that are guessed side by side: the f64 sum
+// of every block first (grid (segments, dim / 4, blocks); 4 waves, one column each), then a block's
+// prefix starts from the sum of the blocks before it.
+constexpr uint32_t kGuessBlock = 1024;
+static __global__ void __launch_bounds__(256) k_seg_chain_bsum(const float *__restrict__ gsum,
+                                                              const uint2 *__restrict__ seg_range, int dim,
+                                                              double *__restrict__ bsum) {
     const int g = blockIdx.x, lane = threadIdx.x & 63, c = blockIdx.y * 4 + (threadIdx.x >> 6);
     if (c >= dim) return;
     const uint2 range = seg_range[g];
     const uint32_t count = range.y - range.x, nP = (count + 31u) / 32u;
+    const uint32_t P0 = blockIdx.z * kGuessBlock;
+    if (P0 >= nP) return;
+    const size_t g0 = seg_group0(range, g);
+    float vin[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+        const uint32_t P = P0 + 64 * k + lane;
+        vin[k] = gsum[(g0 + (P < nP ? P : nP - 1)) * dim + c];
+    }
+    double acc = 0.0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) acc += (P0 + 64 * k + lane < nP) ? (double)vin[k] : 0.0;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+    if (lane == 0) bsum[((size_t)g * gridDim.z + blockIdx.z) * dim + c] = acc;
+}
+
+// grid (segments, dim / 4, blocks); 256 threads = 4 waves, one column each.  bsum == nullptr: one
+// block per column, whatever its length.
+static __global__ void __launch_bounds__(256) k_seg_chain_guess(const float *__restrict__ gsum,
+                                                               const uint2 *__restrict__ seg_range, int dim,
+                                                               const double *__restrict__ bsum,
+                                                               uint16_t *__restrict__ guess) {
+    const int g = blockIdx.x, lane = threadIdx.x & 63, c = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (c >= dim) return;
+    const uint2 range = seg_range[g];
+    const uint32_t count = range.y - range.x, nP_all = (count + 31u) / 32u;
     const size_t g0 = seg_group0(range, g);
     double carry = 0.0;
+    uint32_t P_first = 0, nP = nP_all;
+    if (bsum) {
+        P_first = blockIdx.z * kGuessBlock;
+        if (P_first >= nP_all) return;
+        nP = nP_all - P_first < kGuessBlock ? nP_all : P_first + kGuessBlock;
+        for (uint32_t b = lane; b < blockIdx.z; b += 64) carry += bsum[((size_t)g * gridDim.z + b) * dim + c];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) carry += __shfl_xor(carry, off);
+    }
     constexpr int R = 16;  // batches of 64 groups per round of loads (one memory round trip per round)
-    for (uint32_t P0 = 0; P0 < nP; P0 += 64 * R) {
+    for (uint32_t P0 = P_first; P0 < nP; P0 += 64 * R) {
         float vin[R];
 #pragma unroll
         for (int k = 0; k < R; ++k) {
@@ -441,13 +480,176 @@ static __global__ void __launch_bounds__(256) k_seg_chain_maps(const uint32_t *_
     }
 }
 
-// grid (segments, dim / 4); 256 threads = 4 waves, one column each.
+// The map of the lanes' groups composed over the wave: on return lane p holds the map of the groups
+// of lanes first .. p (lanes outside [first, last) supply the identity), as increments for an even
+// and for an odd start, saturated at 2^25.
+__device__ __forceinline__ void chain_scan_maps(uint32_t &a0, uint32_t &a1, int lane) {
+    const uint32_t cap = 1u << 25;
+    // left, then this lane's map: c_p = l_p + a_[(p + l_p) mod 2]; (0, 0) is the identity, which is what a
+    // lane outside the row supplies
+    auto after_left = [&](uint32_t l0, uint32_t l1) {
+        const uint32_t n0 = l0 + ((l0 & 1u) ? a1 : a0);        // start even: after l0 the parity is l0 & 1
+        const uint32_t n1 = l1 + (((l1 + 1u) & 1u) ? a1 : a0);  // start odd
+        a0 = n0 < cap ? n0 : cap;
+        a1 = n1 < cap ? n1 : cap;
+    };
+    after_left(row_shr<1>(a0, 0u), row_shr<1>(a1, 0u));
+    after_left(row_shr<2>(a0, 0u), row_shr<2>(a1, 0u));
+    after_left(row_shr<4>(a0, 0u), row_shr<4>(a1, 0u));
+    after_left(row_shr<8>(a0, 0u), row_shr<8>(a1, 0u));
+    uint32_t t0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 15), t1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 15);
+    if ((lane >> 4) == 1) after_left(t0, t1);
+    t0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 31), t1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 31);
+    if ((lane >> 4) == 2) after_left(t0, t1);
+    t0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 47), t1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 47);
+    if ((lane >> 4) == 3) after_left(t0, t1);
+}
+
+// Runs of kRunGroups consecutive groups of a long column get their maps composed ahead of the walk
+// (k_seg_chain_runs): a run is "clean" when every group has one guessed binade, the same in all of
+// them (groups of zeros fit any), and a usable map.  The walk then passes a clean run in one step
+// when S is in that binade at the run's start and does not leave it by the run's end — S never
+// decreases, so it is in the binade at every group in between and each group's map applies, which is
+// all the group-by-group walk checks.  Any other run is walked group by group as before.
+constexpr uint32_t kRunGroups = 256;
+constexpr uint32_t kRunClean = 0x80000000u, kRunAnyBinade = 0x40000000u;
+
+// Index of a segment's first run in the per-run table (runs of different segments never share one).
+__device__ __forceinline__ size_t seg_run0(const uint2 range, int g) {
+    return seg_group0(range, g) / kRunGroups + (size_t)g;
+}
+
+// grid (segments, dim / 4, ceil(groups / 1024)); 256 threads = 4 waves, one column each; a wave
+// composes four runs (16 batches of 64 groups, one round of loads).
+static __global__ void __launch_bounds__(256) k_seg_chain_runs(const uint2 *__restrict__ seg_range, int dim,
+                                                              const uint16_t *__restrict__ guess,
+                                                              const uint4 *__restrict__ maps,
+                                                              uint4 *__restrict__ runs) {
+    const int g = blockIdx.x, lane = threadIdx.x & 63, c = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (c >= dim) return;
+    const uint2 range = seg_range[g];
+    const uint32_t count = range.y - range.x, nP = (count + 31u) / 32u;
+    const uint32_t P0 = blockIdx.z * (4u * kRunGroups);
+    if (P0 >= nP) return;
+    const size_t g0 = seg_group0(range, g), r0 = seg_run0(range, g);
+    constexpr int R = 16;
+    uint16_t codeR[R];
+    uint4 mpR[R];
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        const uint32_t idx = P0 + 64u * k + lane;
+        const size_t at = (g0 + (idx < nP ? idx : nP - 1u)) * dim + c;
+        codeR[k] = guess[at];
+        mpR[k] = maps[at];
+    }
+    const uint32_t cap = 1u << 25;
+#pragma unroll
+    for (int run = 0; run < 4; ++run) {
+        const uint32_t Pr = P0 + run * kRunGroups;
+        if (Pr >= nP) break;  // uniform
+        uint32_t c0 = 0, c1 = 0, e = 0;
+        bool clean = true, any_binade = true;
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) {
+            const int k = 4 * run + k4;
+            const uint32_t base = Pr + 64u * k4;
+            const uint32_t left = base >= nP ? 0u : (nP - base < 64u ? nP - base : 64u);
+            if (left == 0u) break;  // uniform
+            const uint16_t code = codeR[k];
+            const uint4 mp = mpR[k];
+            const bool mine = (uint32_t)lane < left;
+            const bool zero = (code & kGuessZero) != 0;
+            const uint32_t elo = code & 255u;
+            const bool usable = (code & kGuessOk) &&
+                                (zero || (!(code & kGuessTwo) && mp.x != kMapInvalid && elo >= 30u && elo <= 250u));
+            if (__ballot(mine && !usable)) clean = false;
+            const unsigned long long binade = __ballot(mine && !zero);
+            if (binade) {
+                const uint32_t ef = (uint32_t)__builtin_amdgcn_readlane((int)elo, __ffsll((long long)binade) - 1);
+                if (any_binade) e = ef;
+                any_binade = false;
+                if (__ballot(mine && !zero && elo != e)) clean = false;
+            }
+            uint32_t a0 = (mine && !zero) ? (mp.x < cap ? mp.x : cap) : 0u;
+            uint32_t a1 = (mine && !zero) ? (mp.y < cap ? mp.y : cap) : 0u;
+            chain_scan_maps(a0, a1, lane);
+            const uint32_t b0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 63), b1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 63);
+            // the run so far, then this batch
+            const uint32_t n0 = c0 + ((c0 & 1u) ? b1 : b0), n1 = c1 + (((c1 + 1u) & 1u) ? b1 : b0);
+            c0 = n0 < cap ? n0 : cap;
+            c1 = n1 < cap ? n1 : cap;
+        }
+        if (lane == 0)
+            runs[(r0 + Pr / kRunGroups) * dim + c] =
+                make_uint4(c0, c1, (clean ? kRunClean : 0u) | (any_binade ? kRunAnyBinade : 0u) | e, 0u);
+    }
+}
+
+// One batch of up to 64 groups (lane = group base + lane) added to S, which is the same value in every
+// lane: runs of usable groups through their composed maps, any other group term by term.
+__device__ __forceinline__ void chain_batch(float &S, uint32_t base, uint32_t left, uint16_t code, uint4 mp,
+                                            const uint32_t *__restrict__ pm, uint32_t count,
+                                            const float *__restrict__ x, int64_t ld, int c, float mean_c, int lane) {
+    const uint32_t elo = code & 255u;
+    const bool zero = (code & kGuessZero) != 0;
+    uint32_t start = 0;  // groups of the batch already added
+    while (start < left) {
+        // S is +0, positive, +inf or a NaN; with the sign bit of a NaN eS is above every guess
+        const uint32_t Sb = __float_as_uint(S), eS = Sb >> 23;
+        const uint32_t s = (Sb & 0x7fffffu) | 0x800000u;  // S / u for a normal S
+        const bool is_lo = elo == eS, is_hi = (code & kGuessTwo) && elo + 1u == eS;
+        uint32_t a0 = is_lo ? mp.x : mp.z, a1 = is_lo ? mp.y : mp.w;
+        // a group of zeros keeps any finite S; another group needs S in the binade of its map
+        const bool mine = (uint32_t)lane >= start && (uint32_t)lane < left;
+        const bool ok = (code & kGuessOk) &&
+                        (zero ? eS < 255u : (eS >= 30u && eS <= 250u && (is_lo || is_hi) && a0 != kMapInvalid));
+        if (zero) a0 = a1 = 0u;
+        // the run of usable groups that starts at `start`
+        const unsigned long long stop = __ballot(mine && !ok) | (left < 64u ? ~0ull << left : 0ull);
+        const uint32_t end = stop ? (uint32_t)__ffsll((long long)stop) - 1u : 64u;
+        bool advanced = false;
+        if (end > start) {
+            const uint32_t cap = 1u << 25;
+            const bool part = (uint32_t)lane >= start && (uint32_t)lane < end;
+            a0 = part ? (a0 < cap ? a0 : cap) : 0u;
+            a1 = part ? (a1 < cap ? a1 : cap) : 0u;
+            // inclusive scan: the map of groups start .. lane, as increments for a start parity
+            chain_scan_maps(a0, a1, lane);
+            const uint32_t send = s + ((s & 1u) ? a1 : a0);
+            const bool fits = part && send <= (1u << 24);
+            const int nv = __popcll(__ballot(fits));  // fits is monotone: the sums never decrease
+            if (nv > 0) {
+                const uint32_t take = (uint32_t)__builtin_amdgcn_readlane((int)send, __builtin_amdgcn_readfirstlane((int)start + nv - 1));
+                // (a subnormal or zero S only passes groups of zeros: take == s and S stays)
+                S = __uint_as_float(take == (1u << 24) ? (eS + 1u) << 23 : (eS << 23) | (take - (1u << 23)));
+                start += (uint32_t)nv;
+                advanced = true;
+            }
+        }
+        if (!advanced) {
+            // the group's terms one by one (positions past the end add +0.0, which changes nothing)
+            const uint32_t P = base + start;
+            float t = 0.0f;
+            if (lane < 32 && P * 32u + (uint32_t)lane < count) {
+                const float d = x[(int64_t)pm[P * 32u + lane] * ld + c] - mean_c;
+                t = d * d;
+            }
+#pragma unroll
+            for (int i = 0; i < 32; ++i) S = S + __shfl(t, i);
+            start += 1u;
+        }
+    }
+}
+
+// grid (segments, dim / 4); 256 threads = 4 waves, one column each.  runs == nullptr: every group is
+// walked (short columns); else the table of k_seg_chain_runs.
 static __global__ void __launch_bounds__(256) k_seg_chain_compose(const uint32_t *__restrict__ perm,
                                                                  const uint2 *__restrict__ seg_range,
                                                                  const float *__restrict__ means, int64_t first,
                                                                  const float *__restrict__ x, int64_t ld, int dim,
                                                                  const uint16_t *__restrict__ guess,
                                                                  const uint4 *__restrict__ maps,
+                                                                 const uint4 *__restrict__ runs,
                                                                  float *__restrict__ var) {
     const int g = blockIdx.x, lane = threadIdx.x & 63, c = blockIdx.y * 4 + (threadIdx.x >> 6);
     if (c >= dim) return;
@@ -457,6 +659,49 @@ static __global__ void __launch_bounds__(256) k_seg_chain_compose(const uint32_t
     const float mean_c = means[(first + g) * dim + c];
     const uint32_t *pm = perm + range.x;
     float S = 0.0f;  // the same value in every lane
+    if (runs) {
+        const size_t r0 = seg_run0(range, g);
+        const uint32_t nR = (nP + kRunGroups - 1u) / kRunGroups;
+        for (uint32_t rb = 0; rb < nR; rb += 64) {
+            const uint32_t ri = rb + lane;
+            const uint4 rm = runs[(r0 + (ri < nR ? ri : nR - 1u)) * dim + c];  // lane = run rb + lane
+            const uint32_t here = nR - rb < 64u ? nR - rb : 64u;
+            for (uint32_t j = 0; j < here; ++j) {
+                const uint32_t c0 = (uint32_t)__builtin_amdgcn_readlane((int)rm.x, (int)j);
+                const uint32_t c1 = (uint32_t)__builtin_amdgcn_readlane((int)rm.y, (int)j);
+                const uint32_t meta = (uint32_t)__builtin_amdgcn_readlane((int)rm.z, (int)j);
+                const uint32_t Sb = __float_as_uint(S), eS = Sb >> 23;
+                const uint32_t s = (Sb & 0x7fffffu) | 0x800000u;
+                const uint32_t send = s + ((s & 1u) ? c1 : c0);
+                const bool binade_ok = (meta & kRunAnyBinade) ? eS < 255u : (eS == (meta & 255u) && eS >= 30u && eS <= 250u);
+                if ((meta & kRunClean) && binade_ok && send <= (1u << 24)) {
+                    // (a run of zeros: send == s and S stays, whatever finite value it has)
+                    if (!(meta & kRunAnyBinade))
+                        S = __uint_as_float(send == (1u << 24) ? (eS + 1u) << 23 : (eS << 23) | (send - (1u << 23)));
+                    continue;
+                }
+                // group by group: the run's four batches
+                const uint32_t Pr = (rb + j) * kRunGroups;
+                uint16_t codeR[4];
+                uint4 mpR[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t idx = Pr + 64u * k + lane;
+                    const size_t at = (g0 + (idx < nP ? idx : nP - 1u)) * dim + c;
+                    codeR[k] = guess[at];
+                    mpR[k] = maps[at];
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t base = Pr + 64u * k;
+                    const uint32_t left = base >= nP ? 0u : (nP - base < 64u ? nP - base : 64u);
+                    chain_batch(S, base, left, codeR[k], mpR[k], pm, count, x, ld, c, mean_c, lane);
+                }
+            }
+        }
+        if (lane == 0) var[(size_t)g * dim + c] = S;
+        return;
+    }
     // Batches of 64 groups at fixed positions (lane = group 64 b + lane), R batches per round of
     // loads: one memory round trip per round instead of one per batch.
     constexpr int R = 16;
@@ -474,78 +719,9 @@ static __global__ void __launch_bounds__(256) k_seg_chain_compose(const uint32_t
 #pragma unroll
         for (int k = 0; k < R; ++k) {
             const uint32_t base = (b0 + k) * 64u;  // first group of the batch
-            // groups in the batch (none past the end: the loop below does not run; uniform)
+            // groups in the batch (none past the end: the loop inside does not run; uniform)
             const uint32_t left = base >= nP ? 0u : (nP - base < 64u ? nP - base : 64u);
-            const uint16_t code = codeR[k];
-            const uint4 mp = mpR[k];
-            const uint32_t elo = code & 255u;
-            const bool zero = (code & kGuessZero) != 0;
-            uint32_t start = 0;  // groups of the batch already added
-            while (start < left) {
-                // S is +0, positive, +inf or a NaN; with the sign bit of a NaN eS is above every guess
-                const uint32_t Sb = __float_as_uint(S), eS = Sb >> 23;
-                const uint32_t s = (Sb & 0x7fffffu) | 0x800000u;  // S / u for a normal S
-                const bool is_lo = elo == eS, is_hi = (code & kGuessTwo) && elo + 1u == eS;
-                uint32_t a0 = is_lo ? mp.x : mp.z, a1 = is_lo ? mp.y : mp.w;
-                // a group of zeros keeps any finite S; another group needs S in the binade of its map
-                const bool mine = (uint32_t)lane >= start && (uint32_t)lane < left;
-                const bool ok = (code & kGuessOk) &&
-                                (zero ? eS < 255u : (eS >= 30u && eS <= 250u && (is_lo || is_hi) && a0 != kMapInvalid));
-                if (zero) a0 = a1 = 0u;
-                // the run of usable groups that starts at `start`
-                const unsigned long long stop = __ballot(mine && !ok) | (left < 64u ? ~0ull << left : 0ull);
-                const uint32_t end = stop ? (uint32_t)__ffsll((long long)stop) - 1u : 64u;
-                bool advanced = false;
-                if (end > start) {
-                    const uint32_t cap = 1u << 25;
-                    const bool part = (uint32_t)lane >= start && (uint32_t)lane < end;
-                    a0 = part ? (a0 < cap ? a0 : cap) : 0u;
-                    a1 = part ? (a1 < cap ? a1 : cap) : 0u;
-                    // inclusive scan: the map of groups start .. lane, as increments for a start parity
-                    // (left, then this lane's map: c_p = l_p + a_[(p + l_p) mod 2]; (0, 0) is the identity, which
-                    // is what a lane outside the row supplies)
-                    auto after_left = [&](uint32_t l0, uint32_t l1) {
-                        const uint32_t n0 = l0 + ((l0 & 1u) ? a1 : a0);        // start even: after l0 the parity is l0 & 1
-                        const uint32_t n1 = l1 + (((l1 + 1u) & 1u) ? a1 : a0);  // start odd
-                        a0 = n0 < cap ? n0 : cap;
-                        a1 = n1 < cap ? n1 : cap;
-                    };
-                    after_left(row_shr<1>(a0, 0u), row_shr<1>(a1, 0u));
-                    after_left(row_shr<2>(a0, 0u), row_shr<2>(a1, 0u));
-                    after_left(row_shr<4>(a0, 0u), row_shr<4>(a1, 0u));
-                    after_left(row_shr<8>(a0, 0u), row_shr<8>(a1, 0u));
-                    {
-                        uint32_t t0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 15), t1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 15);
-                        if ((lane >> 4) == 1) after_left(t0, t1);
-                        t0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 31), t1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 31);
-                        if ((lane >> 4) == 2) after_left(t0, t1);
-                        t0 = (uint32_t)__builtin_amdgcn_readlane((int)a0, 47), t1 = (uint32_t)__builtin_amdgcn_readlane((int)a1, 47);
-                        if ((lane >> 4) == 3) after_left(t0, t1);
-                    }
-                    const uint32_t send = s + ((s & 1u) ? a1 : a0);
-                    const bool fits = part && send <= (1u << 24);
-                    const int nv = __popcll(__ballot(fits));  // fits is monotone: the sums never decrease
-                    if (nv > 0) {
-                        const uint32_t take = (uint32_t)__builtin_amdgcn_readlane((int)send, __builtin_amdgcn_readfirstlane((int)start + nv - 1));
-                        // (a subnormal or zero S only passes groups of zeros: take == s and S stays)
-                        S = __uint_as_float(take == (1u << 24) ? (eS + 1u) << 23 : (eS << 23) | (take - (1u << 23)));
-                        start += (uint32_t)nv;
-                        advanced = true;
-                    }
-                }
-                if (!advanced) {
-                    // the group's terms one by one (positions past the end add +0.0, which changes nothing)
-                    const uint32_t P = base + start;
-                    float t = 0.0f;
-                    if (lane < 32 && P * 32u + (uint32_t)lane < count) {
-                        const float d = x[(int64_t)pm[P * 32u + lane] * ld + c] - mean_c;
-                        t = d * d;
-                    }
-#pragma unroll
-                    for (int i = 0; i < 32; ++i) S = S + __shfl(t, i);
-                    start += 1u;
-                }
-            }
+            chain_batch(S, base, left, codeR[k], mpR[k], pm, count, x, ld, c, mean_c, lane);
         }
     }
     if (lane == 0) var[(size_t)g * dim + c] = S;

@@ -306,16 +306,49 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                                0, st, perm, (const uint2 *)d_range, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
                                var_maps ? (float *)nullptr : d_sq, var_maps ? (float *)ctx->tsvq_gsum.p : (float *)nullptr);
             if (var_maps) {
-                hipLaunchKernelGGL(vq::k_seg_chain_guess, dim3((unsigned)ns, (unsigned)cdiv(dim, 4)), dim3(256), 0, st,
-                                   (const float *)ctx->tsvq_gsum.p, (const uint2 *)d_range, dim,
-                                   (uint16_t *)ctx->tsvq_guess.p);
+                // columns above kGuessBlock groups: the blocks' sums first, then all blocks side by side
+                // (both pay from about 4096 groups per column on: 22 us for the block sums, 48 us for the runs)
+                const unsigned nblk_all = cdiv(cdiv((int64_t)longest, 32), vq::kGuessBlock);
+                const unsigned nblk = nblk_all > 4 ? nblk_all : 1u;
+                double *d_bsum = nullptr;
+                if (nblk > 1) {
+                    const int32_t rc = ensure(ctx, ctx->tsvq_bsum, sizeof(double) * (size_t)ns * nblk * dim);
+                    if (rc != VQ_OK) {
+                        free_means();
+                        (void)hipFree(rp_tmp);
+                        return cleanup_fail(rc);
+                    }
+                    d_bsum = (double *)ctx->tsvq_bsum.p;
+                    hipLaunchKernelGGL(vq::k_seg_chain_bsum, dim3((unsigned)ns, (unsigned)cdiv(dim, 4), nblk), dim3(256), 0,
+                                       st, (const float *)ctx->tsvq_gsum.p, (const uint2 *)d_range, dim, d_bsum);
+                }
+                hipLaunchKernelGGL(vq::k_seg_chain_guess, dim3((unsigned)ns, (unsigned)cdiv(dim, 4), nblk), dim3(256), 0,
+                                   st, (const float *)ctx->tsvq_gsum.p, (const uint2 *)d_range, dim,
+                                   (const double *)d_bsum, (uint16_t *)ctx->tsvq_guess.p);
                 hipLaunchKernelGGL(vq::k_seg_chain_maps, dim3((unsigned)cdiv((int64_t)longest, 64), (unsigned)ns),
                                    dim3(256), 0, st, perm, (const uint2 *)d_range, (const float *)d_smeans, (int64_t)0,
                                    d_x, ld, dim, (const uint16_t *)ctx->tsvq_guess.p, (uint4 *)ctx->tsvq_maps.p);
+                // long columns: the maps of runs of 256 groups composed ahead, so that the walk passes a
+                // clean run in one step
+                uint4 *d_runs = nullptr;
+                if (nblk > 1) {
+                    const size_t nruns = ((size_t)n + vq::kChainGroup * (size_t)kChainSegs) / (32 * vq::kRunGroups) + ns + 2;
+                    const int32_t rc = ensure(ctx, ctx->tsvq_segmaps, sizeof(uint4) * nruns * dim);
+                    if (rc != VQ_OK) {
+                        free_means();
+                        (void)hipFree(rp_tmp);
+                        return cleanup_fail(rc);
+                    }
+                    d_runs = (uint4 *)ctx->tsvq_segmaps.p;
+                    hipLaunchKernelGGL(vq::k_seg_chain_runs,
+                                       dim3((unsigned)ns, (unsigned)cdiv(dim, 4), cdiv(cdiv((int64_t)longest, 32), 4 * vq::kRunGroups)),
+                                       dim3(256), 0, st, (const uint2 *)d_range, dim, (const uint16_t *)ctx->tsvq_guess.p,
+                                       (const uint4 *)ctx->tsvq_maps.p, d_runs);
+                }
                 hipLaunchKernelGGL(vq::k_seg_chain_compose, dim3((unsigned)ns, (unsigned)cdiv(dim, 4)), dim3(256), 0,
                                    st, perm, (const uint2 *)d_range, (const float *)d_smeans, (int64_t)0, d_x, ld, dim,
                                    (const uint16_t *)ctx->tsvq_guess.p, (const uint4 *)ctx->tsvq_maps.p,
-                                   (float *)d_var);
+                                   (const uint4 *)d_runs, (float *)d_var);
             } else {
                 hipLaunchKernelGGL(vq::k_seg_chain32, dim3((unsigned)ns, (unsigned)cdiv(dim, 32)), dim3(256), 0, st,
                                    (const float *)d_sq, (const uint2 *)d_range, dim, (float *)d_var);
