@@ -13,7 +13,7 @@ Prints ONE JSON line (see README of the bench contract):
                events of each launch's own dispatch) during the timed steps; the matrix-core and
                HBM views of the same time and the floor set by the selection's instructions at
                their measured issue rate are secondary fields
-  end_to_end   one pass host rows -> page-locked pack -> upload -> fit -> encode -> codes on the host
+  end_to_end   one pass pageable host rows -> upload -> fit -> encode -> codes on the host
   calibration  measured peaks of the box: plain-copy HBM rate, vector instruction issue rates
   cpu_baseline the C restatement of the reference (oracle/) timed on the host cores on a bounded
                sample of the same workload
@@ -181,38 +181,41 @@ def main():
         "encode_recheck_fraction": round(recheck_pairs / float(n * M), 6),
     }
 
-    # End to end, once: what a host that starts from rows in its own memory pays.  The rows are
-    # packed into page-locked memory (the reference holds one heap vector per row, so a pack is
-    # needed in any case; here it is one copy of the contiguous array), uploaded, trained on,
-    # encoded, and the codes come back.  Not part of `value`.
+    # End to end, once: what a host that starts from rows in its own (pageable) memory pays.  vq_h2d
+    # stages a large pageable upload through page-locked buffers with several host threads while
+    # the copy engine uploads the chunk before; then fit, encode, and the codes come back into
+    # page-locked memory.  For comparison the same rows from a page-locked buffer (no staging).
+    # Not part of `value`.
     end_to_end = None
     if args.end_to_end:
         hx = ctx.host_empty((n, DIM), np.float32)
         hcodes = ctx.host_empty((n, M), np.uint8)
-        hx[:1] = x[:1]  # touch
+        np.copyto(hx, x)
         best = None
-        for _ in range(2):
+        for _ in range(3):
             t0 = time.perf_counter()
-            np.copyto(hx, x)
+            dx.upload(x)           # pageable numpy array
             t1 = time.perf_counter()
-            dx.upload(hx)
-            t2 = time.perf_counter()
             step()
             ctx.sync()
-            t3 = time.perf_counter()
+            t2 = time.perf_counter()
             vq_amd._ffi.lib().vq_d2h(ctx._h, hcodes.ctypes.data, dcodes.ptr, hcodes.nbytes)
+            t3 = time.perf_counter()
+            dx.upload(hx)          # page-locked
             t4 = time.perf_counter()
-            cur = {"pack_ms": (t1 - t0) * 1e3, "h2d_ms": (t2 - t1) * 1e3, "fit_encode_ms": (t3 - t2) * 1e3,
-                   "d2h_codes_ms": (t4 - t3) * 1e3, "total_ms": (t4 - t0) * 1e3}
+            cur = {"upload_ms": (t1 - t0) * 1e3, "fit_encode_ms": (t2 - t1) * 1e3,
+                   "d2h_codes_ms": (t3 - t2) * 1e3, "total_ms": (t3 - t0) * 1e3,
+                   "upload_from_page_locked_ms": (t4 - t3) * 1e3}
             if best is None or cur["total_ms"] < best["total_ms"]:
                 best = cur
         end_to_end = {k_: round(v, 3) for k_, v in best.items()}
         end_to_end["vectors_per_s"] = round(n / (best["total_ms"] * 1e-3), 1)
-        end_to_end["vectors_per_s_without_pack"] = round(
-            n / ((best["total_ms"] - best["pack_ms"]) * 1e-3), 1)
-        end_to_end["h2d_GBs"] = round(x.nbytes / (best["h2d_ms"] * 1e-3) / 1e9, 1)
-        end_to_end["note"] = ("best of 2; pack = one numpy copy of the 512 MB array into page-locked "
-                              "memory on one host thread; synchronous upload; codes back to page-locked memory")
+        end_to_end["upload_GBs"] = round(x.nbytes / (best["upload_ms"] * 1e-3) / 1e9, 1)
+        end_to_end["upload_from_page_locked_GBs"] = round(
+            x.nbytes / (best["upload_from_page_locked_ms"] * 1e-3) / 1e9, 1)
+        end_to_end["note"] = ("best of 3; upload = vq_h2d of the 512 MB pageable array (staged through "
+                              "page-locked chunks by host threads, overlapped with the copy engine); "
+                              "codes back to page-locked memory")
         ctx.host_free(hx)
         ctx.host_free(hcodes)
 

@@ -385,3 +385,19 @@ def test_failures_forced_from_the_host_come_back_as_status_codes(ctx):
     ctx.lbg_fit(dx, 64, 8, 1, 8, 4, 3, init, reseed, dcb)
     want = O.lbg(x, 4, 3, init[0], reseed[0])
     assert np.array_equal(dcb.download()[0].view(np.uint32), want["centroids"].view(np.uint32))
+
+
+@pytest.mark.parametrize("nbytes", [(64 << 20) - 4, 64 << 20, (64 << 20) + 4, (150 << 20) + 12345 * 4])
+def test_large_upload_from_pageable_memory_is_exact(ctx, nbytes):
+    """vq_h2d stages a pageable source of 64 MiB or more through page-locked chunks with several host
+    threads: every byte must arrive, whatever the size relative to the chunks and the threads' slices."""
+    n = nbytes // 4
+    x = np.random.default_rng(nbytes % 997).integers(0, 2 ** 31, n, dtype=np.int64).astype(np.uint32).view(F)
+    d = ctx.empty((n,), F)
+    d.upload(x)
+    assert np.array_equal(d.download().view(np.uint32), x.view(np.uint32))
+    hx = ctx.host_empty((n,), F)   # page-locked source: one direct copy
+    np.copyto(hx, x[::-1])
+    d.upload(hx)
+    assert np.array_equal(d.download().view(np.uint32), x[::-1].view(np.uint32))
+    ctx.host_free(hx)

@@ -32,6 +32,10 @@ struct vq_ctx {
     DevBuf tsvq_means;           // TSVQ build: the means of all nodes, read back once at the end
     void *tsvq_pin = nullptr;    // TSVQ build: page-locked staging of a level's tables and decisions
     size_t tsvq_pin_cap = 0;
+    // vq_h2d from pageable memory: page-locked staging buffers and the events of their uploads
+    static constexpr int kStageBuffers = 3;
+    void *h2d_stage[kStageBuffers] = {nullptr, nullptr, nullptr};
+    hipEvent_t h2d_event[kStageBuffers] = {nullptr, nullptr, nullptr};
     DevBuf tsvq_gsum, tsvq_guess, tsvq_maps;  // per group of 32 squares: sum, binade guess, integer maps
     DevBuf tsvq_bsum, tsvq_segmaps;           // per block of groups: f64 sum; per run of groups: composed map
     int tsvq_var_path = 0;       // 0 = composed integer maps, 1 = one chain of adds per column

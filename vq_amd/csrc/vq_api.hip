@@ -11,6 +11,8 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <atomic>
+#include <thread>
 #include <vector>
 
 #include "ctx.hpp"
@@ -582,6 +584,10 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);
     if (ctx->tsvq_pin) (void)hipHostFree(ctx->tsvq_pin);
+    for (int i = 0; i < vq_ctx::kStageBuffers; ++i) {
+        if (ctx->h2d_stage[i]) (void)hipHostFree(ctx->h2d_stage[i]);
+        if (ctx->h2d_event[i]) (void)hipEventDestroy(ctx->h2d_event[i]);
+    }
     prof_collect(ctx);
     for (hipEvent_t e : ctx->prof_pool) (void)hipEventDestroy(e);
     (void)hipEventDestroy(ctx->ev0);
@@ -636,8 +642,61 @@ int32_t vq_host_free(vq_ctx *ctx, void *h_ptr) {
     return VQ_OK;
 }
 
+// A large upload from pageable memory: host threads stage it chunk by chunk into page-locked buffers
+// while the copy engine uploads the chunk before, instead of the runtime's single-threaded staging.
+static int32_t h2d_staged(vq_ctx *ctx, char *d_dst, const char *h_src, size_t bytes) {
+    constexpr size_t kChunk = 16u << 20;
+    constexpr int NB = vq_ctx::kStageBuffers;
+    for (int i = 0; i < NB; ++i) {
+        if (!ctx->h2d_stage[i]) VQ_HIP(ctx, hipHostMalloc(&ctx->h2d_stage[i], kChunk, hipHostMallocDefault));
+        if (!ctx->h2d_event[i]) VQ_HIP(ctx, hipEventCreateWithFlags(&ctx->h2d_event[i], hipEventDisableTiming));
+    }
+    const size_t nchunks = (bytes + kChunk - 1) / kChunk;
+    const unsigned hw = std::thread::hardware_concurrency();
+    const int T = (int)std::min<unsigned>(8u, std::max<unsigned>(1u, hw / 2));
+    std::atomic<size_t> stageable{(size_t)NB};  // chunks below this index may be staged: their buffer is free
+    std::vector<std::atomic<int>> staged(nchunks);
+    for (auto &a : staged) a.store(0, std::memory_order_relaxed);
+    auto work = [&](int t) {
+        for (size_t c = 0; c < nchunks; ++c) {
+            while (c >= stageable.load(std::memory_order_acquire)) std::this_thread::yield();
+            const size_t len = std::min(kChunk, bytes - c * kChunk);
+            const size_t per = ((len + T - 1) / T + 63) & ~(size_t)63;
+            const size_t lo = std::min(len, per * (size_t)t), hi = std::min(len, lo + per);
+            if (hi > lo) memcpy((char *)ctx->h2d_stage[c % NB] + lo, h_src + c * kChunk + lo, hi - lo);
+            staged[c].fetch_add(1, std::memory_order_release);
+        }
+    };
+    std::vector<std::thread> pool;
+    for (int t = 1; t < T; ++t) pool.emplace_back(work, t);
+    hipError_t err = hipSuccess;
+    std::thread first(work, 0);
+    for (size_t c = 0; c < nchunks; ++c) {
+        while (staged[c].load(std::memory_order_acquire) < T) std::this_thread::yield();
+        const size_t len = std::min(kChunk, bytes - c * kChunk);
+        if (err == hipSuccess)
+            err = hipMemcpyAsync(d_dst + c * kChunk, ctx->h2d_stage[c % NB], len, hipMemcpyHostToDevice, ctx->stream);
+        if (err == hipSuccess) err = hipEventRecord(ctx->h2d_event[c % NB], ctx->stream);
+        // chunk c + 1 takes the buffer of chunk c + 1 - NB: wait for that upload (on an error the
+        // workers are let through to the end, nothing more is uploaded)
+        if (c + 1 >= (size_t)NB && err == hipSuccess) err = hipEventSynchronize(ctx->h2d_event[(c + 1) % NB]);
+        stageable.store(c + 2 > (size_t)NB ? c + 2 : (size_t)NB, std::memory_order_release);
+    }
+    first.join();
+    for (auto &th : pool) th.join();
+    VQ_HIP(ctx, err);
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return VQ_OK;
+}
+
 int32_t vq_h2d(vq_ctx *ctx, void *d_dst, const void *h_src, size_t bytes) {
     if (!ctx || (bytes && (!d_dst || !h_src))) return VQ_ERR_INVALID_ARG;
+    if (bytes >= (64u << 20)) {
+        hipPointerAttribute_t attr;
+        const bool locked = hipPointerGetAttributes(&attr, h_src) == hipSuccess && attr.type == hipMemoryTypeHost;
+        (void)hipGetLastError();  // an unregistered host pointer is reported as an error: that is the pageable case
+        if (!locked) return h2d_staged(ctx, (char *)d_dst, (const char *)h_src, bytes);
+    }
     VQ_HIP(ctx, hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->stream));
     VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return VQ_OK;
