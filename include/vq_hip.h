@@ -118,7 +118,8 @@ int32_t vq_host_free(vq_ctx *ctx, void *h_ptr);
  * layout `&[Vector<f32>]` (src/vector.rs:150-152): the host packs rows into one buffer.
  * vq_h2d of 64 MiB or more from pageable memory is staged by the library: up to eight host threads
  * copy 16 MiB chunks into page-locked buffers of the context while the copy engine uploads the chunk
- * before (about 50 GB/s instead of 18-29 for one plain copy; a page-locked source goes up directly). */
+ * before (about 50 GB/s instead of 18-29 for one plain copy; a page-locked source goes up directly);
+ * vq_d2h into pageable memory does the same in the other direction. */
 int32_t vq_h2d(vq_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
 int32_t vq_d2h(vq_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
 

@@ -702,8 +702,65 @@ int32_t vq_h2d(vq_ctx *ctx, void *d_dst, const void *h_src, size_t bytes) {
     return VQ_OK;
 }
 
+// The other direction: the copy engine fills page-locked chunks, host threads copy the chunk before
+// out to the pageable destination.
+static int32_t d2h_staged(vq_ctx *ctx, char *h_dst, const char *d_src, size_t bytes) {
+    constexpr size_t kChunk = 16u << 20;
+    constexpr int NB = vq_ctx::kStageBuffers;
+    for (int i = 0; i < NB; ++i) {
+        if (!ctx->h2d_stage[i]) VQ_HIP(ctx, hipHostMalloc(&ctx->h2d_stage[i], kChunk, hipHostMallocDefault));
+        if (!ctx->h2d_event[i]) VQ_HIP(ctx, hipEventCreateWithFlags(&ctx->h2d_event[i], hipEventDisableTiming));
+    }
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));  // the staging buffers are idle
+    const size_t nchunks = (bytes + kChunk - 1) / kChunk;
+    const unsigned hw = std::thread::hardware_concurrency();
+    const int T = (int)std::min<unsigned>(8u, std::max<unsigned>(1u, hw / 2));
+    std::atomic<size_t> arrived{0};  // chunks below this index are in their staging buffer
+    std::vector<std::atomic<int>> copied(nchunks);
+    for (auto &a : copied) a.store(0, std::memory_order_relaxed);
+    auto work = [&](int t) {
+        for (size_t c = 0; c < nchunks; ++c) {
+            while (c >= arrived.load(std::memory_order_acquire)) std::this_thread::yield();
+            const size_t len = std::min(kChunk, bytes - c * kChunk);
+            const size_t per = ((len + T - 1) / T + 63) & ~(size_t)63;
+            const size_t lo = std::min(len, per * (size_t)t), hi = std::min(len, lo + per);
+            if (hi > lo) memcpy(h_dst + c * kChunk + lo, (const char *)ctx->h2d_stage[c % NB] + lo, hi - lo);
+            copied[c].fetch_add(1, std::memory_order_release);
+        }
+    };
+    std::vector<std::thread> pool;
+    for (int t = 0; t < T; ++t) pool.emplace_back(work, t);
+    hipError_t err = hipSuccess;
+    size_t issued = 0;
+    auto issue = [&]() {  // the download of chunk `issued` into its buffer
+        const size_t len = std::min(kChunk, bytes - issued * kChunk);
+        if (err == hipSuccess)
+            err = hipMemcpyAsync(ctx->h2d_stage[issued % NB], d_src + issued * kChunk, len, hipMemcpyDeviceToHost, ctx->stream);
+        if (err == hipSuccess) err = hipEventRecord(ctx->h2d_event[issued % NB], ctx->stream);
+        ++issued;
+    };
+    while (issued < nchunks && issued < (size_t)NB) issue();
+    for (size_t c = 0; c < nchunks; ++c) {
+        if (err == hipSuccess) err = hipEventSynchronize(ctx->h2d_event[c % NB]);
+        arrived.store(c + 1, std::memory_order_release);  // (on an error the workers run through: the call fails)
+        if (issued < nchunks) {  // chunk c + NB takes this buffer once the threads have emptied it
+            while (copied[c].load(std::memory_order_acquire) < T) std::this_thread::yield();
+            issue();
+        }
+    }
+    for (auto &th : pool) th.join();
+    VQ_HIP(ctx, err);
+    return VQ_OK;
+}
+
 int32_t vq_d2h(vq_ctx *ctx, void *h_dst, const void *d_src, size_t bytes) {
     if (!ctx || (bytes && (!h_dst || !d_src))) return VQ_ERR_INVALID_ARG;
+    if (bytes >= (64u << 20)) {
+        hipPointerAttribute_t attr;
+        const bool locked = hipPointerGetAttributes(&attr, h_dst) == hipSuccess && attr.type == hipMemoryTypeHost;
+        (void)hipGetLastError();
+        if (!locked) return d2h_staged(ctx, (char *)h_dst, (const char *)d_src, bytes);
+    }
     VQ_HIP(ctx, hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
     VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return VQ_OK;
