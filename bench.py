@@ -2,10 +2,10 @@
 """bench.py — PQ fit + encode throughput on one MI355X, with roofline and CPU baseline.
 
 One step = ProductQuantizer::fit (10 LBG iterations) followed by the encode of every row
-(BASELINE.json configs[1]: 1,000,000 x 128 f32 rows from a mixture of 1,024 isotropic Gaussians,
+(the headline configuration: 1,000,000 x 128 f32 rows from a mixture of 1,024 isotropic Gaussians,
 m = 16, k = 256, Euclidean encode), with the rows already resident in HBM.
 
-Prints ONE JSON line (see README of the bench contract):
+Prints ONE JSON line:
   value        rows / second over fit + encode (whole job, one GPU)
   roofline     the dominant kernel (the assignment pass) against the bound that binds it, the
                vector ALU: algorithmic selection lane-slots per second over the issue peak; its
