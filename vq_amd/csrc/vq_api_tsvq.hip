@@ -25,6 +25,7 @@ struct vq_tree {
     std::vector<int32_t> h_left, h_right, h_split_dim;
     std::vector<float> h_split_val;
     std::vector<int64_t> h_count;
+    void *d_block = nullptr;  // one allocation: centroids, their norms, left and right children
     float *d_centroids = nullptr, *d_cnorm = nullptr;
     int32_t *d_left = nullptr, *d_right = nullptr;
 };
@@ -44,15 +45,23 @@ struct Seg {
     uint32_t lo, hi;
 };
 
-int32_t tree_to_device(vq_ctx *ctx, vq_tree *t) {
+// d_means: the centroids where they already are on the device (the build's node means), else they
+// go up from the host copy.
+int32_t tree_to_device(vq_ctx *ctx, vq_tree *t, const float *d_means = nullptr) {
     size_t nn = (size_t)t->n_nodes, dim = (size_t)t->dim;
-    VQ_HIP(ctx, hipMalloc(&t->d_centroids, sizeof(float) * nn * dim));
-    VQ_HIP(ctx, hipMalloc(&t->d_cnorm, sizeof(float) * nn));
-    VQ_HIP(ctx, hipMalloc(&t->d_left, sizeof(int32_t) * nn));
-    VQ_HIP(ctx, hipMalloc(&t->d_right, sizeof(int32_t) * nn));
+    auto pad = [](size_t z) { return (z + 255) & ~(size_t)255; };
+    const size_t cen_b = pad(sizeof(float) * nn * dim), idx_b = pad(sizeof(int32_t) * nn);
+    VQ_HIP(ctx, hipMalloc(&t->d_block, cen_b + 3 * idx_b));
+    t->d_centroids = (float *)t->d_block;
+    t->d_cnorm = (float *)((char *)t->d_block + cen_b);
+    t->d_left = (int32_t *)((char *)t->d_block + cen_b + idx_b);
+    t->d_right = (int32_t *)((char *)t->d_block + cen_b + 2 * idx_b);
     hipStream_t st = ctx->stream;
-    VQ_HIP(ctx, hipMemcpyAsync(t->d_centroids, t->h_centroids.data(), sizeof(float) * nn * dim,
-                               hipMemcpyHostToDevice, st));
+    if (d_means)
+        VQ_HIP(ctx, hipMemcpyAsync(t->d_centroids, d_means, sizeof(float) * nn * dim, hipMemcpyDeviceToDevice, st));
+    else
+        VQ_HIP(ctx, hipMemcpyAsync(t->d_centroids, t->h_centroids.data(), sizeof(float) * nn * dim,
+                                   hipMemcpyHostToDevice, st));
     VQ_HIP(ctx, hipMemcpyAsync(t->d_left, t->h_left.data(), sizeof(int32_t) * nn, hipMemcpyHostToDevice, st));
     VQ_HIP(ctx, hipMemcpyAsync(t->d_right, t->h_right.data(), sizeof(int32_t) * nn, hipMemcpyHostToDevice, st));
     hipLaunchKernelGGL(vq::k_centroid_norms, dim3(cdiv((int64_t)nn, 256)), dim3(256), 0, st, t->d_centroids,
@@ -64,10 +73,7 @@ int32_t tree_to_device(vq_ctx *ctx, vq_tree *t) {
 
 void tree_release(vq_tree *t) {
     if (!t) return;
-    (void)hipFree(t->d_centroids);
-    (void)hipFree(t->d_cnorm);
-    (void)hipFree(t->d_left);
-    (void)hipFree(t->d_right);
+    (void)hipFree(t->d_block);
     delete t;
 }
 
@@ -129,8 +135,6 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         tree_release(T);
         return rc;
     };
-    void *rp_tmp = nullptr;
-    size_t rp_cap = 0;
     int32_t rc = VQ_OK;
     struct LevelMeans {
         void *d;
@@ -204,7 +208,6 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         if (e__ != hipSuccess) {                                                                  \
             (void)hipGetLastError();                                                              \
             free_means();                                                                         \
-            (void)hipFree(rp_tmp);                                                                \
             return cleanup_fail(fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,   \
                                      "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__,   \
                                      __LINE__));                                                  \
@@ -224,7 +227,6 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             if (rc == VQ_OK) rc = pinned(up_bytes + pad(down_bytes));
             if (rc != VQ_OK) {
                 free_means();
-                (void)hipFree(rp_tmp);
                 return cleanup_fail(rc);
             }
             char *at = (char *)ctx->tsvq_level.p, *h = (char *)ctx->tsvq_pin;
@@ -266,7 +268,6 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         if (e__ != hipSuccess) {                                                                  \
             (void)hipGetLastError();                                                              \
             free_means();                                                                         \
-            (void)hipFree(rp_tmp);                                                                \
             return cleanup_fail(fail(ctx, e__ == hipErrorOutOfMemory ? VQ_ERR_OOM : VQ_ERR_HIP,   \
                                      "%s: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__,   \
                                      __LINE__));                                                  \
@@ -283,7 +284,6 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             const int32_t rc = ensure(ctx, ctx->tsvq_split, total);
             if (rc != VQ_OK) {
                 free_means();
-                (void)hipFree(rp_tmp);
                 return cleanup_fail(rc);
             }
             char *at = (char *)ctx->tsvq_split.p;
@@ -315,7 +315,6 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                     const int32_t rc = ensure(ctx, ctx->tsvq_bsum, sizeof(double) * (size_t)ns * nblk * dim);
                     if (rc != VQ_OK) {
                         free_means();
-                        (void)hipFree(rp_tmp);
                         return cleanup_fail(rc);
                     }
                     d_bsum = (double *)ctx->tsvq_bsum.p;
@@ -336,7 +335,6 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                     const int32_t rc = ensure(ctx, ctx->tsvq_segmaps, sizeof(uint4) * nruns * dim);
                     if (rc != VQ_OK) {
                         free_means();
-                        (void)hipFree(rp_tmp);
                         return cleanup_fail(rc);
                     }
                     d_runs = (uint4 *)ctx->tsvq_segmaps.p;
@@ -394,13 +392,14 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                            ns, (const float *)d_median, flags);
         size_t need = 0;
         SP_HIP(rocprim::exclusive_scan(nullptr, need, flags, scan, 0u, (size_t)n, rocprim::plus<uint32_t>(), st));
-        if (need > rp_cap) {
-            (void)hipFree(rp_tmp);
-            rp_tmp = nullptr;
-            SP_HIP(hipMalloc(&rp_tmp, need));
-            rp_cap = need;
+        {
+            const int32_t rc = ensure(ctx, ctx->tsvq_scan, need);
+            if (rc != VQ_OK) {
+                free_means();
+                return cleanup_fail(rc);
+            }
         }
-        SP_HIP(rocprim::exclusive_scan(rp_tmp, need, flags, scan, 0u, (size_t)n, rocprim::plus<uint32_t>(), st));
+        SP_HIP(rocprim::exclusive_scan(ctx->tsvq_scan.p, need, flags, scan, 0u, (size_t)n, rocprim::plus<uint32_t>(), st));
         hipLaunchKernelGGL(vq::k_seg_partition, dim3(cdiv(n, 256)), dim3(256), 0, st, perm, n,
                            (const uint2 *)d_range, ns, flags, scan, perm2, (uint32_t *)d_nleft);
         SP_HIP(hipGetLastError());
@@ -435,8 +434,6 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         level.swap(next);
         --depth_left;
     }
-    (void)hipFree(rp_tmp);
-    rp_tmp = nullptr;
     T->n_nodes = (int32_t)T->h_left.size();
     T->h_centroids.resize((size_t)T->n_nodes * dim);
     if (means_arena)
@@ -447,10 +444,10 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
             LV_HIP(hipMemcpyAsync(T->h_centroids.data() + (size_t)lm.first_node * dim, lm.d,
                                   sizeof(float) * (size_t)lm.nseg * dim, hipMemcpyDeviceToHost, st));
     LV_HIP(hipStreamSynchronize(st));
-    free_means();
 #undef LV_HIP
 #undef SP_HIP
-    rc = tree_to_device(ctx, T);
+    rc = tree_to_device(ctx, T, means_arena ? (const float *)ctx->tsvq_means.p : nullptr);
+    free_means();
     if (rc != VQ_OK) return cleanup_fail(rc);
     *out = T;
     return VQ_OK;
