@@ -959,18 +959,6 @@ __device__ __forceinline__ float float_from_order_key(uint32_t k) {
     return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
-static __global__ void k_seg_select_init(const uint2 *__restrict__ seg_range, int nseg, SegSelect *__restrict__ sel,
-                                         uint32_t *__restrict__ hist) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < nseg * 512) hist[i] = 0u;
-    if (i < nseg) {
-        const uint2 r = seg_range[i];
-        const uint32_t c = r.y - r.x;
-        sel[2 * i] = SegSelect{0u, (c % 2 == 0) ? c / 2 - 1 : c / 2};
-        sel[2 * i + 1] = SegSelect{0u, c / 2};
-    }
-}
-
 // One workgroup per 4096 positions; pass = 0..3 looks at key bits [31 - 8 pass, 24 - 8 pass].
 static __global__ void __launch_bounds__(256) k_seg_select_hist(const float *__restrict__ vals, int64_t n,
                                                                 const uint2 *__restrict__ seg_range, int nseg,
@@ -1054,16 +1042,22 @@ static __global__ void __launch_bounds__(64) k_seg_select_pick(uint32_t *__restr
     if (lane == 0 && s.rank >= all) sel[i] = SegSelect{s.prefix | (255u << shift), s.rank - all};
 }
 
-static __global__ void k_seg_select_out(const SegSelect *__restrict__ sel, int nseg, float *__restrict__ mids) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < 2 * nseg) mids[i] = float_from_order_key(sel[i].prefix);
-}
-
 // The split dimension of every segment: argmax of its per-dimension sums with the LAST maximal
 // element winning (Iterator::max_by, src/tsvq.rs:102-106); one thread per segment.
-static __global__ void k_seg_argmax_last(const float *__restrict__ var, int nseg, int dim, int *__restrict__ sdim) {
+// The same launch starts the radix select of the middle values: bins cleared, ranks of the two
+// targets of every segment (the lower and the upper middle).  Grid over nseg * 512 bins.
+static __global__ void k_seg_argmax_last(const float *__restrict__ var, int nseg, int dim, int *__restrict__ sdim,
+                                         const uint2 *__restrict__ seg_range, SegSelect *__restrict__ sel,
+                                         uint32_t *__restrict__ hist) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nseg * 512) hist[i] = 0u;
     if (i >= nseg) return;
+    {
+        const uint2 r = seg_range[i];
+        const uint32_t c = r.y - r.x;
+        sel[2 * i] = SegSelect{0u, (c % 2 == 0) ? c / 2 - 1 : c / 2};
+        sel[2 * i + 1] = SegSelect{0u, c / 2};
+    }
     const float *v = var + (size_t)i * dim;
     int best = 0;
     float vb = v[0];
@@ -1084,12 +1078,13 @@ static __global__ void k_seg_argmax_last(const float *__restrict__ var, int nseg
 
 // The median of every segment from its two middle values (src/tsvq.rs:112-117): their f32 sum
 // divided by two for an even count, the middle value otherwise.
-static __global__ void k_seg_median(const float *__restrict__ mids, const uint2 *__restrict__ seg_range, int nseg,
+static __global__ void k_seg_median(const SegSelect *__restrict__ sel, const uint2 *__restrict__ seg_range, int nseg,
                                     float *__restrict__ median) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= nseg) return;
     const uint32_t cnt = seg_range[i].y - seg_range[i].x;
-    const float a = mids[2 * i], b = mids[2 * i + 1];
+    // the selected keys back as floats
+    const float a = float_from_order_key(sel[2 * i].prefix), b = float_from_order_key(sel[2 * i + 1].prefix);
     const float sum = a + b;
     median[i] = (cnt % 2u == 0u) ? sum / 2.0f : a;
 }

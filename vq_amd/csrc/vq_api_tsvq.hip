@@ -260,7 +260,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         if (split.empty()) break;
         // the level's small tables: one grow-only arena of the context instead of nine allocations;
         // split dimension, median and left count of every node side by side, so that one copy returns them
-        void *d_smeans = nullptr, *d_var = nullptr, *d_down = nullptr, *d_mids = nullptr, *d_sel = nullptr,
+        void *d_smeans = nullptr, *d_var = nullptr, *d_down = nullptr, *d_sel = nullptr,
              *d_hist = nullptr;
 #define SP_HIP(call)                                                                              \
     do {                                                                                          \
@@ -275,10 +275,9 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     } while (0)
         {
             const size_t cap = (size_t)std::max(ns, 1024);  // sized once for the usual depths
-            const size_t sizes[6] = {sizeof(float) * cap * dim, sizeof(float) * cap * dim, 3 * sizeof(uint32_t) * cap,
-                                     sizeof(float) * 2 * cap, sizeof(vq::SegSelect) * 2 * cap,
-                                     sizeof(uint32_t) * 512 * cap};
-            void **ptrs[6] = {&d_smeans, &d_var, &d_down, &d_mids, &d_sel, &d_hist};
+            const size_t sizes[5] = {sizeof(float) * cap * dim, sizeof(float) * cap * dim, 3 * sizeof(uint32_t) * cap,
+                                     sizeof(vq::SegSelect) * 2 * cap, sizeof(uint32_t) * 512 * cap};
+            void **ptrs[5] = {&d_smeans, &d_var, &d_down, &d_sel, &d_hist};
             size_t total = 0;
             for (size_t z : sizes) total += (z + 255) & ~(size_t)255;
             const int32_t rc = ensure(ctx, ctx->tsvq_split, total);
@@ -287,7 +286,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                 return cleanup_fail(rc);
             }
             char *at = (char *)ctx->tsvq_split.p;
-            for (int z = 0; z < 6; ++z) {
+            for (int z = 0; z < 5; ++z) {
                 *ptrs[z] = at;
                 at += (sizes[z] + 255) & ~(size_t)255;
             }
@@ -369,23 +368,20 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
                                (float *)d_var);
         SP_HIP(hipGetLastError());
         // split dimension on the device (src/tsvq.rs:102-106); read back with the left counts below
-        hipLaunchKernelGGL(vq::k_seg_argmax_last, dim3(cdiv(ns, 64)), dim3(64), 0, st, (const float *)d_var, ns, dim,
-                           (int *)d_sdim);
+        hipLaunchKernelGGL(vq::k_seg_argmax_last, dim3(cdiv((int64_t)ns * 512, 256)), dim3(256), 0, st,
+                           (const float *)d_var, ns, dim, (int *)d_sdim, (const uint2 *)d_range, (vq::SegSelect *)d_sel,
+                           (uint32_t *)d_hist);
         // split column, middle values by radix select (src/tsvq.rs:109-117)
         hipLaunchKernelGGL(vq::k_seg_gather_col, dim3(cdiv(n, 256)), dim3(256), 0, st, perm, n,
                            (const uint2 *)d_range, ns, (const int *)d_sdim, d_x, ld, vals);
-        hipLaunchKernelGGL(vq::k_seg_select_init, dim3(cdiv((int64_t)ns * 512, 256)), dim3(256), 0, st,
-                           (const uint2 *)d_range, ns, (vq::SegSelect *)d_sel, (uint32_t *)d_hist);
         for (int pass = 0; pass < 4; ++pass) {
             hipLaunchKernelGGL(vq::k_seg_select_hist, dim3(cdiv(n, 4096)), dim3(256), 0, st, (const float *)vals, n,
                                (const uint2 *)d_range, ns, (const vq::SegSelect *)d_sel, pass, (uint32_t *)d_hist);
             hipLaunchKernelGGL(vq::k_seg_select_pick, dim3(2 * ns), dim3(64), 0, st, (uint32_t *)d_hist,
                                (vq::SegSelect *)d_sel, ns, pass);
         }
-        hipLaunchKernelGGL(vq::k_seg_select_out, dim3(cdiv(2 * ns, 64)), dim3(64), 0, st,
-                           (const vq::SegSelect *)d_sel, ns, (float *)d_mids);
         SP_HIP(hipGetLastError());
-        hipLaunchKernelGGL(vq::k_seg_median, dim3(cdiv(ns, 64)), dim3(64), 0, st, (const float *)d_mids,
+        hipLaunchKernelGGL(vq::k_seg_median, dim3(cdiv(ns, 64)), dim3(64), 0, st, (const vq::SegSelect *)d_sel,
                            (const uint2 *)d_range, ns, (float *)d_median);
         // stable partition by `<= median` (src/tsvq.rs:120-123)
         hipLaunchKernelGGL(vq::k_seg_flags, dim3(cdiv(n, 256)), dim3(256), 0, st, vals, n, (const uint2 *)d_range,
