@@ -406,27 +406,25 @@ static __global__ void __launch_bounds__(256) k_seg_chain_guess(const float *__r
     }
 }
 
-// inc[0], inc[1] of one group for a running sum in the binade of exponent field e.
+// inc[0], inc[1] of one group for a running sum in the binade of exponent field e (30 <= e <= 250).
+// A term over the unit, y = t / u = t * 2^(150 - e), is exact (a scaling by a power of two; a product
+// that underflows stays below 1/2 and counts as zero either way), so its integer part, and whether
+// the rest is above or exactly one half, come from a floor and a subtraction, both exact below 2^24.
 __device__ __forceinline__ void chain_group_map(const float (&t)[32], int valid, uint32_t e, uint32_t &inc0,
                                                 uint32_t &inc1) {
+    const float inv_u = __uint_as_float((277u - e) << 23);  // 2^(150 - e)
     uint32_t a0 = 0, a1 = 0, par0 = 0, par1 = 1;
     bool bad = false;
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
         if (i < valid) {
-            const uint32_t tb = __float_as_uint(t[i]);
-            uint32_t et = (tb >> 23) & 255u, m = tb & 0x7fffffu;
-            bad = bad || (tb >> 31) != 0u || et == 255u;
-            if (et == 0u) et = 1u; else m |= 0x800000u;
-            const int sh = (int)e - (int)et;
-            bad = bad || sh < 0;
-            uint32_t q = 0, up = 0, tie = 0;
-            if (sh >= 0 && sh < 25) {
-                q = m >> sh;
-                const uint32_t rem = m & ((1u << sh) - 1u), half = (1u << sh) >> 1;
-                up = rem > half ? 1u : 0u;
-                tie = (sh > 0 && rem == half) ? 1u : 0u;
-            }
+            const float y = t[i] * inv_u;
+            // a negative term, a NaN, an infinity, or a term of a higher binade than the sum's
+            bad = bad || !(y >= 0.0f) || !(y < 16777216.0f);
+            const float f = floorf(y);
+            const float rest = y - f;
+            const uint32_t q = (uint32_t)f;
+            const uint32_t up = rest > 0.5f ? 1u : 0u, tie = rest == 0.5f ? 1u : 0u;
             const uint32_t d0 = q + up + (tie & (par0 + q)), d1 = q + up + (tie & (par1 + q));
             a0 += d0;
             a1 += d1;
