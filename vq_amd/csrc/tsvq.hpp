@@ -413,7 +413,9 @@ static __global__ void __launch_bounds__(256) k_seg_chain_guess(const float *__r
 __device__ __forceinline__ void chain_group_map(const float (&t)[32], int valid, uint32_t e, uint32_t &inc0,
                                                 uint32_t &inc1) {
     const float inv_u = __uint_as_float((277u - e) << 23);  // 2^(150 - e)
-    uint32_t a0 = 0, a1 = 0, par0 = 0, par1 = 1;
+    // s0, s1: the running sum's integer for an even and for an odd start, less the (even) start
+    // itself: their lowest bits are the parities the tie rule asks for
+    uint32_t s0 = 0, s1 = 1;
     bool bad = false;
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
@@ -424,16 +426,15 @@ __device__ __forceinline__ void chain_group_map(const float (&t)[32], int valid,
             const float f = floorf(y);
             const float rest = y - f;
             const uint32_t q = (uint32_t)f;
-            const uint32_t up = rest > 0.5f ? 1u : 0u, tie = rest == 0.5f ? 1u : 0u;
-            const uint32_t d0 = q + up + (tie & (par0 + q)), d1 = q + up + (tie & (par1 + q));
-            a0 += d0;
-            a1 += d1;
-            par0 = (par0 + d0) & 1u;
-            par1 = (par1 + d1) & 1u;
+            const uint32_t tie = rest == 0.5f ? 1u : 0u;
+            const uint32_t step = q + (rest > 0.5f ? 1u : 0u);
+            // a tie goes up when that makes the sum even: when sum + q is odd
+            s0 += step + (tie & (s0 + q));
+            s1 += step + (tie & (s1 + q));
         }
     }
-    inc0 = bad ? kMapInvalid : a0;
-    inc1 = bad ? kMapInvalid : a1;
+    inc0 = bad ? kMapInvalid : s0;
+    inc1 = bad ? kMapInvalid : s1 - 1u;
 }
 
 // Grid (blocks of 64 positions, segments), as k_seg_sqdev32: one thread per (group, column).
