@@ -223,6 +223,35 @@ def test_mfma_path_equals_oracle_and_valu_path(ctx, metric, n, m, k, kind):
         assert frac < 0.05, frac  # the matrix-core pass decides almost every row itself
 
 
+@pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN])
+@pytest.mark.parametrize("n,m,k", [(3000, 4, 256), (1500, 3, 255), (800, 8, 6), (2100, 1, 37), (5000, 16, 254)])
+def test_ties_and_near_ties_inside_a_run_of_four_centroids(ctx, metric, n, m, k):
+    """The matrix-core pass keeps one key per run of four consecutive centroids and picks inside the
+    best run by exact distances.  Duplicates and neighbours one ulp apart inside a run (in one lane
+    half: 4j and 4j + 1; across the halves: 4j + 1 and 4j + 2), a codebook that ends inside a run,
+    and rows that sit exactly on centroids: the oracle's first-smallest choice, and few rows that
+    need the full reference-order scan."""
+    rng = np.random.default_rng(100 * n + k)
+    dim = 8 * m
+    cb = rng.standard_normal((m, k, 8)).astype(F)
+    for j in range(0, k - 3, 8):
+        cb[:, j + 1] = cb[:, j]                                   # exact tie inside a lane half
+        cb[:, j + 2] = np.nextafter(cb[:, j + 1], F(np.inf))      # one ulp away, across the halves
+    if k % 4 >= 2:
+        cb[:, k - 1] = cb[:, k - 2]                               # a tie in the last, partial run
+    x = rng.standard_normal((n, dim)).astype(F)
+    pick = rng.integers(0, k, n // 2)
+    x[: n // 2] = cb[:, pick].transpose(1, 0, 2).reshape(n // 2, dim)   # rows on centroids
+    x[: n // 4] += (rng.standard_normal((n // 4, dim)) * 1e-4).astype(F)
+    dx, dcb = ctx.to_device(x), ctx.to_device(cb)
+    want = O.pq_encode(metric, x, cb).astype(np.uint8)
+    ctx.set_assign_path(0)
+    got = gpu_encode(ctx, metric, dx, n, dim, m, k, dcb)
+    frac = ctx.last_recheck_count() / float(n * m)
+    assert np.array_equal(got, want)
+    assert frac < 0.05, frac
+
+
 def test_lbg_fit_same_result_on_both_assignment_paths(ctx):
     n, dim, m, k, iters = 20000, 128, 16, 256, 5
     x = data.gaussian_mixture(n, dim, 256, 0.05, seed=1)

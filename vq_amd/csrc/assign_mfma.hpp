@@ -1,15 +1,16 @@
 // Nearest-centroid assignment for squared-L2 / Euclidean on the matrix cores, exact by re-check.
 //
 // The scores  s[j] = ||c_j||^2 + ||x||^2 - 2 x.c_j  of 32 rows against 32 centroids at a time come
-// out of the matrix cores.  The running smallest and second-smallest score of every row are kept
-// with the centroid index packed into the 8 low mantissa bits (one v_and_or per score, then five
-// v_min3 / v_med3 per four scores).  The matrix form rounds differently from the reference's
-// sequential (x-c)^2 sum, so a row is only decided from the scores when its two best are further
-// apart than a bound on every error involved (operand splitting, matrix accumulation, the packed
-// bits, the reference's own rounding).  Then the smallest exact distance is provably the same
-// centroid.  Every other (row, block) pair — exact ties, near ties, sqrt collisions under
-// Euclidean, non-finite values — is decided by the reference-order argmin, so the result is
-// bit-identical to the all-VALU path for every input.
+// out of the matrix cores.  The matrix form rounds differently from the reference's sequential
+// (x-c)^2 sum, so a row is only decided from the scores when its best candidates are further
+// apart than a bound on every error involved (operand splitting, matrix accumulation, the index
+// bits packed into the 8 low mantissa bits, the reference's own rounding).  Then the smallest
+// exact distance provably lies where the scores say.  Every other (row, block) pair — exact ties,
+// near ties, sqrt collisions under Euclidean, non-finite values — is decided by the
+// reference-order argmin, so the result is bit-identical to the all-VALU path for every input.
+// The 8-float kernel keeps the two smallest keys over runs of four consecutive centroids (the
+// run's smallest score, tagged with the run's first index) and picks inside the best run by exact
+// distances; the wide kernel keeps the three smallest scores, one tag per score.
 //
 // 8-float column blocks (k_assign_mfma_bf): bf16 matrix cores with split operands; the undecided
 // rows are resolved inside the same wave.  Wider blocks (k_assign_mfma_wide_bf): the same split
@@ -224,8 +225,7 @@ static __global__ void __launch_bounds__(256) k_mfma_bf_prep(const float *__rest
 // ---- the exact path of k_assign_mfma_bf ---------------------------------------------------------
 // Undecided rows of one (tile of 32 rows, column block) are decided by the whole wave in the
 // reference's order (src/utils.rs:63-70, src/pq.rs:166-174): lane l owns centroids l, l + 64,
-// l + 128, l + 192 (loaded once per wave and column block, when its first undecided row turns
-// up), computes their distances to the row in sequential f32 order, keeps the first smallest
+// l + 128, l + 192 (read from the wave's copy in LDS), computes their distances to the row in sequential f32 order, keeps the first smallest
 // (strict '<' over ascending indices), and the smallest (distance, index) pair over the lanes wins.
 // A NaN distance is never chosen unless it is centroid 0's, which is never replaced.  Euclidean
 // compares the roots, as the reference does.  No LDS and, per batch of up to eight rows, one
@@ -241,28 +241,14 @@ __device__ __forceinline__ void lexmin(uint32_t &d, uint32_t &i, uint32_t od, ui
     i = take ? oi : i;
 }
 
-struct ExactCentroids {  // this lane's four centroids of the column block
-    float4 c0[4], c1[4];
-};
-__device__ __forceinline__ void exact_load_centroids(ExactCentroids &ec, const float *__restrict__ cb, int k,
-                                                     int lane) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const int j = lane + 64 * q;
-        const float4 *cp = reinterpret_cast<const float4 *>(cb + (size_t)(j < k ? j : 0) * 8);
-        ec.c0[q] = cp[0];
-        ec.c1[q] = cp[1];
-    }
-}
-
-// todo: ballot of the lanes (below 32) whose row is undecided; rows = first row of the tile.
+// cl: the column block's centroids in LDS (k x 8 floats, this wave's copy).
+// todo: ballot of the lanes (below 32) whose row is undecided; xblk = first row of the tile.
 // Returns the codes of those rows in their lanes (other lanes keep `code`).
 template <int METRIC>
-__device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, const ExactCentroids &ec,
-                                           const float *__restrict__ xblk, int64_t ld, int k, int lane) {
+__device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, const float *cl,
+                                               const float *__restrict__ xblk, int64_t ld, int k, int lane) {
     const float inf = __builtin_inff();
     while (todo) {
-        // the batch: up to eight undecided rows; lane L reads float L % 8 of batch row L / 8
         int src[8];
         int cnt = 0;
         int mine = __builtin_amdgcn_readfirstlane(__ffsll(todo) - 1);
@@ -274,7 +260,7 @@ __device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, co
             if ((lane >> 3) == i) mine = src[i];
         }
         const float val = xblk[(int64_t)mine * ld + (lane & 7)];
-        for (int i = 0; i < cnt; ++i) {  // a loop, not unrolled: the path is rare and code size is not free
+        for (int i = 0; i < cnt; ++i) {
             float xs[8];
 #pragma unroll
             for (int d = 0; d < 8; ++d)
@@ -284,24 +270,23 @@ __device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, co
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int j = lane + 64 * q;
-                const float c[8] = {ec.c0[q].x, ec.c0[q].y, ec.c0[q].z, ec.c0[q].w,
-                                    ec.c1[q].x, ec.c1[q].y, ec.c1[q].z, ec.c1[q].w};
+                const float4 *cp = reinterpret_cast<const float4 *>(cl + (j < k ? j : 0) * 8);
+                const float4 c0 = cp[0], c1 = cp[1];
+                const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
                 float d = d_sq<8>(xs, c);
                 if constexpr (METRIC == M_EUCLID) d = sqrtf(d);
                 if (q == 0) dfirst = d;
                 d = (d == d) ? d : inf;
-                if (j < k && (d < bd || bi == 0x7fffffffu)) {  // ascending j: strict '<' keeps the first
+                if (j < k && (d < bd || bi == 0x7fffffffu)) {
                     bd = d;
                     bi = (uint32_t)j;
                 }
             }
-            // smallest (distance, index) of the wave: four steps inside the rows of 16 lanes, then
-            // the four rows as scalars
             uint32_t kd = __float_as_uint(bd), ki = bi;
-            lexmin(kd, ki, dpp_u32<0xB1>(kd), dpp_u32<0xB1>(ki));    // quad_perm [1,0,3,2]
-            lexmin(kd, ki, dpp_u32<0x4E>(kd), dpp_u32<0x4E>(ki));    // quad_perm [2,3,0,1]
-            lexmin(kd, ki, dpp_u32<0x141>(kd), dpp_u32<0x141>(ki));  // row_half_mirror
-            lexmin(kd, ki, dpp_u32<0x140>(kd), dpp_u32<0x140>(ki));  // row_mirror
+            lexmin(kd, ki, dpp_u32<0xB1>(kd), dpp_u32<0xB1>(ki));
+            lexmin(kd, ki, dpp_u32<0x4E>(kd), dpp_u32<0x4E>(ki));
+            lexmin(kd, ki, dpp_u32<0x141>(kd), dpp_u32<0x141>(ki));
+            lexmin(kd, ki, dpp_u32<0x140>(kd), dpp_u32<0x140>(ki));
             uint32_t rd = (uint32_t)__builtin_amdgcn_readlane((int)kd, 0), ri = (uint32_t)__builtin_amdgcn_readlane((int)ki, 0);
 #pragma unroll
             for (int row = 1; row < 4; ++row)
@@ -309,7 +294,6 @@ __device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, co
                        (uint32_t)__builtin_amdgcn_readlane((int)ki, 16 * row));
             const float d0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(dfirst), 0));
             const int best = (d0 == d0) ? (int)ri : 0;
-            // src[i] with a loop index: a chain of selects over the eight scalars
             int who = src[0];
 #pragma unroll
             for (int u = 1; u < 8; ++u) who = (i == u) ? src[u] : who;
@@ -319,222 +303,226 @@ __device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, co
     return code;
 }
 
-// One wave = TILES tiles of 32 rows and SG consecutive column blocks of 8 floats (SG = 4: one
-// 128-byte line of every row).  256 threads = 4 waves; grid = (row tiles, groups of column blocks),
-// so that the waves are short enough for the last round of workgroups not to leave the chip idle.
-template <int METRIC, bool LBG, int TILES, int SG>
-__global__ void __launch_bounds__(256, (TILES * SG <= 8) ? 4 : 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb) {
+// One wave = one column block of 8 floats against a run of tiles of 32 rows.  The wave keeps the
+// A operands of all the block's centroids in registers (8 blocks of 32 centroids x 2 instructions
+// x 4 registers) and a copy of the block's centroids in LDS, and streams the rows past them: the
+// inner loop reads no memory.  A lane's 16 scores of a tile are four runs of four consecutive
+// centroids; the smallest score of a run, tagged with the run's first index, is the run's key, and
+// the smallest and second-smallest key of the row are kept (two minima and one v_and_or per run,
+// five v_min3 / v_med3 per four runs: 17 vector instructions for 16 scores).  When the two best
+// keys are further apart than the error bound, every centroid outside the best run is provably
+// further from the row than the run's best one, and the reference's choice is the first smallest
+// exact distance among the run's four centroids, which the two lane halves compute from the LDS
+// copy, two centroids each.  Otherwise the row goes through the reference-order argmin.
+// SG = 4: the four waves of a workgroup take the four column blocks of one 128-byte line of the
+// same rows.  SG = 1 (m not a multiple of 4): the four waves take consecutive runs of one block.
+// FULL: 8 blocks of 32 centroids (k above 224), scored without a branch between them.
+template <int METRIC, bool LBG, int SG, bool FULL>
+__global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb, int run_tiles) {
     constexpr int SD = 8;
-    extern __shared__ __attribute__((aligned(16))) float lds_mu[];  // the centres [SG][8], maxc2 [SG]
+    __shared__ __attribute__((aligned(16))) float lds_cb[4][256 * SD];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int nb = tb.nb, m = a.m;
+    const int nb = FULL ? 8 : tb.nb, m = a.m, k = a.k;
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: workgroups id, id + 8,
     // id + 16, ... (the same XCD, dispatched close together) take the column-block groups of one
-    // row tile, so that the lines of those rows are fetched into one L2 once and the code bytes
-    // of a row are merged there before they are written back.
+    // run of rows, so that the code bytes of a row are merged in one L2 before they are written back.
     const int ngroups = m / SG;
     const unsigned per_chunk = 8u * (unsigned)ngroups;
     const unsigned chunk_id = blockIdx.x / per_chunk, rem = blockIdx.x % per_chunk;
-    const int s0 = (int)(rem / 8u) * SG;
-    const int64_t tile_id = (int64_t)chunk_id * 8 + (rem % 8u);
-    if (threadIdx.x < SG * 8) lds_mu[threadIdx.x] = tb.mu[(size_t)s0 * 8 + threadIdx.x];
-    if (threadIdx.x < SG) lds_mu[SG * 8 + threadIdx.x] = tb.maxc2[s0 + threadIdx.x];
-    // LBG: the blocks that have converged, read once (the same in every lane)
-    bool skip[SG];
-#pragma unroll
-    for (int q = 0; q < SG; ++q) skip[q] = LBG ? __builtin_amdgcn_readfirstlane(a.done[s0 + q]) != 0 : false;
-    __syncthreads();
-    const int64_t row_base = (tile_id * 4 + wave) * (32 * TILES);
-    if (row_base >= a.n) return;
+    const int g = (int)(rem / 8u);
+    const int64_t run_id = (int64_t)chunk_id * 8 + (rem % 8u);
+    const int s = SG == 4 ? g * 4 + wave : g;
+    const int64_t tile0 = SG == 4 ? run_id * run_tiles : (run_id * 4 + wave) * run_tiles;
+    const int64_t row0 = tile0 * 32;
+    if (row0 >= a.n) return;
+    if constexpr (LBG) {
+        if (__builtin_amdgcn_readfirstlane(a.done[s]) != 0) return;  // the block has converged
+    }
+    int64_t left = (a.n - row0 + 31) / 32;
+    const int ntiles = (int)(left < run_tiles ? left : run_tiles);
 
-    float xall[TILES][SG][4];  // this lane's dimensions [4h, 4h + 4) of every block
-    uint32_t cw[TILES];
+    // the block's centroids: this wave's copy in LDS (no other wave reads it: no barrier)
+    float *cl = lds_cb[wave];
+    {
+        const float4 *src = reinterpret_cast<const float4 *>(a.cb + (size_t)s * k * SD);
+        float4 *dst = reinterpret_cast<float4 *>(cl);
+        const int nv = 2 * k;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int i = lane + 64 * c;
+            const float4 v = src[i < nv ? i : 0];
+            if (i < nv) dst[i] = v;
+        }
+    }
+    // the A operands of every block of 32 centroids
+    u32x4 A1[8], A2[8];
+    {
+        const u32x4 *ap = tb.atab + (size_t)s * nb * 128 + lane;
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const int bc = b < nb ? b : 0;
+            A1[b] = ap[(size_t)bc * 128];
+            A2[b] = ap[(size_t)bc * 128 + 64];
+        }
+    }
+    float muh[4];  // the centre's dimensions [4h, 4h + 4)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) muh[u] = tb.mu[(size_t)s * 8 + 4 * h + u];
+    const float mc2 = tb.maxc2[s];
+    const uint32_t keep = opaque_vgpr(0xFFFFFF00u);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // rows two tiles ahead (a row past the end reads row 0 and is never stored)
+    const float *xcol = a.x + (int64_t)s * SD + 4 * h;
+    auto row_clamped = [&](int t) -> int64_t {
+        const int64_t row = row0 + 32 * (int64_t)t + r;
+        return row < a.n ? row : 0;
+    };
+    float4 xa = *reinterpret_cast<const float4 *>(xcol + row_clamped(0) * a.ld);
+    float4 xb = *reinterpret_cast<const float4 *>(xcol + row_clamped(1) * a.ld);
+    uint8_t oa = 0, ob = 0;
+    if constexpr (LBG) {
+        oa = a.codes[(size_t)s * a.n + row_clamped(0)];
+        ob = a.codes[(size_t)s * a.n + row_clamped(1)];
+    }
     uint32_t n_exact = 0;
-    uint32_t chg = 0;  // LBG: bit q set when a code of block s0 + q changed in this lane
+    bool chg = false;
+    for (int t = 0; t < ntiles; ++t) {
+        const float4 xc = xa;
+        const uint8_t old = oa;
+        xa = xb;
+        oa = ob;
+        xb = *reinterpret_cast<const float4 *>(xcol + row_clamped(t + 2) * a.ld);
+        if constexpr (LBG) ob = a.codes[(size_t)s * a.n + row_clamped(t + 2)];
+        const float xraw[4] = {xc.x, xc.y, xc.z, xc.w};
+        u32x4 b1, b2;
+        float x2;
+        {
+            float xv[4];  // relative to the block's centre
 #pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-        const int64_t row = row_base + 32 * t + r;
-        cw[t] = 0u;
-        // Unconditional loads (a row past the end reads row 0 and is never stored): loads under a
-        // branch make the compiler wait for every load in flight at each use.
-        const int64_t rc = row < a.n ? row : 0;
-        const float *xr = a.x + rc * a.ld + (int64_t)s0 * SD + 4 * h;
+            for (int u = 0; u < 4; ++u) xv[u] = xraw[u] - muh[u];
+            float p = 0.0f;
 #pragma unroll
-        for (int q = 0; q < SG; ++q)
-#pragma unroll
-            for (int u = 0; u < 4; ++u) xall[t][q][u] = xr[q * SD + u];
-    }
-    const u32x4 *ap = tb.atab + (size_t)s0 * nb * 128 + lane;
-    u32x4 pa1, pa2, qa1, qa2;
-    bool primed = false;
-#pragma unroll
-    for (int q = 0; q < SG; ++q) {
-        const int s = s0 + q;
-        if (skip[q]) {
-            primed = false;
-            continue;
+            for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
+            const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
+            const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
+            const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
+            // this half's share of ||x||^2 in two bf16 parts (it is the same in every score of the
+            // row, so its rounding cancels in their differences), then ones for the parts of ||c||^2
+            const uint32_t p0 = bf16_pack2(p, 0.0f);
+            const float r1 = p - __uint_as_float(p0 << 16);
+            const uint32_t p1 = bf16_pack2(r1, 0.0f);
+            b1 = u32x4{h01, h23, l01, l23};
+            b2 = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), 0x3f803f80u};
+            int pa, pb;
+            swap_halves(__float_as_int(p), pa, pb);
+            x2 = __int_as_float(pa) + __int_as_float(pb);  // lower half's share + upper half's, in both
         }
-        u32x4 b1[TILES], b2[TILES];
-        float x2[TILES];
-        int m1[TILES], m2[TILES];
-        uint8_t old[TILES];  // LBG: the rows' current codes, in flight while the block is scored
+        int m1 = 0x7f800000, m2 = 0x7f800000;  // +inf
+        // One block of 32 centroids.  The tag leaves out the lane half (bit 2), so it is the same in
+        // every lane and lives in scalar registers.
+#define VQ_SCORE_BLOCK(b)                                                                                       \
+    {                                                                                                           \
+        const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};      \
+        floatx16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A1[b]),               \
+                                                               __builtin_bit_cast(bf16x8, b1), zero, 0, 0, 0);  \
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A2[b]),                        \
+                                                      __builtin_bit_cast(bf16x8, b2), acc, 0, 0, 0);            \
+        int key[4];                                                                                             \
+        _Pragma("unroll") for (int p = 0; p < 4; ++p) {                                                         \
+            const int gmin = imin(imin(imin(__float_as_int(acc[4 * p]), __float_as_int(acc[4 * p + 1])),        \
+                                       __float_as_int(acc[4 * p + 2])),                                         \
+                                  __float_as_int(acc[4 * p + 3]));                                              \
+            key[p] = (int)(((uint32_t)gmin & keep) | (uint32_t)(32 * (b) + 8 * p));                             \
+        }                                                                                                       \
+        top2_push4(m1, m2, key[0], key[1], key[2], key[3]);                                                     \
+    }
+        if constexpr (FULL) {
+            VQ_SCORE_BLOCK(0) VQ_SCORE_BLOCK(1) VQ_SCORE_BLOCK(2) VQ_SCORE_BLOCK(3)
+            VQ_SCORE_BLOCK(4) VQ_SCORE_BLOCK(5) VQ_SCORE_BLOCK(6) VQ_SCORE_BLOCK(7)
+        } else {
+            VQ_SCORE_BLOCK(0) VQ_SCORE_BLOCK(1)
+            if (nb > 2) { VQ_SCORE_BLOCK(2) VQ_SCORE_BLOCK(3) }
+            if (nb > 4) { VQ_SCORE_BLOCK(4) VQ_SCORE_BLOCK(5) }
+            if (nb > 6) { VQ_SCORE_BLOCK(6) VQ_SCORE_BLOCK(7) }
+        }
+#undef VQ_SCORE_BLOCK
+        // the partner lane (other half) saw the other 16 centroids of every block
+        m1 |= 4 * h;  // bit 2 of the centroid index: the lane half
+        m2 |= 4 * h;
+        int f1, g1, f2, g2;
+        swap_halves(m1, f1, g1);
+        swap_halves(m2, f2, g2);
+        const float s1 = __int_as_float(imin(f1, g1));
+        const float s2 = __int_as_float(imin(imax(f1, g1), imin(f2, g2)));
+        const int64_t row = row0 + 32 * (int64_t)t + r;
+        const bool mine = h == 0 && row < a.n;
+        const float bound = x2 + mc2;
+        const float margin = 6.103515625e-05f * fabsf(s2) + 1.220703125e-04f * bound;
+        bool sure = (s2 - s1) > margin;  // false for NaN / inf-inf
+        // below 1e-31 the bf16 parts of ||c - mu||^2 may be subnormal, which the matrix cores may
+        // flush: up to 3 * 2^-126 lost, more than the margin allows for at such a bound
+        sure = sure && (bound < 1e29f) && (bound > 1e-31f) && (s1 < 1e29f);
+        const int first = (int)(__float_as_uint(s1) & 0xFFu);  // first centroid of the best run
+        const unsigned long long todo = __ballot(mine && !sure);
+        int code;
+        {
+            // the best run's four centroids, two per lane half, in the reference's order
+            const int j0 = first + 2 * h;
+            const int ja = j0 < k ? j0 : k - 1, jb = j0 + 1 < k ? j0 + 1 : k - 1;
+            const float4 *pa = reinterpret_cast<const float4 *>(cl + ja * SD);
+            const float4 *pb = reinterpret_cast<const float4 *>(cl + jb * SD);
+            const float4 ca0 = pa[0], ca1 = pa[1], cb0 = pb[0], cb1 = pb[1];
+            float xs[8];
 #pragma unroll
-        for (int t = 0; t < TILES; ++t) {
+            for (int u = 0; u < 4; ++u) {
+                int lo, hi;
+                swap_halves(__float_as_int(xraw[u]), lo, hi);
+                xs[u] = __int_as_float(lo);
+                xs[4 + u] = __int_as_float(hi);
+            }
+            const float ca[8] = {ca0.x, ca0.y, ca0.z, ca0.w, ca1.x, ca1.y, ca1.z, ca1.w};
+            const float cc[8] = {cb0.x, cb0.y, cb0.z, cb0.w, cb1.x, cb1.y, cb1.z, cb1.w};
+            float da = d_sq<8>(xs, ca), db = d_sq<8>(xs, cc);
+            if constexpr (METRIC == M_EUCLID) {
+                da = sqrtf(da);
+                db = sqrtf(db);
+            }
+            const bool second = (j0 + 1 < k) && (db < da);  // strict: the first of equals
+            uint32_t kd = __float_as_uint(second ? db : da);
+            const uint32_t ki = (uint32_t)(second ? j0 + 1 : j0);
+            kd = j0 < k ? kd : 0x7f800000u;  // a padding centroid
+            int dlo, dhi, ilo, ihi;
+            swap_halves((int)kd, dlo, dhi);
+            swap_halves((int)ki, ilo, ihi);
+            code = (uint32_t)dhi < (uint32_t)dlo ? ihi : ilo;  // the lower half holds the lower indices
+        }
+        if (todo) {  // the same in every lane: the reference-order argmin of the undecided rows
+            n_exact += (uint32_t)__popcll(todo);
+            code = exact_rows8<METRIC>(todo, code, cl, a.x + (row0 + 32 * (int64_t)t) * a.ld + (int64_t)s * SD, a.ld,
+                                           k, lane);
+        }
+        if (mine) {
             if constexpr (LBG) {
-                const int64_t row = row_base + 32 * t + r;
-                old[t] = a.codes[(size_t)s * a.n + (row < a.n ? row : 0)];
-            }
-            {
-                float xv[4];  // relative to the block's centre
-#pragma unroll
-                for (int u = 0; u < 4; ++u) xv[u] = xall[t][q][u] - lds_mu[q * 8 + 4 * h + u];
-                float p = 0.0f;
-#pragma unroll
-                for (int u = 0; u < 4; ++u) p = __builtin_fmaf(xv[u], xv[u], p);
-                const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
-                const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
-                const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
-                // this half's share of ||x||^2 in two bf16 parts (it is the same in every score of the
-                // row, so its rounding cancels in their differences), then ones for the parts of ||c||^2
-                const uint32_t p0 = bf16_pack2(p, 0.0f);
-                const float r1 = p - __uint_as_float(p0 << 16);
-                const uint32_t p1 = bf16_pack2(r1, 0.0f);
-                b1[t] = u32x4{h01, h23, l01, l23};
-                b2[t] = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), 0x3f803f80u};
-                int pa, pb;
-                swap_halves(__float_as_int(p), pa, pb);
-                x2[t] = __int_as_float(pa) + __int_as_float(pb);  // lower half's share + upper half's, in both
-            }
-            m1[t] = 0x7f800000;  // +inf
-            m2[t] = 0x7f800000;
-        }
-        // One block of 32 centroids against the TILES row tiles.  The packed index leaves out the
-        // lane half (bit 2), so it is the same in every lane and lives in scalar registers.
-        const uint32_t keep = opaque_vgpr(0xFFFFFF00u);
-        auto block = [&](int b, const u32x4 &a1c, const u32x4 &a2c) {
-            const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int t = 0; t < TILES; ++t) {
-                floatx16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    __builtin_bit_cast(bf16x8, a1c), __builtin_bit_cast(bf16x8, b1[t]), zero, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                    __builtin_bit_cast(bf16x8, a2c), __builtin_bit_cast(bf16x8, b2[t]), acc, 0, 0, 0);
-                int key[16];
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    key[v] = pack_tag(acc[v], keep, (uint32_t)(32 * b + 8 * (v / 4) + v % 4));
-#pragma unroll
-                for (int v = 0; v < 16; v += 4)
-                    top2_push4(m1[t], m2[t], key[v], key[v + 1], key[v + 2], key[v + 3]);
-            }
-        };
-        // The A operands of the SG column blocks are one run of SG * nb blocks (nb is even): two
-        // buffers, each refilled two blocks ahead as soon as its block is scored, so the first
-        // blocks of the next column block arrive while this one's rows are decided.
-        const int fb = q * nb;
-        if (!primed) {
-            pa1 = ap[(size_t)fb * 128];
-            pa2 = ap[(size_t)fb * 128 + 64];
-            qa1 = ap[(size_t)(fb + 1) * 128];
-            qa2 = ap[(size_t)(fb + 1) * 128 + 64];
-            primed = true;
-        }
-        for (int b = 0; b < nb; b += 2) {
-            block(b, pa1, pa2);
-            const int f2 = fb + b + 2 < SG * nb ? fb + b + 2 : SG * nb - 2;  // past the end: any valid block
-            pa1 = ap[(size_t)f2 * 128];
-            pa2 = ap[(size_t)f2 * 128 + 64];
-            block(b + 1, qa1, qa2);
-            qa1 = ap[(size_t)(f2 + 1) * 128];
-            qa2 = ap[(size_t)(f2 + 1) * 128 + 64];
-        }
-        const float mc2 = lds_mu[SG * 8 + q];
-        int code[TILES];
-        unsigned long long todo[TILES], any_todo = 0;
-#pragma unroll
-        for (int t = 0; t < TILES; ++t) {
-            // the partner lane (other half) saw the other 16 centroids of every block
-            m1[t] |= 4 * h;  // bit 2 of the centroid index: the lane half
-            m2[t] |= 4 * h;
-            int f1, g1, f2, g2;
-            swap_halves(m1[t], f1, g1);
-            swap_halves(m2[t], f2, g2);
-            const float s1 = __int_as_float(imin(f1, g1));
-            const float s2 = __int_as_float(imin(imax(f1, g1), imin(f2, g2)));
-            const int64_t row = row_base + 32 * t + r;
-            const bool mine = h == 0 && row < a.n;
-            const float bound = x2[t] + mc2;
-            const float margin = 6.103515625e-05f * fabsf(s2) + 1.220703125e-04f * bound;
-            bool sure = (s2 - s1) > margin;  // false for NaN / inf-inf
-            // below 1e-31 the bf16 parts of ||c - mu||^2 may be subnormal, which the matrix cores may
-            // flush: up to 3 * 2^-126 lost, more than the margin allows for at such a bound
-            sure = sure && (bound < 1e29f) && (bound > 1e-31f) && (s1 < 1e29f);
-            code[t] = (int)(__float_as_uint(s1) & 0xFFu);
-            todo[t] = __ballot(mine && !sure);
-            any_todo |= todo[t];
-        }
-        if (any_todo) {  // the same in every lane: the reference-order argmin of the undecided rows
-            ExactCentroids ec;
-            exact_load_centroids(ec, a.cb + (size_t)s * a.k * SD, a.k, lane);
-#pragma unroll
-            for (int t = 0; t < TILES; ++t) {
-                n_exact += (uint32_t)__popcll(todo[t]);
-                if (todo[t])
-                    code[t] = exact_rows8<METRIC>(todo[t], code[t], ec, a.x + (row_base + 32 * t) * a.ld + (int64_t)s * SD,
-                                                  a.ld, a.k, lane);
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < TILES; ++t) {
-            const int64_t row = row_base + 32 * t + r;
-            const bool mine = h == 0 && row < a.n;
-            if (mine) {
-                if constexpr (LBG) {
-                    if (old[t] != (uint8_t)code[t]) {
-                        a.codes[(size_t)s * a.n + row] = (uint8_t)code[t];
-                        chg |= 1u << q;
-                    }
-                } else if (SG == 4 || SG == 2) {
-                    cw[t] |= (uint32_t)code[t] << (8 * q);
-                } else {
-                    a.codes[row * m + s] = (uint8_t)code[t];
+                if (old != (uint8_t)code) {
+                    a.codes[(size_t)s * a.n + row] = (uint8_t)code;
+                    chg = true;
                 }
-            }
-        }
-    }
-    if constexpr (!LBG && (SG == 4 || SG == 2)) {
-        if (h == 0) {
-#pragma unroll
-            for (int t = 0; t < TILES; ++t) {
-                const int64_t row = row_base + 32 * t + r;
-                if (row < a.n) {
-                    if constexpr (SG == 4)
-                        *reinterpret_cast<uint32_t *>(a.codes + row * m + s0) = cw[t];
-                    else
-                        *reinterpret_cast<uint16_t *>(a.codes + row * m + s0) = (uint16_t)cw[t];
-                }
+            } else {
+                a.codes[row * m + s] = (uint8_t)code;
             }
         }
     }
     if constexpr (LBG) {
         // changed[s]: one lane per wave, once per wave, and only where the flag still reads 0 (every
         // store to one address is serialised in its L2 channel; a stale 0 from the vector cache
-        // costs a store, nothing else).  The flags are read together: one memory round trip.
-        uint32_t any = 0;
-#pragma unroll
-        for (int q = 0; q < SG; ++q) any |= __any((chg >> q) & 1u) ? (1u << q) : 0u;
-        if (lane == 0 && any) {
-            int cur[SG];
-#pragma unroll
-            for (int q = 0; q < SG; ++q) cur[q] = a.changed[s0 + q];
-#pragma unroll
-            for (int q = 0; q < SG; ++q)
-                if (((any >> q) & 1u) && cur[q] == 0) a.changed[s0 + q] = 1;
-        }
+        // costs a store, nothing else).
+        if (__any(chg) && lane == 0 && a.changed[s] == 0) a.changed[s] = 1;
     }
     if (lane == 0 && n_exact)
-        atomicAdd(tb.stat + ((tile_id * 4 + wave) & (kStatSlots - 1)) * kStatStride, n_exact);
+        atomicAdd(tb.stat + ((run_id * 4 + wave) & (kStatSlots - 1)) * kStatStride, n_exact);
 }
 
 }  // namespace vq

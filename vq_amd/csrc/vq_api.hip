@@ -19,11 +19,8 @@
 #include "assign_exact.hpp"
 #include "assign_mfma.hpp"
 
-#ifndef VQ_MFMA_TILES
-#define VQ_MFMA_TILES 2  // tiles of 32 rows per wave in the matrix-core assignment
-#endif
-#ifndef VQ_MFMA_SG
-#define VQ_MFMA_SG 4     // column blocks of 8 floats per wave (4: one 128-byte line of each row)
+#ifndef VQ_MFMA_RUN
+#define VQ_MFMA_RUN 8    // tiles of 32 rows per wave in the matrix-core assignment (a power of two)
 #endif
 #include "lbg_update.hpp"
 #include "calibrate.hpp"
@@ -164,18 +161,24 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready, hip
     MfmaTabPtrs t;
     VQ_TRY(mfma_tab_ptrs(ctx, a.m, a.k, t));
     const int nb = t.nb;
-    constexpr int TILES = VQ_MFMA_TILES;
     if (!tables_ready)
         hipLaunchKernelGGL(vq::k_mfma_bf_prep, dim3(a.m), dim3(256), 0, ctx->stream, a.cb, a.m, a.k, nb, t.atab,
                            t.maxc2, t.mu, t.stat);
     vq::MfmaBfTables tb{(const vq::u32x4 *)t.atab, t.maxc2, t.mu, t.stat, nb};
-    // 4 column blocks of 8 floats = one 128-byte line per row
-    constexpr int SG = VQ_MFMA_SG;
-    const bool grouped = a.m % SG == 0;
-    auto kern = grouped ? vq::k_assign_mfma_bf<METRIC, LBG, TILES, SG> : vq::k_assign_mfma_bf<METRIC, LBG, TILES, 1>;
-    const int sg = grouped ? SG : 1;
-    const size_t lds = sizeof(float) * sg * 9;
-    const int64_t blocks = cdiv(cdiv(a.n, 4 * 32 * TILES), 8) * 8 * (a.m / sg);  // tiles in chunks of 8
+    // a workgroup = 4 column blocks of 8 floats (one 128-byte line per row) against one run of row
+    // tiles, or, where m is not a multiple of 4, one column block against four runs
+    const bool grouped = a.m % 4 == 0, full = nb == 8;
+    const void *kern =
+        grouped ? (full ? (const void *)vq::k_assign_mfma_bf<METRIC, LBG, 4, true> : (const void *)vq::k_assign_mfma_bf<METRIC, LBG, 4, false>)
+                : (full ? (const void *)vq::k_assign_mfma_bf<METRIC, LBG, 1, true> : (const void *)vq::k_assign_mfma_bf<METRIC, LBG, 1, false>);
+    // A wave loads the operands of its column block once (16 KB + 8 KB) and amortises them over
+    // its run: 8 tiles of 32 rows where that still leaves several rounds of workgroups per compute unit.
+    const int64_t tiles = cdiv(a.n, 32);
+    const int64_t groups = grouped ? a.m / 4 : a.m;
+    int run_tiles = VQ_MFMA_RUN;
+    while (run_tiles > 1 && cdiv(tiles, (grouped ? 1 : 4) * run_tiles) * groups < 8192) run_tiles >>= 1;
+    const int64_t runs = cdiv(tiles, (grouped ? 1 : 4) * (int64_t)run_tiles);
+    const int64_t blocks = cdiv(runs, 8) * 8 * groups;  // runs in chunks of 8
     if (blocks >= (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * m too large for one launch");
     hipEvent_t ev_a = nullptr, ev_b = nullptr;
     if (ctx->prof_on) {
@@ -185,11 +188,12 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready, hip
     } else if (done) {
         ev_b = ctx->ev_fork;
     }
+    vq::AssignArgs aa = a;
+    void *args[] = {&aa, &tb, &run_tiles};
     if (ev_a || ev_b)
-        hipExtLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), (uint32_t)lds, ctx->stream, ev_a, ev_b, 0u, a,
-                              tb);
+        VQ_HIP(ctx, hipExtLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, 0, ctx->stream, ev_a, ev_b, 0u));
     else
-        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), lds, ctx->stream, a, tb);
+        VQ_HIP(ctx, hipLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, 0, ctx->stream));
     VQ_HIP(ctx, hipGetLastError());
     if (started) *started = ev_a;
     if (done) *done = ev_b;
