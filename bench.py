@@ -36,7 +36,7 @@ PEAK_HBM_GBS = 8000.0
 PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X published dense bf16 matrix peak
 # rocprofv3 FETCH_SIZE / WRITE_SIZE of one LBG launch of k_assign_mfma_bf (KiB per dispatch), scaled by
 # the plain copy kernel (FETCH x 2.000, WRITE x 1.000): profiles/pq_fit_encode_1Mx128.md
-MEASURED_ASSIGN_TRAFFIC_BYTES = int((263610.0 * 2.000 + 12207.0 * 1.000) * 1024)
+MEASURED_ASSIGN_TRAFFIC_BYTES = int((261910.0 * 2.000 + 12562.0 * 1.000) * 1024)
 
 
 def log(*a):
@@ -113,17 +113,20 @@ def main():
     value = n / (ms_per_step * 1e-3)
 
     # Dominant kernel: the assignment pass (k_assign_mfma_bf), timed alone by HIP events on the
-    # library's stream (start and stop events of each launch's own dispatch).  What binds it is the
-    # vector ALU: the n x (m*k) scores come out of the matrix cores (which stay under a third busy)
-    # and every one of them has to pass through the selection of the row's two smallest.
+    # library's stream (start and stop events of each launch's own dispatch).  What binds it is
+    # instruction issue: the n x (m*k) scores come out of the matrix cores, every one of them has
+    # to pass through the selection of the row's two smallest keys on the vector ALU, and on this
+    # chip the two kinds of instruction take turns on a SIMD (one more matrix instruction per tile
+    # lengthens the pass by that instruction's 32 clocks).
     #   algorithmic vector work per row = 2 lane-slots per score (one to tag or compare, one to
     #   select) = 2*m*k = 8,192; the 2*k*D lane-slots of the distance sums are on the matrix cores
     #   and priced there (mfma_* fields), so they are NOT counted against the vector peak.
     #   peak = 78.6 T lane-slots/s (256 CUs x 128 lanes x 2.4 GHz: one instruction per lane per
     #   clock; the published 157.3 TFLOP/s fp32 vector figure counts a fused multiply-add as two).
-    # The instructions the selection is actually made of (v_and_or_b32, v_min3_i32, v_med3_i32)
-    # issue at 4.2 clocks per wave64 on this chip, not 2, and the kernel needs 2.25 per score, so
-    # frac = 0.43 is the ceiling of this formulation; selection_floor_ms prices exactly that.
+    # The kernel spends 17 instructions on 16 scores (v_min_i32 / v_min3_i32 over runs of four
+    # centroids, one v_and_or_b32 tag per run, v_min3_i32 / v_med3_i32 for the two smallest keys),
+    # each 4.2 clocks per wave64 on this chip, not 1; selection_floor_ms prices exactly those, and
+    # issue_floor_ms adds the two matrix instructions per 32 x 32 tile at the nominal clock.
     flop_per_launch = 2.0 * K * DIM * n
     bytes_per_launch = (4.0 * DIM + 2.0 * M) * n
     slots_per_launch = 2.0 * M * K * n
@@ -133,8 +136,9 @@ def main():
     achieved_slots = slots_per_launch / sec / 1e12
     roofline = {
         "bound": "valu",
-        "kernel": "k_assign_mfma_bf (bf16-split matrix-core scores + packed-index top-2 selection on the "
-                  "vector ALU + in-wave exact re-check; the 10 LBG passes and the encode pass)",
+        "kernel": "k_assign_mfma_bf (bf16-split matrix-core scores, top-2 selection over runs of four "
+                  "centroids on the vector ALU, exact pick inside the best run, in-wave exact re-check; "
+                  "the 10 LBG passes and the encode pass)",
         "achieved": round(achieved_slots, 3),
         "peak": PEAK_VALU_TLANESLOTS,
         "unit": "T lane-slots/s",
@@ -157,17 +161,21 @@ def main():
         "hbm_frac": round(bytes_per_launch / sec / 1e9 / PEAK_HBM_GBS, 4),
         "assign_ms_incl_tables": round(assign_ms / max(assign_n, 1), 4),
     }
-    # Measured issue rates of this box (vq_calibrate).  Per four scores the kernel issues
-    # 4 v_and_or_b32 (index tag), 3 v_min3_i32 and 2 v_med3_i32 (top-2 update); one wave64
-    # instruction handles 64 scores.  The floor is the time those instructions alone take with
-    # every SIMD full.
+    # Measured issue rates of this box (vq_calibrate).  Per 16 scores the kernel issues 8 minima
+    # (v_min_i32 / v_min3_i32, one class) for the four runs, 4 v_and_or_b32 (the runs' tags), and
+    # 3 v_min3_i32 + 2 v_med3_i32 (top-2 update); one wave64 instruction handles 64 lanes.  The
+    # selection floor is the time those instructions alone take with every SIMD full; the issue
+    # floor adds the matrix instructions (2 per 32 x 32 tile, 32 clocks each, 1024 SIMDs at 2.4 GHz).
     rate = {name: ctx.calibrate(kind) for kind, name in
             ((1, "v_fma_f32"), (2, "v_min3_i32"), (3, "v_med3_i32"), (4, "v_and_or_b32"), (5, "v_add_u32"))}
     scores = float(n) * M * K
-    floor_ms = scores / 64.0 * (1.0 / rate["v_and_or_b32"] + 0.75 / rate["v_min3_i32"]
-                                + 0.5 / rate["v_med3_i32"]) * 1e3
+    floor_ms = scores / 64.0 * ((11.0 / 16.0) / rate["v_min3_i32"] + 0.25 / rate["v_and_or_b32"]
+                                + 0.125 / rate["v_med3_i32"]) * 1e3
+    mfma_ms = scores / 1024.0 * 2.0 * 32.0 / (1024.0 * 2.4e9) * 1e3
     roofline["selection_floor_ms"] = round(floor_ms, 4)
     roofline["frac_of_selection_floor"] = round(floor_ms / avg_kern_ms, 4)
+    roofline["issue_floor_ms"] = round(floor_ms + mfma_ms, 4)
+    roofline["frac_of_issue_floor"] = round((floor_ms + mfma_ms) / avg_kern_ms, 4)
     calibration = {
         "hbm_copy_GBs_read_plus_write": round(ctx.calibrate(0), 1),
         "valu_wave64_Ginstr_per_s": {k_: round(v / 1e9, 1) for k_, v in rate.items()},

@@ -374,19 +374,26 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
-    // rows two tiles ahead (a row past the end reads row 0 and is never stored)
+    // rows two tiles ahead; the lane's row moves on by 32 per tile, so its offset is added up
+    // rather than multiplied out
     const float *xcol = a.x + (int64_t)s * SD + 4 * h;
-    auto row_clamped = [&](int t) -> int64_t {
-        const int64_t row = row0 + 32 * (int64_t)t + r;
-        return row < a.n ? row : 0;
-    };
-    float4 xa = *reinterpret_cast<const float4 *>(xcol + row_clamped(0) * a.ld);
-    float4 xb = *reinterpret_cast<const float4 *>(xcol + row_clamped(1) * a.ld);
+    const uint8_t *ccol = a.codes + (size_t)s * a.n;
+    const int64_t lane_rows = a.n - (row0 + r);                       // rows from this lane's first to the end
+    const int64_t lane_left = lane_rows > 0 ? (lane_rows + 31) / 32 : 0;
+    // tiles of this run in which the lane has a row; the fetches past the run's end read row 0
+    // (the next run belongs to a workgroup on another XCD: its rows would be fetched into two L2s)
+    const int lane_tiles = (int)(lane_left < run_tiles ? lane_left : run_tiles);
+    const int64_t xstep = 32 * a.ld;
+    int64_t xoff = (row0 + r) * a.ld, coff = row0 + r;                // of the lane's row in tile 0
+    auto fetch_x = [&](int t) { return *reinterpret_cast<const float4 *>(xcol + (t < lane_tiles ? xoff : 0)); };
+    auto fetch_c = [&](int t) { return ccol[t < lane_tiles ? coff : 0]; };
+    float4 xa = fetch_x(0);
     uint8_t oa = 0, ob = 0;
-    if constexpr (LBG) {
-        oa = a.codes[(size_t)s * a.n + row_clamped(0)];
-        ob = a.codes[(size_t)s * a.n + row_clamped(1)];
-    }
+    if constexpr (LBG) oa = fetch_c(0);
+    xoff += xstep;
+    coff += 32;
+    float4 xb = fetch_x(1);
+    if constexpr (LBG) ob = fetch_c(1);
     uint32_t n_exact = 0;
     bool chg = false;
     for (int t = 0; t < ntiles; ++t) {
@@ -394,8 +401,10 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
         const uint8_t old = oa;
         xa = xb;
         oa = ob;
-        xb = *reinterpret_cast<const float4 *>(xcol + row_clamped(t + 2) * a.ld);
-        if constexpr (LBG) ob = a.codes[(size_t)s * a.n + row_clamped(t + 2)];
+        xoff += xstep;
+        coff += 32;
+        xb = fetch_x(t + 2);
+        if constexpr (LBG) ob = fetch_c(t + 2);
         const float xraw[4] = {xc.x, xc.y, xc.z, xc.w};
         u32x4 b1, b2;
         float x2;
