@@ -68,6 +68,32 @@ __device__ __forceinline__ void swap_halves(int v, int &a, int &b) {
     b = (int)r[1];
 }
 
+// v_med3_i32 / v_max3_i32 by name, for the same reason.  Not for operands that a matrix instruction
+// has just written: the compiler does not count wait states for inline assembly.
+__device__ __forceinline__ int imed3a(int a, int b, int c) {
+    int r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ int imax3a(int a, int b, int c) {
+    int r;
+    asm("v_max3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// Four new keys into the running three smallest (m1 <= m2 <= m3): 10 operations.  The smallest
+// comes out of two min3 steps; the second is the smallest of m2 and the two medians; the third
+// is the smallest of everything else that can still be third: the median of those three, the
+// two maxima, and m3.
+__device__ __forceinline__ void top3_push4(int &m1, int &m2, int &m3, int k0, int k1, int k2, int k3) {
+    const int ta = imed3a(m1, k0, k1), xa = imax3a(m1, k0, k1), a1 = imin3(m1, k0, k1);
+    const int tb = imed3a(a1, k2, k3), xb = imax3a(a1, k2, k3);
+    m1 = imin3(a1, k2, k3);
+    const int md = imed3a(m2, ta, tb);
+    m2 = imin3(m2, ta, tb);
+    m3 = imin(imin3(m3, xa, xb), md);
+}
+
 // Four new keys into the running (smallest, second smallest): 5 operations.
 // second smallest of {m1, m2, x, y} with m1 <= m2 is min(m2, med3(m1, x, y)).
 __device__ __forceinline__ void top2_push4(int &m1, int &m2, int k0, int k1, int k2, int k3) {
@@ -542,31 +568,27 @@ namespace vq {
 
 // ---------------------------------------------------------------------------------------------
 // Wide column blocks on the bf16 matrix cores: the operand split of k_assign_mfma_bf applied to
-// every chunk of 8 dimensions (two instructions per chunk and tile of 32 centroids; each lane half
-// owns 4 of the 8 dimensions, the three bf16 parts of its share of ||x||^2 ride in the spare slots
-// of the second instruction).
+// 16 dimensions at a time.  With the high and low bf16 parts of the centroid operand (ah, al) and
+// of the row operand (xh, xl), a tile of 32 rows x 32 centroids takes three instructions per 16
+// dimensions, ah.xh + al.xh + ah.xl, each with all 16 contraction slots in use (each lane half
+// owns 8 of the 16 dimensions).  An earlier shape worked on 8 dimensions with two instructions,
+// {ah, al}.{xh, xh} and {ah, al}.{xl, 0}: a quarter of the slots multiplied zeros.
 // A workgroup = 128 rows; a wave takes one tile of 32 rows against every tile of 32 centroids: 8
-// accumulator tiles (128 registers) that start at ||c - mu||^2.  The centroid operand of a tile and
-// chunk is the 16 bytes {ah, al} as they lie in LDS, used by both instructions:
-//     A . {xh, xh} = ah.xh + al.xh        A . {xl, 0} = ah.xl
-// so the row is split once per chunk for 16 matrix instructions and no operand is assembled in
-// registers (vector and matrix instructions mostly take turns on a SIMD: an earlier shape — two
-// row tiles x four centroid tiles per wave, operands {ah, ah} and {al, 1, ...} built from the LDS
-// word, ||x||^2 fed through spare slots — spent as many cycles on vector work as on the matrix
-// instructions: 0.55 ms per pass at 1M x 256 against 0.39 ms now).  ||x - mu||^2 is summed on the
-// vector ALU and added to the scores before the selection.  The A operands of a chunk (16 KB for
-// 256 centroids) are staged in LDS once per workgroup, double-buffered; the row and the next A
-// chunk are fetched one chunk ahead.
+// accumulator tiles (128 registers) that start at ||c - mu||^2.  The centroid operands of a tile
+// are the 16 bytes of ah and the 16 bytes of al as they lie in LDS, and the row is split once per
+// 16 dimensions for 3 NB matrix instructions, so no operand is assembled in registers (vector
+// and matrix instructions take turns on a SIMD).  ||x - mu||^2 is summed on the vector ALU and
+// added to the scores before the selection.  The A operands of 16 dimensions (16 KB for 256
+// centroids) are staged in LDS once per workgroup, double-buffered; the row and the next A
+// operands are fetched one stage ahead.
 // Error of a score: 3 * 2^-16 (split, as above) + (34 * sd/8 + 16) * 2^-24 (fp32 accumulation, an
-// upper bound: 12 non-zero addends per chunk and the final sum) + 2^-22 (rounding of x - mu and
-// c - mu), per unit of ||x - mu||^2 + ||c - mu||^2; twice that for two candidates.
-#ifndef VQ_WIDE_STAGE_CHUNKS
-#define VQ_WIDE_STAGE_CHUNKS 2
-#endif
+// upper bound: at most 17 additions per instruction, 1.5 instructions per 8 dimensions, and the
+// final sum) + 2^-22 (rounding of x - mu and c - mu), per unit of ||x - mu||^2 + ||c - mu||^2;
+// twice that for two candidates.
 constexpr int kWideCentreMax = 2048;  // widest column block whose centre is staged in LDS
 
 struct MfmaWideBfTables {
-    const u32x4 *atab;     // [m][sd/8][nb][64]  {ah, al} of the lane's four dimensions
+    const u32x4 *atab;     // [m][ceil(sd/16)][nb][2][64]  ah, then al, of the lane's eight dimensions
     const float *c2perm;   // [m][nb][2][16]
     const float *blockmax; // [m][nb]  largest ||c - mu||^2 per block of 32 centroids (NaN if any is NaN)
     const float *mu;       // [m][sd]  centre of every column block: mean of its centroids
@@ -644,7 +666,7 @@ static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *_
     const int s = blockIdx.x, b = blockIdx.y;
     const int i = threadIdx.x & 31, g = threadIdx.x >> 5;
     const int j = b * 32 + i;
-    const int nkc = sd / 8;
+    const int npair = (sd + 15) / 16;
     __shared__ float part[8][32];
     // the same decision in every workgroup of the column block (same values, same order)
     float mm = 0.0f, cc = 0.0f;
@@ -657,37 +679,43 @@ static __global__ void __launch_bounds__(256) k_mfma_wide_bf_prep(const float *_
     if (b == 0 && threadIdx.x == 0) shifted[s] = on ? 1 : 0;
     const float *c = cb + ((size_t)s * k + (j < k ? j : 0)) * sd;
     float p = 0.0f;
-    for (int kc = g; kc < nkc; kc += 8) {
-        const float4 v0 = *reinterpret_cast<const float4 *>(c + kc * 8);
-        const float4 v1 = *reinterpret_cast<const float4 *>(c + kc * 8 + 4);
-        float4 u0 = make_float4(0.f, 0.f, 0.f, 0.f), u1 = u0;
-        if (on) {
-            u0 = *reinterpret_cast<const float4 *>(mu + (size_t)s * sd + kc * 8);
-            u1 = *reinterpret_cast<const float4 *>(mu + (size_t)s * sd + kc * 8 + 4);
-        }
-        const float cv[8] = {v0.x - u0.x, v0.y - u0.y, v0.z - u0.z, v0.w - u0.w,
-                             v1.x - u1.x, v1.y - u1.y, v1.z - u1.z, v1.w - u1.w};
-        uint32_t hw[4], lw[4];  // packed pairs of the high and low parts
+    for (int pr = g; pr < npair; pr += 8) {
+        // lane i + 32 h holds the dimensions 16 pr + 8 h .. + 7 (zeros past the block's width): 16
+        // bytes of high parts, then, 64 entries on, 16 bytes of low parts, each the operand of a
+        // matrix instruction as it lies in LDS
+        u32x4 *dst = atab + (((size_t)s * npair + pr) * nb + b) * 128;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            uint32_t hb[2], lb[2];
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const float x = cv[2 * w + e];
-                p = __builtin_fmaf(x, x, p);
-                const float a = (j < k) ? -2.0f * x : 0.0f;
-                hb[e] = bf16_rne_bits(a);
-                lb[e] = bf16_rne_bits(a - bf16_bits_to_float(hb[e]));
+        for (int h = 0; h < 2; ++h) {
+            const int d0 = 16 * pr + 8 * h;
+            const bool in = d0 < sd;  // sd is a multiple of 8
+            const int dc = in ? d0 : 0;
+            const float4 v0 = *reinterpret_cast<const float4 *>(c + dc);
+            const float4 v1 = *reinterpret_cast<const float4 *>(c + dc + 4);
+            float4 u0 = make_float4(0.f, 0.f, 0.f, 0.f), u1 = u0;
+            if (on) {
+                u0 = *reinterpret_cast<const float4 *>(mu + (size_t)s * sd + dc);
+                u1 = *reinterpret_cast<const float4 *>(mu + (size_t)s * sd + dc + 4);
             }
-            hw[w] = hb[0] | (hb[1] << 16);
-            lw[w] = lb[0] | (lb[1] << 16);
-        }
-        // lane i + 32 h holds {ah[4h..4h+3], al[4h..4h+3]}: the kernel builds instruction 1's operand
-        // {ah, ah} and instruction 2's {al, 1, 1, 1, 0} from it, so that only the 16 bytes that differ
-        // between centroids go through LDS
-        u32x4 *dst = atab + (((size_t)s * nkc + kc) * nb + b) * 64;
+            float cv[8] = {v0.x - u0.x, v0.y - u0.y, v0.z - u0.z, v0.w - u0.w,
+                           v1.x - u1.x, v1.y - u1.y, v1.z - u1.z, v1.w - u1.w};
+            uint32_t hw[4], lw[4];  // packed pairs of the high and low parts
 #pragma unroll
-        for (int h = 0; h < 2; ++h) dst[32 * h + i] = u32x4{hw[2 * h], hw[2 * h + 1], lw[2 * h], lw[2 * h + 1]};
+            for (int w = 0; w < 4; ++w) {
+                uint32_t hb[2], lb[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float x = in ? cv[2 * w + e] : 0.0f;
+                    p = __builtin_fmaf(x, x, p);
+                    const float a = (j < k) ? -2.0f * x : 0.0f;
+                    hb[e] = bf16_rne_bits(a);
+                    lb[e] = bf16_rne_bits(a - bf16_bits_to_float(hb[e]));
+                }
+                hw[w] = hb[0] | (hb[1] << 16);
+                lw[w] = lb[0] | (lb[1] << 16);
+            }
+            dst[32 * h + i] = u32x4{hw[0], hw[1], hw[2], hw[3]};
+            dst[64 + 32 * h + i] = u32x4{lw[0], lw[1], lw[2], lw[3]};
+        }
     }
     part[g][i] = p;
     __syncthreads();
@@ -722,8 +750,7 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 template <bool LBG, int NB>
 __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, MfmaWideBfTables tb) {
     constexpr int NBMAX = 8;
-    constexpr int SC = VQ_WIDE_STAGE_CHUNKS;  // chunks of 8 dimensions per stage (per barrier)
-    __shared__ u32x4 lds_a[2][SC * NBMAX * 64];  // 2 stages x SC chunks x 8 KB
+    __shared__ u32x4 lds_a[2][NBMAX * 128];  // 2 stages x 16 dimensions x 256 centroids x {high, low}: 2 x 16 KB
     __shared__ float lds_c2[NBMAX * 32];
     __shared__ float lds_mu[kWideCentreMax];
     __shared__ uint32_t wg_list[128];
@@ -736,11 +763,11 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
     constexpr int nb = NB;
-    const int sd = tb.sd, nkc = sd / 8;
-    const u32x4 *ag = tb.atab + (size_t)s * nkc * nb * 64;
-    const int chunk16 = nb * 64;  // 16-byte pieces per chunk
+    const int sd = tb.sd, npair = (sd + 15) / 16;
+    const u32x4 *ag = tb.atab + (size_t)s * npair * nb * 128;
+    const int pair16 = nb * 128;  // 16-byte pieces per 16 dimensions
     for (int i = threadIdx.x; i < nb * 32; i += 256) lds_c2[i] = tb.c2perm[(size_t)s * nb * 32 + i];
-    for (int i = threadIdx.x; i < SC * chunk16; i += 256) lds_a[0][i] = ag[i < nkc * chunk16 ? i : nkc * chunk16 - 1];
+    for (int i = threadIdx.x; i < pair16; i += 256) lds_a[0][i] = ag[i];
     if (threadIdx.x == 0) {
         wg_count = 0;
         wg_pcount = 0;
@@ -751,7 +778,7 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
 
     const int64_t row = (int64_t)blockIdx.x * 128 + wave * 32 + r;
     const bool valid = row < a.n;
-    const float *xr = a.x + (valid ? row : 0) * a.ld + (int64_t)s * sd + 4 * h;  // this half's 4 dimensions
+    const float *xr = a.x + (valid ? row : 0) * a.ld + (int64_t)s * sd;
     const bool shifted = tb.shifted[s] != 0;  // uniform
     // the accumulators start at ||c - mu||^2; ||x - mu||^2, the same in every score of a row, is
     // summed on the side and added before the selection
@@ -760,110 +787,119 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[b][v] = lds_c2[(b * 2 + h) * 16 + v];
-    // Loads are unconditional (a row past the end reads row 0 and is never stored; A pieces past
-    // the chunk are clamped): loads under a branch make the compiler wait for every outstanding
-    // load at each use instead of counting them.
-    float4 xn = *reinterpret_cast<const float4 *>(xr);  // the next chunk of the row
+    // Loads are unconditional (a row past the end reads row 0 and is never stored; pieces past
+    // the block's width are clamped and zeroed): loads under a branch make the compiler wait for
+    // every outstanding load at each use instead of counting them.
+    // This half's 8 of the 16 dimensions of a stage: 16 pr + 8 h .. + 7.
+    auto piece = [&](int pr) { return 16 * pr + 8 * h < sd ? 16 * pr + 8 * h : 0; };
+    float4 xn0 = *reinterpret_cast<const float4 *>(xr + piece(0));  // the next piece of the row
+    float4 xn1 = *reinterpret_cast<const float4 *>(xr + piece(0) + 4);
     float x2 = 0.0f;
-    // A stage is SC chunks of 8 dimensions: one barrier per 16 SC matrix instructions of a wave.
-    // Chunks past the last one have zero row operands (they add nothing).
-    const int nst = (nkc + SC - 1) / SC;
-    const int total16 = nkc * chunk16;
-    for (int st = 0; st < nst; ++st) {
+    // A stage is 16 dimensions: with the high and low parts of the centroid operand (ah, al) and of
+    // the row operand (xh, xl), three matrix instructions per tile of 32 centroids,
+    //   ah . xh + al . xh + ah . xl,
+    // every contraction slot of each in use; one barrier per 3 NB matrix instructions of a wave.
+    const int total16 = npair * pair16;
+    for (int st = 0; st < npair; ++st) {
         const int cur = st & 1;
-        const bool more = st + 1 < nst;
+        const bool more = st + 1 < npair;
         // the A operands of the next stage: into registers now, into LDS at the end of this stage
-        u32x4 pre[2 * SC];
+        u32x4 pre[4];
 #pragma unroll
-        for (int q = 0; q < 2 * SC; ++q) {
-            const int i = (st + 1) * SC * chunk16 + (int)threadIdx.x + 256 * q;
+        for (int q = 0; q < 4; ++q) {
+            const int i = (st + 1) * pair16 + (int)threadIdx.x + 256 * q;
             pre[q] = ag[i < total16 ? i : total16 - 1];
         }
-        // The stage's centroid operands are read from LDS four tiles (one group) at a time (reading a
-        // group ahead of its use measured the same and costs 16 registers).
-        constexpr int NG = (NB + 3) / 4;  // groups of four centroid tiles per chunk
-        auto read_group = [&](int sub, int g, u32x4 (&av)[4]) {
+        // operands of this stage from the row piece fetched one stage ago
+        const bool in = 16 * st + 8 * h < sd;
+        float xv[8] = {xn0.x, xn0.y, xn0.z, xn0.w, xn1.x, xn1.y, xn1.z, xn1.w};
+        if (shifted) {
+            const float4 m0 = *reinterpret_cast<const float4 *>(lds_mu + piece(st));
+            const float4 m1 = *reinterpret_cast<const float4 *>(lds_mu + piece(st) + 4);
+            xv[0] -= m0.x;
+            xv[1] -= m0.y;
+            xv[2] -= m0.z;
+            xv[3] -= m0.w;
+            xv[4] -= m1.x;
+            xv[5] -= m1.y;
+            xv[6] -= m1.z;
+            xv[7] -= m1.w;
+        }
+        if (!in) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) xv[u] = 0.0f;
+        }
+        uint32_t hp[4], lp[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            x2 = __builtin_fmaf(xv[2 * u], xv[2 * u], x2);
+            x2 = __builtin_fmaf(xv[2 * u + 1], xv[2 * u + 1], x2);
+            hp[u] = bf16_pack2(xv[2 * u], xv[2 * u + 1]);
+            lp[u] = bf16_pack2(xv[2 * u] - __uint_as_float(hp[u] << 16), xv[2 * u + 1] - __uint_as_float(hp[u] & 0xffff0000u));
+        }
+        const u32x4 bh = u32x4{hp[0], hp[1], hp[2], hp[3]}, bl = u32x4{lp[0], lp[1], lp[2], lp[3]};
+        // fetch the next piece of the row
+        const int nx = st + 1 < npair ? st + 1 : npair - 1;
+        xn0 = *reinterpret_cast<const float4 *>(xr + piece(nx));
+        xn1 = *reinterpret_cast<const float4 *>(xr + piece(nx) + 4);
+        // The stage's centroid operands are read from LDS four tiles (one group) at a time.
+        constexpr int NG = (NB + 3) / 4;  // groups of four centroid tiles
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            u32x4 ah[4], al[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const int b = 4 * g + c < nb ? 4 * g + c : nb - 1;  // past the last block: read it, not multiplied
-                av[c] = lds_a[cur][sub * chunk16 + b * 64 + lane];
+                ah[c] = lds_a[cur][b * 128 + lane];
+                al[c] = lds_a[cur][b * 128 + 64 + lane];
             }
-        };
+            // the three dependent instructions of a tile are three others apart
 #pragma unroll
-        for (int sub = 0; sub < SC; ++sub) {
-            const int kc = SC * st + sub;
-            const bool live = kc < nkc;  // uniform
-            const int kcc = live ? kc : nkc - 1;
-            // operands of this chunk from the row piece fetched one chunk ago.  With the centroid
-            // operand A = {ah, al} (as it lies in LDS, no register shuffling):
-            //   A . {xh, xh} = ah.xh + al.xh      A . {xl, 0} = ah.xl
-            float xv[4] = {xn.x, xn.y, xn.z, xn.w};
-            if (shifted) {
-                const float4 mn = *reinterpret_cast<const float4 *>(lds_mu + kcc * 8 + 4 * h);
-                xv[0] -= mn.x;
-                xv[1] -= mn.y;
-                xv[2] -= mn.z;
-                xv[3] -= mn.w;
-            }
-            if (!live) xv[0] = xv[1] = xv[2] = xv[3] = 0.0f;
+            for (int c = 0; c < 4; ++c)
+                if (4 * g + c < nb)
+                    acc[4 * g + c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8, ah[c]), __builtin_bit_cast(bf16x8, bh), acc[4 * g + c], 0, 0, 0);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) x2 = __builtin_fmaf(xv[u], xv[u], x2);
-            const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
-            const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
-            const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
-            const u32x4 b1 = u32x4{h01, h23, h01, h23}, b2 = u32x4{l01, l23, 0u, 0u};
-            // fetch the next chunk of the row
-            const int nx = kc + 1 < nkc ? kc + 1 : nkc - 1;
-            xn = *reinterpret_cast<const float4 *>(xr + nx * 8);
+            for (int c = 0; c < 4; ++c)
+                if (4 * g + c < nb)
+                    acc[4 * g + c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8, al[c]), __builtin_bit_cast(bf16x8, bh), acc[4 * g + c], 0, 0, 0);
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                u32x4 av[4];
-                read_group(sub, g, av);
-                {
-                    // the first instruction of every tile, then the second: the two dependent
-                    // instructions of a tile are three others apart
-#pragma unroll
-                    for (int c = 0; c < 4; ++c)
-                        if (4 * g + c < nb)
-                            acc[4 * g + c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                                __builtin_bit_cast(bf16x8, av[c]), __builtin_bit_cast(bf16x8, b1), acc[4 * g + c], 0, 0, 0);
-#pragma unroll
-                    for (int c = 0; c < 4; ++c)
-                        if (4 * g + c < nb)
-                            acc[4 * g + c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                                __builtin_bit_cast(bf16x8, av[c]), __builtin_bit_cast(bf16x8, b2), acc[4 * g + c], 0, 0, 0);
-                }
-            }
+            for (int c = 0; c < 4; ++c)
+                if (4 * g + c < nb)
+                    acc[4 * g + c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8, ah[c]), __builtin_bit_cast(bf16x8, bl), acc[4 * g + c], 0, 0, 0);
         }
         if (more) {
 #pragma unroll
-            for (int q = 0; q < 2 * SC; ++q) {
+            for (int q = 0; q < 4; ++q) {
                 const int i = threadIdx.x + 256 * q;
-                if (i < SC * chunk16) lds_a[cur ^ 1][i] = pre[q];
+                if (i < pair16) lds_a[cur ^ 1][i] = pre[q];
             }
         }
         lds_barrier();
     }
     x2 += __shfl_xor(x2, 32);  // both halves' shares of ||x - mu||^2
-    // the three smallest scores of the row (index in the low 8 bits, one v_and_or per score)
-    auto push = [](int &m1, int &m2, int &m3, int key) {
-        m3 = imed3(m2, m3, key);
-        m2 = imed3(m1, m2, key);
-        m1 = imin(m1, key);
-    };
+    // the three smallest scores of the row, the index in the low 8 bits (one v_and_or per score; the
+    // tag leaves out the lane half, bit 2, so it is the same in every lane: a scalar operand)
     int m1 = 0x7f800000, m2 = 0x7f800000, m3 = 0x7f800000;
     const uint32_t keep = opaque_vgpr(0xFFFFFF00u);
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-            push(m1, m2, m3, pack_tag(acc[b][v] + x2, keep, (uint32_t)(32 * b + 8 * (v / 4) + v % 4) | (uint32_t)(4 * h)));
+        for (int v = 0; v < 16; v += 4) {
+            int key[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                key[u] = pack_tag(acc[b][v + u] + x2, keep, (uint32_t)(32 * b + 8 * (v / 4) + u));
+            top3_push4(m1, m2, m3, key[0], key[1], key[2], key[3]);
+        }
     }
     {
+        m1 |= 4 * h;
+        m2 |= 4 * h;
         const int o1 = __shfl_xor(m1, 32), o2 = __shfl_xor(m2, 32), o3 = __shfl_xor(m3, 32);
-        push(m1, m2, m3, o1);
-        push(m1, m2, m3, o2);
-        push(m1, m2, m3, o3);
+        top3_push4(m1, m2, m3, o1, o2, o3, 0x7f800000);
     }
     const uint32_t i1 = (uint32_t)m1 & 0xFFu, i2 = (uint32_t)m2 & 0xFFu;
     if (h == 0) {

@@ -232,7 +232,8 @@ int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const ui
 template <int METRIC, bool LBG>
 int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     const int nb = (a.k + 31) / 32, nkc = sd / 8, nsl = (sd + 31) / 32;
-    const size_t n_atab = (size_t)a.m * nkc * nb * 128 * 4, n_c2 = (size_t)a.m * nb * 32;  // floats
+    // A operands: 2 x 64 lanes x 16 bytes per (s, 16 dimensions, block of 32 centroids)
+    const size_t n_atab = (size_t)a.m * ((sd + 15) / 16) * nb * 128 * 4, n_c2 = (size_t)a.m * nb * 32;  // floats
     VQ_TRY(ensure(ctx, ctx->mfma_tab, sizeof(float) * (n_atab + n_c2 + (size_t)a.m * nb + (size_t)a.m * sd + a.m + 2 * (size_t)a.m * nsl + 8) + 64));
     // header (two counts), the list for the all-centroid check, the list for the two-candidate check
     const size_t n_pairs = (size_t)a.n * a.m;
@@ -250,8 +251,8 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     hipLaunchKernelGGL(vq::k_mfma_wide_bf_prep, dim3(a.m, nb), dim3(256), 0, ctx->stream, a.cb, mu, norms, shifted,
                        a.m, a.k, nb, sd,
                        (vq::u32x4 *)atab, c2perm, maxc2, count);
-    // two candidates, each: operand split 3 * 2^-16, fp32 accumulation (34 per chunk + 16) * 2^-24,
-    // rounding of the differences from the centre 2^-22
+    // two candidates, each: operand split 3 * 2^-16, fp32 accumulation (34 per 8 dimensions + 16)
+    // * 2^-24 (an upper bound), rounding of the differences from the centre 2^-22
     const float kappa = 2.0f * (3.0f * 1.52587890625e-05f + (34.0f * nkc + 16.0f + 4.0f) * 5.9604644775390625e-08f);
     vq::MfmaWideBfTables tb{(const vq::u32x4 *)atab, c2perm, maxc2, mu, shifted, list, count, pairs, nb, sd, kappa};
     {
