@@ -579,8 +579,8 @@ namespace vq {
 // 16 dimensions for 3 NB matrix instructions, so no operand is assembled in registers (vector
 // and matrix instructions take turns on a SIMD).  ||x - mu||^2 is summed on the vector ALU and
 // added to the scores before the selection.  The A operands of 16 dimensions (16 KB for 256
-// centroids) are staged in LDS once per workgroup, double-buffered; the row and the next A
-// operands are fetched one stage ahead.
+// centroids) are staged in LDS once per workgroup, double-buffered; the next A operands are
+// fetched one stage ahead, the row two.
 // Error of a score: 3 * 2^-16 (split, as above) + (34 * sd/8 + 16) * 2^-24 (fp32 accumulation, an
 // upper bound: at most 17 additions per instruction, 1.5 instructions per 8 dimensions, and the
 // final sum) + 2^-22 (rounding of x - mu and c - mu), per unit of ||x - mu||^2 + ||c - mu||^2;
@@ -794,6 +794,9 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     auto piece = [&](int pr) { return 16 * pr + 8 * h < sd ? 16 * pr + 8 * h : 0; };
     float4 xn0 = *reinterpret_cast<const float4 *>(xr + piece(0));  // the next piece of the row
     float4 xn1 = *reinterpret_cast<const float4 *>(xr + piece(0) + 4);
+    const int second = npair > 1 ? 1 : 0;
+    float4 xf0 = *reinterpret_cast<const float4 *>(xr + piece(second));  // and the one after it
+    float4 xf1 = *reinterpret_cast<const float4 *>(xr + piece(second) + 4);
     float x2 = 0.0f;
     // A stage is 16 dimensions: with the high and low parts of the centroid operand (ah, al) and of
     // the row operand (xh, xl), three matrix instructions per tile of 32 centroids,
@@ -838,10 +841,12 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
             lp[u] = bf16_pack2(xv[2 * u] - __uint_as_float(hp[u] << 16), xv[2 * u + 1] - __uint_as_float(hp[u] & 0xffff0000u));
         }
         const u32x4 bh = u32x4{hp[0], hp[1], hp[2], hp[3]}, bl = u32x4{lp[0], lp[1], lp[2], lp[3]};
-        // fetch the next piece of the row
-        const int nx = st + 1 < npair ? st + 1 : npair - 1;
-        xn0 = *reinterpret_cast<const float4 *>(xr + piece(nx));
-        xn1 = *reinterpret_cast<const float4 *>(xr + piece(nx) + 4);
+        // fetch the row two stages ahead
+        const int nx = st + 2 < npair ? st + 2 : npair - 1;
+        xn0 = xf0;
+        xn1 = xf1;
+        xf0 = *reinterpret_cast<const float4 *>(xr + piece(nx));
+        xf1 = *reinterpret_cast<const float4 *>(xr + piece(nx) + 4);
         // The stage's centroid operands are read from LDS four tiles (one group) at a time.
         constexpr int NG = (NB + 3) / 4;  // groups of four centroid tiles
 #pragma unroll

@@ -206,10 +206,12 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready, hip
 template <int METRIC, bool LBG>
 int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const uint32_t *list,
                           const uint32_t *count) {
-    const size_t lds = sizeof(float) * 4 * vq::kWideRows * (size_t)sd;
-    if (lds > 160 * 1024) return fail(ctx, VQ_ERR_UNSUPPORTED, "sub_dim %d too large", sd);
     const bool vec = sd % 4 == 0 && (reinterpret_cast<uintptr_t>(a.cb) & 15) == 0;
     const bool listed = list != nullptr;
+    size_t lds = sizeof(float) * 4 * vq::kWideRows * (size_t)sd;
+    // a handful of listed pairs: one per workgroup, the row and slices of every centroid in LDS
+    if (listed) lds = std::max(lds, sizeof(float) * ((size_t)sd + vq::kPairWgLdsFloats));
+    if (lds > 160 * 1024) return fail(ctx, VQ_ERR_UNSUPPORTED, "sub_dim %d too large", sd);
     auto pick = [&](auto L, auto V) {
         constexpr bool LISTED = decltype(L)::value, VEC = decltype(V)::value;
         return reinterpret_cast<const void *>(vq::k_assign_wide_exact<METRIC, LBG, LISTED, VEC>);
