@@ -27,6 +27,7 @@ struct AssignArgs {
     uint8_t *codes;       // LBG mode: [m][n] in place (old -> new); encode mode: [n][m]
     int *changed;         // LBG mode: changed[s] set to 1 when any code of block s differs
     const int *done;      // LBG mode: blocks with done[s] != 0 are skipped
+    float *dist = nullptr;  // encode mode, k_assign_mfma_bf only: [n][m] distance of the chosen centroid, or null
 };
 
 // Called by the lanes of a wave that changed a code.  Every store to one address is serialised

@@ -269,10 +269,11 @@ __device__ __forceinline__ void lexmin(uint32_t &d, uint32_t &i, uint32_t od, ui
 
 // cl: the column block's centroids in LDS (k x 8 floats, this wave's copy).
 // todo: ballot of the lanes (below 32) whose row is undecided; xblk = first row of the tile.
-// Returns the codes of those rows in their lanes (other lanes keep `code`).
+// Returns the codes of those rows in their lanes, and their distances in dist (other lanes keep
+// `code` and `dist`).
 template <int METRIC>
-__device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, const float *cl,
-                                               const float *__restrict__ xblk, int64_t ld, int k, int lane) {
+__device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, float &dist, const float *cl,
+                                           const float *__restrict__ xblk, int64_t ld, int k, int lane) {
     const float inf = __builtin_inff();
     while (todo) {
         int src[8];
@@ -323,7 +324,10 @@ __device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, co
             int who = src[0];
 #pragma unroll
             for (int u = 1; u < 8; ++u) who = (i == u) ? src[u] : who;
-            if (lane == who) code = best;
+            if (lane == who) {
+                code = best;
+                dist = (d0 == d0) ? __uint_as_float(rd) : d0;  // the chosen centroid's distance as computed
+            }
         }
     }
     return code;
@@ -503,6 +507,7 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
         const int first = (int)(__float_as_uint(s1) & 0xFFu);  // first centroid of the best run
         const unsigned long long todo = __ballot(mine && !sure);
         int code;
+        float dist;  // of the chosen centroid, as the reference computes it
         {
             // the best run's four centroids, two per lane half, in the reference's order
             const int j0 = first + 2 * h;
@@ -533,10 +538,11 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
             swap_halves((int)kd, dlo, dhi);
             swap_halves((int)ki, ilo, ihi);
             code = (uint32_t)dhi < (uint32_t)dlo ? ihi : ilo;  // the lower half holds the lower indices
+            dist = __uint_as_float((uint32_t)dhi < (uint32_t)dlo ? (uint32_t)dhi : (uint32_t)dlo);
         }
         if (todo) {  // the same in every lane: the reference-order argmin of the undecided rows
             n_exact += (uint32_t)__popcll(todo);
-            code = exact_rows8<METRIC>(todo, code, cl, a.x + (row0 + 32 * (int64_t)t) * a.ld + (int64_t)s * SD, a.ld,
+            code = exact_rows8<METRIC>(todo, code, dist, cl, a.x + (row0 + 32 * (int64_t)t) * a.ld + (int64_t)s * SD, a.ld,
                                            k, lane);
         }
         if (mine) {
@@ -547,6 +553,7 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
                 }
             } else {
                 a.codes[row * m + s] = (uint8_t)code;
+                if (a.dist) a.dist[row * m + s] = dist;  // for the caller that merges chunks of a larger codebook
             }
         }
     }

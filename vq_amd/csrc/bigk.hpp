@@ -80,10 +80,13 @@ __device__ __forceinline__ float pair_distance(const float *__restrict__ x, cons
 // A chunk whose own first distance is NaN reports local index 0 whatever follows (nothing is
 // below NaN), while the loop over all k centroids would carry the earlier chunks' minimum into
 // it: such a pair walks the chunk again with the running minimum, one centroid at a time.
+// win_d: the winners' distances where the assignment kernel has written them (the same arithmetic),
+// else null and the distance is computed here.
 template <int METRIC>
 __global__ void __launch_bounds__(256) k_chunk_merge(const float *__restrict__ x, int64_t n, int64_t ld, int m,
                                                      int sd, int kc, const float *__restrict__ chunk,
-                                                     const uint8_t *__restrict__ win8, int base,
+                                                     const uint8_t *__restrict__ win8,
+                                                     const float *__restrict__ win_d, int base,
                                                      float *__restrict__ best_d, uint16_t *__restrict__ out) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n * m) return;
@@ -92,7 +95,7 @@ __global__ void __launch_bounds__(256) k_chunk_merge(const float *__restrict__ x
     const float *xr = x + row * ld + (int64_t)s * sd;
     const float *cs = chunk + (size_t)s * kc * sd;
     const int w = win8[i];
-    const float d = pair_distance<METRIC>(xr, cs + (size_t)w * sd, sd);
+    const float d = win_d ? win_d[i] : pair_distance<METRIC>(xr, cs + (size_t)w * sd, sd);
     if (base == 0) {
         best_d[i] = d;
         out[i] = (uint16_t)w;

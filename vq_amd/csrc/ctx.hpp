@@ -50,7 +50,7 @@ struct vq_ctx {
     DevBuf tmp_a, tmp_b, tmp_c, tmp_d, tmp_e, tmp_f;  // scratch of the RVQ / OPQ / TSVQ entry points
     // codebooks above 256 centroids: chunk tables, chunk winners, running minimum, merged codes,
     // the LBG's assignment, sort keys in and out, the sort's workspace, per-cluster tables, flags
-    DevBuf big_chunk, big_win, big_best, big_fresh, big_codes, big_keys, big_sorted, big_sort_tmp, big_tables,
+    DevBuf big_chunk, big_win, big_wind, big_best, big_fresh, big_codes, big_keys, big_sorted, big_sort_tmp, big_tables,
         big_flags;
     // optional per-kernel-class timing (HIP events on the stream)
     bool prof_on = false;
@@ -169,8 +169,11 @@ int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t 
                      int32_t k_max = 256);
 
 // Launchers defined in vq_api.hip, used by the RVQ / OPQ entry points.
+// d_dist (optional, n x m floats): receives the chosen centroids' distances where the kernel that runs
+// computes them anyway; *dist_written says whether it did.
 int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
-                     int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes);
+                     int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes, float *d_dist = nullptr,
+                     bool *dist_written = nullptr);
 
 // Defined in vq_api_bigk.hip: the same for any k up to 65536 with 16-bit codes, and the LBG above
 // 256 centroids (arguments as vq_lbg_fit, already validated).

@@ -506,7 +506,9 @@ int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t 
 
 
 int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
-                  int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes) {
+                  int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes, float *d_dist,
+                  bool *dist_written) {
+    if (dist_written) *dist_written = false;
     VQ_TRY(check_common(ctx, d_x, n, ld, m, sd, k));
     if (!d_codebooks || !d_codes) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: null pointer");
     if (reinterpret_cast<uintptr_t>(d_codes) & 3)
@@ -533,6 +535,13 @@ int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, i
         hipLaunchKernelGGL(vq::k_centroid_norms, dim3(cdiv((int64_t)m * k, 256)), dim3(256), 0,
                            ctx->stream, d_codebooks, (int64_t)m * k, sd, cnorm);
         a.cnorm = cnorm;
+    }
+    // the 8-float matrix-core kernel has the chosen centroid's exact distance at hand
+    if (d_dist && dist_written &&
+        ((metric == VQ_SQEUCLIDEAN && mfma_applicable<vq::M_SQ, false>(ctx, a, sd)) ||
+         (metric == VQ_EUCLIDEAN && mfma_applicable<vq::M_EUCLID, false>(ctx, a, sd)))) {
+        a.dist = d_dist;
+        *dist_written = true;
     }
     ProfSpan sp(ctx, VQ_PROF_ENCODE);
     return launch_assign<false>(ctx, metric, a, sd);
@@ -586,7 +595,7 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
                       &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tsvq_split, &ctx->tsvq_level, &ctx->tsvq_means, &ctx->tsvq_scan, &ctx->tsvq_bsum, &ctx->tsvq_segmaps, &ctx->tsvq_gsum, &ctx->tsvq_guess, &ctx->tsvq_maps, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f,
-                      &ctx->big_chunk, &ctx->big_win, &ctx->big_best, &ctx->big_fresh, &ctx->big_codes, &ctx->big_keys,
+                      &ctx->big_chunk, &ctx->big_win, &ctx->big_wind, &ctx->big_best, &ctx->big_fresh, &ctx->big_codes, &ctx->big_keys,
                       &ctx->big_sorted, &ctx->big_sort_tmp, &ctx->big_tables, &ctx->big_flags};
     for (DevBuf *b : bufs)
         if (b->p) (void)hipFree(b->p);

@@ -17,9 +17,9 @@ namespace {
 
 template <int METRIC>
 void launch_merge(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int m, int sd, int kc, const float *chunk,
-                  const uint8_t *win, int base, float *best, uint16_t *out) {
+                  const uint8_t *win, const float *win_d, int base, float *best, uint16_t *out) {
     hipLaunchKernelGGL(vq::k_chunk_merge<METRIC>, dim3(cdiv(n * m, 256)), dim3(256), 0, ctx->stream, d_x, n, ld, m, sd,
-                       kc, chunk, win, base, best, out);
+                       kc, chunk, win, win_d, base, best, out);
 }
 
 }  // namespace
@@ -48,19 +48,24 @@ int32_t assign_codes_u16(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t 
     }
     VQ_TRY(ensure(ctx, ctx->big_chunk, sizeof(float) * (size_t)m * vq::kChunk * sd));
     VQ_TRY(ensure(ctx, ctx->big_best, sizeof(float) * pairs));
+    VQ_TRY(ensure(ctx, ctx->big_wind, sizeof(float) * pairs));
     float *chunk = (float *)ctx->big_chunk.p;
     float *best = (float *)ctx->big_best.p;
+    float *wind = (float *)ctx->big_wind.p;
     for (int base = 0; base < k; base += vq::kChunk) {
         const int kc = std::min(vq::kChunk, k - base);
         hipLaunchKernelGGL(vq::k_chunk_tables, dim3(cdiv((int64_t)m * kc * sd, 256)), dim3(256), 0, ctx->stream,
                            d_codebooks, m, k, sd, base, kc, chunk);
         VQ_HIP(ctx, hipGetLastError());
-        VQ_TRY(assign_codes(ctx, metric, d_x, n, ld, m, sd, kc, chunk, win));
+        // the winners' distances come with the codes where the assignment kernel computes them anyway
+        bool have_d = false;
+        VQ_TRY(assign_codes(ctx, metric, d_x, n, ld, m, sd, kc, chunk, win, wind, &have_d));
+        const float *wd = have_d ? wind : nullptr;
         switch (metric) {
-        case VQ_SQEUCLIDEAN: launch_merge<vq::M_SQ>(ctx, d_x, n, ld, m, sd, kc, chunk, win, base, best, d_codes); break;
-        case VQ_EUCLIDEAN: launch_merge<vq::M_EUCLID>(ctx, d_x, n, ld, m, sd, kc, chunk, win, base, best, d_codes); break;
-        case VQ_COSINE: launch_merge<vq::M_COS>(ctx, d_x, n, ld, m, sd, kc, chunk, win, base, best, d_codes); break;
-        default: launch_merge<vq::M_L1>(ctx, d_x, n, ld, m, sd, kc, chunk, win, base, best, d_codes); break;
+        case VQ_SQEUCLIDEAN: launch_merge<vq::M_SQ>(ctx, d_x, n, ld, m, sd, kc, chunk, win, wd, base, best, d_codes); break;
+        case VQ_EUCLIDEAN: launch_merge<vq::M_EUCLID>(ctx, d_x, n, ld, m, sd, kc, chunk, win, wd, base, best, d_codes); break;
+        case VQ_COSINE: launch_merge<vq::M_COS>(ctx, d_x, n, ld, m, sd, kc, chunk, win, wd, base, best, d_codes); break;
+        default: launch_merge<vq::M_L1>(ctx, d_x, n, ld, m, sd, kc, chunk, win, wd, base, best, d_codes); break;
         }
         VQ_HIP(ctx, hipGetLastError());
     }
