@@ -415,7 +415,12 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
     const int lane_tiles = (int)(lane_left < run_tiles ? lane_left : run_tiles);
     const int64_t xstep = 32 * a.ld;
     int64_t xoff = (row0 + r) * a.ld, coff = row0 + r;                // of the lane's row in tile 0
-    auto fetch_x = [&](int t) { return *reinterpret_cast<const float4 *>(xcol + (t < lane_tiles ? xoff : 0)); };
+    // rows may start at any float (any leading dimension): a 16-byte load that only claims 4-byte alignment
+    typedef float rowpiece __attribute__((ext_vector_type(4), aligned(4)));
+    auto fetch_x = [&](int t) {
+        const rowpiece v = *reinterpret_cast<const rowpiece *>(xcol + (t < lane_tiles ? xoff : 0));
+        return make_float4(v[0], v[1], v[2], v[3]);
+    };
     auto fetch_c = [&](int t) { return ccol[t < lane_tiles ? coff : 0]; };
     float4 xa = fetch_x(0);
     uint8_t oa = 0, ob = 0;
