@@ -110,9 +110,14 @@ def main():
 
         x = data.gaussian_mixture(n, dim, 1024, 0.05, seed=1)
         streams = data.index_streams(n, m, k, iters, seed=1)
-        t0 = time.perf_counter()
-        q = api.OptimizedProductQuantizer.fit(x, m, k, iters, outer, api.Distance.Euclidean, 0, streams=streams)
-        out["c3_opq_fit_host_classes_ms_incl_pack_and_upload"] = (time.perf_counter() - t0) * 1e3
+        # the first call of a process also pays for the library's first allocations and the clock's ramp
+        each = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            q = api.OptimizedProductQuantizer.fit(x, m, k, iters, outer, api.Distance.Euclidean, 0, streams=streams)
+            each.append(round((time.perf_counter() - t0) * 1e3, 3))
+        out["c3_opq_fit_host_classes_ms_incl_pack_and_upload"] = min(each[1:])
+        out["c3_opq_fit_ms_each"] = each
         R = q.rotation().astype(np.float64)
         out["c3_rotation_orthogonality_err"] = float(np.abs(R.T @ R - np.eye(dim)).max())
         dx = ctx.to_device(x)
