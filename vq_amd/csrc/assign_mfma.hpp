@@ -351,7 +351,9 @@ template <int METRIC, bool LBG, int SG, bool FULL>
 __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb, int run_tiles) {
     constexpr int SD = 8;
     __shared__ __attribute__((aligned(16))) float lds_cb[4][256 * SD];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wave's number through readfirstlane: what follows from it (column block, first row, base
+    // addresses) is then uniform for the compiler and lives in scalar registers
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int r = lane & 31, h = lane >> 5;
     const int nb = FULL ? 8 : tb.nb, m = a.m, k = a.k;
     // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: workgroups id, id + 8,
@@ -404,24 +406,25 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
-    // rows two tiles ahead; the lane's row moves on by 32 per tile, so its offset is added up
-    // rather than multiplied out
-    const float *xcol = a.x + (int64_t)s * SD + 4 * h;
-    const uint8_t *ccol = a.codes + (size_t)s * a.n;
+    // rows two tiles ahead.  Addresses are a scalar base (the run's first row) plus a 32-bit lane
+    // offset that moves on by 32 rows per tile (the host keeps the run's extent below 2^31 bytes).
+    const float *xrun = a.x + row0 * a.ld + (int64_t)s * SD;          // uniform
+    const uint8_t *crun = a.codes + (size_t)s * a.n + row0;           // uniform (LBG: [m][n] codes)
     const int64_t lane_rows = a.n - (row0 + r);                       // rows from this lane's first to the end
     const int64_t lane_left = lane_rows > 0 ? (lane_rows + 31) / 32 : 0;
-    // tiles of this run in which the lane has a row; the fetches past the run's end read row 0
-    // (the next run belongs to a workgroup on another XCD: its rows would be fetched into two L2s)
+    // tiles of this run in which the lane has a row; the fetches past the run's end read the run's
+    // first row (the next run belongs to a workgroup on another XCD: its rows would be fetched into two L2s)
     const int lane_tiles = (int)(lane_left < run_tiles ? lane_left : run_tiles);
-    const int64_t xstep = 32 * a.ld;
-    int64_t xoff = (row0 + r) * a.ld, coff = row0 + r;                // of the lane's row in tile 0
+    const uint32_t xstep = 128u * (uint32_t)a.ld;                                          // bytes per tile
+    uint32_t xoff = 4u * ((uint32_t)r * (uint32_t)a.ld + 4u * (uint32_t)h), coff = (uint32_t)r;  // of the lane's row in tile 0
     // rows may start at any float (any leading dimension): a 16-byte load that only claims 4-byte alignment
     typedef float rowpiece __attribute__((ext_vector_type(4), aligned(4)));
     auto fetch_x = [&](int t) {
-        const rowpiece v = *reinterpret_cast<const rowpiece *>(xcol + (t < lane_tiles ? xoff : 0));
+        const char *p = reinterpret_cast<const char *>(xrun) + (t < lane_tiles ? xoff : 16u * (uint32_t)h);
+        const rowpiece v = *reinterpret_cast<const rowpiece *>(p);
         return make_float4(v[0], v[1], v[2], v[3]);
     };
-    auto fetch_c = [&](int t) { return ccol[t < lane_tiles ? coff : 0]; };
+    auto fetch_c = [&](int t) { return crun[t < lane_tiles ? coff : 0u]; };
     float4 xa = fetch_x(0);
     uint8_t oa = 0, ob = 0;
     if constexpr (LBG) oa = fetch_c(0);
@@ -501,8 +504,7 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
         swap_halves(m2, f2, g2);
         const float s1 = __int_as_float(imin(f1, g1));
         const float s2 = __int_as_float(imin(imax(f1, g1), imin(f2, g2)));
-        const int64_t row = row0 + 32 * (int64_t)t + r;
-        const bool mine = h == 0 && row < a.n;
+        const bool mine = h == 0 && t < lane_tiles;  // the lane's row of this tile exists
         const float bound = x2 + mc2;
         const float margin = 6.103515625e-05f * fabsf(s2) + 1.220703125e-04f * bound;
         bool sure = (s2 - s1) > margin;  // false for NaN / inf-inf
@@ -551,14 +553,16 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
                                            k, lane);
         }
         if (mine) {
+            const uint32_t rr = 32u * (uint32_t)t + (uint32_t)r;  // row within the run
             if constexpr (LBG) {
                 if (old != (uint8_t)code) {
-                    a.codes[(size_t)s * a.n + row] = (uint8_t)code;
+                    a.codes[(size_t)s * a.n + row0 + rr] = (uint8_t)code;
                     chg = true;
                 }
             } else {
-                a.codes[row * m + s] = (uint8_t)code;
-                if (a.dist) a.dist[row * m + s] = dist;  // for the caller that merges chunks of a larger codebook
+                const size_t out0 = (size_t)row0 * m + s;  // uniform
+                a.codes[out0 + rr * (uint32_t)m] = (uint8_t)code;
+                if (a.dist) a.dist[out0 + rr * (uint32_t)m] = dist;  // for the caller that merges chunks of a larger codebook
             }
         }
     }

@@ -299,6 +299,8 @@ bool mfma_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     if (ctx->assign_path == 1) return false;
     if (METRIC != vq::M_SQ && METRIC != vq::M_EUCLID) return false;
     if (sd != 8 || (reinterpret_cast<uintptr_t>(a.cb) & 15) != 0) return false;  // float4 centroid loads
+    // the kernel addresses the rows of a wave's run (at most 288 of them) with 32-bit offsets
+    if (a.ld > (1 << 20) || a.m > (1 << 16)) return false;
     return a.k <= 256;
 }
 
