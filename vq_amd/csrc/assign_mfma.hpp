@@ -794,7 +794,11 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
 
     const int64_t row = (int64_t)blockIdx.x * 128 + wave * 32 + r;
     const bool valid = row < a.n;
-    const float *xr = a.x + (valid ? row : 0) * a.ld + (int64_t)s * sd;
+    // the workgroup's first row is a scalar base, the lane's row a 32-bit byte offset from it (the
+    // host keeps 128 rows below 2^31 bytes); a row past the end reads the workgroup's first row
+    const char *xwg = reinterpret_cast<const char *>(a.x + (int64_t)blockIdx.x * 128 * a.ld + (int64_t)s * sd);
+    const uint32_t xlane = valid ? 4u * (uint32_t)(wave * 32 + r) * (uint32_t)a.ld : 0u;
+    auto row_piece = [&](int d) { return *reinterpret_cast<const float4 *>(xwg + (xlane + 4u * (uint32_t)d)); };
     const bool shifted = tb.shifted[s] != 0;  // uniform
     // the accumulators start at ||c - mu||^2; ||x - mu||^2, the same in every score of a row, is
     // summed on the side and added before the selection
@@ -808,11 +812,11 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     // every outstanding load at each use instead of counting them.
     // This half's 8 of the 16 dimensions of a stage: 16 pr + 8 h .. + 7.
     auto piece = [&](int pr) { return 16 * pr + 8 * h < sd ? 16 * pr + 8 * h : 0; };
-    float4 xn0 = *reinterpret_cast<const float4 *>(xr + piece(0));  // the next piece of the row
-    float4 xn1 = *reinterpret_cast<const float4 *>(xr + piece(0) + 4);
+    float4 xn0 = row_piece(piece(0));  // the next piece of the row
+    float4 xn1 = row_piece(piece(0) + 4);
     const int second = npair > 1 ? 1 : 0;
-    float4 xf0 = *reinterpret_cast<const float4 *>(xr + piece(second));  // and the one after it
-    float4 xf1 = *reinterpret_cast<const float4 *>(xr + piece(second) + 4);
+    float4 xf0 = row_piece(piece(second));  // and the one after it
+    float4 xf1 = row_piece(piece(second) + 4);
     float x2 = 0.0f;
     // A stage is 16 dimensions: with the high and low parts of the centroid operand (ah, al) and of
     // the row operand (xh, xl), three matrix instructions per tile of 32 centroids,
@@ -826,8 +830,9 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         u32x4 pre[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int i = (st + 1) * pair16 + (int)threadIdx.x + 256 * q;
-            pre[q] = ag[i < total16 ? i : total16 - 1];
+            const uint32_t i = (uint32_t)((st + 1) * pair16) + threadIdx.x + 256u * (uint32_t)q;
+            const uint32_t ic = i < (uint32_t)total16 ? i : (uint32_t)total16 - 1u;
+            pre[q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(ag) + 16u * ic);
         }
         // operands of this stage from the row piece fetched one stage ago
         const bool in = 16 * st + 8 * h < sd;
@@ -861,8 +866,8 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         const int nx = st + 2 < npair ? st + 2 : npair - 1;
         xn0 = xf0;
         xn1 = xf1;
-        xf0 = *reinterpret_cast<const float4 *>(xr + piece(nx));
-        xf1 = *reinterpret_cast<const float4 *>(xr + piece(nx) + 4);
+        xf0 = row_piece(piece(nx));
+        xf1 = row_piece(piece(nx) + 4);
         // The stage's centroid operands are read from LDS four tiles (one group) at a time.
         constexpr int NG = (NB + 3) / 4;  // groups of four centroid tiles
 #pragma unroll

@@ -288,9 +288,10 @@ bool mfma_wide_applicable(const vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     if (ctx->assign_path == 1 || ctx->no_alloc) return false;  // its lists grow with n: not for a fixed scratch
     if (METRIC != vq::M_SQ && METRIC != vq::M_EUCLID) return false;
     if (sd < 16 || sd % 8 != 0 || a.k > 256 || a.m > 65535) return false;
-    // float4 row and centroid loads
+    // float4 row and centroid loads; the rows of a workgroup and the operand table within 32-bit byte offsets
     if (a.ld % 4 != 0 || ((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.cb)) & 15) != 0)
         return false;
+    if (a.ld > (1 << 20) || sd > (1 << 16)) return false;
     return (int64_t)a.n * a.m < (1LL << 32);
 }
 
