@@ -835,7 +835,6 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
             pre[q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(ag) + 16u * ic);
         }
         // operands of this stage from the row piece fetched one stage ago
-        const bool in = 16 * st + 8 * h < sd;
         float xv[8] = {xn0.x, xn0.y, xn0.z, xn0.w, xn1.x, xn1.y, xn1.z, xn1.w};
         if (shifted) {
             const float4 m0 = *reinterpret_cast<const float4 *>(lds_mu + piece(st));
@@ -849,9 +848,11 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
             xv[6] -= m1.z;
             xv[7] -= m1.w;
         }
-        if (!in) {
+        if (st == npair - 1 && (sd & 8) != 0) {  // uniform: a width that is an odd multiple of 8 ends in the lower half
+            if (h != 0) {
 #pragma unroll
-            for (int u = 0; u < 8; ++u) xv[u] = 0.0f;
+                for (int u = 0; u < 8; ++u) xv[u] = 0.0f;
+            }
         }
         uint32_t hp[4], lp[4];
 #pragma unroll
