@@ -148,9 +148,11 @@ static __global__ void k_big_init(BigLbg st, int m) {
 }
 
 // New codes (n x m, from the merge) into the assignment ([m][n]); src/utils.rs:66-72.  Also the
-// sort key of the pair: column block, code, row.
+// sort key of the pair: the row in bits 0-31, the code in the code_bits above them, the column
+// block above that.  The keys are written block by block in row order, so a stable sort on the
+// bits from 32 up lists every cluster's members in row order.
 static __global__ void __launch_bounds__(256) k_big_commit(BigLbg st, const uint16_t *__restrict__ fresh, int64_t n,
-                                                           int m, uint64_t *__restrict__ keys) {
+                                                           int m, int code_bits, uint64_t *__restrict__ keys) {
     const int s = blockIdx.y;
     const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (row >= n) return;
@@ -164,16 +166,16 @@ static __global__ void __launch_bounds__(256) k_big_commit(BigLbg st, const uint
             mark_changed(st.changed + s);
         }
     }
-    keys[(size_t)s * n + row] = ((uint64_t)s << 48) | ((uint64_t)c << 32) | (uint64_t)row;
+    keys[(size_t)s * n + row] = ((uint64_t)s << (32 + code_bits)) | ((uint64_t)c << 32) | (uint64_t)row;
 }
 
 // Sorted keys -> first position and size of every cluster that has members.
 static __global__ void __launch_bounds__(256) k_big_bounds(BigLbg st, const uint64_t *__restrict__ sorted, int64_t n,
-                                                           int m, int k) {
+                                                           int m, int k, int code_bits) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n * m) return;
-    const uint32_t sc = (uint32_t)(sorted[i] >> 32);  // (block << 16) | code
-    const int s = (int)(sc >> 16), j = (int)(sc & 0xffffu);
+    const uint32_t sc = (uint32_t)(sorted[i] >> 32);  // (block << code_bits) | code
+    const int s = (int)(sc >> code_bits), j = (int)(sc & ((1u << code_bits) - 1u));
     const int64_t in_block = i - (int64_t)s * n;
     const bool first = i == 0 || (uint32_t)(sorted[i - 1] >> 32) != sc;
     const bool last = i + 1 == n * m || (uint32_t)(sorted[i + 1] >> 32) != sc;

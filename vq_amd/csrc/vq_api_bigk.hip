@@ -88,12 +88,15 @@ int32_t lbg_fit_big(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_
     VQ_TRY(ensure(ctx, ctx->big_sorted, sizeof(uint64_t) * pairs));
     VQ_TRY(ensure(ctx, ctx->idx, sizeof(uint32_t) * mk));
     VQ_TRY(ensure(ctx, ctx->reseed, sizeof(uint32_t) * ((size_t)m * n_reseed + 1)));
-    // keys: row in bits 0-31, code in 32-47, column block from 48
-    unsigned end_bit = 48;
-    while (end_bit < 64 && ((uint64_t)(m - 1) >> (end_bit - 48)) != 0) ++end_bit;
+    // keys: row in bits 0-31, code in the next code_bits, column block above; they are written block by
+    // block in row order, so the sort covers the bits from 32 up only (a radix sort is stable)
+    int code_bits = 1;
+    while ((1 << code_bits) < k) ++code_bits;
+    unsigned end_bit = 32u + (unsigned)code_bits;
+    while (end_bit < 64 && ((uint64_t)(m - 1) >> (end_bit - 32u - (unsigned)code_bits)) != 0) ++end_bit;
     uint64_t *keys = (uint64_t *)ctx->big_keys.p, *sorted = (uint64_t *)ctx->big_sorted.p;
     size_t sort_bytes = 0;
-    VQ_HIP(ctx, rocprim::radix_sort_keys(nullptr, sort_bytes, keys, sorted, pairs, 0u, end_bit, st));
+    VQ_HIP(ctx, rocprim::radix_sort_keys(nullptr, sort_bytes, keys, sorted, pairs, 32u, end_bit, st));
     VQ_TRY(ensure(ctx, ctx->big_sort_tmp, sort_bytes));
 
     vq::BigLbg S;
@@ -132,12 +135,12 @@ int32_t lbg_fit_big(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_
         }
         ProfSpan sp(ctx, VQ_PROF_LBG_UPDATE);
         hipLaunchKernelGGL(vq::k_big_commit, dim3(cdiv(n, 256), m), dim3(256), 0, st, S, (const uint16_t *)fresh, n, m,
-                           keys);
+                           code_bits, keys);
         VQ_HIP(ctx, hipGetLastError());
-        VQ_HIP(ctx, rocprim::radix_sort_keys(ctx->big_sort_tmp.p, sort_bytes, keys, sorted, pairs, 0u, end_bit, st));
+        VQ_HIP(ctx, rocprim::radix_sort_keys(ctx->big_sort_tmp.p, sort_bytes, keys, sorted, pairs, 32u, end_bit, st));
         VQ_HIP(ctx, hipMemsetAsync(S.count, 0, sizeof(uint32_t) * mk, st));
         hipLaunchKernelGGL(vq::k_big_bounds, dim3(cdiv((int64_t)pairs, 256)), dim3(256), 0, st, S,
-                           (const uint64_t *)sorted, n, m, k);
+                           (const uint64_t *)sorted, n, m, k, code_bits);
         hipLaunchKernelGGL(vq::k_big_plan, dim3(m), dim3(256), 0, st, S, k);
         hipLaunchKernelGGL(vq::k_big_small_means, dim3(cdiv((int64_t)k * sd, 256), m), dim3(256), 0, st, S,
                            (const uint64_t *)sorted, d_x, n, ld, k, sd, (const uint32_t *)ctx->reseed.p, n_reseed,
