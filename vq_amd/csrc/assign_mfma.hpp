@@ -348,7 +348,8 @@ __device__ __forceinline__ int exact_rows8(unsigned long long todo, int code, fl
 // same rows.  SG = 1 (m not a multiple of 4): the four waves take consecutive runs of one block.
 // FULL: 8 blocks of 32 centroids (k above 224), scored without a branch between them.
 template <int METRIC, bool LBG, int SG, bool FULL>
-__global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb, int run_tiles) {
+__global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfTables tb, int run_tiles, int64_t nruns,
+                                                            int64_t run_stride) {
     constexpr int SD = 8;
     __shared__ __attribute__((aligned(16))) float lds_cb[4][256 * SD];
     // the wave's number through readfirstlane: what follows from it (column block, first row, base
@@ -363,16 +364,12 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
     const unsigned per_chunk = 8u * (unsigned)ngroups;
     const unsigned chunk_id = blockIdx.x / per_chunk, rem = blockIdx.x % per_chunk;
     const int g = (int)(rem / 8u);
-    const int64_t run_id = (int64_t)chunk_id * 8 + (rem % 8u);
+    const int64_t run_first = (int64_t)chunk_id * 8 + (rem % 8u);
     const int s = SG == 4 ? g * 4 + wave : g;
-    const int64_t tile0 = SG == 4 ? run_id * run_tiles : (run_id * 4 + wave) * run_tiles;
-    const int64_t row0 = tile0 * 32;
-    if (row0 >= a.n) return;
+    if (run_first >= nruns) return;
     if constexpr (LBG) {
         if (__builtin_amdgcn_readfirstlane(a.done[s]) != 0) return;  // the block has converged
     }
-    int64_t left = (a.n - row0 + 31) / 32;
-    const int ntiles = (int)(left < run_tiles ? left : run_tiles);
 
     // the block's centroids: this wave's copy in LDS (no other wave reads it: no barrier)
     float *cl = lds_cb[wave];
@@ -406,6 +403,16 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
+    uint32_t n_exact = 0;
+    bool chg = false;
+    // The workgroup walks over its runs of rows (run_first, run_first + run_stride, ...) with the
+    // operands it has loaded: the grid is a few workgroups per compute unit, not one per run.
+    for (int64_t run_id = run_first; run_id < nruns; run_id += run_stride) {
+    const int64_t tile0 = SG == 4 ? run_id * run_tiles : (run_id * 4 + wave) * run_tiles;
+    const int64_t row0 = tile0 * 32;
+    if (row0 >= a.n) break;  // SG == 1: the last run may end before this wave's share
+    const int64_t left = (a.n - row0 + 31) / 32;
+    const int ntiles = (int)(left < run_tiles ? left : run_tiles);
     // rows two tiles ahead.  Addresses are a scalar base (the run's first row) plus a 32-bit lane
     // offset that moves on by 32 rows per tile (the host keeps the run's extent below 2^31 bytes).
     const float *xrun = a.x + row0 * a.ld + (int64_t)s * SD;          // uniform
@@ -432,8 +439,6 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
     coff += 32;
     float4 xb = fetch_x(1);
     if constexpr (LBG) ob = fetch_c(1);
-    uint32_t n_exact = 0;
-    bool chg = false;
     for (int t = 0; t < ntiles; ++t) {
         const float4 xc = xa;
         const uint8_t old = oa;
@@ -566,6 +571,7 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
             }
         }
     }
+    }  // runs
     if constexpr (LBG) {
         // changed[s]: one lane per wave, once per wave, and only where the flag still reads 0 (every
         // store to one address is serialised in its L2 channel; a stale 0 from the vector cache
@@ -573,7 +579,7 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
         if (__any(chg) && lane == 0 && a.changed[s] == 0) a.changed[s] = 1;
     }
     if (lane == 0 && n_exact)
-        atomicAdd(tb.stat + ((run_id * 4 + wave) & (kStatSlots - 1)) * kStatStride, n_exact);
+        atomicAdd(tb.stat + ((run_first * 4 + wave) & (kStatSlots - 1)) * kStatStride, n_exact);
 }
 
 }  // namespace vq

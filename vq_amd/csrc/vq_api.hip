@@ -22,6 +22,9 @@
 #ifndef VQ_MFMA_RUN
 #define VQ_MFMA_RUN 8    // tiles of 32 rows per wave in the matrix-core assignment (a power of two)
 #endif
+#ifndef VQ_MFMA_WGS
+#define VQ_MFMA_WGS 3072 // workgroups of the matrix-core assignment: four rounds of three per compute unit
+#endif
 #include "lbg_update.hpp"
 #include "calibrate.hpp"
 
@@ -177,8 +180,13 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready, hip
     const int64_t groups = grouped ? a.m / 4 : a.m;
     int run_tiles = VQ_MFMA_RUN;
     while (run_tiles > 1 && cdiv(tiles, (grouped ? 1 : 4) * run_tiles) * groups < 8192) run_tiles >>= 1;
-    const int64_t runs = cdiv(tiles, (grouped ? 1 : 4) * (int64_t)run_tiles);
-    const int64_t blocks = cdiv(runs, 8) * 8 * groups;  // runs in chunks of 8
+    int64_t runs = cdiv(tiles, (grouped ? 1 : 4) * (int64_t)run_tiles);
+    // a workgroup walks over several runs with the operands it has loaded once; the grid is a few
+    // rounds of the three workgroups a compute unit holds (768: the slowest workgroup sets the
+    // time; one workgroup per run: the operands are loaded 15,000 times), a multiple of 8 per group
+    int64_t run_stride = std::max<int64_t>(8, (VQ_MFMA_WGS / groups) / 8 * 8);
+    run_stride = std::min<int64_t>(run_stride, cdiv(runs, 8) * 8);
+    const int64_t blocks = run_stride * groups;
     if (blocks >= (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * m too large for one launch");
     hipEvent_t ev_a = nullptr, ev_b = nullptr;
     if (ctx->prof_on) {
@@ -189,7 +197,7 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready, hip
         ev_b = ctx->ev_fork;
     }
     vq::AssignArgs aa = a;
-    void *args[] = {&aa, &tb, &run_tiles};
+    void *args[] = {&aa, &tb, &run_tiles, &runs, &run_stride};
     if (ev_a || ev_b)
         VQ_HIP(ctx, hipExtLaunchKernel(kern, dim3((unsigned)blocks), dim3(256), args, 0, ctx->stream, ev_a, ev_b, 0u));
     else
