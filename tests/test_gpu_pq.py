@@ -54,6 +54,7 @@ LBG_CASES = [
     (70000, 16, 2, 3, 3, "same"),      # sub_dim 8: one huge cluster, empties re-seeded
     (13000, 24, 3, 5, 3, "normal"),    # sub_dim 8 but m % 4 != 0 -> per-part leaves, gather path
     (13000, 6, 1, 4, 3, "normal"),     # sub_dim 6, clusters above 1024 -> per-part leaves
+    (300001, 32, 4, 256, 2, "normal"), # sub_dim 8: a workgroup of the assignment walks over several runs of rows
 ]
 
 
@@ -177,6 +178,8 @@ def test_errors_match_reference_panics(ctx):
     (5000, 16, 256, "uniform"), (1000, 16, 256, "mixture"), (700, 4, 100, "normal"),
     (513, 1, 1, "normal"), (64, 2, 33, "grid"), (2000, 16, 256, "offset"), (300, 3, 7, "same"),
     (900, 16, 256, "nonfinite"),
+    # enough rows for a workgroup to walk over several runs of rows, the last one partial
+    (200001, 4, 256, "uniform"), (150001, 3, 200, "normal"),
 ])
 def test_mfma_path_equals_oracle_and_valu_path(ctx, metric, n, m, k, kind):
     """sub_dim 8: the default path is the matrix-core pass + exact re-check.  It must give the
