@@ -111,12 +111,17 @@ __device__ __forceinline__ void top2_push4(int &m1, int &m2, int k0, int k1, int
 // (round-to-nearest-even twice).  With a = -2c, the lanes of half h = lane / 32 own dimensions
 // [4h, 4h + 4) of the block and the 8 contraction slots of that half hold
 //     instruction 1:  ah . xh  (4 slots)   ah . xl  (4 slots)
-//     instruction 2:  al . xh  (4 slots)   1 . (three bf16 parts of the half's share of ||x||^2)
-// so a lane loads and splits only its own 16 bytes of the row, both halves do the same work, and
-// the accumulator starts at ||c||^2: the result is the score ||c||^2 + ||x||^2 - 2 x.c with an
-// error of at most 3 * 2^-16 * sum|a_t||x_t| <= 3 * 2^-16 (||x||^2 + ||c||^2) from the dropped
-// terms (a ex, x ea, al xl) plus at most 2^-17.9 (||x||^2 + ||c||^2) from the fp32 accumulation of
-// the 2 x 17 addends.  Two candidates compared: below 2^-13.2 (||x||^2 + max ||c||^2); the test
+//     instruction 2:  al . xh  (4 slots)   1 . (the half's share of ||x||^2, one slot; an empty
+//                                               slot; ||c||^2 in three bf16 parts over the two halves)
+// so a lane loads and splits only its own 16 bytes of the row and both halves do the same work:
+// the result is the score ||c||^2 + ||x||^2 - 2 x.c + delta with an error of at most
+// 3 * 2^-16 * sum|a_t||x_t| <= 3 * 2^-16 (||x||^2 + ||c||^2) from the dropped terms (a ex, x ea,
+// al xl) plus at most 2^-17.9 (||x||^2 + ||c||^2) from the fp32 accumulation of the 2 x 15
+// addends.  delta: the share of ||x||^2 rides as ONE bf16 number rounded up, 0 <= delta <
+// 2^-7 ||x||^2; the product 1 . share is exact and the same addend in every score of the row, so
+// delta cancels in the difference of two scores (it lengthens the partial sums, and with them the
+// accumulation bound, by under 1 %), and rounding up keeps scores of near-zero distances from
+// turning negative.  Two candidates compared: below 2^-13.2 (||x||^2 + max ||c||^2); the test
 // uses 2^-13, plus 2^-14 |second| for the packed bits and the reference's own rounding.  bf16
 // keeps the fp32 exponent range, so no scaling is needed; non-finite values fail the test.
 // x and c here are the row and the centroid minus the block's centre mu (rounded to fp32): the
@@ -461,13 +466,12 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
             const uint32_t h01 = bf16_pack2(xv[0], xv[1]), h23 = bf16_pack2(xv[2], xv[3]);
             const uint32_t l01 = bf16_pack2(xv[0] - __uint_as_float(h01 << 16), xv[1] - __uint_as_float(h01 & 0xffff0000u));
             const uint32_t l23 = bf16_pack2(xv[2] - __uint_as_float(h23 << 16), xv[3] - __uint_as_float(h23 & 0xffff0000u));
-            // this half's share of ||x||^2 in two bf16 parts (it is the same in every score of the
-            // row, so its rounding cancels in their differences), then ones for the parts of ||c||^2
-            const uint32_t p0 = bf16_pack2(p, 0.0f);
-            const float r1 = p - __uint_as_float(p0 << 16);
-            const uint32_t p1 = bf16_pack2(r1, 0.0f);
+            // this half's share of ||x||^2 as one bf16 number rounded up (p >= 0; the same in every score
+            // of the row, so its rounding cancels in their differences, and rounding up keeps the
+            // scores from turning negative), then ones for the parts of ||c||^2
+            const uint32_t p0 = (__float_as_uint(p) + 0xFFFFu) >> 16;
             b1 = u32x4{h01, h23, l01, l23};
-            b2 = u32x4{h01, h23, (p0 & 0xffffu) | (p1 << 16), 0x3f803f80u};
+            b2 = u32x4{h01, h23, p0, 0x3f803f80u};
             int pa, pb;
             swap_halves(__float_as_int(p), pa, pb);
             x2 = __int_as_float(pa) + __int_as_float(pb);  // lower half's share + upper half's, in both
