@@ -291,10 +291,10 @@ __global__ void __launch_bounds__(256) k_crosscov_mfma(const float *__restrict__
                                                        double *__restrict__ part) {
     // a wave owns TWO tiles of 16 output rows (32 dimensions of y), so every operand of x it
     // fetches feeds two matrix instructions
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ti = 2 * (blockIdx.y * 4 + w), nti = DIM / 16;
     if (ti >= nti) return;
-    const bool two = ti + 1 < nti;
+    const bool two = ti + 1 < nti;  // without a second tile acc1 repeats acc0 and is not stored
     b0 += 128 * blockIdx.z;
     const int kk = lane >> 4, jj = lane & 15;
     const int64_t lo = (int64_t)blockIdx.x * rows_per_chunk;
@@ -305,46 +305,80 @@ __global__ void __launch_bounds__(256) k_crosscov_mfma(const float *__restrict__
         acc0[tj] = doublex4{0.0, 0.0, 0.0, 0.0};
         acc1[tj] = doublex4{0.0, 0.0, 0.0, 0.0};
     }
-    // Operands are fetched kAhead steps (of 4 rows) ahead.  The loads are unconditional — an
-    // address past the chunk is clamped to the lane's first row and the value zeroed afterwards —
-    // because a load under a branch makes the compiler wait for every load in flight at its use.
-    constexpr int kAhead = 4;
-    const int64_t base_row = lo + (lo + kk < hi ? kk : 0);  // the chunk is not empty: lo < hi
-    const float *yp = yr + base_row * (int64_t)DIM + 16 * ti + jj;
-    const float *yp1 = two ? yp + 16 : yp;
-    const float *xp = x + base_row * (int64_t)DIM + b0 + jj;
-    float a0[kAhead], a1[kAhead], b[kAhead][NT];
-    bool ok[kAhead];
-#pragma unroll
-    for (int u = 0; u < kAhead; ++u) {
-        ok[u] = lo + 4 * u + kk < hi;
-        const int64_t off = ok[u] ? (int64_t)(4 * u) * DIM : 0;
-        a0[u] = yp[off];
-        a1[u] = yp1[off];
-#pragma unroll
-        for (int tj = 0; tj < NT; ++tj) b[u][tj] = xp[off + 16 * tj];
-    }
-    for (int64_t r = lo; r < hi; r += 4 * kAhead) {
+    // Addresses: a scalar base that moves on by four rows per step plus one fixed 32-bit lane
+    // offset (and the column tile as the instruction's immediate), so the loop spends no vector
+    // instruction on them; the vector ALU and the matrix cores take turns on a SIMD, and what the
+    // loop still needs of the first is the conversions to f64.
+    const int nsteps = (int)((hi - lo) / 4);  // steps in which every lane has a row
+    const int tail = (int)((hi - lo) % 4);
+    uint32_t lane_off = 4u * ((uint32_t)kk * (uint32_t)DIM + (uint32_t)jj);
+    const int64_t stepb = 16 * (int64_t)DIM;
+    const char *ybase = reinterpret_cast<const char *>(yr + lo * (int64_t)DIM + 16 * ti);
+    const char *xbase = reinterpret_cast<const char *>(x + lo * (int64_t)DIM + b0);
+    const int ysec = two ? 64 : 0;
+    auto ldf = [](const char *base, uint32_t off, int imm) {
+        return *reinterpret_cast<const float *>(base + (uint64_t)off + imm);
+    };
+    if (nsteps > 0) {
+        // Operands are fetched kAhead steps ahead.  The loads are unconditional (a load under a
+        // branch makes the compiler wait for every load in flight at its use): past the last
+        // whole step they read that step again and the values are dropped.
+        constexpr int kAhead = 4;
+        float a0[kAhead], a1[kAhead], b[kAhead][NT];
 #pragma unroll
         for (int u = 0; u < kAhead; ++u) {
-            const double ac0 = ok[u] ? (double)a0[u] : 0.0, ac1 = (ok[u] && two) ? (double)a1[u] : 0.0;
-            double bc[NT];
+            const int st = u < nsteps ? u : nsteps - 1;
+            const char *yb = ybase + st * stepb, *xb = xbase + st * stepb;
+            a0[u] = ldf(yb, lane_off, 0);
+            a1[u] = ldf(yb + ysec, lane_off, 0);
 #pragma unroll
-            for (int tj = 0; tj < NT; ++tj) bc[tj] = ok[u] ? (double)b[u][tj] : 0.0;
-            const int64_t rn = r + 4 * (u + kAhead);  // first row of the step this slot holds next
-            ok[u] = rn + kk < hi;
-            const int64_t off = ok[u] ? (rn - lo) * (int64_t)DIM : 0;
-            a0[u] = yp[off];
-            a1[u] = yp1[off];
+            for (int tj = 0; tj < NT; ++tj) b[u][tj] = ldf(xb, lane_off, 64 * tj);
+            // in step order: the loop waits for the oldest loads only
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int i = 0; i < nsteps; i += kAhead) {
 #pragma unroll
-            for (int tj = 0; tj < NT; ++tj) b[u][tj] = xp[off + 16 * tj];
-            if (r + 4 * u < hi) {  // the same in every lane
+            for (int u = 0; u < kAhead; ++u) {
+                double ac0 = (double)a0[u], ac1 = (double)a1[u];
+                double bc[NT];
 #pragma unroll
-                for (int tj = 0; tj < NT; ++tj) {
-                    acc0[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(ac0, bc[tj], acc0[tj], 0, 0, 0);
-                    acc1[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(ac1, bc[tj], acc1[tj], 0, 0, 0);
+                for (int tj = 0; tj < NT; ++tj) bc[tj] = (double)b[u][tj];
+                // The conversions stay here (the empty statements pin them: a conversion moved
+                // below the slot's next loads would need copies of the old values, and a wait for
+                // them), so the slot's registers are free for those loads; and the lane offset
+                // stays a 32-bit register beside a scalar base.
+                asm volatile("" : "+v"(ac0), "+v"(ac1));
+#pragma unroll
+                for (int tj = 0; tj < NT; ++tj) asm volatile("" : "+v"(bc[tj]));
+                asm volatile("" : "+v"(lane_off));
+                const int nx = i + u + kAhead;  // the step this slot holds next
+                const int st = nx < nsteps ? nx : nsteps - 1;
+                const char *yb = ybase + st * stepb, *xb = xbase + st * stepb;
+                a0[u] = ldf(yb, lane_off, 0);
+                a1[u] = ldf(yb + ysec, lane_off, 0);
+#pragma unroll
+                for (int tj = 0; tj < NT; ++tj) b[u][tj] = ldf(xb, lane_off, 64 * tj);
+                __builtin_amdgcn_sched_barrier(0);
+                if (i + u < nsteps) {  // the same in every lane
+#pragma unroll
+                    for (int tj = 0; tj < NT; ++tj) {
+                        acc0[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(ac0, bc[tj], acc0[tj], 0, 0, 0);
+                        acc1[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(ac1, bc[tj], acc1[tj], 0, 0, 0);
+                    }
                 }
             }
+        }
+    }
+    if (tail) {  // the chunk's last one to three rows: zeros in the lanes of the missing rows
+        const bool ok = kk < tail;
+        const char *yb = ybase + nsteps * stepb, *xb = xbase + nsteps * stepb;
+        const uint32_t off = ok ? lane_off : 4u * (uint32_t)jj;
+        const double ac0 = ok ? (double)ldf(yb, off, 0) : 0.0, ac1 = ok ? (double)ldf(yb + ysec, off, 0) : 0.0;
+#pragma unroll
+        for (int tj = 0; tj < NT; ++tj) {
+            const double bc = ok ? (double)ldf(xb, off, 64 * tj) : 0.0;
+            acc0[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(ac0, bc, acc0[tj], 0, 0, 0);
+            acc1[tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(ac1, bc, acc1[tj], 0, 0, 0);
         }
     }
     double *out = part + (size_t)blockIdx.x * DIM * DIM;
