@@ -85,6 +85,24 @@ def test_lbg_fit_matches_oracle_bitwise(ctx, n, dim, m, k, iters, kind):
     assert np.array_equal(got.view(np.uint32), want["codebooks"].view(np.uint32))
 
 
+def test_column_blocks_of_one_group_stop_at_different_iterations(ctx):
+    """src/utils.rs:104-106 per column block: blocks 0 and 2 of a group of four hold constant rows and
+    stop after their first pass, blocks 1 and 3 go on (the group's streaming sums are one workgroup)."""
+    rng = np.random.default_rng(77)
+    n, dim, m, k, iters = 40000, 64, 8, 5, 6
+    x = rng.standard_normal((n, dim)).astype(F)
+    for s in (0, 2, 4, 5, 6, 7):
+        x[:, 8 * s:8 * s + 8] = x[0, 8 * s:8 * s + 8]
+    init, reseed = data.index_streams(n, m, k, iters, seed=5)
+    want = O.pq_fit(x, m, k, iters, init, reseed)
+    assert want["rc"] == 0
+    got, it, used, _, _ = gpu_lbg(ctx, x, m, k, iters, init, reseed)
+    assert len(set(want["iters"][:4].tolist())) > 1 and want["iters"][4:].max() < iters
+    assert np.array_equal(it, want["iters"])
+    assert np.array_equal(used, want["reseeds"])
+    assert np.array_equal(got.view(np.uint32), want["codebooks"].view(np.uint32))
+
+
 @pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN, O.COSINE, O.MANHATTAN])
 @pytest.mark.parametrize("n,dim,m,k,kind", [
     (1000, 128, 16, 256, "uniform"),

@@ -530,14 +530,17 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const 
 // accumulator in LDS in rank order (round r: the lanes of rank r, all on different clusters) —
 // so every cluster receives its rows of this part in row order, one at a time, starting from
 // 0.0.  Emits the per-part sums (k_lbg_hist counts the members, on another stream at the same
-// time); no floating-point atomics.
+// time); no floating-point atomics.  The four waves meet at a workgroup barrier before every
+// chunk (the barrier waits for nothing else: the prefetches stay in flight): each of them reads
+// a different 32-byte quarter of the same lines, and waves that drift apart by the length of
+// their prefetch queues find those lines gone from the compute unit's cache.
 static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const float *__restrict__ x, int64_t n,
                                                             int64_t ld) {
     const int g = blockIdx.y, b = blockIdx.x;
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int s = 4 * g + w;
     __shared__ float4 acc_lo[4][kMaxK], acc_hi[4][kMaxK];  // components 0-3 and 4-7 of every cluster
-    if (st.done[s]) return;  // uniform per wave; the waves never synchronise with each other
+    if (st.done[4 * g] && st.done[4 * g + 1] && st.done[4 * g + 2] && st.done[4 * g + 3]) return;
     float4 *alo = acc_lo[w], *ahi = acc_hi[w];
     for (int i = lane; i < kMaxK; i += 64) {
         alo[i] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -546,51 +549,63 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
     __builtin_amdgcn_wave_barrier();
     const int64_t lo = (int64_t)b * kPartRows;
     const int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
-    const uint8_t *__restrict__ codes = st.codes + (size_t)s * n;
+    constexpr int PF = 3;
+    const int rows = (int)(hi - lo);
+    const int nchunks = (rows + 63) / 64, rows_last = rows - 64 * (nchunks - 1);
+    const int nsteps = (nchunks + PF - 1) / PF * PF;  // chunk steps of the loop below, one barrier each
+    if (st.done[s]) {  // this wave's column block has stopped: it only keeps the others' barriers company
+        for (int c = 0; c < nsteps; ++c) __builtin_amdgcn_s_barrier();
+        return;
+    }
     // The sub-vectors and codes of the next PF chunks are kept in flight: one chunk's arithmetic
-    // is far shorter than a memory round trip.
-    constexpr int PF = 4;
+    // is far shorter than a memory round trip.  The loads are unconditional and in chunk order (a
+    // load under a branch, or out of order, makes the compiler wait for every load in flight at
+    // the first use): a lane without a row in the part's last chunk reads that chunk's first row,
+    // the fetches past the last chunk read that chunk again, and both are dropped.
     float4 b0[PF], b1[PF];
-    uint32_t bc[PF];
+    uint8_t bc[PF];  // (bytes until they are used: widened where they are loaded, they would be waited for there)
     // Lanes 2p and 2p+1 fetch the two 16-byte halves of row p of the chunk (b0) and of row 32 + p
     // (b1): one load instruction touches each 64-byte piece of a line once instead of twice.  The
     // neighbours then swap a half, so that lane 2p owns row p and lane 2p + 1 owns row 32 + p.
     const int pr = lane >> 1, hf = lane & 1;
     const int ridx = hf ? 32 + pr : pr;  // this lane's row of a chunk
-    const float *xp = x + (lo + pr) * ld + (int64_t)s * 8 + 4 * hf;
-    const uint8_t *cp = codes + lo + ridx;
-    const int64_t xstep = 64 * ld, xhalf = 32 * ld;
-    const int rows = (int)(hi - lo);
-    int fetched = 0;  // first row of the chunk being fetched
+    // addresses: a scalar base per chunk plus 32-bit lane offsets (a part spans 4096 rows: the
+    // host keeps the leading dimension below 2^20 floats)
+    const char *xbase = reinterpret_cast<const char *>(x + lo * ld + (int64_t)s * 8);
+    const uint8_t *cbase = st.codes + (size_t)s * n + lo;
+    const uint32_t hoff = 16u * (uint32_t)hf;
+    const uint32_t f0 = 4u * (uint32_t)pr * (uint32_t)ld + hoff, f1 = f0 + 128u * (uint32_t)ld;
+    const uint32_t l0 = pr < rows_last ? f0 : hoff, l1 = 32 + pr < rows_last ? f1 : hoff;
+    const uint32_t lc = ridx < rows_last ? (uint32_t)ridx : 0u;
+    const int64_t chunkb = 256 * ld;  // bytes of 64 rows
+    auto fetch = [&](int chunk, float4 &d0, float4 &d1, uint8_t &dc) {
+        const int cc = chunk < nchunks ? chunk : nchunks - 1;  // uniform
+        const bool last = cc == nchunks - 1;
+        const char *xb = xbase + cc * chunkb;
+        const uint8_t *cb = cbase + 64 * cc;
+        d0 = *reinterpret_cast<const float4 *>(xb + (uint64_t)(last ? l0 : f0));
+        d1 = *reinterpret_cast<const float4 *>(xb + (uint64_t)(last ? l1 : f1));
+        dc = cb[last ? lc : (uint32_t)ridx];
+    };
 #pragma unroll
     for (int u = 0; u < PF; ++u) {
-        b0[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-        b1[u] = b0[u];
-        bc[u] = 0u;
-        if (fetched + pr < rows) b0[u] = *reinterpret_cast<const float4 *>(xp);
-        if (fetched + 32 + pr < rows) b1[u] = *reinterpret_cast<const float4 *>(xp + xhalf);
-        if (fetched + ridx < rows) bc[u] = *cp;
-        xp += xstep;
-        cp += 64;
-        fetched += 64;
+        fetch(u, b0[u], b1[u], bc[u]);
+        __builtin_amdgcn_sched_barrier(0);
     }
     // lanes whose row comes before this lane's row
     const unsigned long long even = 0x5555555555555555ull, below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     const unsigned long long ltm = hf ? (even | (~even & below)) : (even & below);
     const uint32_t lt_lo = (uint32_t)ltm, lt_hi = (uint32_t)(ltm >> 32);
-    for (int base = 0; base < rows; base += 64 * PF) {
+    for (int base = 0; base < nsteps; base += PF) {
 #pragma unroll
         for (int u = 0; u < PF; ++u) {
-            if (base + 64 * u >= rows) break;  // uniform
-            bool pending = base + 64 * u + ridx < rows;
+            // (a chunk past the part's end has no pending lane and falls through: an exit from here,
+            // which the compiler routes past the loop's head, would make it wait there for every
+            // load in flight)
+            __builtin_amdgcn_s_barrier();  // step base + u of nsteps
+            const bool pending = 64 * (base + u) + ridx < rows;
             const float4 fa = b0[u], fb = b1[u];
-            const uint32_t c = pending ? bc[u] : 0u;
-            if (fetched + pr < rows) b0[u] = *reinterpret_cast<const float4 *>(xp);
-            if (fetched + 32 + pr < rows) b1[u] = *reinterpret_cast<const float4 *>(xp + xhalf);
-            if (fetched + ridx < rows) bc[u] = *cp;
-            xp += xstep;
-            cp += 64;
-            fetched += 64;
+            uint32_t c = pending ? (uint32_t)bc[u] : 0u;
             // swap: the even lane sends its half of row 32 + p, the odd lane its half of row p
             const float4 snd = hf ? fa : fb;
             float4 rcv;
@@ -598,8 +613,14 @@ static __global__ void __launch_bounds__(256) k_lbg_stream8(LbgState st, const f
             rcv.y = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(snd.y), 0xB1, 0xF, 0xF, true));
             rcv.z = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(snd.z), 0xB1, 0xF, 0xF, true));
             rcv.w = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(snd.w), 0xB1, 0xF, 0xF, true));
-            const float4 v0 = hf ? rcv : fa;  // components 0-3 of this lane's row
-            const float4 v1 = hf ? fb : rcv;  // components 4-7
+            float4 v0 = hf ? rcv : fa;  // components 0-3 of this lane's row
+            float4 v1 = hf ? fb : rcv;  // components 4-7
+            // the slot's registers are free from here on (the empty statement pins the selects
+            // above it): its next loads go out now
+            asm volatile("" : "+v"(v0.x), "+v"(v0.y), "+v"(v0.z), "+v"(v0.w), "+v"(v1.x), "+v"(v1.y), "+v"(v1.z),
+                         "+v"(v1.w), "+v"(c));
+            fetch(base + u + PF, b0[u], b1[u], bc[u]);
+            __builtin_amdgcn_sched_barrier(0);
             // Lanes of the same cluster, found with one wave ballot per code bit: a lane differs
             // from lane j when some bit of its code differs from j's bit in the ballot.
             const unsigned long long vb = __ballot(pending);

@@ -964,7 +964,8 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
     const int nparts = (int)((n + vq::kPartRows - 1) / vq::kPartRows);
     const int nseg = (nparts + vq::kScanSeg - 1) / vq::kScanSeg;
     // streaming sums of the large clusters: 32-byte sub-vectors, 4 per 128-byte line, aligned rows
-    const bool stream = sd == 8 && m % 4 == 0 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0;
+    const bool stream = sd == 8 && m % 4 == 0 && ld % 4 == 0 && ld <= (1 << 20) &&
+                        (reinterpret_cast<uintptr_t>(d_x) & 15) == 0;  // (32-bit lane offsets inside a chunk)
     const int64_t leaf_cap64 = stream ? (int64_t)k : (int64_t)k * nparts;
     if (leaf_cap64 * sd > (1LL << 31)) return fail(ctx, VQ_ERR_UNSUPPORTED, "n * k * sub_dim too large");
     const int leaf_cap = (int)leaf_cap64;
