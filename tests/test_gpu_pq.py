@@ -360,6 +360,35 @@ def test_rows_with_leading_dimension_and_offset(ctx, sd, m, k, pad, shift):
     assert np.array_equal(dcb2.download().view(np.uint32), w["codebooks"].view(np.uint32))
 
 
+def test_leading_dimension_beyond_the_kernels_32_bit_offsets(ctx):
+    """A row stride above 2^20 floats: the matrix-core assignment and the streaming sums address a
+    run of rows with 32-bit offsets and leave such input to the other kernels; codes and centroids
+    are the oracle's all the same.  The rows sit in a device buffer that is mostly never written."""
+    n, sd, m, k, ld = 130, 8, 4, 16, (1 << 20) + 8
+    dim = sd * m
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((n, dim)).astype(F)
+    from vq_amd import _ffi
+    dbuf = ctx.empty((n, ld), F)
+    for i in range(n):  # row i of the wide buffer
+        row = np.ascontiguousarray(x[i])
+        ctx._check(_ffi.lib().vq_h2d(ctx._h, dbuf.ptr + 4 * i * ld, row.ctypes.data, row.nbytes))
+    cb = np.ascontiguousarray(x[rng.choice(n, k, replace=False)].reshape(k, m, sd).transpose(1, 0, 2))
+    dcb = ctx.to_device(cb)
+    dcodes = ctx.empty((n, m), np.uint8)
+    for metric in (O.SQEUCLIDEAN, O.EUCLIDEAN):
+        want = O.pq_encode(metric, x, cb).astype(np.uint8)
+        ctx.assign(metric, dbuf, n, ld, m, sd, k, dcb, dcodes)
+        assert np.array_equal(dcodes.download(), want)
+    init, reseed = data.index_streams(n, m, k, 3, seed=11)
+    w = O.pq_fit(x, m, k, 3, init, reseed)
+    assert w["rc"] == 0
+    dcb2 = ctx.empty((m, k, sd), F)
+    it, _ = ctx.lbg_fit(dbuf, n, ld, m, sd, k, 3, init, reseed, dcb2)
+    assert np.array_equal(it, w["iters"])
+    assert np.array_equal(dcb2.download().view(np.uint32), w["codebooks"].view(np.uint32))
+
+
 @pytest.mark.parametrize("path", [0, 1])
 def test_timing_classes_count_every_pass(ctx, path):
     """The per-class timers (measurement only): a fit of `iters` passes yields `iters` spans of the
