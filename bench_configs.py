@@ -60,8 +60,10 @@ def main():
                 # (epsilon = 0: the mean residual norm, src/rvq.rs:131-141, cannot stop the fit and is skipped,
                 # as the host class does)
 
-        rvq_fit()
-        out["c4_rvq_fit_ms"] = timed(rvq_fit)
+        rvq_fit()  # first call: workspace allocations
+        each = [round(timed(rvq_fit), 3) for _ in range(3)]  # (the clock is still ramping during the first)
+        out["c4_rvq_fit_ms"] = min(each[1:])
+        out["c4_rvq_fit_ms_each"] = each
         dall = ctx.empty((n, stages), np.uint8)
         drec = ctx.empty((n, dim), np.uint16)
         enc = lambda: ctx.rvq_encode(vq_amd.EUCLIDEAN, dx, n, dim, dim, stages, k, dcb, 0.0, dall, None, drec)
