@@ -517,9 +517,9 @@ __device__ __forceinline__ void wide_argmin(const AssignArgs &a, int sd, int s, 
 // The wave's share of the groups of NR rows (or listed pairs).
 template <int METRIC, bool LBG, bool LISTED, bool VEC, int NR>
 __device__ __forceinline__ void wide_exact_groups(const AssignArgs &a, int sd, const uint32_t *__restrict__ list,
-                                                  int64_t total, float *lds_x, int lane, int wave) {
+                                                  int64_t total, float *lds_x, int lane, int wave, unsigned nblocks) {
     const int64_t groups = (total + NR - 1) / NR;
-    for (int64_t grp = (int64_t)blockIdx.x * 4 + wave; grp < groups; grp += (int64_t)gridDim.x * 4) {
+    for (int64_t grp = (int64_t)blockIdx.x * 4 + wave; grp < groups; grp += (int64_t)nblocks * 4) {
         int64_t rows[NR];
         int ss[NR];
 #pragma unroll
@@ -701,33 +701,6 @@ __device__ __forceinline__ void wide_exact_pair_wg(const AssignArgs &a, int sd, 
     }
 }
 
-template <int METRIC, bool LBG, bool LISTED, bool VEC>
-__global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd, const uint32_t *__restrict__ list,
-                                                           const uint32_t *__restrict__ list_count) {
-    extern __shared__ float lds_wide[];  // 4 waves x 8 rows x sd
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    float *lds_x = lds_wide + (size_t)wave * kWideRows * sd;
-    const int64_t total = LISTED ? (int64_t)*list_count : a.n;
-    if constexpr (LBG && !LISTED) {
-        if (a.done[blockIdx.y]) return;
-    }
-    if constexpr (LISTED && VEC && (METRIC == M_SQ || METRIC == M_EUCLID)) {
-        // a handful of pairs: one per workgroup, one centroid per thread
-        if (total <= (int64_t)gridDim.x && a.k <= 256) {
-            if ((int64_t)blockIdx.x < total) wide_exact_pair_wg<METRIC, LBG>(a, sd, list[blockIdx.x], lds_wide);
-            return;
-        }
-    }
-    if constexpr (LISTED) {
-        // a short list: one pair per wave, so that the pass is as long as one pair's scan, not eight
-        if (total <= (int64_t)gridDim.x * 4) {
-            wide_exact_groups<METRIC, LBG, LISTED, VEC, 1>(a, sd, list, total, lds_x, lane, wave);
-            return;
-        }
-    }
-    wide_exact_groups<METRIC, LBG, LISTED, VEC, kWideRows>(a, sd, list, total, lds_x, lane, wave);
-}
-
 // Exact decision between two candidate centroids per listed (row, column block) pair — the
 // pairs the matrix-core pass narrowed down to its two best scores.  Lanes 2i and 2i + 1 take
 // candidates c1 and c2 of entry i: each accumulates its distance in the reference's order
@@ -735,13 +708,13 @@ __global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd,
 // reference's strict '<' scan restricted to the only two centroids that can win it.  Euclidean
 // compares the roots, as the reference does.  Requires sd % 4 == 0 and 16-byte aligned rows
 // and centroids.
+// Workgroup `block` of `nblocks` that share the list.
 template <int METRIC, bool LBG>
-__global__ void __launch_bounds__(256) k_assign_wide_pair(AssignArgs a, int sd, const uint2 *__restrict__ pairs,
-                                                          const uint32_t *__restrict__ pair_count) {
-    const uint32_t total = *pair_count;
+__device__ __forceinline__ void wide_pair_blocks(const AssignArgs &a, int sd, const uint2 *__restrict__ pairs,
+                                                 uint32_t total, unsigned block, unsigned nblocks) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float inf = __builtin_inff();
-    for (uint64_t base = ((uint64_t)blockIdx.x * 4 + wave) * 32; base < total; base += (uint64_t)gridDim.x * 4 * 32) {
+    for (uint64_t base = ((uint64_t)block * 4 + wave) * 32; base < total; base += (uint64_t)nblocks * 4 * 32) {
         const uint64_t e = base + (lane >> 1);
         const bool active = e < total;
         const uint2 ent = pairs[active ? e : base];
@@ -777,6 +750,44 @@ __global__ void __launch_bounds__(256) k_assign_wide_pair(AssignArgs a, int sd, 
             }
         }
     }
+}
+
+template <int METRIC, bool LBG, bool LISTED, bool VEC>
+__global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd, const uint32_t *__restrict__ list,
+                                                           const uint32_t *__restrict__ list_count,
+                                                           const uint2 *__restrict__ pairs,
+                                                           const uint32_t *__restrict__ pair_count,
+                                                           unsigned exact_blocks) {
+    extern __shared__ float lds_wide[];  // 4 waves x 8 rows x sd
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // The workgroups from exact_blocks on take the list of pairs with two candidates: the two
+    // follow-ups of the matrix-core pass are short and independent, and run side by side in one launch.
+    if constexpr (LISTED && (METRIC == M_SQ || METRIC == M_EUCLID)) {
+        if (blockIdx.x >= exact_blocks) {
+            wide_pair_blocks<METRIC, LBG>(a, sd, pairs, *pair_count, blockIdx.x - exact_blocks, gridDim.x - exact_blocks);
+            return;
+        }
+    }
+    float *lds_x = lds_wide + (size_t)wave * kWideRows * sd;
+    const int64_t total = LISTED ? (int64_t)*list_count : a.n;
+    if constexpr (LBG && !LISTED) {
+        if (a.done[blockIdx.y]) return;
+    }
+    if constexpr (LISTED && VEC && (METRIC == M_SQ || METRIC == M_EUCLID)) {
+        // a handful of pairs: one per workgroup, one centroid per thread
+        if (total <= (int64_t)exact_blocks && a.k <= 256) {
+            if ((int64_t)blockIdx.x < total) wide_exact_pair_wg<METRIC, LBG>(a, sd, list[blockIdx.x], lds_wide);
+            return;
+        }
+    }
+    if constexpr (LISTED) {
+        // a short list: one pair per wave, so that the pass is as long as one pair's scan, not eight
+        if (total <= (int64_t)exact_blocks * 4) {
+            wide_exact_groups<METRIC, LBG, LISTED, VEC, 1>(a, sd, list, total, lds_x, lane, wave, exact_blocks);
+            return;
+        }
+    }
+    wide_exact_groups<METRIC, LBG, LISTED, VEC, kWideRows>(a, sd, list, total, lds_x, lane, wave, exact_blocks);
 }
 
 }  // namespace vq

@@ -58,7 +58,7 @@ static __device__ __align__(256) unsigned char scratch[kNoAllocBytes];
 
 template <int METRIC, bool LBG>
 int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const uint32_t *list,
-                          const uint32_t *count);
+                          const uint32_t *count, const uint2 *pairs = nullptr, const uint32_t *pair_count = nullptr);
 
 template <int SD, int G, int METRIC, bool LBG>
 int32_t launch_static(vq_ctx *ctx, const vq::AssignArgs &a) {
@@ -213,7 +213,7 @@ int32_t launch_mfma(vq_ctx *ctx, const vq::AssignArgs &a, bool tables_ready, hip
 // undecided pairs of the matrix-core pass.
 template <int METRIC, bool LBG>
 int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const uint32_t *list,
-                          const uint32_t *count) {
+                          const uint32_t *count, const uint2 *pairs, const uint32_t *pair_count) {
     const bool vec = sd % 4 == 0 && (reinterpret_cast<uintptr_t>(a.cb) & 15) == 0;
     const bool listed = list != nullptr;
     size_t lds = sizeof(float) * 4 * vq::kWideRows * (size_t)sd;
@@ -230,9 +230,11 @@ int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const ui
         VQ_HIP(ctx, hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int64_t groups = (a.n + vq::kWideRows - 1) / vq::kWideRows;
     dim3 grid(listed ? 2048u : (unsigned)std::min<int64_t>((groups + 3) / 4, 1 << 20), listed ? 1u : (unsigned)a.m);
+    unsigned exact_blocks = grid.x;
+    if (pairs) grid.x += 512u;  // the workgroups of the two-candidate list
     vq::AssignArgs aa = a;
     int sdv = sd;
-    void *args[] = {&aa, &sdv, (void *)&list, (void *)&count};
+    void *args[] = {&aa, &sdv, (void *)&list, (void *)&count, (void *)&pairs, (void *)&pair_count, &exact_blocks};
     VQ_HIP(ctx, hipLaunchKernel(kern, grid, dim3(256), args, lds, ctx->stream));
     return VQ_OK;
 }
@@ -284,11 +286,9 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     }
     VQ_HIP(ctx, hipGetLastError());
     ctx->recheck_src = 2;
-    // undecided pairs with two candidates, then the few that need every centroid
-    hipLaunchKernelGGL((vq::k_assign_wide_pair<METRIC, LBG>), dim3(512), dim3(256), 0, ctx->stream, a, sd,
-                       (const uint2 *)pairs, (const uint32_t *)(count + 1));
-    VQ_HIP(ctx, hipGetLastError());
-    return launch_wide_exact<METRIC, LBG>(ctx, a, sd, list, count);
+    // undecided pairs with two candidates and the few that need every centroid, in one launch
+    return launch_wide_exact<METRIC, LBG>(ctx, a, sd, list, count, (const uint2 *)pairs,
+                                          (const uint32_t *)(count + 1));
 }
 
 template <int METRIC, bool LBG>
