@@ -15,8 +15,12 @@ Prints ONE JSON line:
                their measured issue rate are secondary fields
   end_to_end   one pass pageable host rows -> upload -> fit -> encode -> codes on the host
   calibration  measured peaks of the box: plain-copy HBM rate, vector instruction issue rates
-  cpu_baseline the C restatement of the reference (oracle/) timed on the host cores on a bounded
-               sample of the same workload
+  cpu_baseline the C restatement of the reference (oracle/) timed on the host cores on the same
+               workload with the same index streams; `parity` compares its codebooks and codes with
+               the buffers the timed steps wrote
+  other_configs  after the headline measurement: the OPQ, RVQ and TSVQ configurations at full size
+               (bench_configs.py), each with its times, its dominant kernel against its bound and
+               the parity triple against the oracle on a sample
 """
 import argparse
 import json
@@ -56,6 +60,8 @@ def main():
                     help="skip the one-off host-to-codes measurement")
     ap.add_argument("--cpu-sample", type=int, default=1_000_000,
                     help="rows of the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--configs", default="c3,c4,c5",
+                    help="other configurations to run after the headline measurement (\"\" = none)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -87,15 +93,19 @@ def main():
                           "copy_calibration_bytes_written": n * DIM * 4, "launches": 3}))
         return
 
+    iters_seen = []
+
     def step():
-        ctx.lbg_fit(dx, n, DIM, M, sd, K, ITERS, init, reseed, dcb)
+        it, _ = ctx.lbg_fit(dx, n, DIM, M, sd, K, ITERS, init, reseed, dcb)
         ctx.assign(vq_amd.EUCLIDEAN, dx, n, DIM, M, sd, K, dcb, dcodes)
+        iters_seen.append(it)
 
     for _ in range(args.warmup):
         step()
     ctx.sync()
     ctx.prof_enable(True)
     ctx.sync()
+    del iters_seen[:]
     t0 = time.perf_counter()
     ctx.timer_start()
     for _ in range(args.steps):
@@ -109,6 +119,10 @@ def main():
     kern_ms, kern_n = ctx.prof_read(vq_amd._ffi.PROF_ASSIGN_KERNEL)
     ctx.prof_enable(False)
     recheck_pairs = ctx.last_recheck_count()
+    # what the timed steps left in their output buffers, and how many LBG iterations each column
+    # block ran in them (a block that converges leaves its later passes at once: the line says so)
+    timed_cb, timed_codes = dcb.download(), dcodes.download()
+    timed_iters = np.concatenate(iters_seen) if iters_seen else np.zeros(1, np.int32)
     ms_per_step = wall_ms / args.steps
     value = n / (ms_per_step * 1e-3)
 
@@ -176,10 +190,28 @@ def main():
     roofline["frac_of_selection_floor"] = round(floor_ms / avg_kern_ms, 4)
     roofline["issue_floor_ms"] = round(floor_ms + mfma_ms, 4)
     roofline["frac_of_issue_floor"] = round((floor_ms + mfma_ms) / avg_kern_ms, 4)
+    # The peak above is the packed / dual-rate one.  The selection's instruction class (v_min3_i32,
+    # v_med3_i32, v_and_or_b32) issues one wave64 per 4 clocks and SIMD: 256 CUs x 64 lanes x 2.4 GHz.
+    roofline["peak_of_selection_class"] = PEAK_VALU_TLANESLOTS / 2.0
+    roofline["frac_of_selection_class_peak"] = round(achieved_slots / (PEAK_VALU_TLANESLOTS / 2.0), 4)
+    # Do matrix and vector instructions of a SIMD run side by side?  (ms: matrix alone, vector alone,
+    # together.)  From different waves they take turns (together = sum), which is why issue_floor_ms
+    # adds them; behind a matrix instruction of the SAME wave independent vector instructions issue
+    # in its shadow, all but about a quarter of its 32 clocks — the kernel places half a block's
+    # selection behind each matrix instruction for that reason.
+    ov = {}
+    for mode, name in ((0, "different_waves_8_min3_per_mfma"), (1, "same_wave_7_min3_per_mfma"),
+                       (2, "same_wave_3_min3_per_mfma")):
+        (t_m, t_v, t_b), waves = ctx.calibrate_overlap(mode)
+        ov[name] = {"mfma_alone_ms": round(t_m, 4), "valu_alone_ms": round(t_v, 4), "together_ms": round(t_b, 4),
+                    "together_over_sum": round(t_b / (t_m + t_v), 3), "together_over_max": round(t_b / max(t_m, t_v), 3)}
+        if mode == 0:
+            ov[name]["waves_per_simd_number_mfma_then_valu"] = list(waves)
     calibration = {
         "hbm_copy_GBs_read_plus_write": round(ctx.calibrate(0), 1),
         "valu_wave64_Ginstr_per_s": {k_: round(v / 1e9, 1) for k_, v in rate.items()},
         "valu_fma_TFLOPs": round(rate["v_fma_f32"] * 128.0 / 1e12, 1),
+        "mfma_valu_overlap": ov,
     }
     breakdown = {
         "lbg_assign_ms_per_step": round(assign_ms / args.steps, 3),
@@ -187,6 +219,10 @@ def main():
         "encode_ms_per_step": round(enc_ms / args.steps, 3),
         "gpu_event_ms_per_step": round(gpu_ms / args.steps, 3),
         "encode_recheck_fraction": round(recheck_pairs / float(n * M), 6),
+        # LBG iterations run per column block over the timed steps: 10 = no block stopped early, every
+        # timed pass did its full work
+        "lbg_iters_run_min": int(timed_iters.min()),
+        "lbg_iters_run_max": int(timed_iters.max()),
     }
 
     # End to end, once: what a host that starts from rows in its own (pageable) memory pays.  vq_h2d
@@ -227,14 +263,16 @@ def main():
         ctx.host_free(hx)
         ctx.host_free(hcodes)
 
-    # CPU baseline + parity on a bounded sample of the same rows
+    # CPU baseline on the same rows with the same index streams, and parity of what the TIMED steps
+    # wrote (codebooks and codes of the last timed step) against it
     cpu = None
     parity = None
     if args.cpu_sample > 0:
         from oracle import oracle as O
         ns = min(args.cpu_sample, n)
-        xs = np.ascontiguousarray(x[:ns])
-        init_s, reseed_s = data.index_streams(ns, M, K, ITERS, seed=2)
+        full = ns == n
+        xs = x if full else np.ascontiguousarray(x[:ns])
+        init_s, reseed_s = (init, reseed) if full else data.index_streams(ns, M, K, ITERS, seed=2)
         threads = min(os.cpu_count() or 1, 16)
         t0 = time.perf_counter()
         ref = O.pq_fit_encode(O.EUCLIDEAN, xs, M, K, ITERS, init_s, reseed_s, threads=threads)
@@ -247,21 +285,31 @@ def main():
             "reference_published": "3,751 vectors/s (266.6 s for 1M x 128 uniform rows, "
                                    "i7-1355U laptop, reference README.md:79-80)",
         }
-        dxs = ctx.to_device(xs)
-        dcb_s = ctx.empty((M, K, sd), np.float32)
-        dcodes_s = ctx.empty((ns, M), np.uint8)
-        ctx.lbg_fit(dxs, ns, DIM, M, sd, K, ITERS, init_s, reseed_s, dcb_s)
-        ctx.assign(vq_amd.EUCLIDEAN, dxs, ns, DIM, M, sd, K, dcb_s, dcodes_s)
-        g_cb, g_codes = dcb_s.download(), dcodes_s.download()
+        if full:
+            g_cb, g_codes = timed_cb, timed_codes
+            dcodes_s, dcb_s = dcodes, dcb
+        else:
+            dxs = ctx.to_device(xs)
+            dcb_s = ctx.empty((M, K, sd), np.float32)
+            dcodes_s = ctx.empty((ns, M), np.uint8)
+            ctx.lbg_fit(dxs, ns, DIM, M, sd, K, ITERS, init_s, reseed_s, dcb_s)
+            ctx.assign(vq_amd.EUCLIDEAN, dxs, ns, DIM, M, sd, K, dcb_s, dcodes_s)
+            g_cb, g_codes = dcb_s.download(), dcodes_s.download()
         num = np.sqrt(((g_cb.astype(np.float64) - ref["codebooks"]) ** 2).sum())
         den = np.sqrt((ref["codebooks"].astype(np.float64) ** 2).sum())
         # reconstruction MSE of the f16 reconstructions (src/bin/utils.rs:50-67), both sides
         dre = ctx.empty((ns, DIM), np.uint16)
+        if full:
+            dcodes_s.upload(g_codes)
+            dcb_s.upload(g_cb)
         ctx.decode_f16(dcodes_s, ns, M, sd, K, dcb_s, dre)
         mse_gpu = O.mse_f16(xs, dre.download())
         mse_ref = O.mse_f16(xs, O.pq_decode_f16(ref["codes"], ref["codebooks"]))
+        dre.free()
         parity = {
             "sample_rows": ns,
+            "compared": "the codebooks and codes the timed steps wrote (same rows, same index streams)" if full
+                        else "a separate fit + encode of the sample",
             "mse_gpu": float(mse_gpu), "mse_ref": float(mse_ref),
             "mse_rel_diff": float(abs(mse_gpu - mse_ref) / mse_ref) if mse_ref else 0.0,
             "code_mismatch_rate": float(np.mean(g_codes != ref["codes"].astype(np.uint8))),
@@ -269,6 +317,13 @@ def main():
             "centroids_bit_identical": bool(np.array_equal(g_cb.view(np.uint32),
                                                            ref["codebooks"].view(np.uint32))),
         }
+
+    # the other configurations, after the headline measurement (bench_configs.py)
+    others = None
+    which = [c for c in args.configs.split(",") if c]
+    if which and n == N_ROWS:
+        import bench_configs
+        others = bench_configs.other_configs(ctx, log, which, x_c2=x, dx_c2=dx)
 
     out = {
         "metric": "PQ fit+encode vectors/sec at 1M x 128, m=16, k=256 (10 LBG iterations)",
@@ -293,6 +348,7 @@ def main():
         "breakdown": breakdown,
         "end_to_end": end_to_end,
         "parity": parity,
+        "other_configs": others,
     }
     print(json.dumps(out), flush=True)
 

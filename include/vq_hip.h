@@ -98,6 +98,17 @@ enum {
     VQ_CALIB_VALU_ADD = 5
 };
 int32_t vq_calibrate(vq_ctx *ctx, int32_t what, double *h_rate);
+/* Whether the matrix and the vector instructions of one SIMD run side by side or take turns
+ * (measurement only; no counterpart in the reference).  Every SIMD holds 8 waves.
+ *   mode 0  four waves of a SIMD issue chains of v_mfma_f32_32x32x16_bf16 (4096 each), the other four
+ *           chains of v_min3_i32 (8 x 4096 each): the two kinds come from different waves
+ *   mode 1  every wave issues both in one instruction stream, 7 independent v_min3_i32 after each
+ *           matrix instruction;  mode 2: the same with 3
+ * h_ms[0] = milliseconds of the matrix instructions alone, h_ms[1] of the vector instructions alone,
+ * h_ms[2] of both together (same counts).  h_waves (nullable, 8 numbers; mode 0 only, else zeros):
+ * how many waves of the last launch ran on SIMD 0..3 of their compute unit, first the matrix waves,
+ * then the vector waves — equal numbers mean every SIMD held both kinds.  Synchronises. */
+int32_t vq_calibrate_overlap(vq_ctx *ctx, int32_t mode, double *h_ms, uint32_t *h_waves);
 
 /* Number of (row, block) pairs the most recent matrix-core assignment pass left to the exact
  * re-check (0 if that path has not run).  Synchronises.  Measurement only. */

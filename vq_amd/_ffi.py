@@ -29,6 +29,7 @@ SYMBOLS = {
     "vq_ctx_set_assign_path": (_i32, [_vp, _i32]),
     "vq_ctx_set_tsvq_variance_path": (_i32, [_vp, _i32]),
     "vq_calibrate": (_i32, [_vp, _i32, C.POINTER(C.c_double)]),
+    "vq_calibrate_overlap": (_i32, [_vp, _i32, C.POINTER(C.c_double), C.POINTER(C.c_uint32)]),
     "vq_ctx_last_recheck_count": (_i32, [_vp, C.POINTER(C.c_uint32)]),
     "vq_ctx_last_recheck_split": (_i32, [_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "vq_procrustes_rotation": (_i32, [_vp, _vp, _i32, _vp]),
@@ -232,6 +233,16 @@ class Context:
         out = C.c_double(0)
         self._check(_lib.vq_calibrate(self._h, what, C.byref(out)))
         return out.value
+
+    def calibrate_overlap(self, mode):
+        """Milliseconds of (matrix instructions alone, vector instructions alone, both together) on
+        every SIMD; mode 0: from different waves, 1 / 2: one stream with 7 / 3 vector instructions
+        per matrix instruction.  Second value: waves per SIMD number (mode 0: four counts of the matrix
+        waves, four of the vector waves)."""
+        out = (C.c_double * 3)()
+        waves = (C.c_uint32 * 8)()
+        self._check(_lib.vq_calibrate_overlap(self._h, mode, out, waves))
+        return tuple(out), tuple(waves)
 
     def set_tsvq_variance_path(self, path):
         """0: composed integer maps (default); 1: one chain of adds per column."""

@@ -479,31 +479,68 @@ __global__ void __launch_bounds__(256, 3) k_assign_mfma_bf(AssignArgs a, MfmaBfT
         int m1 = 0x7f800000, m2 = 0x7f800000;  // +inf
         // One block of 32 centroids.  The tag leaves out the lane half (bit 2), so it is the same in
         // every lane and lives in scalar registers.
-#define VQ_SCORE_BLOCK(b)                                                                                       \
+        // The scores of block b + 1 are made while block b's go through the selection: a matrix
+        // instruction holds back the vector instructions of OTHER waves of its SIMD for as long as it
+        // runs, but independent vector instructions of its own wave issue in its shadow, so every
+        // matrix instruction is followed by half a block's selection from the same wave.
+#define VQ_MFMA_1(b, acc)                                                                                       \
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A1[b]),                            \
+                                                  __builtin_bit_cast(bf16x8, b1), zero, 0, 0, 0);
+#define VQ_MFMA_2(b, acc)                                                                                       \
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A2[b]),                            \
+                                                  __builtin_bit_cast(bf16x8, b2), acc, 0, 0, 0);
+#define VQ_RUN_KEY(b, acc, p)                                                                                   \
     {                                                                                                           \
-        const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};      \
-        floatx16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A1[b]),               \
-                                                               __builtin_bit_cast(bf16x8, b1), zero, 0, 0, 0);  \
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, A2[b]),                        \
-                                                      __builtin_bit_cast(bf16x8, b2), acc, 0, 0, 0);            \
-        int key[4];                                                                                             \
-        _Pragma("unroll") for (int p = 0; p < 4; ++p) {                                                         \
-            const int gmin = imin(imin(imin(__float_as_int(acc[4 * p]), __float_as_int(acc[4 * p + 1])),        \
-                                       __float_as_int(acc[4 * p + 2])),                                         \
-                                  __float_as_int(acc[4 * p + 3]));                                              \
-            key[p] = (int)(((uint32_t)gmin & keep) | (uint32_t)(32 * (b) + 8 * p));                             \
-        }                                                                                                       \
-        top2_push4(m1, m2, key[0], key[1], key[2], key[3]);                                                     \
+        const int gmin = imin(imin(imin(__float_as_int(acc[4 * p]), __float_as_int(acc[4 * p + 1])),            \
+                                   __float_as_int(acc[4 * p + 2])),                                             \
+                              __float_as_int(acc[4 * p + 3]));                                                  \
+        key[p] = (int)(((uint32_t)gmin & keep) | (uint32_t)(32 * (b) + 8 * p));                                 \
     }
+        // selection of block b (scores in cur) with the matrix instructions of block nb (into nxt) in between
+#define VQ_SCORE_BLOCK(b, cur, nb, nxt, more)                                                                   \
+    {                                                                                                           \
+        int key[4];                                                                                             \
+        if (more) { VQ_MFMA_1(nb, nxt) }                                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                                      \
+        VQ_RUN_KEY(b, cur, 0) VQ_RUN_KEY(b, cur, 1)                                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                                      \
+        if (more) { VQ_MFMA_2(nb, nxt) }                                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                                      \
+        VQ_RUN_KEY(b, cur, 2) VQ_RUN_KEY(b, cur, 3)                                                             \
+        top2_push4(m1, m2, key[0], key[1], key[2], key[3]);                                                     \
+        __builtin_amdgcn_sched_barrier(0);                                                                      \
+    }
+        const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        floatx16 accA, accB;
+        VQ_MFMA_1(0, accA)
+        VQ_MFMA_2(0, accA)
         if constexpr (FULL) {
-            VQ_SCORE_BLOCK(0) VQ_SCORE_BLOCK(1) VQ_SCORE_BLOCK(2) VQ_SCORE_BLOCK(3)
-            VQ_SCORE_BLOCK(4) VQ_SCORE_BLOCK(5) VQ_SCORE_BLOCK(6) VQ_SCORE_BLOCK(7)
+            VQ_SCORE_BLOCK(0, accA, 1, accB, true) VQ_SCORE_BLOCK(1, accB, 2, accA, true)
+            VQ_SCORE_BLOCK(2, accA, 3, accB, true) VQ_SCORE_BLOCK(3, accB, 4, accA, true)
+            VQ_SCORE_BLOCK(4, accA, 5, accB, true) VQ_SCORE_BLOCK(5, accB, 6, accA, true)
+            VQ_SCORE_BLOCK(6, accA, 7, accB, true) VQ_SCORE_BLOCK(7, accB, 0, accA, false)
         } else {
-            VQ_SCORE_BLOCK(0) VQ_SCORE_BLOCK(1)
-            if (nb > 2) { VQ_SCORE_BLOCK(2) VQ_SCORE_BLOCK(3) }
-            if (nb > 4) { VQ_SCORE_BLOCK(4) VQ_SCORE_BLOCK(5) }
-            if (nb > 6) { VQ_SCORE_BLOCK(6) VQ_SCORE_BLOCK(7) }
+            VQ_SCORE_BLOCK(0, accA, 1, accB, true)
+            if (nb > 2) {
+                VQ_SCORE_BLOCK(1, accB, 2, accA, true) VQ_SCORE_BLOCK(2, accA, 3, accB, true)
+                if (nb > 4) {
+                    VQ_SCORE_BLOCK(3, accB, 4, accA, true) VQ_SCORE_BLOCK(4, accA, 5, accB, true)
+                    if (nb > 6) {
+                        VQ_SCORE_BLOCK(5, accB, 6, accA, true) VQ_SCORE_BLOCK(6, accA, 7, accB, true)
+                        VQ_SCORE_BLOCK(7, accB, 0, accA, false)
+                    } else {
+                        VQ_SCORE_BLOCK(5, accB, 0, accA, false)
+                    }
+                } else {
+                    VQ_SCORE_BLOCK(3, accB, 0, accA, false)
+                }
+            } else {
+                VQ_SCORE_BLOCK(1, accB, 0, accA, false)
+            }
         }
+#undef VQ_MFMA_1
+#undef VQ_MFMA_2
+#undef VQ_RUN_KEY
 #undef VQ_SCORE_BLOCK
         // the partner lane (other half) saw the other 16 centroids of every block
         m1 |= 4 * h;  // bit 2 of the centroid index: the lane half

@@ -860,6 +860,53 @@ int32_t vq_calibrate(vq_ctx *ctx, int32_t what, double *h_rate) {
     return VQ_OK;
 }
 
+int32_t vq_calibrate_overlap(vq_ctx *ctx, int32_t mode, double *h_ms, uint32_t *h_waves) {
+    if (!ctx || !h_ms || mode < 0 || mode > 2)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: overlap calibration mode %d", mode);
+    VQ_HIP(ctx, hipSetDevice(ctx->device));
+    hipStream_t st = ctx->stream;
+    hipDeviceProp_t prop;
+    VQ_HIP(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    const unsigned waves_per_cu = 32u;  // 8 on every SIMD
+    VQ_TRY(ensure(ctx, ctx->tmp_a, 256));
+    uint32_t *sink = (uint32_t *)ctx->tmp_a.p, *where = sink + 8;
+    const int n_mfma = 4096;
+    const int vpm = mode == 0 ? 8 : mode == 1 ? 7 : 3;  // vector instructions per matrix instruction
+    const int n_valu = n_mfma * vpm;
+    for (int which = 0; which < 3; ++which) {
+        const int nm = which == 1 ? 0 : n_mfma, nv = which == 0 ? 0 : n_valu;
+        float best = 1e30f, ms = 0.f;
+        for (int rep = 0; rep < 4; ++rep) {
+            VQ_HIP(ctx, hipMemsetAsync(where, 0, 8 * sizeof(uint32_t), st));
+            VQ_HIP(ctx, hipEventRecord(ctx->ev0, st));
+            if (mode == 0)
+                hipLaunchKernelGGL((vq::k_calib_overlap<0, 8>), dim3((unsigned)prop.multiProcessorCount * waves_per_cu / 8u),
+                                   dim3(512), 0, st, nm, nv, 1u, sink, where);
+            else if (mode == 1)
+                hipLaunchKernelGGL((vq::k_calib_overlap<1, 7>), dim3((unsigned)prop.multiProcessorCount * waves_per_cu / 4u),
+                                   dim3(256), 0, st, nm, nv, 1u, sink, where);
+            else
+                hipLaunchKernelGGL((vq::k_calib_overlap<1, 3>), dim3((unsigned)prop.multiProcessorCount * waves_per_cu / 4u),
+                                   dim3(256), 0, st, nm, nv, 1u, sink, where);
+            VQ_HIP(ctx, hipGetLastError());
+            VQ_HIP(ctx, hipEventRecord(ctx->ev1, st));
+            VQ_HIP(ctx, hipEventSynchronize(ctx->ev1));
+            VQ_HIP(ctx, hipEventElapsedTime(&ms, ctx->ev0, ctx->ev1));
+            if (rep > 0 && ms < best) best = ms;
+        }
+        h_ms[which] = best;
+    }
+    if (h_waves) {
+        if (mode == 0) {
+            VQ_HIP(ctx, hipMemcpyAsync(h_waves, where, 8 * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+            VQ_HIP(ctx, hipStreamSynchronize(st));
+        } else {
+            for (int i = 0; i < 8; ++i) h_waves[i] = 0u;
+        }
+    }
+    return VQ_OK;
+}
+
 int32_t vq_ctx_set_tsvq_variance_path(vq_ctx *ctx, int32_t path) {
     if (!ctx || (path != 0 && path != 1)) return VQ_ERR_INVALID_ARG;
     ctx->tsvq_var_path = path;
