@@ -86,10 +86,11 @@ def _kernel_avg(ctx, fn):
 
 
 # ---- c3: OPQ ---------------------------------------------------------------------------------
-def opq_fit_device(ctx, dx, n, dim, m, k, iters, outer, streams, metric, bufs=None, snapshots=()):
+def opq_fit_device(ctx, dx, n, dim, m, k, iters, outer, streams, metric, bufs=None, snapshots=(), trace=None):
     """OptimizedProductQuantizer::fit (src/opq.rs:90-205) on rows already in HBM, the calls of the
-    host class (vq_amd/host/vq.hpp) one by one.  Returns (rotation f32, codebooks device array,
-    {outer iteration: (rotation, codebooks)} for the iterations named in snapshots)."""
+    host class (vq_amd/host/vq.hpp) one by one.  Returns (rotation f32, buffers,
+    {outer iteration: (rotation, codebooks)} for the iterations named in snapshots).  trace (a list):
+    receives (rows the iteration trained on, its codebooks, A, R) of every outer iteration."""
     import vq_amd
     sd = dim // m
     init, reseed = streams
@@ -101,6 +102,7 @@ def opq_fit_device(ctx, dx, n, dim, m, k, iters, outer, streams, metric, bufs=No
     R = np.eye(dim, dtype=F)
     snaps = {}
     for it in range(outer):
+        rows = drot.download() if trace is not None else None
         ctx.lbg_fit(drot, n, dim, m, sd, k, iters, init, reseed, dcb)       # 127-142
         ctx.assign(metric, drot, n, dim, m, sd, k, dcb, dcodes)             # 146-163
         ctx.decode_f32(dcodes, n, m, sd, k, dcb, drec)                      # 164-167
@@ -110,6 +112,8 @@ def opq_fit_device(ctx, dx, n, dim, m, k, iters, outer, streams, metric, bufs=No
         ctx.rotate(dx, n, dim, dim, dR, drot)                               # 186-194
         if it + 1 in snapshots:
             snaps[it + 1] = (R.copy(), dcb.download())
+        if trace is not None:
+            trace.append((rows, dcb.download(), dcodes.download(), A, R.copy()))
     return R, bufs, snaps
 
 
@@ -174,7 +178,9 @@ def run_c3(ctx, log, x=None, dx=None):
     xs = np.ascontiguousarray(x[:ns])
     st_s = data.index_streams(ns, m, k, iters, seed=3)
     dxs = ctx.to_device(xs)
-    _, sb, snaps = opq_fit_device(ctx, dxs, ns, dim, m, k, iters, outer, st_s, vq_amd.EUCLIDEAN, snapshots=(1, 3, 5))
+    trace = []
+    _, sb, snaps = opq_fit_device(ctx, dxs, ns, dim, m, k, iters, outer, st_s, vq_amd.EUCLIDEAN, snapshots=(1, 3, 5),
+                                  trace=trace)
     par = {}
     t0 = time.perf_counter()
     for it in (1, 3, 5):
@@ -198,19 +204,36 @@ def run_c3(ctx, log, x=None, dx=None):
             "mse_gpu": mse_g, "mse_ref": mse_r, "mse_rel_diff": _rel(mse_g, mse_r)}
         for b in (dRg, dcbg, drec):
             b.free()
-    # How much of that is the algorithm's own sensitivity: the oracle against itself with ONE element
-    # of the sample moved by one unit in the last place.  From the second outer iteration on the two
-    # sides train on rotated rows that differ in their last bits (the rotation is a tolerance
-    # quantity: a matrix product and an SVD whose rounding the reference leaves to nalgebra), and
-    # Lloyd iterations amplify such differences — a row that changes its cluster moves two centroids.
-    xp = xs.copy()
-    xp[0, 0] = np.nextafter(xp[0, 0], F(2.0))
+    # Where the difference from the second outer iteration on comes from.  (1) Step by step along the
+    # GPU's own trajectory: the oracle, given the rows each outer iteration of the GPU trained on,
+    # must reproduce that iteration's codebooks and codes bit for bit and its rotation update to
+    # rounding, so nothing but the rotated rows' last bits separates the two runs (the rotation is a
+    # tolerance quantity: a matrix product and an SVD whose rounding the reference leaves to
+    # nalgebra; the library's product runs on the matrix cores, the oracle's is a sequential sum).
+    step = []
+    for it, (rows, cbg, codes_g, A_g, R_g) in enumerate(trace):
+        ref_cb = O.pq_fit(rows, m, k, iters, st_s[0], st_s[1])["codebooks"]
+        ref_codes = O.pq_encode(O.EUCLIDEAN, rows, ref_cb).astype(np.uint8)
+        rec = ref_cb[np.arange(m)[None, :], ref_codes.astype(np.int64)].reshape(ns, dim).astype(np.float64)
+        A_ref = (rec.T @ rows.astype(np.float64)).astype(F).astype(np.float64)
+        step.append({"outer": it + 1,
+                     "centroids_bit_identical": bool(np.array_equal(cbg.view(np.uint32), ref_cb.view(np.uint32))),
+                     "code_mismatch_rate": float(np.mean(codes_g != ref_codes)),
+                     "cross_cov_rel_diff": _rel_l2(A_g, A_ref),
+                     "rotation_max_abs_diff_f32": float(np.abs(R_g - O.procrustes(A_ref).astype(F)).max())})
+    par["stepwise_from_the_rows_the_gpu_trained_on"] = step
+    # (2) The algorithm's own sensitivity: the oracle against itself when every input value moves by
+    # at most one unit in the last place (a random half of them up, the other half down) — Lloyd
+    # iterations amplify such differences, a row that changes its cluster moves two centroids.
+    rng = np.random.default_rng(11)
+    up = rng.random(xs.shape) < 0.5
+    xp = np.where(up, np.nextafter(xs, F(np.inf)), np.nextafter(xs, F(-np.inf))).astype(F)
     for it in (1, 3, 5):
         a = O.opq_fit(O.EUCLIDEAN, xs, m, k, iters, it, st_s[0], st_s[1])
         b = O.opq_fit(O.EUCLIDEAN, xp, m, k, iters, it, st_s[0], st_s[1])
         ca = O.opq_encode(O.EUCLIDEAN, xs, a["rotation"], a["codebooks"])
         cb_ = O.opq_encode(O.EUCLIDEAN, xs, b["rotation"], b["codebooks"])
-        par[f"outer_{it}"]["oracle_vs_oracle_one_ulp_in_one_input"] = {
+        par[f"outer_{it}"]["oracle_vs_oracle_inputs_moved_one_ulp"] = {
             "centroid_rel_l2": _rel_l2(b["codebooks"], a["codebooks"]),
             "code_mismatch_rate": float(np.mean(ca != cb_))}
     par["sample"] = (f"first {ns} rows, own index streams (seed 3); oracle = vqo_opq_fit (host Jacobi SVD), "

@@ -281,13 +281,25 @@ int32_t vq_rotate(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t 
                   float *d_y);
 
 /* h_A[a*dim + b] = sum_i d_y[i][a] * d_x[i][b], both n x dim compact — the matrix A = Y X^T of
- * src/opq.rs:172-179, accumulated in f64 in a fixed order.  dim <= 128.  Synchronises. */
+ * src/opq.rs:172-179, accumulated in f64 in a fixed order (f64 matrix instructions when dim is a
+ * multiple of 16).  dim <= 4096.  Synchronises. */
 int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n, int32_t dim, double *h_A);
 
 /* h_R = V U^T for h_A = U S V^T (both dim x dim, row-major, host memory): the rotation update of
- * src/opq.rs:180-183, by a one-sided Jacobi SVD in f64 on the device.  dim even, 2 <= dim <= 128.
- * Synchronises. */
+ * src/opq.rs:180-183.  dim <= 4096, any parity.  V U^T is the orthogonal polar factor of A^T, unique
+ * for a non-singular A, and is computed
+ *   - for dim <= 512 by Newton-Schulz steps in f64 on the matrix cores; when they have not
+ *     converged within their step limit (A singular, condition number above about 1e6, or
+ *     non-finite), and for larger dim,
+ *   - by a one-sided Jacobi SVD in f64: on the device for even dim <= 128, otherwise the same
+ *     routine in host code of this library (the reference runs its SVD on the host as well);
+ *     directions a singular A leaves open are completed to an orthonormal basis.
+ * The result is a tolerance quantity (the reference's nalgebra SVD is not restated): both ways
+ * agree to about 1e-10 for condition numbers up to 1e6.  Synchronises. */
 int32_t vq_procrustes_rotation(vq_ctx *ctx, const double *h_A, int32_t dim, double *h_R);
+/* 0 (default): as above; 1: the SVD only.  The switch exists for measurement and tests.  No
+ * counterpart in the reference. */
+int32_t vq_ctx_set_procrustes_path(vq_ctx *ctx, int32_t path);
 
 /* ---- tree-structured VQ (src/tsvq.rs) ------------------------------------------------------ */
 

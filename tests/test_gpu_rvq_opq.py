@@ -162,6 +162,51 @@ def test_procrustes_rotation_is_the_polar_factor(ctx, dim):
     assert np.array_equal(ctx.procrustes_rotation(np.zeros((dim, dim))), np.eye(dim))
 
 
+@pytest.mark.parametrize("dim", [2, 5, 16, 40, 128, 130, 200])
+@pytest.mark.parametrize("cond", [1.0, 50.0, 1e4, 1e6])
+def test_procrustes_rotation_newton_schulz_and_svd_agree(ctx, dim, cond):
+    """The two ways to R = V U^T (src/opq.rs:180-183) — Newton-Schulz steps to the polar factor of
+    A^T on the f64 matrix cores (the default) and the one-sided Jacobi SVD — on matrices of a given
+    condition number, against each other, against numpy's SVD and against the polar-factor
+    properties.  The polar factor moves by about eps * cond under rounding, whichever way it is
+    computed, so the tolerance follows cond."""
+    rng = np.random.default_rng(1000 * dim + int(np.log10(cond)))
+    U, _ = np.linalg.qr(rng.standard_normal((dim, dim)))
+    V, _ = np.linalg.qr(rng.standard_normal((dim, dim)))
+    sv = np.geomspace(1.0, 1.0 / cond, dim) * 37.0
+    A = (U * sv) @ V.T
+    tol = 1e-11 + 3e-15 * cond
+    ctx.set_procrustes_path(1)
+    R_svd = ctx.procrustes_rotation(A)
+    ctx.set_procrustes_path(0)
+    R = ctx.procrustes_rotation(A)
+    u, _, vt = np.linalg.svd(A)
+    assert np.abs(R - vt.T @ u.T).max() <= tol
+    assert np.abs(R - R_svd).max() <= tol
+    assert np.abs(R.T @ R - np.eye(dim)).max() <= 1e-11
+    P = R @ A
+    assert np.abs(P - P.T).max() <= 1e-9 * np.abs(A).max()
+    assert np.array_equal(R, ctx.procrustes_rotation(A))  # deterministic
+
+
+def test_procrustes_rotation_that_newton_schulz_cannot_take_falls_to_the_svd(ctx):
+    """Singular, nearly singular (condition number 1e13) and non-finite matrices leave the
+    Newton-Schulz steps without convergence; the SVD path answers, as it does when it is the only
+    path."""
+    rng = np.random.default_rng(5)
+    dim = 64
+    U, _ = np.linalg.qr(rng.standard_normal((dim, dim)))
+    V, _ = np.linalg.qr(rng.standard_normal((dim, dim)))
+    for sv in (np.geomspace(1.0, 1e-13, dim), np.r_[np.ones(dim - 3), np.zeros(3)]):
+        A = (U * sv) @ V.T
+        ctx.set_procrustes_path(1)
+        want = ctx.procrustes_rotation(A)
+        ctx.set_procrustes_path(0)
+        got = ctx.procrustes_rotation(A)
+        assert np.array_equal(got, want)
+        assert np.abs(got.T @ got - np.eye(dim)).max() <= 1e-10
+
+
 @pytest.mark.parametrize("dim,rank", [(4, 2), (16, 10), (64, 63), (128, 100), (7, 3), (130, 60)])
 def test_procrustes_rotation_of_a_singular_matrix_is_orthogonal(ctx, dim, rank):
     """Directions that A leaves open (zero singular values; an all-zero column such as a padded

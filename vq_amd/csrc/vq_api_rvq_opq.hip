@@ -4,11 +4,14 @@
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
+#include <cmath>
+#include <cstring>
 #include <vector>
 
 #include "ctx.hpp"
 #include "rvq_opq.hpp"
 #include "procrustes_host.hpp"
+#include "polar.hpp"
 
 using namespace vqh;
 
@@ -99,6 +102,93 @@ int32_t rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int
                                d_codebooks, (const CodeT *)d_codes, stages, (const uint8_t *)used, d_recon_f16);
     }
     VQ_HIP(ctx, hipGetLastError());
+    return VQ_OK;
+}
+
+}  // namespace
+
+namespace {
+
+// R = the orthogonal polar factor of A^T by Newton-Schulz steps (polar.hpp).  *done = false when the
+// iteration has not converged within its step limit (the caller then takes the SVD).
+int32_t polar_newton_schulz(vq_ctx *ctx, const double *h_A, int dim, double *h_R, bool *done) {
+    *done = false;
+    if (dim > vq::kPolarMaxDim) return VQ_OK;
+    const int P = (dim + 15) / 16 * 16;
+    const size_t total = (size_t)P * P;
+    // |A|_1 and |A|_inf: largest column and row sums of |a|
+    std::vector<double> colsum((size_t)dim, 0.0);
+    double norm_inf = 0.0;
+    for (int i = 0; i < dim; ++i) {
+        double r = 0.0;
+        for (int j = 0; j < dim; ++j) {
+            const double v = std::fabs(h_A[(size_t)i * dim + j]);
+            r += v;
+            colsum[j] += v;
+        }
+        norm_inf = std::max(norm_inf, r);
+    }
+    double norm_1 = 0.0;
+    for (double c : colsum) norm_1 = std::max(norm_1, c);
+    double fro = 0.0;
+    for (size_t e = 0; e < (size_t)dim * dim; ++e) fro += h_A[e] * h_A[e];
+    // two upper bounds of the largest singular value; the smaller one
+    const double scale = std::min(std::sqrt(fro), std::sqrt(norm_1) * std::sqrt(norm_inf));
+    if (!(scale > 0.0) || !std::isfinite(scale)) return VQ_OK;  // zero or non-finite: the SVD path decides
+    std::vector<double> x0(total, 0.0);  // A^T / scale, zero-padded to P x P
+    const double inv = 1.0 / scale;
+    for (int i = 0; i < dim; ++i)
+        for (int j = 0; j < dim; ++j) x0[(size_t)j * P + i] = h_A[(size_t)i * dim + j] * inv;
+    VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(double) * total));
+    VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * total));
+    VQ_TRY(ensure(ctx, ctx->tmp_f, 1024));
+    double *X[2] = {(double *)ctx->tmp_a.p, (double *)ctx->tmp_b.p};
+    unsigned long long *errs = (unsigned long long *)ctx->tmp_f.p;  // kPolarMaxSteps of them, then the flags
+    int *fin = (int *)(errs + vq::kPolarMaxSteps);
+    static_assert(sizeof(unsigned long long) * vq::kPolarMaxSteps + sizeof(int) * (vq::kPolarMaxSteps + 2) <= 1024,
+                  "step tables");
+    hipStream_t st = ctx->stream;
+    VQ_HIP(ctx, hipMemsetAsync(ctx->tmp_f.p, 0, 1024, st));
+    VQ_HIP(ctx, hipMemcpyAsync(X[0], x0.data(), sizeof(double) * total, hipMemcpyHostToDevice, st));
+    const unsigned strips = (unsigned)(P / 16), waves = strips < 8u ? strips : 8u;
+    const size_t lds = sizeof(double) * 16 * (size_t)P;
+    if (lds > 48 * 1024)
+        VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(vq::k_polar_step<0>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    unsigned long long h_errs[vq::kPolarMaxSteps];
+    int s = 0, last = -1;
+    double low = 1e-3;  // assumed lower bound of the singular values after the first (plain) step
+    while (s < vq::kPolarMaxSteps && last < 0) {
+        const int upto = std::min(vq::kPolarMaxSteps, s == 0 ? 16 : s + 6);
+        for (; s < upto; ++s) {
+            double rho = 1.0;
+            if (s > 0 && low < 0.9) {
+                rho = std::sqrt(3.0 / (1.0 + low + low * low));
+                low = rho * low * (3.0 - rho * rho * low * low) * 0.5;
+            }
+            if (P == 128)
+                hipLaunchKernelGGL(vq::k_polar_step<8>, dim3(strips), dim3(64 * waves), lds, st,
+                                   (const double *)X[s & 1], P, dim, s, rho, errs, fin, X[(s + 1) & 1]);
+            else
+                hipLaunchKernelGGL(vq::k_polar_step<0>, dim3(strips), dim3(64 * waves), lds, st,
+                                   (const double *)X[s & 1], P, dim, s, rho, errs, fin, X[(s + 1) & 1]);
+        }
+        VQ_HIP(ctx, hipGetLastError());
+        VQ_HIP(ctx, hipMemcpyAsync(h_errs, errs, sizeof(unsigned long long) * s, hipMemcpyDeviceToHost, st));
+        VQ_HIP(ctx, hipStreamSynchronize(st));
+        for (int t = 0; t < s && last < 0; ++t) {
+            double e;
+            std::memcpy(&e, &h_errs[t], sizeof e);
+            if (e < vq::kPolarLastStepErr) last = t;
+        }
+    }
+    if (last < 0) return VQ_OK;
+    std::vector<double> r(total);
+    VQ_HIP(ctx, hipMemcpyAsync(r.data(), X[(last + 1) & 1], sizeof(double) * total, hipMemcpyDeviceToHost, st));
+    VQ_HIP(ctx, hipStreamSynchronize(st));
+    for (int i = 0; i < dim; ++i)
+        for (int j = 0; j < dim; ++j) h_R[(size_t)i * dim + j] = r[(size_t)i * P + j];
+    *done = true;
     return VQ_OK;
 }
 
@@ -261,18 +351,35 @@ int32_t vq_cross_cov(vq_ctx *ctx, const float *d_y, const float *d_x, int64_t n,
     return VQ_OK;
 }
 
+int32_t vq_ctx_set_procrustes_path(vq_ctx *ctx, int32_t path) {
+    if (!ctx || (path != 0 && path != 1)) return VQ_ERR_INVALID_ARG;
+    ctx->procrustes_path = path;
+    return VQ_OK;
+}
+
 int32_t vq_procrustes_rotation(vq_ctx *ctx, const double *h_A, int32_t dim, double *h_R) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
     if (!h_A || !h_R || dim < 1) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
     if (dim > 4096) return fail(ctx, VQ_ERR_UNSUPPORTED, "rotation update: dim %d above 4096", dim);
     const size_t total = (size_t)dim * dim;
-    // sizes the device kernel does not take: the same Jacobi SVD on the host (the reference runs
-    // its SVD on the host as well, src/opq.rs:180)
-    if (dim > vq::kJacobiMax || dim % 2 != 0) {
+    // First the polar factor by Newton-Schulz steps on the f64 matrix cores (any dim up to 512); a
+    // matrix that does not converge there — singular, badly conditioned, non-finite — takes the
+    // one-sided Jacobi SVD: on the device for even dim up to 128, else the same routine on the host
+    // (the reference runs its SVD on the host as well, src/opq.rs:180).
+    if (dim > vq::kPolarMaxDim && (dim > vq::kJacobiMax || dim % 2 != 0)) {
         vqh::procrustes_host(h_A, (size_t)dim, h_R);
         return VQ_OK;
     }
     VQ_HIP(ctx, hipSetDevice(ctx->device));
+    if (ctx->procrustes_path == 0) {
+        bool done = false;
+        VQ_TRY(polar_newton_schulz(ctx, h_A, dim, h_R, &done));
+        if (done) return VQ_OK;
+    }
+    if (dim > vq::kJacobiMax || dim % 2 != 0) {
+        vqh::procrustes_host(h_A, (size_t)dim, h_R);
+        return VQ_OK;
+    }
     const int half = dim / 2;
     VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(double) * total));
     VQ_TRY(ensure(ctx, ctx->tmp_b, sizeof(double) * total));
