@@ -367,7 +367,8 @@ def run_c5(ctx, log):
         out[f"descend_{name}_ms"] = round(ms, 4)
         gbs = bytes_row * n / (ms * 1e-3) / 1e9
         out[f"descend_{name}_roofline"] = {
-            "kernel": "k_tsvq_descend_reg", "bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+            "kernel": "k_tsvq_descend_w (one inner product per node, the two distances where it cannot decide)"
+                      if metric == vq_amd.COSINE else "k_tsvq_descend_reg (two distances per node)", "bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
             "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
             "algorithmic_bytes": "4*D + 1 = 513 per row"}
     tree.free()

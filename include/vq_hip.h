@@ -324,6 +324,16 @@ int32_t vq_tree_download(const vq_tree *tree, float *h_centroids, int32_t *h_lef
  * leaf reached; `<=` goes left, single children are followed.  Asynchronous. */
 int32_t vq_tsvq_descend(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld,
                         const vq_tree *tree, int32_t *d_leaf);
+/* How vq_tsvq_descend decides a node under cosine, squared Euclidean and Euclidean distance when
+ * the row fits in registers (dim a multiple of 32 up to 128):
+ *   0 (default)  by the sign of one inner product with a vector of the node (the difference of the
+ *                children's normalised centroids, or of the centroids with a norm term), whenever
+ *                its value clears a proven bound on every rounding error of the reference's two
+ *                sums; otherwise, for that row, by those two sums
+ *   1            by the two sums always
+ * Both give the reference's leaves bit for bit; the switch exists for measurement and tests.
+ * Manhattan always takes the two sums.  No counterpart in the reference. */
+int32_t vq_ctx_set_tsvq_descend_path(vq_ctx *ctx, int32_t path);
 /* d_out[i] = f16(centroid of leaf d_leaf[i]) (src/tsvq.rs:241-248), n x dim.  Asynchronous. */
 int32_t vq_tsvq_decode_f16(vq_ctx *ctx, const vq_tree *tree, const int32_t *d_leaf, int64_t n,
                            uint16_t *d_out);

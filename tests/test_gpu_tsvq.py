@@ -171,3 +171,82 @@ def test_variance_paths_agree_with_the_oracle_on_edge_data(ctx, kind, n, dim, de
             assert_same_tree(ctx.tsvq_build(dx, n, dim, dim, depth).download(), want_tree)
     finally:
         ctx.set_tsvq_variance_path(0)
+
+
+def _hand_tree(ctx, cen, depth):
+    """A complete binary tree of the given depth over the rows of cen (breadth-first ids)."""
+    nn = 2 ** (depth + 1) - 1
+    assert len(cen) == nn
+    left = np.array([2 * i + 1 if 2 * i + 2 < nn else -1 for i in range(nn)], np.int32)
+    right = np.array([2 * i + 2 if 2 * i + 2 < nn else -1 for i in range(nn)], np.int32)
+    return ctx.tree_create(cen, left, right), dict(centroids=cen, left=left, right=right)
+
+
+@pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN, O.COSINE])
+@pytest.mark.parametrize("dim", [32, 64, 128])
+@pytest.mark.parametrize("kind", ["ties", "near_ties", "scales", "zero_norms", "non_finite", "far_offset",
+                                  "equal_children"])
+def test_descent_by_one_inner_product_agrees_with_the_two_distances(ctx, metric, dim, kind):
+    """The default descent decides a node by the sign of one inner product when its value clears a
+    bound on every rounding error of the reference's two sums, else by those sums.  Both paths
+    against the oracle on data made to sit on the boundary: rows equidistant from both children
+    (exactly, and to within a few units in the last place of the sums), magnitudes from 1e-20 to
+    1e18 (outside the range the bound is proven for), zero rows and zero centroids (the cosine's own
+    rule), NaN and infinities, children that only differ far from the origin, identical children."""
+    rng = np.random.default_rng([dim, metric, len(kind)])
+    depth = 4
+    nn = 2 ** (depth + 1) - 1
+    cen = rng.standard_normal((nn, dim)).astype(F)
+    n = 3000
+    q = rng.standard_normal((n, dim)).astype(F)
+    if kind == "ties":
+        cen = np.round(cen * 2).astype(F)
+        q = np.round(q * 2).astype(F)
+        # rows on the bisector of the root's children: the mean of the two plus a vector orthogonal to their difference
+        d = (cen[1] - cen[2]).astype(np.float64)
+        for i in range(0, n, 3):
+            v = np.round(rng.standard_normal(dim) * 2)
+            j = int(np.argmax(np.abs(d)))
+            v[j] = 0.0
+            q[i] = ((cen[1] + cen[2]) / 2 + v).astype(F)
+    elif kind == "near_ties":
+        mid = ((cen[1].astype(np.float64) + cen[2]) / 2)
+        d = (cen[1] - cen[2]).astype(np.float64)
+        for i in range(n):
+            v = rng.standard_normal(dim)
+            v -= d * (v @ d) / (d @ d)  # orthogonal to the difference: equidistant in exact arithmetic
+            row = (mid + v + d * rng.uniform(-3e-7, 3e-7)).astype(F)
+            q[i] = row if metric != O.COSINE else (v + rng.uniform(-3e-7, 3e-7) * (cen[1] / np.linalg.norm(cen[1])
+                                                                            - cen[2] / np.linalg.norm(cen[2]))).astype(F)
+    elif kind == "scales":
+        q = (q * np.exp(rng.uniform(np.log(1e-20), np.log(1e18), (n, 1)))).astype(F)
+        cen = (cen * np.exp(rng.uniform(np.log(1e-18), np.log(1e16), (nn, 1)))).astype(F)
+    elif kind == "zero_norms":
+        q[::5] = 0.0
+        cen[[1, 4, 9, 20]] = 0.0
+        q[1::7, : dim // 2] = 0.0
+    elif kind == "non_finite":
+        q[::11, 3] = np.nan
+        q[5::13, 7] = np.inf
+        q[6::17, 2] = -np.inf
+        cen[6, 1] = np.nan
+        cen[11, 0] = np.inf
+    elif kind == "far_offset":
+        cen = (1000.0 + cen * 1e-3).astype(F)
+        q = (1000.0 + q * 1e-3).astype(F)
+    else:
+        cen[2] = cen[1]
+        cen[8] = cen[7]
+    tree, otree = _hand_tree(ctx, cen, depth)
+    with np.errstate(all="ignore"):
+        want = O.tsvq_descend(metric, q, otree)
+    dq = ctx.to_device(q)
+    dleaf = ctx.empty(n, np.int32)
+    try:
+        for path in (0, 1):
+            ctx.set_tsvq_descend_path(path)
+            ctx.tsvq_descend(metric, dq, n, dim, tree, dleaf)
+            got = dleaf.download()
+            assert np.array_equal(got, want), (path, int((got != want).sum()))
+    finally:
+        ctx.set_tsvq_descend_path(0)

@@ -30,6 +30,7 @@ SYMBOLS = {
     "vq_ctx_set_tsvq_variance_path": (_i32, [_vp, _i32]),
     "vq_calibrate": (_i32, [_vp, _i32, C.POINTER(C.c_double)]),
     "vq_ctx_set_procrustes_path": (_i32, [_vp, _i32]),
+    "vq_ctx_set_tsvq_descend_path": (_i32, [_vp, _i32]),
     "vq_calibrate_overlap": (_i32, [_vp, _i32, C.POINTER(C.c_double), C.POINTER(C.c_uint32)]),
     "vq_ctx_last_recheck_count": (_i32, [_vp, C.POINTER(C.c_uint32)]),
     "vq_ctx_last_recheck_split": (_i32, [_vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
@@ -360,6 +361,10 @@ class Context:
         A = np.empty((dim, dim), np.float64)
         self._check(_lib.vq_cross_cov(self._h, d_y.ptr, d_x.ptr, n, dim, A.ctypes.data))
         return A
+
+    def set_tsvq_descend_path(self, path):
+        """0: one inner product per node where it decides (default); 1: two distances per node always."""
+        self._check(_lib.vq_ctx_set_tsvq_descend_path(self._h, path))
 
     def set_procrustes_path(self, path):
         """0: Newton-Schulz polar factor first, the SVD when it does not converge (default); 1: SVD only."""

@@ -1386,6 +1386,235 @@ __global__ void __launch_bounds__(512) k_tsvq_descend_reg(const float *__restric
     }  // batches
 }
 
+// ---- descent decided by one inner product per node, exact where that cannot decide ---------------
+// Cosine: the reference goes left iff dl <= dr with dl = 1 - (x.cl) / (|x| |cl|) (src/tsvq.rs:167-171,
+// src/distances.rs:141-151), which in exact arithmetic is the sign of x.w, w = cl / |cl| - cr / |cr|.
+// Squared Euclidean and Euclidean: the sign of x.w + b, w = 2 (cl - cr), b = |cr|^2 - |cl|^2.  So a
+// node costs one vector of the table below instead of two centroids, and one chain of fused
+// multiply-adds instead of two of rounded products.  The rounded sums of the reference can only
+// differ from that sign when the value is small, and how small is bounded (u = 2^-24, D <= 128):
+//   cosine   each of dl, dr is within 133.2 u of its exact value (129 u for the sequential sum of D
+//            rounded products, relative to |x| |c|; 2 u for the product of the norms and the division;
+//            2 u for 1 - q), the computed x.w within 260.1 u |x| of the exact one (4 u |x| from the
+//            rounding of w, 256 u |x| from the sum): |x.w| > 600 u na decides, na the computed |x|.
+//   L2       each of the sums within 131 u of its exact value, relatively; the roots of two sums that
+//            differ by more than 6 u, relatively, differ after rounding; the computed x.w + b within
+//            131 u S of the exact one, S = 4 |x|^2 + 2 (|cl|^2 + |cr|^2) >= both sums together:
+//            |x.w + b| > 300 u (4 x2 + s) decides, x2 the computed |x|^2, s rounded up.
+// Everything else — near ties, norms outside [1e-15, 1e15] (zero norms have their own rule in the
+// reference, huge ones overflow), non-finite values (they fail the comparison) — is decided for that
+// lane by the two sums in the reference's order, read from global memory.  Manhattan has no such form
+// and keeps the two-centroid kernel.
+constexpr float kDescendCosMargin = 600.0f * 5.9604644775390625e-08f;
+constexpr float kDescendL2Margin = 300.0f * 5.9604644775390625e-08f;
+
+// Tables for the nodes below kTopNodes, one wave per node: w[node][DIM], and per node
+//   cosine: sc[node] = kDescendCosMargin, or +inf when a child's norm is outside [1e-15, 1e15]
+//   L2:     sc[2 node] = b, sc[2 node + 1] = kDescendL2Margin * s (+inf when s is not in [1e-30, 1e30])
+// Nodes without two children get zeros and +inf (they are never consulted).
+template <bool COS>
+static __global__ void __launch_bounds__(64) k_tsvq_wtable(const float *__restrict__ cen,
+                                                           const float *__restrict__ cnorm,
+                                                           const int *__restrict__ left,
+                                                           const int *__restrict__ right, int dim,
+                                                           float *__restrict__ w, float *__restrict__ sc) {
+    const int node = blockIdx.x, lane = threadIdx.x;
+    const int l = left[node], r = right[node];
+    const bool both = l >= 0 && r >= 0;
+    const float inf = __builtin_inff();
+    if (!both) {
+        for (int t = lane; t < dim; t += 64) w[(size_t)node * dim + t] = 0.0f;
+        if (lane == 0) {
+            if (COS) {
+                sc[node] = inf;
+            } else {
+                sc[2 * node] = 0.0f;
+                sc[2 * node + 1] = inf;
+            }
+        }
+        return;
+    }
+    const float *cl = cen + (size_t)l * dim, *cr = cen + (size_t)r * dim;
+    if constexpr (COS) {
+        const float nl = cnorm[l], nr = cnorm[r];
+        for (int t = lane; t < dim; t += 64) {
+            const float a = cl[t] / nl, b = cr[t] / nr;
+            w[(size_t)node * dim + t] = a - b;
+        }
+        const bool ok = nl >= 1e-15f && nl <= 1e15f && nr >= 1e-15f && nr <= 1e15f;
+        if (lane == 0) sc[node] = ok ? kDescendCosMargin : inf;
+    } else {
+        double sl = 0.0, sr = 0.0;
+        for (int t = lane; t < dim; t += 64) {
+            const float a = cl[t], b = cr[t];
+            w[(size_t)node * dim + t] = 2.0f * (a - b);
+            sl += (double)a * (double)a;
+            sr += (double)b * (double)b;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            sl += __shfl_xor(sl, off);
+            sr += __shfl_xor(sr, off);
+        }
+        if (lane == 0) {
+            const double s = 2.0 * (sl + sr);
+            const bool ok = s >= 1e-30 && s <= 1e30;  // false for NaN
+            sc[2 * node] = (float)(sr - sl);
+            sc[2 * node + 1] = ok ? (float)(s * 1.000001) * kDescendL2Margin : inf;
+        }
+    }
+}
+
+// The walk of k_tsvq_descend_reg with the decision above: the table of the first kTopNodes nodes
+// in LDS (same layout and stride), the row in registers.  METRIC: M_SQ, M_EUCLID or M_COS.
+template <int METRIC, int DIM>
+__global__ void __launch_bounds__(512) k_tsvq_descend_w(const float *__restrict__ x, int64_t n, int64_t ld,
+                                                       const float *__restrict__ cen,
+                                                       const float *__restrict__ cnorm,
+                                                       const int *__restrict__ left,
+                                                       const int *__restrict__ right, int n_nodes,
+                                                       const float *__restrict__ wtab,
+                                                       const float *__restrict__ sctab, int *__restrict__ leaf) {
+    constexpr int TS = DIM + 4;
+    constexpr bool COS = METRIC == M_COS;
+    __shared__ float top[kTopNodes * TS];
+    __shared__ int lds_child[2 * kTopNodes];
+    __shared__ float lds_sc[2 * kTopNodes];
+    const int lane = threadIdx.x & 63;
+    const int ntop = n_nodes < kTopNodes ? n_nodes : kTopNodes;
+    for (int e = threadIdx.x; e < ntop; e += 512) {
+        lds_child[2 * e] = left[e];
+        lds_child[2 * e + 1] = right[e];
+        if constexpr (COS) {
+            lds_sc[e] = sctab[e];
+        } else {
+            lds_sc[2 * e] = sctab[2 * e];
+            lds_sc[2 * e + 1] = sctab[2 * e + 1];
+        }
+    }
+    for (int e = threadIdx.x; e < ntop * (DIM / 4); e += 512) {
+        const int nd = e / (DIM / 4), pc = e % (DIM / 4);
+        *reinterpret_cast<float4 *>(&top[nd * TS + pc * 4]) =
+            *reinterpret_cast<const float4 *>(wtab + (size_t)nd * DIM + pc * 4);
+    }
+    __syncthreads();
+    const int64_t nbatch = (n + 63) / 64;
+    for (int64_t batch = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 6); batch < nbatch; batch += (int64_t)gridDim.x * 8) {
+        const int64_t row0 = batch * 64;  // one wave = 64 rows
+        float xr[DIM];
+        {
+            const int64_t row = row0 + lane < n ? row0 + lane : n - 1;  // past the end: the last row, not stored
+            const float4 *xp = reinterpret_cast<const float4 *>(x + row * ld);
+#pragma unroll
+            for (int q = 0; q < DIM / 4; ++q) {
+                const float4 v = xp[q];
+                xr[q * 4 + 0] = v.x;
+                xr[q * 4 + 1] = v.y;
+                xr[q * 4 + 2] = v.z;
+                xr[q * 4 + 3] = v.w;
+            }
+        }
+        // |x|^2 in the reference's order (the exact step's cosine needs it so; the margins take it as it is)
+        float sa = 0.0f;
+#pragma unroll
+        for (int t = 0; t < DIM; ++t) {
+            float p = xr[t] * xr[t];
+            sa = sa + p;
+        }
+        const float na = sqrtf(sa);
+        // the row's own share of the margin; a row whose norm is out of range (or not finite) never
+        // passes the test: +inf
+        const float inf = __builtin_inff();
+        float mrow;
+        if constexpr (COS)
+            mrow = (na >= 1e-15f && na <= 1e15f) ? na : inf;
+        else
+            mrow = (sa <= 1e30f) ? 4.0f * kDescendL2Margin * sa : inf;  // false for NaN
+        int node = 0;
+        bool active = row0 + lane < n;
+        while (__any(active)) {
+            int l = -1, r = -1;
+            if (active) {
+                if (node < ntop) {
+                    l = lds_child[2 * node];
+                    r = lds_child[2 * node + 1];
+                } else {
+                    l = left[node];
+                    r = right[node];
+                }
+            }
+            const bool both = l >= 0 && r >= 0;
+            bool undecided = both;
+            if (both && node < ntop) {
+                const float *pw = &top[node * TS];
+                float f0 = 0.0f, f1 = 0.0f, f2 = 0.0f, f3 = 0.0f;
+#pragma unroll
+                for (int q = 0; q < DIM / 4; ++q) {
+                    const float4 a = *reinterpret_cast<const float4 *>(pw + q * 4);
+                    f0 = __builtin_fmaf(xr[q * 4 + 0], a.x, f0);
+                    f1 = __builtin_fmaf(xr[q * 4 + 1], a.y, f1);
+                    f2 = __builtin_fmaf(xr[q * 4 + 2], a.z, f2);
+                    f3 = __builtin_fmaf(xr[q * 4 + 3], a.w, f3);
+                }
+                float f = (f0 + f1) + (f2 + f3);
+                float theta;
+                if constexpr (COS) {
+                    theta = lds_sc[node] * mrow;
+                } else {
+                    f += lds_sc[2 * node];
+                    theta = lds_sc[2 * node + 1] + mrow;
+                }
+                // (inf * 0 and inf - inf give NaN, which fails both tests)
+                if (f > theta) {
+                    node = l;
+                    undecided = false;
+                } else if (f < -theta) {
+                    node = r;
+                    undecided = false;
+                }
+            } else if (!both) {
+                if (l >= 0)
+                    node = l;
+                else if (r >= 0)
+                    node = r;
+                else
+                    active = false;
+            }
+            if (__any(undecided)) {
+                if (undecided) {
+                    // the two sums in the reference's order (src/tsvq.rs:167-171), from global memory
+                    const float4 *pl = reinterpret_cast<const float4 *>(cen + (size_t)l * DIM);
+                    const float4 *pr = reinterpret_cast<const float4 *>(cen + (size_t)r * DIM);
+                    float al = 0.0f, ar = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < DIM / 4; ++q) {
+                        const float4 a = pl[q], b = pr[q];
+                        tsvq_step<METRIC>(al, ar, xr[q * 4 + 0], a.x, b.x);
+                        tsvq_step<METRIC>(al, ar, xr[q * 4 + 1], a.y, b.y);
+                        tsvq_step<METRIC>(al, ar, xr[q * 4 + 2], a.z, b.z);
+                        tsvq_step<METRIC>(al, ar, xr[q * 4 + 3], a.w, b.w);
+                    }
+                    float dl, dr;
+                    if constexpr (COS) {
+                        float nl = cnorm[l], nr = cnorm[r];
+                        float ql = al / (na * nl), qr = ar / (na * nr);
+                        dl = (na == 0.0f || nl == 0.0f) ? 1.0f : 1.0f - ql;
+                        dr = (na == 0.0f || nr == 0.0f) ? 1.0f : 1.0f - qr;
+                    } else if constexpr (METRIC == M_EUCLID) {
+                        dl = sqrtf(al);
+                        dr = sqrtf(ar);
+                    } else {
+                        dl = al;
+                        dr = ar;
+                    }
+                    node = (dl <= dr) ? l : r;
+                }
+            }
+        }
+        if (row0 + lane < n) leaf[row0 + lane] = node;
+    }  // batches
+}
+
 // out[i][t] = f16(centroid[leaf[i]][t])   (src/tsvq.rs:242-248)
 static __global__ void __launch_bounds__(256) k_tsvq_decode_f16(const int *__restrict__ leaf, int64_t n, int dim,
                                                          const float *__restrict__ cen,

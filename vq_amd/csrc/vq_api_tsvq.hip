@@ -28,6 +28,9 @@ struct vq_tree {
     void *d_block = nullptr;  // one allocation: centroids, their norms, left and right children
     float *d_centroids = nullptr, *d_cnorm = nullptr;
     int32_t *d_left = nullptr, *d_right = nullptr;
+    // per node below vq::kTopNodes: the vector and the scalars that decide a descent step by one
+    // inner product (cosine; squared Euclidean and Euclidean)
+    float *d_wcos = nullptr, *d_sccos = nullptr, *d_wl2 = nullptr, *d_scl2 = nullptr;
 };
 
 namespace {
@@ -51,11 +54,18 @@ int32_t tree_to_device(vq_ctx *ctx, vq_tree *t, const float *d_means = nullptr) 
     size_t nn = (size_t)t->n_nodes, dim = (size_t)t->dim;
     auto pad = [](size_t z) { return (z + 255) & ~(size_t)255; };
     const size_t cen_b = pad(sizeof(float) * nn * dim), idx_b = pad(sizeof(int32_t) * nn);
-    VQ_HIP(ctx, hipMalloc(&t->d_block, cen_b + 3 * idx_b));
-    t->d_centroids = (float *)t->d_block;
-    t->d_cnorm = (float *)((char *)t->d_block + cen_b);
-    t->d_left = (int32_t *)((char *)t->d_block + cen_b + idx_b);
-    t->d_right = (int32_t *)((char *)t->d_block + cen_b + 2 * idx_b);
+    const size_t ntop = std::min<size_t>(nn, (size_t)vq::kTopNodes);
+    const size_t w_b = pad(sizeof(float) * ntop * dim), sc_b = pad(sizeof(float) * 2 * ntop);
+    VQ_HIP(ctx, hipMalloc(&t->d_block, cen_b + 3 * idx_b + 2 * w_b + 2 * sc_b));
+    char *base = (char *)t->d_block;
+    t->d_centroids = (float *)base;
+    t->d_cnorm = (float *)(base + cen_b);
+    t->d_left = (int32_t *)(base + cen_b + idx_b);
+    t->d_right = (int32_t *)(base + cen_b + 2 * idx_b);
+    t->d_wcos = (float *)(base + cen_b + 3 * idx_b);
+    t->d_wl2 = (float *)(base + cen_b + 3 * idx_b + w_b);
+    t->d_sccos = (float *)(base + cen_b + 3 * idx_b + 2 * w_b);
+    t->d_scl2 = (float *)(base + cen_b + 3 * idx_b + 2 * w_b + sc_b);
     hipStream_t st = ctx->stream;
     if (d_means)
         VQ_HIP(ctx, hipMemcpyAsync(t->d_centroids, d_means, sizeof(float) * nn * dim, hipMemcpyDeviceToDevice, st));
@@ -66,6 +76,10 @@ int32_t tree_to_device(vq_ctx *ctx, vq_tree *t, const float *d_means = nullptr) 
     VQ_HIP(ctx, hipMemcpyAsync(t->d_right, t->h_right.data(), sizeof(int32_t) * nn, hipMemcpyHostToDevice, st));
     hipLaunchKernelGGL(vq::k_centroid_norms, dim3(cdiv((int64_t)nn, 256)), dim3(256), 0, st, t->d_centroids,
                        (int64_t)nn, (int)dim, t->d_cnorm);
+    hipLaunchKernelGGL(vq::k_tsvq_wtable<true>, dim3((unsigned)ntop), dim3(64), 0, st, t->d_centroids, t->d_cnorm,
+                       t->d_left, t->d_right, (int)dim, t->d_wcos, t->d_sccos);
+    hipLaunchKernelGGL(vq::k_tsvq_wtable<false>, dim3((unsigned)ntop), dim3(64), 0, st, t->d_centroids, t->d_cnorm,
+                       t->d_left, t->d_right, (int)dim, t->d_wl2, t->d_scl2);
     VQ_HIP(ctx, hipGetLastError());
     VQ_HIP(ctx, hipStreamSynchronize(st));
     return VQ_OK;
@@ -507,6 +521,12 @@ int32_t vq_tree_download(const vq_tree *tree, float *h_centroids, int32_t *h_lef
     return VQ_OK;
 }
 
+int32_t vq_ctx_set_tsvq_descend_path(vq_ctx *ctx, int32_t path) {
+    if (!ctx || (path != 0 && path != 1)) return VQ_ERR_INVALID_ARG;
+    ctx->tsvq_descend_path = path;
+    return VQ_OK;
+}
+
 int32_t vq_tsvq_descend(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld,
                         const vq_tree *tree, int32_t *d_leaf) {
     if (!ctx || !tree) return VQ_ERR_INVALID_ARG;
@@ -521,6 +541,31 @@ int32_t vq_tsvq_descend(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n
         int cus = 0;
         VQ_HIP(ctx, hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device));
         dim3 g(std::min<unsigned>(cdiv(n, 512), (unsigned)std::max(cus, 1))), b(512);
+        // cosine and (squared) Euclidean: a step decided by one inner product with the node's vector,
+        // the two sums of the reference only where that cannot decide
+        if (ctx->tsvq_descend_path == 0 && metric != VQ_MANHATTAN && metric >= VQ_SQEUCLIDEAN && metric <= VQ_COSINE) {
+            const bool cosine = metric == VQ_COSINE;
+            const float *wt = cosine ? tree->d_wcos : tree->d_wl2, *sc = cosine ? tree->d_sccos : tree->d_scl2;
+#define DESC_W(M, D)                                                                                   \
+    hipLaunchKernelGGL((vq::k_tsvq_descend_w<M, D>), g, b, 0, ctx->stream, d_x, n, ld, tree->d_centroids, \
+                       tree->d_cnorm, tree->d_left, tree->d_right, (int)tree->h_left.size(), wt, sc, d_leaf)
+#define DESC_WDIM(M)                                                                                   \
+    switch (tree->dim) {                                                                               \
+    case 32: DESC_W(M, 32); break;                                                                     \
+    case 64: DESC_W(M, 64); break;                                                                     \
+    case 96: DESC_W(M, 96); break;                                                                     \
+    default: DESC_W(M, 128); break;                                                                    \
+    }
+            switch (metric) {
+            case VQ_SQEUCLIDEAN: DESC_WDIM(vq::M_SQ); break;
+            case VQ_EUCLIDEAN: DESC_WDIM(vq::M_EUCLID); break;
+            default: DESC_WDIM(vq::M_COS); break;
+            }
+#undef DESC_WDIM
+#undef DESC_W
+            VQ_HIP(ctx, hipGetLastError());
+            return VQ_OK;
+        }
 #define DESC_REG(M, D)                                                                                \
     hipLaunchKernelGGL((vq::k_tsvq_descend_reg<M, D>), g, b, 0, ctx->stream, d_x, n, ld,              \
                        tree->d_centroids, tree->d_cnorm, tree->d_left, tree->d_right, (int)tree->h_left.size(),    \
