@@ -209,19 +209,25 @@ int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int6
 int32_t vq_assign_u16(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                       int32_t sub_dim, int32_t k, const float *d_codebooks, uint16_t *d_codes);
 
-/* vq_assign for callers that cannot allocate device memory (code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
- * arguments, same codes, bit for bit; the call makes no hipMalloc / hipFree and never grows the
- * context's workspace.  The tables of the matrix-core kernel (8-float column blocks under
- * squared-L2 / Euclidean) and the centroid norms (cosine) live in one fixed array of 1.2 MB of
+/* vq_assign for callers that cannot allocate device memory (tight serving loops, harnesses that
+ * forbid hipMalloc, code that must not call an allocator between two points).  No counterpart in the
+ * reference.  Same arguments, same codes, bit for bit; the call makes no hipMalloc / hipFree and
+ * never grows the context's workspace.  The tables of the matrix-core kernel (8-float column blocks
+ * under squared-L2 / Euclidean) and the centroid norms (cosine) live in one fixed array of 1.2 MB of
  * device memory that the library holds on every GPU it runs on until the process ends.
- *   limit: m <= 1024 and m * (k rounded up to a multiple of 64) <= 16384 (e.g. m = 64, k = 256);
- *          beyond it VQ_ERR_UNSUPPORTED, and nothing is launched.
+ *   limit (for the shapes that use the array: cosine, and 8-float column blocks under squared-L2 /
+ *          Euclidean on the default assignment path): m <= 1024 and m * (k rounded up to a multiple
+ *          of 64) <= 16384 (e.g. m = 64, k = 256); beyond it VQ_ERR_UNSUPPORTED, and nothing is
+ *          launched.  Other shapes (Manhattan, other widths) need no scratch and have no such limit.
  *   wider column blocks under squared-L2 / Euclidean take the vector-ALU kernel (the matrix-core
  *   kernel for them keeps lists that grow with n).
- * Every context on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
- * contexts, two threads) race on it; a call leaves nothing the next one depends on.
- * Asynchronous. */
+ * This is the one exception to "distinct contexts are independent": a GPU has ONE such array, and
+ * calls that use it must not overlap in time on that GPU.  Calls of one context follow each other on
+ * its stream.  A call from another context is accepted once everything on the stream of the context
+ * that used the array last has finished, and returns VQ_ERR_UNSUPPORTED before (its kernels would
+ * overwrite tables that kernels in flight still read).  A call leaves nothing the next one depends on.
+ * The call has not been exercised under HIP graph capture (it sets a function attribute on its
+ * first use of a kernel).  Asynchronous. */
 int32_t vq_assign_noalloc(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                           int32_t sub_dim, int32_t k, const float *d_codebooks, uint8_t *d_codes);
 

@@ -234,6 +234,9 @@ def test_host_classes_under_ubsan():
     import sys
     if os.environ.get("VQ_HOST_LIB"):
         pytest.skip("already the sanitizer run")
+    if not os.environ.get("VQ_SANITIZERS_ON_GPU"):
+        pytest.skip("a sanitizer runtime inside a process that drives the GPU: only with VQ_SANITIZERS_ON_GPU=1 "
+                    "(the host mirror runs under the sanitizers without a GPU in tests/test_host_sanitized.py)")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     lib = os.path.join(root, "vq_amd", "libvqhost_ubsan.so")
     assert os.path.exists(lib), "build it with `python -m vq_amd.build`"
@@ -254,6 +257,9 @@ def test_host_classes_under_asan():
     import sys
     if os.environ.get("VQ_HOST_LIB"):
         pytest.skip("already the sanitizer run")
+    if not os.environ.get("VQ_SANITIZERS_ON_GPU"):
+        pytest.skip("a sanitizer runtime inside a process that drives the GPU: only with VQ_SANITIZERS_ON_GPU=1 "
+                    "(the host mirror runs under the sanitizers without a GPU in tests/test_host_sanitized.py)")
     from tests.test_oracle_sanitized import asan_env
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     lib = os.path.join(root, "vq_amd", "libvqhost_asan.so")

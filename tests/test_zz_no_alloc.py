@@ -110,3 +110,52 @@ def test_noalloc_on_a_fresh_context_first(ctx):
         assert c2.last_recheck_count() >= 0
     finally:
         c2.close()
+
+
+def test_noalloc_from_a_second_context_is_refused_while_the_first_is_running(ctx):
+    """One scratch array per GPU: a call from another context while the stream of the context that
+    used the array last is still busy is refused (VQ_ERR_UNSUPPORTED) instead of racing on the
+    tables; once that stream has drained the other context may use the array."""
+    import vq_amd
+    n = 2_000_000
+    x1, cb1 = _case(51, n, 16, 8, 256)
+    x2, cb2 = _case(52, 3000, 8, 8, 64)
+    dx1, dcb1 = ctx.to_device(x1), ctx.to_device(cb1)
+    g1 = ctx.empty((n, 16), np.uint8)
+    c2 = vq_amd.Context(0)
+    try:
+        dx2, dcb2 = c2.to_device(x2), c2.to_device(cb2)
+        g2 = c2.empty((3000, 8), np.uint8)
+        ctx.sync()
+        for _ in range(4):  # about a millisecond of kernels on the first context's stream
+            ctx.assign_noalloc(1, dx1, n, 128, 16, 8, 256, dcb1, g1)
+        with pytest.raises(vq_amd.VqError) as e:
+            c2.assign_noalloc(1, dx2, 3000, 64, 8, 8, 64, dcb2, g2)
+        assert e.value.code == vq_amd._ffi.ERR_UNSUPPORTED and "another context" in str(e.value)
+        # a shape that does not use the array is not concerned
+        xm, cbm = _case(53, 500, 2, 5, 9)
+        gm = c2.empty((500, 2), np.uint8)
+        c2.assign_noalloc(3, c2.to_device(xm), 500, 10, 2, 5, 9, c2.to_device(cbm), gm)
+        assert np.array_equal(gm.download(), O.pq_encode(3, xm, cbm).astype(np.uint8))
+        ctx.sync()
+        c2.assign_noalloc(1, dx2, 3000, 64, 8, 8, 64, dcb2, g2)
+        assert np.array_equal(g2.download(), O.pq_encode(1, x2, cb2).astype(np.uint8))
+        # and back: the first context again, after the second one's stream has drained
+        c2.sync()
+        ctx.assign_noalloc(1, dx1, n, 128, 16, 8, 256, dcb1, g1)
+        w1 = ctx.empty((n, 16), np.uint8)
+        ctx.assign(1, dx1, n, 128, 16, 8, 256, dcb1, w1)
+        assert np.array_equal(g1.download(), w1.download())
+    finally:
+        c2.close()
+
+
+def test_noalloc_limit_only_binds_the_shapes_that_use_the_scratch(ctx):
+    """Manhattan, and squared-L2 on a width without a matrix-core kernel, keep nothing in the fixed
+    array: a shape far beyond its size goes through."""
+    x, cb = _case(61, 300, 128, 6, 256)   # 128 x 256 cells: twice what the array holds
+    dx, dcb = ctx.to_device(x), ctx.to_device(cb)
+    for metric in (0, 3):
+        out = ctx.empty((300, 128), np.uint8)
+        ctx.assign_noalloc(metric, dx, 300, 768, 128, 6, 256, dcb, out)
+        assert np.array_equal(out.download(), O.pq_encode(metric, x, cb).astype(np.uint8))

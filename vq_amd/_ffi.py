@@ -180,6 +180,12 @@ class Context:
 
     def close(self):
         if self._h:
+            if self._pinned:
+                # arrays handed out by host_empty() view this memory: after close() they dangle
+                import warnings
+                warnings.warn(f"Context.close(): {len(self._pinned)} page-locked array(s) from host_empty() were "
+                              "not released with host_free(); their memory is freed now and the arrays "
+                              "must not be used any more", ResourceWarning, stacklevel=2)
             for p in list(self._pinned.values()):
                 _lib.vq_host_free(self._h, p)
             self._pinned.clear()
@@ -205,8 +211,10 @@ class Context:
         return DeviceArray(self, host.shape, host.dtype).upload(host)
 
     def host_empty(self, shape, dtype):
-        """A numpy array over page-locked host memory (vq_host_alloc); release it with
-        host_free(array) once no view of it is in use."""
+        """A numpy array over page-locked host memory (vq_host_alloc).  The array does not own the
+        memory: release it with host_free(array) once no view of it is in use, and before the
+        context is closed — close() frees what is left (with a ResourceWarning), after which the
+        array and every view of it point at freed memory."""
         dtype = np.dtype(dtype)
         shape = tuple(int(s) for s in np.atleast_1d(shape))
         nbytes = int(np.prod(shape)) * dtype.itemsize

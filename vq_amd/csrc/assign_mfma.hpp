@@ -865,24 +865,10 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     float4 xf0 = row_piece(piece(second));  // and the one after it
     float4 xf1 = row_piece(piece(second) + 4);
     float x2 = 0.0f;
-    // A stage is 16 dimensions: with the high and low parts of the centroid operand (ah, al) and of
-    // the row operand (xh, xl), three matrix instructions per tile of 32 centroids,
-    //   ah . xh + al . xh + ah . xl,
-    // every contraction slot of each in use; one barrier per 3 NB matrix instructions of a wave.
-    const int total16 = npair * pair16;
-    for (int st = 0; st < npair; ++st) {
-        const int cur = st & 1;
-        const bool more = st + 1 < npair;
-        // the A operands of the next stage: into registers now, into LDS at the end of this stage
-        u32x4 pre[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint32_t i = (uint32_t)((st + 1) * pair16) + threadIdx.x + 256u * (uint32_t)q;
-            const uint32_t ic = i < (uint32_t)total16 ? i : (uint32_t)total16 - 1u;
-            pre[q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(ag) + 16u * ic);
-        }
-        // operands of this stage from the row piece fetched one stage ago
-        float xv[8] = {xn0.x, xn0.y, xn0.z, xn0.w, xn1.x, xn1.y, xn1.z, xn1.w};
+    // The row operands of a stage: this half's 8 dimensions relative to the centre, their share of
+    // ||x - mu||^2, and their high and low bf16 parts.
+    auto split = [&](int st, const float4 &p0, const float4 &p1, u32x4 &bh, u32x4 &bl) {
+        float xv[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
         if (shifted) {
             const float4 m0 = *reinterpret_cast<const float4 *>(lds_mu + piece(st));
             const float4 m1 = *reinterpret_cast<const float4 *>(lds_mu + piece(st) + 4);
@@ -909,15 +895,40 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
             hp[u] = bf16_pack2(xv[2 * u], xv[2 * u + 1]);
             lp[u] = bf16_pack2(xv[2 * u] - __uint_as_float(hp[u] << 16), xv[2 * u + 1] - __uint_as_float(hp[u] & 0xffff0000u));
         }
-        const u32x4 bh = u32x4{hp[0], hp[1], hp[2], hp[3]}, bl = u32x4{lp[0], lp[1], lp[2], lp[3]};
-        // fetch the row two stages ahead
-        const int nx = st + 2 < npair ? st + 2 : npair - 1;
-        xn0 = xf0;
-        xn1 = xf1;
+        bh = u32x4{hp[0], hp[1], hp[2], hp[3]};
+        bl = u32x4{lp[0], lp[1], lp[2], lp[3]};
+    };
+    // A stage is 16 dimensions: with the high and low parts of the centroid operand (ah, al) and of
+    // the row operand (xh, xl), three matrix instructions per tile of 32 centroids,
+    //   ah . xh + al . xh + ah . xl,
+    // every contraction slot of each in use; one barrier per 3 NB matrix instructions of a wave.
+    // The row operands of stage st + 1 are made while the matrix instructions of stage st run: a
+    // matrix instruction holds back the vector instructions of the other waves of its SIMD, but
+    // independent vector instructions of its own wave issue in its shadow.
+    const int total16 = npair * pair16;
+    u32x4 bh, bl;
+    split(0, xn0, xn1, bh, bl);
+    xn0 = xf0;
+    xn1 = xf1;
+    {
+        const int nx = 2 < npair ? 2 : npair - 1;
         xf0 = row_piece(piece(nx));
         xf1 = row_piece(piece(nx) + 4);
+    }
+    for (int st = 0; st < npair; ++st) {
+        const int cur = st & 1;
+        const bool more = st + 1 < npair;
+        // the A operands of the next stage: into registers now, into LDS at the end of this stage
+        u32x4 pre[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t i = (uint32_t)((st + 1) * pair16) + threadIdx.x + 256u * (uint32_t)q;
+            const uint32_t ic = i < (uint32_t)total16 ? i : (uint32_t)total16 - 1u;
+            pre[q] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(ag) + 16u * ic);
+        }
         // The stage's centroid operands are read from LDS four tiles (one group) at a time.
         constexpr int NG = (NB + 3) / 4;  // groups of four centroid tiles
+        u32x4 nbh = bh, nbl = bl;
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
             u32x4 ah[4], al[4];
@@ -933,6 +944,15 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
                 if (4 * g + c < nb)
                     acc[4 * g + c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                         __builtin_bit_cast(bf16x8, ah[c]), __builtin_bit_cast(bf16x8, bh), acc[4 * g + c], 0, 0, 0);
+            if (g == 0 && more) {
+                // next stage's row operands, behind the first matrix instructions of this stage
+                split(st + 1, xn0, xn1, nbh, nbl);
+                const int nx = st + 3 < npair ? st + 3 : npair - 1;
+                xn0 = xf0;
+                xn1 = xf1;
+                xf0 = row_piece(piece(nx));
+                xf1 = row_piece(piece(nx) + 4);
+            }
 #pragma unroll
             for (int c = 0; c < 4; ++c)
                 if (4 * g + c < nb)
@@ -944,6 +964,8 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
                     acc[4 * g + c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                         __builtin_bit_cast(bf16x8, ah[c]), __builtin_bit_cast(bf16x8, bl), acc[4 * g + c], 0, 0, 0);
         }
+        bh = nbh;
+        bl = nbl;
         if (more) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {

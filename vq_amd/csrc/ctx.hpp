@@ -43,6 +43,8 @@ struct vq_ctx {
     DevBuf mfma_tab, mfma_list, mfma_stat;  // tables, re-check list and counters of the matrix-core assignment
     int recheck_src = 0;         // where the last pass counted its undecided pairs: 1 mfma_stat, 2 mfma_list, 3 the fixed scratch
     int assign_path = 0;         // 0 = matrix cores where a kernel exists, 1 = vector ALU only
+    int compute_units = 0;       // of the context's GPU (0: not asked for yet)
+    int decode_lds_set[4] = {0, 0, 0, 0};  // dynamic-LDS limit already granted to the four resident decode kernels
     int tsvq_descend_path = 0;   // 0 = one inner product per node where it decides (cosine, L2), 1 = two distances per node always
     int procrustes_path = 0;     // 0 = Newton-Schulz polar factor first, SVD when it does not converge; 1 = SVD only
     // vq_assign_noalloc: the device address of this GPU's file-scope scratch array, and whether a

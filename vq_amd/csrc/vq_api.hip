@@ -12,6 +12,7 @@
 #include <cstring>
 #include <string>
 #include <atomic>
+#include <mutex>
 #include <thread>
 #include <vector>
 
@@ -53,6 +54,12 @@ constexpr size_t kNoAllocNormOff = kNoAllocStatOff + sizeof(uint32_t) * vq::kSta
 constexpr size_t kNoAllocBytes = kNoAllocNormOff + sizeof(float) * kNoAllocMaxCells;  // centroid norms (cosine)
 static_assert(kNoAllocStatOff % 256 == 0 && kNoAllocNormOff % 256 == 0, "scratch areas stay 256-byte aligned");
 static __device__ __align__(256) unsigned char scratch[kNoAllocBytes];
+// The context whose calls used a GPU's array last (null: none yet).  Another context may take the
+// array over once everything on that context's stream has finished; until then its calls are
+// refused, because their kernels would overwrite tables that kernels in flight still read.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+vq_ctx *g_scratch_owner[kMaxDevices];
 
 // ---- assignment dispatch -------------------------------------------------------------------
 
@@ -455,13 +462,21 @@ int32_t launch_decode_resident(vq_ctx *ctx, const CodeT *d_codes, int64_t n, int
     if (sd % (F16 ? 8 : 4) != 0 || lds > 128 * 1024 || n * m < (1 << 16)) return VQ_OK;
     if ((reinterpret_cast<uintptr_t>(d_codebooks) | reinterpret_cast<uintptr_t>(d_out)) & 15) return VQ_OK;
     auto kern = k_decode_resident<F16, CodeT>;
-    VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)lds));
-    hipDeviceProp_t prop;
-    VQ_HIP(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    // the kernel's LDS limit and the number of compute units: asked for once per context and kernel
+    const int slot = (F16 ? 2 : 0) + (sizeof(CodeT) == 2 ? 1 : 0);
+    if ((size_t)ctx->decode_lds_set[slot] < lds) {
+        VQ_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));
+        ctx->decode_lds_set[slot] = 128 * 1024;
+    }
+    if (ctx->compute_units == 0) {
+        int cus = 0;
+        VQ_HIP(ctx, hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device));
+        ctx->compute_units = cus > 0 ? cus : 1;
+    }
     const int64_t pieces = (int64_t)n * m * (F16 ? sd / 8 : sd / 4);
     const unsigned per_cu = lds <= 64 * 1024 ? 2u : 1u;
-    const unsigned wgs = (unsigned)std::min<int64_t>((int64_t)prop.multiProcessorCount * per_cu, cdiv(pieces, 4096));
+    const unsigned wgs = (unsigned)std::min<int64_t>((int64_t)ctx->compute_units * per_cu, cdiv(pieces, 4096));
     hipLaunchKernelGGL(kern, dim3(wgs), dim3(1024), lds, ctx->stream, d_codes, n, m, sd, k, d_codebooks,
                        (vq::u32x4 *)d_out);
     VQ_HIP(ctx, hipGetLastError());
@@ -616,6 +631,10 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
         if (ctx->h2d_event[i]) (void)hipEventDestroy(ctx->h2d_event[i]);
     }
     prof_collect(ctx);
+    if (ctx->device >= 0 && ctx->device < kMaxDevices) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (g_scratch_owner[ctx->device] == ctx) g_scratch_owner[ctx->device] = nullptr;
+    }
     for (hipEvent_t e : ctx->prof_pool) (void)hipEventDestroy(e);
     (void)hipEventDestroy(ctx->ev0);
     (void)hipEventDestroy(ctx->ev1);
@@ -694,10 +713,22 @@ static int32_t h2d_staged(vq_ctx *ctx, char *d_dst, const char *h_src, size_t by
             staged[c].fetch_add(1, std::memory_order_release);
         }
     };
+    // (the staging buffers may still be the source of an earlier call's uploads that failed half way)
+    VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
     std::vector<std::thread> pool;
-    for (int t = 1; t < T; ++t) pool.emplace_back(work, t);
+    std::thread first;
+    try {
+        for (int t = 1; t < T; ++t) pool.emplace_back(work, t);
+        first = std::thread(work, 0);
+    } catch (const std::exception &) {
+        // no threads to be had: let the ones that started run through, then one plain copy
+        stageable.store(nchunks + (size_t)NB, std::memory_order_release);
+        for (auto &th : pool) th.join();
+        VQ_HIP(ctx, hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->stream));
+        VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        return VQ_OK;
+    }
     hipError_t err = hipSuccess;
-    std::thread first(work, 0);
     for (size_t c = 0; c < nchunks; ++c) {
         while (staged[c].load(std::memory_order_acquire) < T) std::this_thread::yield();
         const size_t len = std::min(kChunk, bytes - c * kChunk);
@@ -711,6 +742,7 @@ static int32_t h2d_staged(vq_ctx *ctx, char *d_dst, const char *h_src, size_t by
     }
     first.join();
     for (auto &th : pool) th.join();
+    if (err != hipSuccess) (void)hipStreamSynchronize(ctx->stream);  // uploads already enqueued read the staging buffers
     VQ_HIP(ctx, err);
     VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
     return VQ_OK;
@@ -756,7 +788,17 @@ static int32_t d2h_staged(vq_ctx *ctx, char *h_dst, const char *d_src, size_t by
         }
     };
     std::vector<std::thread> pool;
-    for (int t = 0; t < T; ++t) pool.emplace_back(work, t);
+    try {
+        for (int t = 0; t < T; ++t) pool.emplace_back(work, t);
+    } catch (const std::exception &) {
+        // no threads to be had: the ones that started copy nothing that is not there yet (nothing
+        // has arrived), so they are let through and one plain copy does the work
+        arrived.store(nchunks, std::memory_order_release);
+        for (auto &th : pool) th.join();
+        VQ_HIP(ctx, hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+        VQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        return VQ_OK;
+    }
     hipError_t err = hipSuccess;
     size_t issued = 0;
     auto issue = [&]() {  // the download of chunk `issued` into its buffer
@@ -776,6 +818,7 @@ static int32_t d2h_staged(vq_ctx *ctx, char *h_dst, const char *d_src, size_t by
         }
     }
     for (auto &th : pool) th.join();
+    if (err != hipSuccess) (void)hipStreamSynchronize(ctx->stream);  // downloads already enqueued write the staging buffers
     VQ_HIP(ctx, err);
     return VQ_OK;
 }
@@ -1179,13 +1222,32 @@ int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int6
 int32_t vq_assign_noalloc(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                           int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
-    // the tables of the call must fit the fixed scratch: column blocks x centroids padded to 64
-    if (m > 0 && k > 0 && k <= vq::kMaxK) {
+    // Which shapes touch the fixed scratch: the matrix-core kernel of 8-float column blocks (its
+    // tables and counters) and the cosine kernels (the centroid norms).  Only they are bound by its
+    // size, and only they need the GPU's one array for themselves.
+    const bool uses_scratch =
+        metric == VQ_COSINE ||
+        ((metric == VQ_SQEUCLIDEAN || metric == VQ_EUCLIDEAN) && sd == 8 && ctx->assign_path == 0);
+    if (uses_scratch && m > 0 && k > 0 && k <= vq::kMaxK) {
+        // the tables of the call must fit: column blocks x centroids padded to 64
         const int64_t cells = (int64_t)m * 64 * ((k + 63) / 64);
         if (m > kNoAllocMaxM || cells > kNoAllocMaxCells)
             return fail(ctx, VQ_ERR_UNSUPPORTED,
                         "vq_assign_noalloc: m * k (k padded to 64) = %lld exceeds the fixed scratch of %d "
                         "(use vq_assign, which may allocate)", (long long)cells, kNoAllocMaxCells);
+        if (ctx->device < 0 || ctx->device >= kMaxDevices)
+            return fail(ctx, VQ_ERR_UNSUPPORTED, "vq_assign_noalloc: device %d", ctx->device);
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        vq_ctx *owner = g_scratch_owner[ctx->device];
+        if (owner && owner != ctx) {
+            const hipError_t busy = hipStreamQuery(owner->stream);
+            (void)hipGetLastError();
+            if (busy != hipSuccess)
+                return fail(ctx, VQ_ERR_UNSUPPORTED,
+                            "vq_assign_noalloc: the fixed scratch of GPU %d is in use by another context whose "
+                            "stream has not finished (calls that use it must not overlap on one GPU)", ctx->device);
+        }
+        g_scratch_owner[ctx->device] = ctx;
     }
     // no timing spans (their events are created on demand) and no workspace growth inside the call
     const bool prof = ctx->prof_on;
