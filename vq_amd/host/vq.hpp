@@ -618,6 +618,9 @@ public:
                                   streams->reseed.data() + st * (size_t)streams->n_reseed, streams->n_reseed, cb,
                                   nullptr, nullptr));  // rvq.rs:107
             ++produced;
+            // The residuals are a local of the reference's fit (rvq.rs:103) and nothing follows the
+            // last stage: its residual update and norm test (111-141) cannot be observed and are left out.
+            if (st + 1 == stages) break;
             if (k < 2)  // rvq.rs:113-115
                 dcodes.narrow().upload(zeros.data(), n);
             else
