@@ -377,6 +377,26 @@ def run_c5(ctx, log):
             "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
             "algorithmic_bytes": "4*D + 1 = 513 per row"}
     tree.free()
+    # The configuration's wording ("2-means with 10 LBG iterations per node") as the explicit,
+    # non-default mode: the split is lbg_quantize with k = 2 instead of the reference's median split.
+    lbg_iters = 10
+    draws = np.random.default_rng(5).integers(0, 2 ** 32, (2 ** depth - 1, 2 + lbg_iters), dtype=np.uint64).astype(np.uint32)
+    ctx.tsvq_build_kmeans(dx, n, dim, dim, depth, lbg_iters, draws).free()
+    kb = []
+    for i in range(3):
+        ctx.sync()
+        t0 = time.perf_counter()
+        tk = ctx.tsvq_build_kmeans(dx, n, dim, dim, depth, lbg_iters, draws)
+        kb.append(round((time.perf_counter() - t0) * 1e3, 3))
+        if i < 2:
+            tk.free()
+    out["kmeans_mode"] = {"note": "explicit non-default mode (vq_tsvq_build_kmeans): 2-means split with 10 LBG iterations "
+                                  "per node; not the reference's behaviour (src/tsvq.rs:87-123 splits at the median)",
+                          "tsvq_build_ms": min(kb), "tsvq_build_ms_each": kb, "nodes": tk.n_nodes}
+    f = lambda: ctx.tsvq_descend(vq_amd.COSINE, dx, n, dim, tk, dleaf)
+    f()
+    out["kmeans_mode"]["descend_cosine_ms"] = round(_timed(ctx, f, 5), 4)
+    tk.free()
     dx.free()
     dleaf.free()
 
@@ -409,8 +429,26 @@ def run_c5(ctx, log):
         mse_g, mse_r = O.mse_f16(xs, dre.download()), O.mse_f16(xs, rec_r)
         par[name] = {"leaf_mismatch_rate": float(np.mean(dl.download() != leaf_r)),
                      "mse_gpu": mse_g, "mse_ref": mse_r, "mse_rel_diff": _rel(mse_g, mse_r)}
-    out["parity"] = par
     tg.free()
+    # the 2-means mode on a smaller sample (the oracle runs ten LBG iterations per node)
+    nk = 50_000
+    xk = np.ascontiguousarray(xs[:nk])
+    t0 = time.perf_counter()
+    rk, _ = _bfs_order(O.tsvq_fit_kmeans(xk, depth, lbg_iters, draws))
+    cpu_k = time.perf_counter() - t0
+    dxk = ctx.to_device(xk)
+    gk_tree = ctx.tsvq_build_kmeans(dxk, nk, dim, dim, depth, lbg_iters, draws)
+    gk = gk_tree.download()
+    same = gk["n_nodes"] == rk["n_nodes"]
+    par["kmeans_mode"] = {
+        "sample": f"first {nk} rows; oracle build {cpu_k:.1f} s",
+        "tree_structure_equal": bool(same and np.array_equal(gk["left"], rk["left"]) and np.array_equal(gk["right"], rk["right"])),
+        "centroid_rel_l2": _rel_l2(gk["centroids"], rk["centroids"]) if same else None,
+        "centroids_bit_identical": bool(same and np.array_equal(gk["centroids"].view(np.uint32),
+                                                                rk["centroids"].view(np.uint32)))}
+    gk_tree.free()
+    dxk.free()
+    out["parity"] = par
     for b in (dxs, dl, dre):
         b.free()
     log(f"[configs] c5 done: build {out['tsvq_build_ms']} ms, descent {out['descend_cosine_ms']} / "

@@ -317,6 +317,25 @@ typedef struct vq_tree vq_tree;
  * numbered breadth-first (root 0, left before right).  Synchronises. */
 int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim,
                       int32_t max_depth, vq_tree **out);
+/* The same tree built with 2-means splits instead of the median split — NOT the reference's
+ * behaviour (src/tsvq.rs:87-123 splits at the median of the maximum-variance coordinate, which
+ * vq_tsvq_build reproduces); an explicit mode for callers that want a k-means tree (2-means with a
+ * number of LBG iterations per node).  Everything else of TSVQNode::fit stays: the node's centroid
+ * is the mean of its rows (76), a node is a leaf at depth 0 or with at most one row (78), a child
+ * exists only if non-empty and strictly smaller than its parent (128, 135).  The split is
+ * lbg_quantize (src/utils.rs:32-109) with k = 2 on the node's rows in row order; a row goes left
+ * when the first of the two returned centroids is its nearest (squared L2, strict '<').
+ *   h_draws          (2^max_depth - 1) * draws_per_node values: the node at position h of the
+ *                    complete binary tree (root 1, children 2h and 2h + 1) owns
+ *                    h_draws[(h - 1) * draws_per_node ..].  With c rows in the node, its initial
+ *                    centroids are its rows number d[0] % c and d[1] % (c - 1), plus one if that is
+ *                    not below the first (k distinct rows, utils.rs:54), and the i-th empty
+ *                    cluster it meets takes its row number d[2 + i] % c (utils.rs:100).
+ *   draws_per_node   >= 2 + lbg_iters (one cluster can be empty per iteration)
+ * max_depth <= 20.  Synchronises. */
+int32_t vq_tsvq_build_kmeans(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim,
+                             int32_t max_depth, int32_t lbg_iters, const uint32_t *h_draws,
+                             int32_t draws_per_node, vq_tree **out);
 /* A tree from host arrays (children must have larger indices than their parent; -1 = none). */
 int32_t vq_tree_create(vq_ctx *ctx, int32_t n_nodes, int32_t dim, const float *h_centroids,
                        const int32_t *h_left, const int32_t *h_right, vq_tree **out);

@@ -245,6 +245,29 @@ def tsvq_fit(x, max_depth):
                 split_dim=sdim[:nn], split_val=sval[:nn], count=cnt[:nn])
 
 
+def tsvq_fit_kmeans(x, max_depth, lbg_iters, draws):
+    """TSVQ with 2-means splits (vqo_tsvq_fit_kmeans): draws is ((2**max_depth - 1), per_node) uint32."""
+    x = _f32(x)
+    n, dim = x.shape
+    draws = _u32(draws).reshape(2 ** max_depth - 1 if max_depth > 0 else 0, -1) if max_depth > 0 \
+        else np.zeros((0, 2 + lbg_iters), np.uint32)
+    max_nodes = min(2 * n, 2 ** (max_depth + 1)) + 1
+    cen = np.zeros((max_nodes, dim), np.float32)
+    left = np.zeros(max_nodes, np.int32)
+    right = np.zeros(max_nodes, np.int32)
+    cnt = np.zeros(max_nodes, np.int64)
+    fn = lib().vqo_tsvq_fit_kmeans
+    fn.restype = C.c_int64
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int64, C.c_int64,
+                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+    d = np.ascontiguousarray(draws if draws.size else np.zeros((1, 2 + lbg_iters), np.uint32))
+    nn = fn(x.ctypes.data, n, dim, max_depth, lbg_iters, d.ctypes.data, d.shape[1], max_nodes, cen.ctypes.data,
+            left.ctypes.data, right.ctypes.data, cnt.ctypes.data)
+    assert nn > 0, nn
+    return dict(n_nodes=nn, centroids=cen[:nn], left=left[:nn], right=right[:nn],
+                split_dim=np.full(nn, -1, np.int32), split_val=np.zeros(nn, np.float32), count=cnt[:nn])
+
+
 def tsvq_descend(metric, x, tree):
     x = _f32(x)
     n, dim = x.shape

@@ -590,6 +590,93 @@ int64_t vqo_tsvq_fit(const float *x, int64_t n, int64_t dim, int64_t max_depth, 
     return B.n_nodes;
 }
 
+/* ---- TSVQ with 2-means splits (NOT the reference's behaviour) ------------------
+ * The reference splits a node at the median of its maximum-variance coordinate
+ * (src/tsvq.rs:87-123, vqo_tsvq_fit above).  This variant keeps everything else of
+ * TSVQNode::fit (node centroid = mean_vector of its rows, 76; leaf at depth 0 or with
+ * <= 1 row, 78; a child only if non-empty and strictly smaller, 128,135) and replaces
+ * the split by lbg_quantize (src/utils.rs:32-109, vqo_lbg above) with k = 2 on the
+ * node's rows, taken in row order: a row goes left when the first of the two returned
+ * centroids is its nearest (squared L2, strict '<': ties to the first).
+ * Randomness crosses as draws: node at heap position h (root 1, children 2h, 2h+1)
+ * owns draws[(h-1)*per_node ..]; with c rows, the initial rows are the node's rows
+ * number i0 = d[0] % c and i1 = d[1] % (c-1), plus one if i1 >= i0 (distinct), and the
+ * i-th empty cluster takes row number d[2+i] % c.  Built from parts that are pinned
+ * (vqo_lbg, vqo_mean_rows); the composition has no counterpart to compare with. */
+typedef struct {
+    tsvq_build_t b;
+    int64_t lbg_iters;
+    const uint32_t *draws;
+    int64_t per_node;
+    int64_t max_heap;
+} tsvq_km_t;
+
+static int32_t tsvq_km_node(tsvq_km_t *K, const uint32_t *rows, int64_t cnt, int64_t depth, int64_t heap) {
+    tsvq_build_t *B = &K->b;
+    if (B->n_nodes >= B->max_nodes) {
+        B->overflow = 1;
+        return -1;
+    }
+    int32_t me = (int32_t)B->n_nodes++;
+    int64_t dim = B->dim;
+    float *cen = B->centroids + (int64_t)me * dim;
+    vqo_mean_rows(B->x, dim, 0, dim, rows, cnt, cen);
+    B->left[me] = -1;
+    B->right[me] = -1;
+    if (B->node_count) B->node_count[me] = cnt;
+    if (depth == 0 || cnt <= 1) return me;
+    const uint32_t *d = K->draws + (heap - 1) * K->per_node;
+    float *xn = (float *)malloc(sizeof(float) * (size_t)cnt * (size_t)dim);
+    for (int64_t p = 0; p < cnt; ++p)
+        memcpy(xn + p * dim, B->x + (int64_t)rows[p] * dim, sizeof(float) * (size_t)dim);
+    uint32_t init[2];
+    init[0] = (uint32_t)(d[0] % (uint64_t)cnt);
+    init[1] = (uint32_t)(d[1] % (uint64_t)(cnt - 1));
+    if (init[1] >= init[0]) init[1] += 1;
+    int64_t nres = K->per_node - 2;
+    uint32_t *reseed = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)(nres > 0 ? nres : 1));
+    for (int64_t i = 0; i < nres; ++i) reseed[i] = (uint32_t)(d[2 + i] % (uint64_t)cnt);
+    float *c2 = (float *)malloc(sizeof(float) * 2 * (size_t)dim);
+    int rc = vqo_lbg(xn, cnt, dim, 0, dim, 2, K->lbg_iters, init, reseed, nres, c2, NULL, NULL, NULL);
+    uint32_t *l = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)cnt);
+    uint32_t *r = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)cnt);
+    int64_t nl = 0, nr = 0;
+    for (int64_t p = 0; p < cnt; ++p) {
+        if (argmin_d2(xn + p * dim, c2, 2, dim) == 0)
+            l[nl++] = rows[p];
+        else
+            r[nr++] = rows[p];
+    }
+    free(xn);
+    free(reseed);
+    free(c2);
+    if (rc != 0) B->overflow = 2; /* re-seed draws exhausted */
+    if (nl > 0 && nl < cnt) B->left[me] = tsvq_km_node(K, l, nl, depth - 1, 2 * heap);
+    if (nr > 0 && nr < cnt) B->right[me] = tsvq_km_node(K, r, nr, depth - 1, 2 * heap + 1);
+    free(l);
+    free(r);
+    return me;
+}
+
+/* Returns the number of nodes, -10 for empty input, -20 if max_nodes is too small,
+ * -21 if per_node < 2 + lbg_iters (a node can meet one empty cluster per iteration),
+ * -22 if the re-seed draws ran out.  draws: (2^max_depth - 1) * per_node values. */
+int64_t vqo_tsvq_fit_kmeans(const float *x, int64_t n, int64_t dim, int64_t max_depth, int64_t lbg_iters,
+                            const uint32_t *draws, int64_t per_node, int64_t max_nodes, float *centroids,
+                            int32_t *left, int32_t *right, int64_t *node_count) {
+    if (n == 0) return -10;
+    if (per_node < 2 + lbg_iters) return -21;
+    tsvq_km_t K = {{x, dim, centroids, left, right, NULL, NULL, node_count, max_nodes, 0, 0},
+                   lbg_iters, draws, per_node, 0};
+    uint32_t *rows = (uint32_t *)malloc(sizeof(uint32_t) * (size_t)n);
+    for (int64_t i = 0; i < n; ++i) rows[i] = (uint32_t)i;
+    tsvq_km_node(&K, rows, n, max_depth, 1);
+    free(rows);
+    if (K.b.overflow == 1) return -20;
+    if (K.b.overflow == 2) return -22;
+    return K.b.n_nodes;
+}
+
 /* TSVQNode::quantize_with_distance (src/tsvq.rs:162-181) for every row:
  * leaf[i] = node index of the leaf reached. */
 void vqo_tsvq_descend(int metric, const float *x, int64_t n, int64_t dim, const float *centroids,

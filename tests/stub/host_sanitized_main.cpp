@@ -123,6 +123,10 @@ int main() {
         auto t = TSVQ::create(rows, 3, Distance(Distance::CosineDistance));
         CHECK(t.quantize(rows[3]).len() == dim);
         CHECK(t.quantize_batch(rows).size() == n);
+        auto k = TSVQ::create_kmeans(rows, 3, 4, Distance(Distance::Euclidean), 11);
+        CHECK(k.quantize_batch(rows).size() == n);
+        std::vector<uint32_t> wrong(5, 0u);
+        CHECK(!message_of([&] { TSVQ::create_kmeans(rows, 3, 4, Distance(Distance::Euclidean), 11, &wrong); }).empty());
     }
     // the flat C entry points, as the Python binding drives them
     {

@@ -237,6 +237,12 @@ int32_t vq_tsvq_build(vq_ctx *, const float *x, int64_t n, int64_t ld, int32_t d
     *out = t;
     return VQ_OK;
 }
+int32_t vq_tsvq_build_kmeans(vq_ctx *c, const float *x, int64_t n, int64_t ld, int32_t dim, int32_t max_depth,
+                             int32_t lbg_iters, const uint32_t *draws, int32_t per_node, vq_tree **out) {
+    if (per_node < 2 + lbg_iters) return bad(c, VQ_ERR_INVALID_ARG, "Invalid parameter: draws");
+    if (max_depth > 0) touch(draws, (((size_t)1 << max_depth) - 1) * (size_t)per_node);
+    return vq_tsvq_build(c, x, n, ld, dim, max_depth, out);
+}
 int32_t vq_tree_free(vq_ctx *, vq_tree *t) {
     delete t;
     return VQ_OK;

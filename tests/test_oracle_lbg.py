@@ -360,3 +360,34 @@ def test_opq_rotation_is_orthogonal_and_quirk_is_kept():
     codes = O.opq_encode(O.EUCLIDEAN, x, r2["rotation"], r2["codebooks"])
     assert np.array_equal(codes, O.pq_encode(O.EUCLIDEAN, O.rotate(x, r2["rotation"]),
                                              r2["codebooks"]))
+
+
+def test_tsvq_kmeans_oracle_closed_forms():
+    """vqo_tsvq_fit_kmeans (2-means splits, not the reference's median split) on inputs whose answer
+    is known: two separated blobs split into the blobs, with exact means; identical rows cannot be
+    split (every row ties with the first centroid: the right side is empty, the node stays a leaf);
+    depth 0 is the mean of everything; the split only depends on the node's own draws."""
+    rng = np.random.default_rng(0)
+    n, dim = 400, 6
+    lab = rng.integers(0, 2, n).astype(bool)
+    x = (rng.standard_normal((n, dim)) * 0.1 + np.where(lab[:, None], 5.0, -5.0)).astype(np.float32)
+    draws = rng.integers(0, 2 ** 32, (1, 12), dtype=np.uint64).astype(np.uint32)
+    t = O.tsvq_fit_kmeans(x, 1, 10, draws)
+    assert t["n_nodes"] == 3 and sorted(t["count"][1:].tolist()) == sorted([int(lab.sum()), int((~lab).sum())])
+    for child in (1, 2):
+        members = lab if t["centroids"][child][0] > 0 else ~lab
+        acc = np.zeros(dim, np.float32)
+        for r in x[members]:
+            acc = acc + r
+        assert np.array_equal(t["centroids"][child], acc / np.float32(members.sum()))
+    same = np.tile(np.array([[1.5, -2.0, 3.0]], np.float32), (10, 1))
+    t = O.tsvq_fit_kmeans(same, 3, 10, rng.integers(0, 2 ** 32, (7, 12), dtype=np.uint64).astype(np.uint32))
+    assert t["n_nodes"] == 1 and np.array_equal(t["centroids"][0], same[0])
+    t0 = O.tsvq_fit_kmeans(x, 0, 10, np.zeros((0, 12), np.uint32))
+    assert t0["n_nodes"] == 1
+    # draws of other nodes do not matter: the root's split is the same under different draws for the children
+    d2 = rng.integers(0, 2 ** 32, (3, 12), dtype=np.uint64).astype(np.uint32)
+    d3 = d2.copy()
+    d3[1:] = rng.integers(0, 2 ** 32, (2, 12), dtype=np.uint64).astype(np.uint32)
+    a, b = O.tsvq_fit_kmeans(x, 2, 10, d2), O.tsvq_fit_kmeans(x, 2, 10, d3)
+    assert a["count"][1] == b["count"][1]

@@ -65,6 +65,7 @@ SYMBOLS = {
     "vq_rotate": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp, _vp]),
     "vq_cross_cov": (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
     "vq_tsvq_build": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, C.POINTER(_vp)]),
+    "vq_tsvq_build_kmeans": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _i32, C.POINTER(_vp)]),
     "vq_tree_create": (_i32, [_vp, _i32, _i32, _vp, _vp, _vp, C.POINTER(_vp)]),
     "vq_tree_free": (_i32, [_vp, _vp]),
     "vq_tree_info": (_i32, [_vp, C.POINTER(_i32), C.POINTER(_i32)]),
@@ -388,6 +389,16 @@ class Context:
     def tsvq_build(self, d_x, n, ld, dim, max_depth):
         h = _vp()
         self._check(_lib.vq_tsvq_build(self._h, d_x.ptr, n, ld, dim, max_depth, C.byref(h)))
+        return Tree(self, h)
+
+    def tsvq_build_kmeans(self, d_x, n, ld, dim, max_depth, lbg_iters, draws):
+        """The tree with 2-means splits (not the reference's median split).  draws: uint32 array of
+        shape (2**max_depth - 1, per_node), per_node >= 2 + lbg_iters."""
+        draws = np.ascontiguousarray(draws, np.uint32)
+        per_node = draws.shape[-1] if draws.ndim > 1 else int(draws.size)
+        h = _vp()
+        self._check(_lib.vq_tsvq_build_kmeans(self._h, d_x.ptr, n, ld, dim, max_depth, lbg_iters,
+                                              draws.ctypes.data if draws.size else None, per_node, C.byref(h)))
         return Tree(self, h)
 
     def tree_create(self, centroids, left, right):

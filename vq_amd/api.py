@@ -219,6 +219,19 @@ class TSVQ(_Quantizer):
         _check(_h.vqh_tsvq_new(_p(x), _i64(n), _i64(dim), _i64(max_depth), kind, C.c_double(p), C.byref(h)))
         return cls(h.value)
 
+    @classmethod
+    def new_kmeans(cls, training_data, max_depth, lbg_iters, distance, seed, draws=None):
+        """Not in the crate: the tree with 2-means splits (lbg_quantize with k = 2 per node) instead of
+        the median split.  draws (optional): (2**max_depth - 1, 2 + lbg_iters) uint32."""
+        x = _rows(training_data)
+        n, dim = x.shape
+        kind, p = _dist(distance)
+        d = None if draws is None else np.ascontiguousarray(draws, np.uint32)
+        h = _vp()
+        _check(_h.vqh_tsvq_new_kmeans(_p(x), _i64(n), _i64(dim), _i64(max_depth), _i64(lbg_iters), kind, C.c_double(p),
+                                      _u64(seed), _p(d), C.byref(h)))
+        return cls(h.value)
+
     def leaves(self, data):
         x = _rows(data)
         out = np.zeros(x.shape[0], np.int32)

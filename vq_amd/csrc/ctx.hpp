@@ -31,6 +31,7 @@ struct vq_ctx {
     DevBuf tsvq_level;           // TSVQ build: the level's uploaded tables and the leaf sums of its node means
     DevBuf tsvq_means;           // TSVQ build: the means of all nodes, read back once at the end
     DevBuf tsvq_scan;            // TSVQ build: workspace of the partition's prefix scan
+    DevBuf tsvq_km;              // TSVQ build with 2-means splits: centroids, part sums, flags, draws of a level
     void *tsvq_pin = nullptr;    // TSVQ build: page-locked staging of a level's tables and decisions
     size_t tsvq_pin_cap = 0;
     // vq_h2d from pageable memory: page-locked staging buffers and the events of their uploads

@@ -620,7 +620,7 @@ int32_t vq_ctx_destroy(vq_ctx *ctx) {
     if (ctx->side) (void)hipStreamSynchronize(ctx->side);
     DevBuf *bufs[] = {&ctx->flags, &ctx->tables, &ctx->hist, &ctx->perm, &ctx->leaf_desc,
                       &ctx->leaf_sum, &ctx->codes, &ctx->idx, &ctx->reseed, &ctx->cnorm,
-                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tsvq_split, &ctx->tsvq_level, &ctx->tsvq_means, &ctx->tsvq_scan, &ctx->tsvq_bsum, &ctx->tsvq_segmaps, &ctx->tsvq_gsum, &ctx->tsvq_guess, &ctx->tsvq_maps, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f,
+                      &ctx->seg, &ctx->part_sum, &ctx->mfma_tab, &ctx->mfma_list, &ctx->mfma_stat, &ctx->tsvq_sq, &ctx->tsvq_split, &ctx->tsvq_level, &ctx->tsvq_means, &ctx->tsvq_scan, &ctx->tsvq_km, &ctx->tsvq_bsum, &ctx->tsvq_segmaps, &ctx->tsvq_gsum, &ctx->tsvq_guess, &ctx->tsvq_maps, &ctx->tmp_a, &ctx->tmp_b, &ctx->tmp_c, &ctx->tmp_d, &ctx->tmp_e, &ctx->tmp_f,
                       &ctx->big_chunk, &ctx->big_win, &ctx->big_wind, &ctx->big_best, &ctx->big_fresh, &ctx->big_codes, &ctx->big_keys,
                       &ctx->big_sorted, &ctx->big_sort_tmp, &ctx->big_tables, &ctx->big_flags};
     for (DevBuf *b : bufs)

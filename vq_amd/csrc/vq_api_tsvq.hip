@@ -12,6 +12,7 @@
 #include "ctx.hpp"
 #include "assign_exact.hpp"
 #include "tsvq.hpp"
+#include "tsvq_kmeans.hpp"
 
 using namespace vqh;
 
@@ -46,6 +47,14 @@ int tree_depth(uint64_t count) {
 struct Seg {
     int32_t node;
     uint32_t lo, hi;
+    uint64_t heap = 1;  // position in the complete binary tree: root 1, children 2 h and 2 h + 1
+};
+
+// The 2-means split (vq_tsvq_build_kmeans): LBG iterations per node and the nodes' draws.
+struct KmOpts {
+    int32_t lbg_iters;
+    const uint32_t *h_draws;
+    int32_t per_node;
 };
 
 // d_means: the centroids where they already are on the device (the build's node means), else they
@@ -95,8 +104,28 @@ void tree_release(vq_tree *t) {
 
 extern "C" {
 
+static int32_t tsvq_build_impl(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, int32_t max_depth,
+                               const KmOpts *km, vq_tree **out);
+
 int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, int32_t max_depth,
                       vq_tree **out) {
+    return tsvq_build_impl(ctx, d_x, n, ld, dim, max_depth, nullptr, out);
+}
+
+int32_t vq_tsvq_build_kmeans(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, int32_t max_depth,
+                             int32_t lbg_iters, const uint32_t *h_draws, int32_t draws_per_node, vq_tree **out) {
+    if (!ctx || !out) return VQ_ERR_INVALID_ARG;
+    *out = nullptr;
+    if (max_depth > 20) return fail(ctx, VQ_ERR_UNSUPPORTED, "2-means tree: max_depth %d above 20", max_depth);
+    if (lbg_iters < 0 || draws_per_node < 2 + lbg_iters || (max_depth > 0 && !h_draws))
+        return fail(ctx, VQ_ERR_INVALID_ARG,
+                    "Invalid parameter: a node needs 2 + lbg_iters draws (two initial rows, one re-seed per iteration)");
+    KmOpts km{lbg_iters, h_draws, draws_per_node};
+    return tsvq_build_impl(ctx, d_x, n, ld, dim, max_depth, &km, out);
+}
+
+static int32_t tsvq_build_impl(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t dim, int32_t max_depth,
+                               const KmOpts *km, vq_tree **out) {
     if (!ctx || !out) return VQ_ERR_INVALID_ARG;
     *out = nullptr;
     if (n == 0) return fail(ctx, VQ_ERR_EMPTY_INPUT, "Empty input: at least one vector is required.");
@@ -136,7 +165,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     vq_tree *T = new vq_tree;
     T->device = ctx->device;
     T->dim = dim;
-    std::vector<Seg> level{{0, 0u, (uint32_t)n}};
+    std::vector<Seg> level{{0, 0u, (uint32_t)n, 1}};
     T->h_left.push_back(-1);
     T->h_right.push_back(-1);
     T->h_split_dim.push_back(-1);
@@ -150,6 +179,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         return rc;
     };
     int32_t rc = VQ_OK;
+    int km_err = 0;  // 2-means: a node ran out of re-seed draws
     struct LevelMeans {
         void *d;
         int32_t first_node;
@@ -158,6 +188,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
     std::vector<LevelMeans> level_means;  // device means of every level, read back after the last one
     std::vector<uint2> desc;
     std::vector<uint4> info;
+    std::vector<uint32_t> km_draws, km_first;  // 2-means: the splitting nodes' draws and first parts
     // The means of all nodes in one workspace buffer when the deepest possible tree stays small (nodes
     // are numbered level by level, so a level's means are one run of it); else an allocation per level.
     const uint64_t max_nodes = std::min<uint64_t>(2 * (uint64_t)n - 1, (2ull << std::min(max_depth, 40)) - 1);
@@ -308,6 +339,91 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         int *d_sdim = (int *)d_down;
         float *d_median = (float *)d_down + ns;
         uint32_t *d_nleft = (uint32_t *)d_down + 2 * (size_t)ns;
+        if (km) {
+            // ---- 2-means split: lbg_quantize with k = 2 on every splitting node's rows ----------
+            km_first.assign((size_t)ns + 1, 0u);
+            for (int i = 0; i < ns; ++i)
+                km_first[i + 1] = km_first[i] + (uint32_t)cdiv((int64_t)(range[i].y - range[i].x), vq::kKmPart);
+            const uint32_t parts = km_first[ns];
+            km_draws.resize((size_t)ns * km->per_node);
+            for (int i = 0; i < ns; ++i)
+                memcpy(km_draws.data() + (size_t)i * km->per_node,
+                       km->h_draws + (size_t)(level[split[i]].heap - 1) * km->per_node, sizeof(uint32_t) * km->per_node);
+            auto pad4 = [](size_t z) { return (z + 255) & ~(size_t)255; };
+            const size_t sz[6] = {sizeof(float) * 2 * (size_t)ns * dim, sizeof(uint32_t) * ((size_t)ns + 1),
+                                  sizeof(float) * 2 * (size_t)parts * dim, sizeof(uint32_t) * 2 * (size_t)parts,
+                                  sizeof(int) * (4 * (size_t)ns + 1), sizeof(uint32_t) * (size_t)ns * km->per_node};
+            size_t total = 0;
+            for (size_t z : sz) total += pad4(z);
+            {
+                const int32_t rc = ensure(ctx, ctx->tsvq_km, total);
+                if (rc != VQ_OK) {
+                    free_means();
+                    return cleanup_fail(rc);
+                }
+            }
+            char *at = (char *)ctx->tsvq_km.p;
+            vq::KmState S{};
+            S.perm = perm;
+            S.range = (const uint2 *)d_range;
+            S.per_node = km->per_node;
+            S.ns = ns;
+            S.cen = (float *)at;
+            at += pad4(sz[0]);
+            S.part_first = (uint32_t *)at;
+            at += pad4(sz[1]);
+            S.part_sum = (float *)at;
+            at += pad4(sz[2]);
+            S.part_cnt = (uint32_t *)at;
+            at += pad4(sz[3]);
+            int *fl = (int *)at;
+            at += pad4(sz[4]);
+            S.changed = fl;
+            S.done = fl + ns;
+            S.used = fl + 2 * (size_t)ns;
+            S.iters = fl + 3 * (size_t)ns;
+            S.err = fl + 4 * (size_t)ns;
+            uint32_t *d_draws = (uint32_t *)at;
+            S.draws = d_draws;
+            S.codes = (uint8_t *)vals;  // the split column's buffer is not used in this mode
+            SP_HIP(hipMemcpyAsync(S.part_first, km_first.data(), sz[1], hipMemcpyHostToDevice, st));
+            SP_HIP(hipMemcpyAsync(d_draws, km_draws.data(), sz[5], hipMemcpyHostToDevice, st));
+            SP_HIP(hipMemsetAsync(S.codes, 0, (size_t)n, st));  // assignments = vec![0; n], utils.rs:55
+            SP_HIP(hipMemsetAsync(S.err, 0, sizeof(int), st));
+            hipLaunchKernelGGL(vq::k_km_init, dim3(ns), dim3(256), 0, st, S, d_x, ld, dim);
+            const bool reg = dim % 32 == 0 && dim <= 128 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0;
+            auto assign = [&](bool lbg, uint32_t *fl_out) {
+                const dim3 grid(cdiv(n, 256)), block(256);
+#define KM_REG(D)                                                                                          \
+    if (lbg)                                                                                               \
+        hipLaunchKernelGGL((vq::k_km_assign_reg<true, D>), grid, block, 0, st, S, n, d_x, ld, fl_out);     \
+    else                                                                                                   \
+        hipLaunchKernelGGL((vq::k_km_assign_reg<false, D>), grid, block, 0, st, S, n, d_x, ld, fl_out)
+                if (reg) {
+                    switch (dim) {
+                    case 32: KM_REG(32); break;
+                    case 64: KM_REG(64); break;
+                    case 96: KM_REG(96); break;
+                    default: KM_REG(128); break;
+                    }
+                } else if (lbg) {
+                    hipLaunchKernelGGL(vq::k_km_assign<true>, grid, block, 0, st, S, n, d_x, ld, dim, fl_out);
+                } else {
+                    hipLaunchKernelGGL(vq::k_km_assign<false>, grid, block, 0, st, S, n, d_x, ld, dim, fl_out);
+                }
+#undef KM_REG
+            };
+            const unsigned sum_threads = dim <= 64 ? 64u : dim <= 128 ? 128u : 256u;
+            for (int it = 0; it < km->lbg_iters; ++it) {
+                assign(true, nullptr);
+                hipLaunchKernelGGL(vq::k_km_partsum, dim3(parts), dim3(sum_threads), 0, st, S, d_x, ld, dim);
+                hipLaunchKernelGGL(vq::k_km_update, dim3(ns), dim3(256), 0, st, S, d_x, ld, dim);
+            }
+            // rows whose nearest of the two final centroids is the first go left
+            assign(false, flags);
+            SP_HIP(hipGetLastError());
+            SP_HIP(hipMemcpyAsync(&km_err, S.err, sizeof(int), hipMemcpyDeviceToHost, st));
+        } else {
         // the means of the splitting nodes, compacted on the device
         hipLaunchKernelGGL(vq::k_gather_means, dim3(cdiv((int64_t)ns * dim, 256)), dim3(256), 0, st,
                            (const float *)d_means, (const int *)d_split, ns, dim, (float *)d_smeans);
@@ -400,6 +516,7 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         // stable partition by `<= median` (src/tsvq.rs:120-123)
         hipLaunchKernelGGL(vq::k_seg_flags, dim3(cdiv(n, 256)), dim3(256), 0, st, vals, n, (const uint2 *)d_range,
                            ns, (const float *)d_median, flags);
+        }  // median split
         size_t need = 0;
         SP_HIP(rocprim::exclusive_scan(nullptr, need, flags, scan, 0u, (size_t)n, rocprim::plus<uint32_t>(), st));
         {
@@ -420,26 +537,31 @@ int32_t vq_tsvq_build(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int3
         const float *median = (const float *)h_down + ns;
         const uint32_t *nleft = (const uint32_t *)h_down + 2 * (size_t)ns;
         std::swap(perm, perm2);
+        if (km && km_err) {
+            free_means();
+            return cleanup_fail(fail(ctx, VQ_ERR_RESEED_EXHAUSTED, "2-means tree: a node met more empty clusters than it has draws"));
+        }
 
         // ---- children (src/tsvq.rs:126-141) ---------------------------------------------------
         std::vector<Seg> next;
         for (int i = 0; i < ns; ++i) {
             const Seg &sg = level[split[i]];
             uint32_t cnt = sg.hi - sg.lo, nl = nleft[i], nr = cnt - nl;
-            T->h_split_dim[sg.node] = sdim[i];
-            T->h_split_val[sg.node] = median[i];
-            auto add_child = [&](uint32_t lo, uint32_t hi) {
+            T->h_split_dim[sg.node] = km ? -1 : sdim[i];
+            T->h_split_val[sg.node] = km ? 0.f : median[i];
+            const uint64_t heap = sg.heap;
+            auto add_child = [&](uint32_t lo, uint32_t hi, uint64_t child_heap) {
                 int32_t id = (int32_t)T->h_left.size();
                 T->h_left.push_back(-1);
                 T->h_right.push_back(-1);
                 T->h_split_dim.push_back(-1);
                 T->h_split_val.push_back(0.f);
                 T->h_count.push_back((int64_t)hi - lo);
-                next.push_back({id, lo, hi});
+                next.push_back({id, lo, hi, child_heap});
                 return id;
             };
-            if (nl > 0 && nl < cnt) T->h_left[sg.node] = add_child(sg.lo, sg.lo + nl);
-            if (nr > 0 && nr < cnt) T->h_right[sg.node] = add_child(sg.lo + nl, sg.hi);
+            if (nl > 0 && nl < cnt) T->h_left[sg.node] = add_child(sg.lo, sg.lo + nl, 2 * heap);
+            if (nr > 0 && nr < cnt) T->h_right[sg.node] = add_child(sg.lo + nl, sg.hi, 2 * heap + 1);
         }
         level.swap(next);
         --depth_left;

@@ -715,6 +715,44 @@ public:
         return t;
     }
 
+    // NOT in the crate: the same tree with 2-means splits (lbg_quantize with k = 2 and lbg_iters
+    // iterations on every node's rows) instead of the median split of src/tsvq.rs:87-123.  The node at
+    // position h of the complete binary tree (root 1) draws from a generator seeded with seed + h:
+    // two initial rows, one re-seed row per iteration; or the caller passes the draws themselves,
+    // (2^max_depth - 1) x (2 + lbg_iters) values.
+    static TSVQ create_kmeans(const Rows &training_data, size_t max_depth, size_t lbg_iters, Distance distance,
+                              uint64_t seed, const std::vector<uint32_t> *draws = nullptr,
+                              std::shared_ptr<Device> dev = Device::shared()) {
+        if (training_data.empty()) throw VqError::EmptyInput();
+        if (max_depth > 20) throw VqError::InvalidParameter("max_depth above 20 for a 2-means tree");
+        size_t dim = training_data.dim(), n = training_data.size();
+        training_data.expect_dim(dim);
+        const size_t per_node = 2 + lbg_iters, positions = ((size_t)1 << max_depth) - 1;
+        std::vector<uint32_t> own;
+        if (!draws) {
+            own.resize(positions * per_node);
+            for (size_t h = 1; h <= positions; ++h) {
+                uint64_t s = seed + h;
+                for (size_t i = 0; i < per_node; ++i) own[(h - 1) * per_node + i] = (uint32_t)IndexStreams::splitmix(s);
+            }
+            draws = &own;
+        } else if (draws->size() != positions * per_node) {
+            throw VqError::InvalidParameter("a 2-means tree needs (2^max_depth - 1) * (2 + lbg_iters) draws");
+        }
+        TSVQ t;
+        t.dev_ = dev;
+        t.distance = distance;
+        t.dim_ = dim;
+        DeviceBuffer<float> dx(dev, n * dim);
+        dx.upload(training_data.data(), dx.size());
+        vq_tree *tree = nullptr;
+        dev->check(vq_tsvq_build_kmeans(dev->ctx(), dx.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)max_depth,
+                                        (int32_t)lbg_iters, draws->data(), (int32_t)per_node, &tree));
+        std::shared_ptr<Device> keep = dev;
+        t.tree_ = std::shared_ptr<vq_tree>(tree, [keep](vq_tree *p) { vq_tree_free(keep->ctx(), p); });
+        return t;
+    }
+
     // src/tsvq.rs:231-249
     Vector<f16> quantize(const Vector<float> &vector) const {
         if (vector.len() != dim_) throw VqError::DimensionMismatch(dim_, vector.len());

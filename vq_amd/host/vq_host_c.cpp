@@ -131,6 +131,24 @@ int vqh_tsvq_new(const float *x, int64_t n, int64_t dim, int64_t max_depth, int 
     });
 }
 
+// the tree with 2-means splits (not in the crate); draws: nullable, (2^max_depth - 1) * (2 + lbg_iters) values
+int vqh_tsvq_new_kmeans(const float *x, int64_t n, int64_t dim, int64_t max_depth, int64_t lbg_iters, int distance,
+                        double p, uint64_t seed, const uint32_t *draws, void **out) {
+    return guarded([&] {
+        auto rows = rows_of(x, n, dim);
+        std::vector<uint32_t> d;
+        if (draws && max_depth <= 20)
+            d.assign(draws, draws + (((size_t)1 << max_depth) - 1) * (size_t)(2 + lbg_iters));
+        auto o = std::make_unique<Obj>();
+        o->kind = 4;
+        o->dim = dim;
+        o->tsvq = std::make_unique<vq::TSVQ>(vq::TSVQ::create_kmeans(
+            rows, (size_t)max_depth, (size_t)lbg_iters, vq::Distance((vq::Distance::Kind)distance, p), seed,
+            draws ? &d : nullptr));
+        *out = o.release();
+    });
+}
+
 // quantize(&Vector<f32>) of whichever quantizer obj holds; len is the vector's own length
 // *out_len (nullable) receives the length of the returned vector
 int vqh_quantize(void *obj, const float *v, int64_t len, uint16_t *out, int64_t *out_len) {
