@@ -3,7 +3,7 @@
 
 `bench.py` measures the headline PQ workload and then calls `other_configs()` of this module, so
 that its one JSON line also carries, for each of these, the times, the dominant kernel with its
-fraction of the bound that SURVEY-style accounting gives it, and the parity triple (code mismatch
+fraction of the peak of the unit that bounds it, and the parity triple (code mismatch
 rate, centroid relative L2, reconstruction-MSE relative difference) against the CPU oracle on a
 sample the oracle finishes in seconds:
 
@@ -12,9 +12,10 @@ sample the oracle finishes in seconds:
   c4  RVQ   1,000,000 x 256, 8 stages, k = 256, 10 LBG iterations, epsilon = 0   (src/bin/eval_rvq.rs)
   c5  TSVQ  1,000,000 x 128 unit rows, depth 8; cosine, then Manhattan descent  (src/bin/eval_tsvq.rs)
 
-    python bench_configs.py [c3] [c4] [c5]
+    python bench_configs.py [c3] [c4] [c5] [--no-parity]
 
-prints the same object alone.  Inputs are the seeded generators of vq_amd/synth.py.
+prints the same object alone; --no-parity leaves out the comparisons with the oracle, so that a
+profile of the command holds dispatches of the full-size workloads only.  Inputs are the seeded generators of vq_amd/synth.py.
 """
 import json
 import os
@@ -117,7 +118,7 @@ def opq_fit_device(ctx, dx, n, dim, m, k, iters, outer, streams, metric, bufs=No
     return R, bufs, snaps
 
 
-def run_c3(ctx, log, x=None, dx=None):
+def run_c3(ctx, log, x=None, dx=None, parity=True):
     import vq_amd
     from oracle import oracle as O
     from vq_amd import api
@@ -172,6 +173,8 @@ def run_c3(ctx, log, x=None, dx=None):
     del q
     for b in bufs.values():
         b.free()
+    if not parity:
+        return out
 
     # parity against the oracle after 1, 3 and 5 outer iterations, on the first rows of the same data
     ns = 20_000
@@ -262,7 +265,7 @@ def rvq_fit_device(ctx, dx, dres, dcb, dcodes, n, dim, stages, k, iters, init, r
         ctx.residual_sub(dres, n, dim, dim, k, cbp, dcodes)
 
 
-def run_c4(ctx, log):
+def run_c4(ctx, log, parity=True):
     import vq_amd
     from oracle import oracle as O
     from vq_amd import synth as data
@@ -303,6 +306,10 @@ def run_c4(ctx, log):
     out["recheck_fraction_last_stage"] = {"all_centroids": allc / n, "two_candidates": two / n}
     for b in (dx, dres, dall, drec):
         b.free()
+    if not parity:
+        dcb.free()
+        dcodes.free()
+        return out
 
     # parity on a sample: whole fit and encode against the oracle
     ns, st_s = 20_000, 4
@@ -338,7 +345,7 @@ def run_c4(ctx, log):
 
 
 # ---- c5: TSVQ --------------------------------------------------------------------------------
-def run_c5(ctx, log):
+def run_c5(ctx, log, parity=True):
     import vq_amd
     from oracle import oracle as O
     from vq_amd import synth as data
@@ -399,6 +406,8 @@ def run_c5(ctx, log):
     tk.free()
     dx.free()
     dleaf.free()
+    if not parity:
+        return out
 
     # parity on a sample: whole build and both descents against the oracle
     ns = 200_000
@@ -456,22 +465,24 @@ def run_c5(ctx, log):
     return out
 
 
-def other_configs(ctx, log, which=("c3", "c4", "c5"), x_c2=None, dx_c2=None):
+def other_configs(ctx, log, which=("c3", "c4", "c5"), x_c2=None, dx_c2=None, parity=True):
     out = {}
     if "c3" in which:
-        out["c3_opq"] = run_c3(ctx, log, x_c2, dx_c2)
+        out["c3_opq"] = run_c3(ctx, log, x_c2, dx_c2, parity)
     if "c4" in which:
-        out["c4_rvq"] = run_c4(ctx, log)
+        out["c4_rvq"] = run_c4(ctx, log, parity)
     if "c5" in which:
-        out["c5_tsvq"] = run_c5(ctx, log)
+        out["c5_tsvq"] = run_c5(ctx, log, parity)
     return out
 
 
 def main():
     import vq_amd
-    which = sys.argv[1:] or ["c3", "c4", "c5"]
+    args = sys.argv[1:]
+    parity = "--no-parity" not in args  # full-size dispatches only: what the profiles are taken with
+    which = [a for a in args if not a.startswith("--")] or ["c3", "c4", "c5"]
     ctx = vq_amd.Context(0)
-    print(json.dumps(other_configs(ctx, lambda *a: print(*a, file=sys.stderr, flush=True), which), indent=1))
+    print(json.dumps(other_configs(ctx, lambda *a: print(*a, file=sys.stderr, flush=True), which, parity=parity), indent=1))
 
 
 if __name__ == "__main__":
