@@ -52,7 +52,10 @@ def _data(kind, n, dim, seed):
     ("blobs", 50000, 32, 2, 10), ("outliers", 20000, 16, 3, 10), ("outliers", 70000, 128, 2, 4),
     ("duplicates", 6000, 12, 4, 10), ("integers", 12000, 10, 5, 10), ("normal", 500, 7, 8, 10),
     ("normal", 4097, 24, 1, 10), ("blobs", 8192, 64, 3, 0), ("normal", 100, 5, 0, 10),
-    ("normal", 2, 3, 4, 10), ("blobs", 150000, 128, 3, 10)])
+    ("normal", 2, 3, 4, 10), ("blobs", 150000, 128, 3, 10),
+    # the row widths of the one-pass kernel (multiples of 32 up to 128) with parts that end inside a tile
+    ("blobs", 30000, 64, 4, 10), ("normal", 25001, 96, 3, 10), ("outliers", 9000, 96, 5, 6),
+    ("duplicates", 12345, 32, 6, 10), ("integers", 40000, 64, 2, 10)])
 def test_kmeans_build_matches_oracle(ctx, kind, n, dim, depth, iters):
     x = _data(kind, n, dim, seed=n + dim)
     draws = _draws(depth * 1000 + iters, depth, iters)

@@ -182,6 +182,169 @@ static __global__ void __launch_bounds__(256) k_km_assign_reg(KmState st, int64_
     }
 }
 
+// Assignment and part sums of one LBG iteration in one pass over the rows (DIM a multiple of 32 up to
+// 128, 16-byte aligned rows).  One workgroup of 512 threads per part, which walks the part in tiles of
+// 128 positions through two LDS buffers.  Waves 0-3 bring a tile in with coalesced loads (a row is read
+// by DIM / 4 neighbouring lanes; the next tile's loads in flight meanwhile), lay it out in LDS with a row stride of
+// DIM + 4 floats (which both access patterns below read without bank conflicts) and find the code of
+// every row against the node's two centroids, in the operation order of k_km_assign_reg.  Waves
+// 4-7 work one tile behind: thread (component c, cluster j) adds the tile's rows of its cluster to its
+// sum in row order.  A row of the other cluster is added as +0.0 (its bits under an all-zero mask): the
+// sum starts at +0.0 and a sum of floats is -0.0 only if every term is, so that addition changes
+// nothing, and the sums are the part sums of k_km_partsum, bit for bit.
+// Dynamic LDS: km_assign_sum_lds(DIM) bytes.
+constexpr int kKmTile = 128;
+constexpr size_t km_assign_sum_lds(int dim) { return (size_t)2 * kKmTile * (dim + 4) * sizeof(float); }
+
+template <int DIM>
+static __global__ void __launch_bounds__(512) k_km_assign_sum(KmState st, const float *__restrict__ x, int64_t ld) {
+    constexpr int TR = kKmTile;
+    constexpr int STRIDE = DIM + 4;
+    constexpr int D4 = DIM / 4;             // float4 per row
+    constexpr int RPS = 256 / D4;           // rows per sweep of the 256 loading threads (the first RPS * D4 of them load)
+    constexpr int K = (TR + RPS - 1) / RPS; // sweeps per tile
+    static_assert(DIM % 32 == 0 && DIM <= 128, "row shape");
+    extern __shared__ __attribute__((aligned(16))) float tile[];  // [2][TR][STRIDE]
+    __shared__ __attribute__((aligned(16))) float lds_c[2 * DIM];
+    __shared__ __attribute__((aligned(16))) uint32_t lds_sel[2][2][TR];  // [buffer][cluster][row]: all ones where the row is the cluster's
+    __shared__ uint32_t lds_cnt[2];
+    __shared__ uint32_t lds_perm[kKmPart];  // the part's row ids
+    __shared__ uint8_t lds_old[kKmPart];    // and the codes they come with
+    const uint32_t part = blockIdx.x;
+    int lo = 0, hi = st.ns - 1;
+    while (lo < hi) {  // the segment this part belongs to: part_first is ascending
+        const int mid = (lo + hi + 1) >> 1;
+        if (st.part_first[mid] <= part)
+            lo = mid;
+        else
+            hi = mid - 1;
+    }
+    const int g = lo;
+    if (st.done[g]) return;  // the same in the whole workgroup
+    // (the same in every lane: told to the compiler, so that the loops below are scalar loops)
+    const uint32_t rx = __builtin_amdgcn_readfirstlane(st.range[g].x), ry = __builtin_amdgcn_readfirstlane(st.range[g].y);
+    const uint32_t pf = __builtin_amdgcn_readfirstlane(st.part_first[g]);
+    const uint32_t p0 = rx + (part - pf) * (uint32_t)kKmPart;
+    const uint32_t p1 = p0 + kKmPart < ry ? p0 + kKmPart : ry;
+    const uint32_t np = p1 - p0;  // positions in this part
+    const int ntiles = (int)((np + TR - 1) / TR);
+    const int tid = threadIdx.x, lt = tid & 255;
+    const bool producer = tid < 256;
+    const int lrow = lt / D4, lcol = lt % D4;  // a loading thread's place in a sweep
+    const bool loader = producer && lt < RPS * D4;
+    for (uint32_t q = tid; q < np; q += 512) {
+        lds_perm[q] = st.perm[p0 + q];
+        lds_old[q] = st.codes[p0 + q];
+    }
+    for (int t = tid; t < 2 * DIM; t += 512) lds_c[t] = st.cen[(size_t)g * 2 * DIM + t];
+    if (tid < 2) lds_cnt[tid] = 0u;
+    __syncthreads();
+    // The loads of a tile are unconditional (a row past the tile's end reads the tile's last row instead,
+    // and its value never reaches a sum): loads under a branch would make every wait a wait for all of them.
+    // (The loaded values are assigned component by component: as a copy of the 16-byte struct from global
+    // memory the staging array stays in scratch memory.)
+    float4 stage[K];
+    auto fetch = [&](int t, float4(&stg)[K]) {
+        const uint32_t base = (uint32_t)t * TR;
+        const uint32_t rows = np - base < (uint32_t)TR ? np - base : (uint32_t)TR;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const uint32_t row = (uint32_t)(k * RPS + lrow);
+            const float4 v = reinterpret_cast<const float4 *>(x + (int64_t)lds_perm[base + (row < rows ? row : rows - 1u)] * ld)[lcol];
+            stg[k] = make_float4(v.x, v.y, v.z, v.w);
+        }
+    };
+    if (producer) fetch(0, stage);
+    const int c = lt % DIM, j = lt / DIM;  // a summing thread's chain (lt < 2 * DIM)
+    const bool summer = !producer && lt < 2 * DIM;
+    float acc = 0.0f;
+    uint32_t n0 = 0, n1 = 0;
+    bool any_changed = false;
+    // rows [64 * half, 64 * half + 64) of the tile in buffer b into the chains
+    auto sum_half = [&](int b, int half) {
+        const float *tb = tile + (size_t)b * TR * STRIDE + (size_t)(64 * half) * STRIDE + c;
+        const uint4 *sel = reinterpret_cast<const uint4 *>(&lds_sel[b][j][64 * half]);
+#pragma unroll 4
+        for (int r4 = 0; r4 < 16; ++r4) {
+            const uint4 m = sel[r4];
+            const float v0 = tb[(4 * r4 + 0) * STRIDE], v1 = tb[(4 * r4 + 1) * STRIDE];
+            const float v2 = tb[(4 * r4 + 2) * STRIDE], v3 = tb[(4 * r4 + 3) * STRIDE];
+            acc = acc + __uint_as_float(__float_as_uint(v0) & m.x);
+            acc = acc + __uint_as_float(__float_as_uint(v1) & m.y);
+            acc = acc + __uint_as_float(__float_as_uint(v2) & m.z);
+            acc = acc + __uint_as_float(__float_as_uint(v3) & m.w);
+        }
+    };
+    auto step = [&](int i, float4(&stg)[K]) {
+        const int b = i & 1;
+        // first half: tile i into LDS, tile i + 1 on its way | rows 0..63 of tile i - 1 into the sums
+        if (producer) {
+            if (i < ntiles) {
+                float *tb = tile + (size_t)b * TR * STRIDE;
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    if (loader && k * RPS + lrow < TR)
+                        *reinterpret_cast<float4 *>(tb + (k * RPS + lrow) * STRIDE + 4 * lcol) = stg[k];
+                fetch(i + 1 < ntiles ? i + 1 : i, stg);  // (unconditional: the last tile is asked for twice)
+            }
+        } else if (summer && i >= 1) {
+            sum_half(b ^ 1, 0);
+        }
+        lds_only_barrier();  // (not __syncthreads: the loads of the next tile stay in flight)
+        // second half: codes of tile i | rows 64..127 of tile i - 1
+        if (producer) {
+            if (i < ntiles) {
+                // lanes l and l + 32 of a wave take one row: the distance to the first centroid in the
+                // lower lane, to the second in the upper one (each a chain of its own, as in the reference)
+                const int prow = ((lt >> 6) << 5) | (lt & 31), which = (lt >> 5) & 1;
+                const uint32_t q = (uint32_t)i * TR + prow;
+                const float *xr = tile + (size_t)b * TR * STRIDE + prow * STRIDE;
+                const float *cp = lds_c + which * DIM;
+                float d = 0.0f;
+#pragma unroll 8
+                for (int qq = 0; qq < D4; ++qq) {
+                    const float4 v = *reinterpret_cast<const float4 *>(xr + 4 * qq);
+                    const float4 a = *reinterpret_cast<const float4 *>(cp + 4 * qq);
+                    const float xv[4] = {v.x, v.y, v.z, v.w}, ca[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const float e = xv[u] - ca[u];
+                        const float sq = e * e;
+                        d = d + sq;
+                    }
+                }
+                const float other = __shfl_xor(d, 32);
+                if (which == 0) {
+                    uint32_t is0 = 0u, is1 = 0u;  // neither cluster: a position past the part's end
+                    if (q < np) {
+                        const uint8_t code = other < d ? 1 : 0;  // strict '<': ties and NaN stay with the first
+                        if (lds_old[q] != code) {
+                            st.codes[p0 + q] = code;
+                            any_changed = true;
+                        }
+                        is1 = code ? 0xffffffffu : 0u;
+                        is0 = ~is1;
+                        n1 += code;
+                        n0 += 1u - code;
+                    }
+                    lds_sel[b][0][prow] = is0;
+                    lds_sel[b][1][prow] = is1;
+                }
+            }
+        } else if (summer && i >= 1) {
+            sum_half(b ^ 1, 1);
+        }
+        lds_only_barrier();
+    };
+    for (int i = 0; i <= ntiles; ++i) step(i, stage);
+    if (any_changed && st.changed[g] == 0) st.changed[g] = 1;
+    if (n0) atomicAdd(&lds_cnt[0], n0);
+    if (n1) atomicAdd(&lds_cnt[1], n1);
+    __syncthreads();
+    if (summer) st.part_sum[((size_t)part * 2 + j) * DIM + c] = acc;
+    if (tid < 2) st.part_cnt[(size_t)part * 2 + tid] = lds_cnt[tid];
+}
+
 // One workgroup per part (4096 consecutive rows of a node's array): thread t owns components t, t +
 // blockDim, ... and adds the part's rows to the sum of their cluster in row order, from 0.0; thread 0
 // counts.  blockDim: 64, 128 or 256 (the smallest that covers dim, so that short rows leave no idle waves).
@@ -340,7 +503,17 @@ static __global__ void __launch_bounds__(256) k_km_update(KmState st, const floa
             const float dv = __uint2float_rn(m);
             for (int t = threadIdx.x; t < dim; t += 256) {
                 float acc = 0.0f;
-                for (uint32_t q = 0; q < nparts; ++q) acc = acc + st.part_sum[((size_t)(f + q) * 2 + j) * dim + t];
+                const float *ps = st.part_sum + ((size_t)f * 2 + j) * dim + t;
+                const size_t pstride = (size_t)2 * dim;
+                uint32_t q = 0;
+                for (; q + 8 <= nparts; q += 8) {  // eight loads in flight, added in part order
+                    float v[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) v[u] = ps[(size_t)(q + u) * pstride];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) acc = acc + v[u];
+                }
+                for (; q < nparts; ++q) acc = acc + ps[(size_t)q * pstride];
                 out[t] = (m <= (uint32_t)kKmSeqMax) ? st.part_sum[((size_t)f * 2 + j) * dim + t] / dv : acc / dv;
             }
         }

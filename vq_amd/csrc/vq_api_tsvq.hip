@@ -414,9 +414,36 @@ static int32_t tsvq_build_impl(vq_ctx *ctx, const float *d_x, int64_t n, int64_t
 #undef KM_REG
             };
             const unsigned sum_threads = dim <= 64 ? 64u : dim <= 128 ? 128u : 256u;
+            // the fused kernel where a workgroup may hold its two tiles in LDS, else the two kernels apart
+            const void *fused = nullptr;
+            if (reg) {
+                int optin = 0;
+                SP_HIP(hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, ctx->device));
+                const size_t lds = vq::km_assign_sum_lds(dim);
+                if (lds + 24 * 1024 <= (size_t)optin) {  // (+ the kernel's static LDS: the part's row ids, masks, centroids)
+                    switch (dim) {
+                    case 32: fused = reinterpret_cast<const void *>(vq::k_km_assign_sum<32>); break;
+                    case 64: fused = reinterpret_cast<const void *>(vq::k_km_assign_sum<64>); break;
+                    case 96: fused = reinterpret_cast<const void *>(vq::k_km_assign_sum<96>); break;
+                    default: fused = reinterpret_cast<const void *>(vq::k_km_assign_sum<128>); break;
+                    }
+                    if (lds > 48 * 1024)
+                        SP_HIP(hipFuncSetAttribute(fused, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                }
+            }
             for (int it = 0; it < km->lbg_iters; ++it) {
-                assign(true, nullptr);
-                hipLaunchKernelGGL(vq::k_km_partsum, dim3(parts), dim3(sum_threads), 0, st, S, d_x, ld, dim);
+                if (fused) {  // assignment and part sums in one pass over the rows
+                    const size_t lds = vq::km_assign_sum_lds(dim);
+                    switch (dim) {
+                    case 32: hipLaunchKernelGGL(vq::k_km_assign_sum<32>, dim3(parts), dim3(512), lds, st, S, d_x, ld); break;
+                    case 64: hipLaunchKernelGGL(vq::k_km_assign_sum<64>, dim3(parts), dim3(512), lds, st, S, d_x, ld); break;
+                    case 96: hipLaunchKernelGGL(vq::k_km_assign_sum<96>, dim3(parts), dim3(512), lds, st, S, d_x, ld); break;
+                    default: hipLaunchKernelGGL(vq::k_km_assign_sum<128>, dim3(parts), dim3(512), lds, st, S, d_x, ld); break;
+                    }
+                } else {
+                    assign(true, nullptr);
+                    hipLaunchKernelGGL(vq::k_km_partsum, dim3(parts), dim3(sum_threads), 0, st, S, d_x, ld, dim);
+                }
                 hipLaunchKernelGGL(vq::k_km_update, dim3(ns), dim3(256), 0, st, S, d_x, ld, dim);
             }
             // rows whose nearest of the two final centroids is the first go left
