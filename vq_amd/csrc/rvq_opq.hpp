@@ -263,6 +263,7 @@ static __global__ void __launch_bounds__(256) k_crosscov_partial(const float *__
             if (e < total) {
                 int a = e / db, b = e % db;
                 double s = acc[u];
+#pragma unroll 1
                 for (int r = 0; r < rows; ++r) s += (double)ly[r * da + a] * (double)lx[r * db + b];
                 acc[u] = s;
             }
@@ -621,6 +622,7 @@ static __global__ void __launch_bounds__(512) k_rotate_mfma_resident(const float
             for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[t][b][v] = 0.0f;
+#pragma unroll 1
         for (int kc0 = 0; kc0 < NKC; kc0 += kRotAhead) {
 #pragma unroll
             for (int u = 0; u < kRotAhead; ++u) {
