@@ -292,6 +292,9 @@ def test_lbg_fit_same_result_on_both_assignment_paths(ctx):
     (3000, 1, 256, 256, "normal"), (1000, 2, 64, 100, "uniform"), (513, 4, 16, 33, "grid"),
     (700, 1, 128, 256, "offset"), (300, 1, 24, 7, "same"), (640, 1, 256, 64, "nonfinite"),
     (257, 3, 32, 1, "normal"),
+    # long lists of rows for the all-centroid check in a single column block (eight rows per workgroup)
+    (5000, 1, 40, 100, "offset"), (20000, 1, 256, 256, "offset"), (3000, 1, 72, 256, "same"),
+    (2500, 1, 136, 255, "nonfinite"),
 ])
 def test_wide_mfma_path_equals_oracle_and_valu_path(ctx, metric, n, m, sd, k, kind):
     """sub_dim a multiple of 8 above 8 (RVQ stages use the full dimension): chunked matrix-core

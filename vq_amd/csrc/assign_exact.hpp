@@ -517,9 +517,10 @@ __device__ __forceinline__ void wide_argmin(const AssignArgs &a, int sd, int s, 
 // The wave's share of the groups of NR rows (or listed pairs).
 template <int METRIC, bool LBG, bool LISTED, bool VEC, int NR>
 __device__ __forceinline__ void wide_exact_groups(const AssignArgs &a, int sd, const uint32_t *__restrict__ list,
-                                                  int64_t total, float *lds_x, int lane, int wave, unsigned nblocks) {
+                                                  int64_t total, float *lds_x, int lane, int wave, unsigned block,
+                                                  unsigned nblocks) {
     const int64_t groups = (total + NR - 1) / NR;
-    for (int64_t grp = (int64_t)blockIdx.x * 4 + wave; grp < groups; grp += (int64_t)nblocks * 4) {
+    for (int64_t grp = (int64_t)block * 4 + wave; grp < groups; grp += (int64_t)nblocks * 4) {
         int64_t rows[NR];
         int ss[NR];
 #pragma unroll
@@ -701,6 +702,174 @@ __device__ __forceinline__ void wide_exact_pair_wg(const AssignArgs &a, int sd, 
     }
 }
 
+// Listed rows of a single column block (m == 1) eight at a time by a whole workgroup: the scheme of
+// wide_exact_pair_wg with eight rows in LDS, so that the codebook is read once per eight rows (a
+// wave that takes a listed row on its own reads every centroid for that row alone: 256 KB per row
+// at k = 256, D = 256, which is what bounds a list of a few thousand rows).  Thread j keeps eight
+// distances to centroid j, each a sequential chain over the sub-vector in the reference's order.
+// lds: 8 rows (8 * sd floats), 8 x 16 floats of reduction space, 256 x 33 floats of centroid slices.
+constexpr int kRowsWg = 8;
+constexpr int kRowsWgLdsFloats = kRowsWg * 16 + 256 * 33;  // beside the rows
+template <int METRIC, bool LBG>
+__device__ __forceinline__ void wide_exact_rows_wg(const AssignArgs &a, int sd, const uint32_t *__restrict__ list,
+                                                   int64_t total, unsigned block, unsigned nblocks, float *lds) {
+    static_assert(METRIC == M_SQ || METRIC == M_EUCLID, "squared L2 / Euclidean");
+    constexpr int NR = kRowsWg;
+    const int j = threadIdx.x, lane = j & 63, wave = j >> 6, k = a.k;
+    float *red = lds + NR * sd;                      // [NR][16]
+    float *slice = red + NR * 16 + wave * 64 * 33;   // this wave's 64 centroids x 33
+    const float *cbs = a.cb;
+    const int sub = lane >> 3, piece = lane & 7;     // centroid within a group of 8, float4 within the slice
+    const int nsl = (sd + 31) / 32;
+    const float inf = __builtin_inff();
+    for (int64_t grp = block; grp * NR < total; grp += nblocks) {
+        int64_t rows[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            const int64_t e = grp * NR + i;
+            rows[i] = list[e < total ? e : total - 1];  // (m == 1: an entry is a row; the tail repeats the last one)
+        }
+#pragma unroll
+        for (int i = 0; i < NR; ++i)
+            for (int t = j; t < sd; t += 256) lds[i * sd + t] = a.x[rows[i] * a.ld + t];
+        __syncthreads();
+        float4 pre[8];
+        auto fetch = [&](int sl) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int c = 64 * wave + 8 * i + sub;
+                const int d = 32 * sl + 4 * piece;
+                const float4 v = *reinterpret_cast<const float4 *>(cbs + (size_t)(c < k ? c : 0) * sd + (d < sd ? d : 0));
+                pre[i] = make_float4(v.x, v.y, v.z, v.w);
+            }
+        };
+        fetch(0);
+        float acc[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) acc[i] = 0.0f;
+        for (int sl = 0; sl < nsl; ++sl) {
+            __builtin_amdgcn_wave_barrier();  // the lanes have read the previous slice
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float *dst = slice + (8 * i + sub) * 33 + 4 * piece;
+                dst[0] = pre[i].x;
+                dst[1] = pre[i].y;
+                dst[2] = pre[i].z;
+                dst[3] = pre[i].w;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            fetch(sl + 1 < nsl ? sl + 1 : sl);
+            const float *mine = slice + lane * 33;
+            const int nd = sd - 32 * sl < 32 ? sd - 32 * sl : 32;
+            if (nd == 32) {
+#pragma unroll
+                for (int t4 = 0; t4 < 8; ++t4) {
+                    const float c0 = mine[4 * t4], c1 = mine[4 * t4 + 1], c2 = mine[4 * t4 + 2], c3 = mine[4 * t4 + 3];
+#pragma unroll
+                    for (int i = 0; i < NR; ++i) {
+                        const float4 xv = *reinterpret_cast<const float4 *>(lds + i * sd + 32 * sl + 4 * t4);
+                        wide_step<METRIC>(acc[i], xv.x, c0);
+                        wide_step<METRIC>(acc[i], xv.y, c1);
+                        wide_step<METRIC>(acc[i], xv.z, c2);
+                        wide_step<METRIC>(acc[i], xv.w, c3);
+                    }
+                }
+            } else {
+                for (int t = 0; t < nd; ++t) {
+                    const float cv = mine[t];
+#pragma unroll
+                    for (int i = 0; i < NR; ++i) wide_step<METRIC>(acc[i], lds[i * sd + 32 * sl + t], cv);
+                }
+            }
+        }
+        // per row: the smallest (distance, index), the reference's strict '<' scan
+        float dd[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            dd[i] = (j < k && acc[i] == acc[i]) ? acc[i] : inf;  // a NaN distance never wins
+            float bd = dd[i];
+            int bi = j < k ? j : 0x7fffffff;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const float od = __shfl_xor(bd, off);
+                const int oi = __shfl_xor(bi, off);
+                const bool take = (od < bd) || (od == bd && oi < bi);
+                bd = take ? od : bd;
+                bi = take ? oi : bi;
+            }
+            if (lane == 0) {
+                red[i * 16 + wave] = bd;
+                reinterpret_cast<int *>(red)[i * 16 + 4 + wave] = bi;
+            }
+            if (j == 0) red[i * 16 + 12] = acc[i];  // centroid 0's distance as computed
+        }
+        __syncthreads();
+        int best[NR];
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            float bd = red[i * 16];
+            int bi = reinterpret_cast<int *>(red)[i * 16 + 4];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) {
+                const float od = red[i * 16 + w];
+                const int oi = reinterpret_cast<int *>(red)[i * 16 + 4 + w];
+                const bool take = (od < bd) || (od == bd && oi < bi);
+                bd = take ? od : bd;
+                bi = take ? oi : bi;
+            }
+            best[i] = bi;
+            if constexpr (METRIC == M_EUCLID) {
+                // the reference compares the roots: first index whose root equals the smallest root
+                const float sr = sqrtf(bd);
+                int fi = (j < k && sqrtf(dd[i]) == sr) ? j : 0x7fffffff;
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) {
+                    const int oi = __shfl_xor(fi, off);
+                    fi = oi < fi ? oi : fi;
+                }
+                if (lane == 0) reinterpret_cast<int *>(red)[i * 16 + 8 + wave] = fi;
+            }
+        }
+        if constexpr (METRIC == M_EUCLID) {
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                const int *rf = reinterpret_cast<const int *>(red) + i * 16 + 8;
+                int bi = rf[0];
+#pragma unroll
+                for (int w = 1; w < 4; ++w) bi = rf[w] < bi ? rf[w] : bi;
+                best[i] = bi;
+            }
+        }
+        if (j < NR) {
+            // thread i writes row i's code
+            int bi = 0;
+            int64_t row = 0;
+#pragma unroll
+            for (int i = 0; i < NR; ++i)
+                if (i == j) {
+                    bi = best[i];
+                    row = rows[i];
+                }
+            const float d0 = red[j * 16 + 12];
+            if (!(d0 == d0)) bi = 0;  // NaN at index 0 is never displaced
+            if (grp * NR + j < total) {
+                if constexpr (LBG) {
+                    uint8_t *p = a.codes + row;
+                    if (*p != (uint8_t)bi) {
+                        *p = (uint8_t)bi;
+                        mark_changed(a.changed);
+                    }
+                } else {
+                    a.codes[row] = (uint8_t)bi;
+                }
+            }
+        }
+        __syncthreads();  // the rows and the reduction space are written again by the next group
+    }
+}
+
 // Exact decision between two candidate centroids per listed (row, column block) pair — the
 // pairs the matrix-core pass narrowed down to its two best scores.  Lanes 2i and 2i + 1 take
 // candidates c1 and c2 of entry i: each accumulates its distance in the reference's order
@@ -760,13 +929,17 @@ __global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd,
                                                            unsigned exact_blocks) {
     extern __shared__ float lds_wide[];  // 4 waves x 8 rows x sd
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    // The workgroups from exact_blocks on take the list of pairs with two candidates: the two
-    // follow-ups of the matrix-core pass are short and independent, and run side by side in one launch.
+    // The first gridDim.x - exact_blocks workgroups take the list of pairs with two candidates: the two
+    // follow-ups of the matrix-core pass are independent and run side by side in one launch (the
+    // pairs first: workgroups start in index order, and behind a long list of rows they would wait).
+    unsigned block = blockIdx.x;
     if constexpr (LISTED && (METRIC == M_SQ || METRIC == M_EUCLID)) {
-        if (blockIdx.x >= exact_blocks) {
-            wide_pair_blocks<METRIC, LBG>(a, sd, pairs, *pair_count, blockIdx.x - exact_blocks, gridDim.x - exact_blocks);
+        const unsigned pair_blocks = gridDim.x - exact_blocks;
+        if (block < pair_blocks) {
+            wide_pair_blocks<METRIC, LBG>(a, sd, pairs, *pair_count, block, pair_blocks);
             return;
         }
+        block -= pair_blocks;
     }
     float *lds_x = lds_wide + (size_t)wave * kWideRows * sd;
     const int64_t total = LISTED ? (int64_t)*list_count : a.n;
@@ -775,19 +948,24 @@ __global__ void __launch_bounds__(256) k_assign_wide_exact(AssignArgs a, int sd,
     }
     if constexpr (LISTED && VEC && (METRIC == M_SQ || METRIC == M_EUCLID)) {
         // a handful of pairs: one per workgroup, one centroid per thread
-        if (total <= (int64_t)exact_blocks && a.k <= 256) {
-            if ((int64_t)blockIdx.x < total) wide_exact_pair_wg<METRIC, LBG>(a, sd, list[blockIdx.x], lds_wide);
+        if (a.k <= 256 && total <= (a.m == 1 ? 1024 : (int64_t)exact_blocks)) {
+            if ((int64_t)block < total) wide_exact_pair_wg<METRIC, LBG>(a, sd, list[block], lds_wide);
+            return;
+        }
+        // rows of a single column block: eight per workgroup, the codebook read once per eight
+        if (a.k <= 256 && a.m == 1) {
+            wide_exact_rows_wg<METRIC, LBG>(a, sd, list, total, block, exact_blocks, lds_wide);
             return;
         }
     }
     if constexpr (LISTED) {
         // a short list: one pair per wave, so that the pass is as long as one pair's scan, not eight
         if (total <= (int64_t)exact_blocks * 4) {
-            wide_exact_groups<METRIC, LBG, LISTED, VEC, 1>(a, sd, list, total, lds_x, lane, wave, exact_blocks);
+            wide_exact_groups<METRIC, LBG, LISTED, VEC, 1>(a, sd, list, total, lds_x, lane, wave, block, exact_blocks);
             return;
         }
     }
-    wide_exact_groups<METRIC, LBG, LISTED, VEC, kWideRows>(a, sd, list, total, lds_x, lane, wave, exact_blocks);
+    wide_exact_groups<METRIC, LBG, LISTED, VEC, kWideRows>(a, sd, list, total, lds_x, lane, wave, block, exact_blocks);
 }
 
 }  // namespace vq

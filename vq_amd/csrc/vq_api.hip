@@ -226,6 +226,8 @@ int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const ui
     size_t lds = sizeof(float) * 4 * vq::kWideRows * (size_t)sd;
     // a handful of listed pairs: one per workgroup, the row and slices of every centroid in LDS
     if (listed) lds = std::max(lds, sizeof(float) * ((size_t)sd + vq::kPairWgLdsFloats));
+    // ... or eight rows of a single column block per workgroup
+    if (listed && a.m == 1) lds = std::max(lds, sizeof(float) * ((size_t)vq::kRowsWg * sd + vq::kRowsWgLdsFloats));
     if (lds > 160 * 1024) return fail(ctx, VQ_ERR_UNSUPPORTED, "sub_dim %d too large", sd);
     auto pick = [&](auto L, auto V) {
         constexpr bool LISTED = decltype(L)::value, VEC = decltype(V)::value;
@@ -238,7 +240,7 @@ int32_t launch_wide_exact(vq_ctx *ctx, const vq::AssignArgs &a, int sd, const ui
     const int64_t groups = (a.n + vq::kWideRows - 1) / vq::kWideRows;
     dim3 grid(listed ? 2048u : (unsigned)std::min<int64_t>((groups + 3) / 4, 1 << 20), listed ? 1u : (unsigned)a.m);
     unsigned exact_blocks = grid.x;
-    if (pairs) grid.x += 512u;  // the workgroups of the two-candidate list
+    if (pairs) grid.x += 1024u;  // the workgroups of the two-candidate list (they come first in the grid)
     vq::AssignArgs aa = a;
     int sdv = sd;
     void *args[] = {&aa, &sdv, (void *)&list, (void *)&count, (void *)&pairs, (void *)&pair_count, &exact_blocks};
