@@ -308,6 +308,81 @@ static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t 
     }
 }
 
+// The same scatter by a workgroup of four waves per (part, column block), for the shapes whose
+// every row is listed (no streaming sums): wave w ranks the rows [1024 w, 1024 w + 1024) of the
+// part.  A first sweep counts the codes of each quarter, so that a wave's first position inside
+// cluster j is the part's position plus the members in the quarters before its own; the order of
+// the rows inside a cluster stays the row order.  One wave per part is a chain of 64 dependent
+// LDS round trips per part and a handful of waves on the whole GPU when there is one column block.
+static __global__ void __launch_bounds__(256) k_lbg_scatter_wg(LbgState st, int64_t n) {
+    const int s = blockIdx.y, b = blockIdx.x;
+    if (st.done[s]) return;
+    constexpr int kQuarter = kPartRows / 4;
+    __shared__ uint32_t cntq[4][kMaxK];
+    __shared__ uint32_t base[4][kMaxK];
+    __shared__ __attribute__((aligned(16))) uint8_t pcodes[kPartRows];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const uint8_t *codes = st.codes + (size_t)s * n;
+    uint32_t *perm = st.perm + (size_t)s * n;
+    const int64_t lo = (int64_t)b * kPartRows;
+    const int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
+    const int rows = (int)(hi - lo);
+    for (int j = threadIdx.x; j < 4 * kMaxK; j += 256) (&cntq[0][0])[j] = 0u;
+    // the part's codes into LDS, 16 per thread
+    {
+        const int64_t r0 = lo + 16 * (int64_t)threadIdx.x;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (((uintptr_t)(codes + lo) & 15) == 0 && r0 + 16 <= hi) {
+            v = *reinterpret_cast<const uint4 *>(codes + r0);
+        } else {
+            uint32_t q[4] = {0u, 0u, 0u, 0u};
+            for (int u = 0; u < 16; ++u)
+                if (r0 + u < hi) q[u >> 2] |= (uint32_t)codes[r0 + u] << (8 * (u & 3));
+            v = make_uint4(q[0], q[1], q[2], q[3]);
+        }
+        reinterpret_cast<uint4 *>(pcodes)[threadIdx.x] = v;
+    }
+    __syncthreads();
+    const int q0 = w * kQuarter, q1 = q0 + kQuarter < rows ? q0 + kQuarter : rows;
+    for (int i = q0 + lane; i < q1; i += 64) atomicAdd(&cntq[w][pcodes[i]], 1u);
+    __syncthreads();
+    {
+        const uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
+        const uint32_t *start = st.start + (size_t)s * kMaxK;
+        const int j = threadIdx.x;  // kMaxK == 256 threads
+        uint32_t run = start[j] + h[j];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            base[q][j] = run;
+            run += cntq[q][j];
+        }
+    }
+    __syncthreads();
+    uint32_t *mybase = base[w];
+    const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    for (int i0 = q0; i0 < q1; i0 += 64) {
+        const int i = i0 + lane;
+        const bool valid = i < q1;
+        const uint32_t c = valid ? pcodes[i] : 0u;
+        uint64_t mask = __ballot(valid);
+#pragma unroll
+        for (int bit = 0; bit < 8; ++bit) {
+            const bool set = (c >> bit) & 1u;
+            const uint64_t bal = __ballot(set);
+            mask &= set ? bal : ~bal;
+        }
+        // lanes with equal code and valid: mask (invalid lanes have a stale mask, unused)
+        const uint32_t rank = (uint32_t)__popcll(mask & lt);
+        const uint32_t tot = (uint32_t)__popcll(mask);
+        uint32_t pos = 0;
+        if (valid) pos = mybase[c] + rank;
+        __builtin_amdgcn_wave_barrier();  // one wave per table, LDS in program order: reads above, updates below
+        if (valid && rank == 0) mybase[c] += tot;
+        __builtin_amdgcn_wave_barrier();
+        if (valid) perm[pos] = (uint32_t)(lo + i);
+    }
+}
+
 // One lane per (leaf, component): sequential sum of the leaf's members in list order.
 static __global__ void __launch_bounds__(256) k_lbg_leafsum(LbgState st, const float *__restrict__ x,
                                                      int64_t n, int64_t ld, int sd) {
@@ -506,9 +581,11 @@ static __global__ void __launch_bounds__(256) k_lbg_finalize(LbgState st, const 
         sum = ls[0];
     } else {
         if (st.stream) return;  // k_lbg_combine8 writes the large clusters
-        // the per-part sums in part order; sixteen loads in flight, the adds one chain
+        // the per-part sums in part order; 64 loads in flight (the kernel's time is memory round
+        // trips; with 245 parts of a million rows the 64 MB of leaf sums then come in at the HBM rate),
+        // the adds one chain
         sum = 0.0f;
-        constexpr int B = 16;
+        constexpr int B = 64;
         const int np = st.nparts;
         for (int p = 0; p < np; p += B) {
             float v[B];

@@ -1166,7 +1166,10 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
         hipLaunchKernelGGL(vq::k_lbg_scan_seg, dim3(nseg, m), dim3(256), 0, gs, S);
         hipLaunchKernelGGL(vq::k_lbg_plan, dim3(m), dim3(256), 0, gs, S, k);
         hipLaunchKernelGGL(vq::k_lbg_scan_blocks, dim3(nseg, m), dim3(256), 0, gs, S);
-        hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nparts, m), dim3(64), 0, gs, S, n);
+        if (stream)
+            hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nparts, m), dim3(64), 0, gs, S, n);
+        else  // every row is listed: four waves per part
+            hipLaunchKernelGGL(vq::k_lbg_scatter_wg, dim3(nparts, m), dim3(256), 0, gs, S, n);
         if (leaf_wg) {
             // leaves are the few clusters of up to 1024 members beside the streaming kernel
             hipLaunchKernelGGL(vq::k_lbg_leafsum_wg, dim3(leaf_cap, m), dim3(256), 0, gs, S, d_x, n, ld, sd,
