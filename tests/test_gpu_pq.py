@@ -55,6 +55,8 @@ LBG_CASES = [
     (13000, 24, 3, 5, 3, "normal"),    # sub_dim 8 but m % 4 != 0 -> per-part leaves, gather path
     (13000, 6, 1, 4, 3, "normal"),     # sub_dim 6, clusters above 1024 -> per-part leaves
     (300001, 32, 4, 256, 2, "normal"), # sub_dim 8: a workgroup of the assignment walks over several runs of rows
+    (4200000, 2, 1, 5, 2, "normal"),   # 1026 parts of 4096 rows in 33 scan segments (the plan walks them eight at a time)
+    (4200000, 8, 1, 3, 2, "uniform"),  # the same at sub_dim 8 without the streaming sums (m % 4 != 0)
 ]
 
 

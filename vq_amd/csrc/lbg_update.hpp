@@ -146,7 +146,7 @@ static __global__ void __launch_bounds__(256) k_lbg_plan(LbgState st, int k) {
     side_chain_priority();
     const int s = blockIdx.x, j = threadIdx.x;
     if (st.done[s]) return;
-    __shared__ uint32_t sh_cnt[kMaxK], sh_leaf[kMaxK], sh_empty[kMaxK], sh_small[kMaxK];
+    __shared__ uint32_t sh_cnt[4], sh_leaf[4], sh_empty[4], sh_small[4];  // totals of the four waves
     uint32_t run = 0;
     uint32_t *h = st.seg + (size_t)s * st.nseg * kMaxK + j;
     for (int g0 = 0; g0 < st.nseg; g0 += 8) {
@@ -165,18 +165,33 @@ static __global__ void __launch_bounds__(256) k_lbg_plan(LbgState st, int k) {
     const bool big = cnt > (uint32_t)kSeqMax;
     const uint32_t nl = small ? 1u : ((big && !st.stream) ? (uint32_t)st.nparts : 0u);
     const uint32_t emp = (live && cnt == 0) ? 1u : 0u;
-    sh_cnt[j] = cnt;
-    sh_leaf[j] = nl;
-    sh_empty[j] = emp;
-    sh_small[j] = small ? 1u : 0u;
+    // exclusive prefixes over j: inside a wave by shuffles, the three waves before by their totals
+    // (a serial walk per thread is 4 x 255 dependent LDS reads for the last one: 10 us on this chain)
+    uint32_t ic = cnt, il = nl, ie = emp, is = small ? 1u : 0u;  // inclusive inside the wave
+    const int lane = j & 63, wv = j >> 6;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t oc = __shfl_up(ic, off), ol = __shfl_up(il, off), oe = __shfl_up(ie, off), os = __shfl_up(is, off);
+        if (lane >= off) {
+            ic += oc;
+            il += ol;
+            ie += oe;
+            is += os;
+        }
+    }
+    if (lane == 63) {
+        sh_cnt[wv] = ic;
+        sh_leaf[wv] = il;
+        sh_empty[wv] = ie;
+        sh_small[wv] = is;
+    }
     __syncthreads();
-    // exclusive prefixes over j (k <= 256: a serial walk per thread is cheap and simple)
-    uint32_t pc = 0, pl = 0, pe = 0, ps = 0;
-    for (int i = 0; i < j; ++i) {
-        pc += sh_cnt[i];
-        pl += sh_leaf[i];
-        pe += sh_empty[i];
-        ps += sh_small[i];
+    uint32_t pc = ic - cnt, pl = il - nl, pe = ie - emp, ps = is - (small ? 1u : 0u);
+    for (int u = 0; u < wv; ++u) {
+        pc += sh_cnt[u];
+        pl += sh_leaf[u];
+        pe += sh_empty[u];
+        ps += sh_small[u];
     }
     const size_t sj = (size_t)s * kMaxK + j;
     st.count[sj] = cnt;
