@@ -256,13 +256,21 @@ def rvq_fit_device(ctx, dx, dres, dcb, dcodes, n, dim, stages, k, iters, init, r
     the last stage, which nothing can observe (the residuals are a local of fit) unless
     final_residual asks for it."""
     ctx.copy_f32(dres, dx, n * dim)
+    prev = None  # the codebook of a residual update that rides on the next stage's fit (vq_lbg_fit_residual)
     for st in range(stages):
         cbp = dcb.ptr + st * k * dim * 4
-        ctx.lbg_fit(dres, n, dim, 1, dim, k, iters, init[st], reseed[st], cbp)
+        if prev is None:
+            ctx.lbg_fit(dres, n, dim, 1, dim, k, iters, init[st], reseed[st], cbp)
+        else:
+            ctx.lbg_fit_residual(dres, n, dim, dim, k, iters, init[st], reseed[st], cbp, prev, k, dcodes)
+        prev = None
         if st + 1 == stages and not final_residual:
             break
         ctx.assign(metric, dres, n, dim, 1, dim, k, cbp, dcodes)
-        ctx.residual_sub(dres, n, dim, dim, k, cbp, dcodes)
+        if st + 1 < stages:
+            prev = cbp
+        else:
+            ctx.residual_sub(dres, n, dim, dim, k, cbp, dcodes)
 
 
 def run_c4(ctx, log, parity=True):

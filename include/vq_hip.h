@@ -257,6 +257,21 @@ int32_t vq_residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_
 int32_t vq_residual_sub_u16(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
                             const float *d_codebook, const uint16_t *d_codes);
 
+/* The residual update of one stage and the training of the next in one call (src/rvq.rs:103-129 across
+ * two turns of the stage loop): d_res[i] -= d_prev_codebook[d_prev_codes[i]] for every row, exactly as
+ * vq_residual_sub does, then vq_lbg_fit with m = 1, sub_dim = dim on the updated rows, exactly as
+ * vq_lbg_fit does (same arguments, same results bit for bit; on return d_res holds the updated
+ * residual).  Where the fit's first assignment pass is the matrix-core pass over one wide column block
+ * (dim a multiple of 8 from 16 on, k <= 256, 16-byte aligned rows and codebooks, max_iters >= 1) that
+ * pass applies the update as it reads the rows and writes them back in place, which saves the
+ * separate pass over the rows; otherwise the two steps run one after the other.  d_prev_codes: n uint8
+ * codes below k_prev <= 256.  After an error d_res may or may not have been updated.  Synchronises
+ * like vq_lbg_fit. */
+int32_t vq_lbg_fit_residual(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
+                            int32_t max_iters, const uint32_t *h_init_idx, const uint32_t *h_reseed_stream,
+                            int32_t n_reseed, float *d_codebook, const float *d_prev_codebook, int32_t k_prev,
+                            const uint8_t *d_prev_codes, int32_t *h_iters_run, int32_t *h_reseeds_used);
+
 /* *h_out = (sum_i sqrt(sum_t x[i][t]^2)) / n — the early-stop statistic of src/rvq.rs:131-138.
  * Row norms follow the reference's sequential f32 order; the sum over rows (a Rayon sum of
  * unspecified order in the reference) is a fixed-shape f64 tree.  Synchronises. */

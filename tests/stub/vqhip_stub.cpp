@@ -162,6 +162,14 @@ int32_t vq_residual_sub_u16(vq_ctx *, float *res, int64_t n, int64_t ld, int32_t
                             const uint16_t *codes) {
     return residual_any(res, n, ld, dim, k, cb, codes);
 }
+int32_t vq_lbg_fit_residual(vq_ctx *c, float *res, int64_t n, int64_t ld, int32_t dim, int32_t k, int32_t iters,
+                            const uint32_t *init, const uint32_t *reseed, int32_t n_reseed, float *cb,
+                            const float *prev_cb, int32_t k_prev, const uint8_t *prev_codes, int32_t *iters_run,
+                            int32_t *used) {
+    const int32_t rc = vq_residual_sub(c, res, n, ld, dim, k_prev, prev_cb, prev_codes);
+    if (rc != VQ_OK) return rc;
+    return vq_lbg_fit(c, res, n, ld, 1, dim, k, iters, init, reseed, n_reseed, cb, iters_run, used);
+}
 int32_t vq_mean_l2norm(vq_ctx *, const float *x, int64_t n, int64_t ld, int32_t dim, float *out) {
     double s = 0;
     for (int64_t i = 0; i < n; ++i) {

@@ -42,6 +42,72 @@ def gpu_rvq_fit(ctx, metric, x, stages, k, iters, eps, init, reseed):
     return dcb.download()[:produced], dres.download(), np.array(norms, F), dcb
 
 
+@pytest.mark.parametrize("n,dim,ld,k,k_prev,iters,kind", [
+    (5000, 256, 256, 256, 256, 3, "normal"),   # the RVQ stage shape: the first pass applies the update
+    (1000, 40, 40, 7, 5, 4, "normal"),         # an odd multiple of 8: the last stage's upper half is past the width
+    (333, 16, 24, 3, 200, 2, "normal"),        # rows inside a wider buffer, n not a multiple of 128
+    (4097, 128, 128, 64, 1, 3, "integers"),    # exact ties; a previous codebook of one centroid
+    (700, 64, 64, 16, 9, 2, "nonfinite"),
+    (900, 72, 72, 5, 4, 0, "normal"),          # no pass to ride on: the two steps one after the other
+    (900, 12, 12, 5, 4, 3, "normal"),          # a width without the matrix-core pass: the same
+    (600, 8, 8, 4, 3, 3, "normal"),            # the 8-float kernel: the same
+])
+def test_lbg_fit_residual_equals_the_two_steps(ctx, n, dim, ld, k, k_prev, iters, kind):
+    """vq_lbg_fit_residual = vq_residual_sub, then vq_lbg_fit: same residual, codebook, iteration and
+    re-seed counts, bit for bit, on the shapes where the first pass applies the update and on those
+    where it cannot; and the oracle's residual update and fit on the same inputs."""
+    rng = np.random.default_rng(n + dim + k)
+    if kind == "integers":
+        x = np.round(rng.standard_normal((n, ld)) * 2).astype(F)
+        prev = np.round(rng.standard_normal((k_prev, dim)) * 2).astype(F)
+    else:
+        x = rng.standard_normal((n, ld)).astype(F)
+        prev = rng.standard_normal((k_prev, dim)).astype(F)
+    if kind == "nonfinite":
+        x[::17, 3] = np.inf
+        x[5::29, 11] = np.nan
+        prev[2, 7] = -np.inf
+    codes = rng.integers(0, k_prev, n).astype(np.uint8)
+    init, reseed = data.index_streams(n, 1, k, max(iters, 1), seed=n)
+    dprev, dcodes = ctx.to_device(prev), ctx.to_device(codes)
+    # the two steps
+    da = ctx.to_device(x)
+    cba = ctx.empty((k, dim), F)
+    ctx.residual_sub(da, n, ld, dim, k_prev, dprev, dcodes)
+    it_a, used_a = ctx.lbg_fit(da, n, ld, 1, dim, k, iters, init[0], reseed[0], cba)
+    # the one call
+    db = ctx.to_device(x)
+    cbb = ctx.empty((k, dim), F)
+    it_b, used_b = ctx.lbg_fit_residual(db, n, ld, dim, k, iters, init[0], reseed[0], cbb, dprev, k_prev, dcodes)
+    ra, rb = da.download(), db.download()
+    assert np.array_equal(ra.view(np.uint32), rb.view(np.uint32))
+    assert np.array_equal(cba.download().view(np.uint32), cbb.download().view(np.uint32))
+    assert np.array_equal(it_a, it_b) and np.array_equal(used_a, used_b)
+    # against the arithmetic itself: one f32 subtraction per element (src/rvq.rs:127), columns past dim untouched
+    if kind != "nonfinite":  # (the bits of a NaN that a subtraction makes differ between CPU and GPU)
+        want = x.copy()
+        want[:, :dim] = x[:, :dim] - prev[codes]
+        assert np.array_equal(rb.view(np.uint32), want.view(np.uint32))
+        ref = O.pq_fit(np.ascontiguousarray(want[:, :dim]), 1, k, iters, init, reseed)
+        assert np.array_equal(cbb.download().view(np.uint32), ref["codebooks"].reshape(k, dim).view(np.uint32))
+    for b in (dprev, dcodes, da, db, cba, cbb):
+        b.free()
+
+
+def test_lbg_fit_residual_argument_errors(ctx):
+    import vq_amd
+    x = np.zeros((100, 16), F)
+    d, cb, prev, codes = ctx.to_device(x), ctx.empty((4, 16), F), ctx.to_device(np.zeros((4, 16), F)), \
+        ctx.to_device(np.zeros(100, np.uint8))
+    init, reseed = data.index_streams(100, 1, 4, 2, seed=1)
+    with pytest.raises(vq_amd.VqError):
+        ctx.lbg_fit_residual(d, 100, 16, 16, 4, 2, init[0], reseed[0], cb, 0, 4, codes)  # no previous codebook
+    with pytest.raises(vq_amd.VqError):
+        ctx.lbg_fit_residual(d, 100, 16, 16, 4, 2, init[0], reseed[0], cb, prev, 300, codes)  # codes are 8-bit
+    with pytest.raises(vq_amd.VqError):
+        ctx.lbg_fit_residual(d, 3, 16, 16, 4, 2, init[0], reseed[0], cb, prev, 4, codes)  # fewer rows than clusters
+
+
 @pytest.mark.parametrize("metric", [O.SQEUCLIDEAN, O.EUCLIDEAN, O.COSINE, O.MANHATTAN])
 @pytest.mark.parametrize("n,dim,stages,k,iters", [(1000, 10, 2, 2, 50), (600, 32, 3, 16, 5),
                                                     (400, 256, 2, 8, 3), (3000, 6, 2, 2, 4)])

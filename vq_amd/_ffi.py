@@ -48,6 +48,8 @@ SYMBOLS = {
     "vq_prof_read": (_i32, [_vp, _i32, C.POINTER(C.c_double), C.POINTER(_i64)]),
     "vq_lbg_fit": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp,
                           _vp]),
+    "vq_lbg_fit_residual": (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp, _i32, _vp,
+                                   _vp, _vp]),
     "vq_assign": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_assign_noalloc": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
     "vq_assign_u16": (_i32, [_vp, _i32, _vp, _i64, _i64, _i32, _i32, _i32, _vp, _vp]),
@@ -302,6 +304,21 @@ class Context:
                                     init_idx.ctypes.data, reseed_stream.ctypes.data if n_reseed
                                     else None, n_reseed, _ptr(d_codebooks), iters.ctypes.data,
                                     used.ctypes.data))
+        return iters, used
+
+    def lbg_fit_residual(self, d_res, n, ld, dim, k, max_iters, init_idx, reseed_stream, d_codebook,
+                         d_prev_codebook, k_prev, d_prev_codes):
+        """d_res[i] -= d_prev_codebook[d_prev_codes[i]], then lbg_fit (m = 1) on the updated rows."""
+        init_idx = np.ascontiguousarray(init_idx, np.uint32).reshape(-1)
+        reseed_stream = np.ascontiguousarray(reseed_stream, np.uint32).reshape(1, -1) \
+            if np.size(reseed_stream) else np.zeros((1, 0), np.uint32)
+        n_reseed = reseed_stream.shape[1]
+        iters = np.zeros(1, np.int32)
+        used = np.zeros(1, np.int32)
+        self._check(_lib.vq_lbg_fit_residual(self._h, _ptr(d_res), n, ld, dim, k, max_iters,
+                                             init_idx.ctypes.data, reseed_stream.ctypes.data if n_reseed
+                                             else None, n_reseed, _ptr(d_codebook), _ptr(d_prev_codebook),
+                                             k_prev, _ptr(d_prev_codes), iters.ctypes.data, used.ctypes.data))
         return iters, used
 
     def assign(self, metric, d_x, n, ld, m, sub_dim, k, d_codebooks, d_codes):

@@ -810,8 +810,14 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // grid (ceil(n/128), m); 256 threads = 4 waves, one tile of 32 rows each against every centroid.
 // NB = tiles of 32 centroids (tb.nb), a template parameter so that the chains of matrix
 // instructions are straight-line code.
-template <bool LBG, int NB>
+// PEND (LBG mode, one column block): the rows are a residual whose update by the previous stage's
+// codebook is still pending, x[i] -= pend_cb[pend_codes[i]] (src/rvq.rs:124-129).  A workgroup first
+// updates its own 128 rows in place — whole rows per wave instruction, one f32 subtraction per
+// element, as the separate pass would — and then scores them as any other rows, which it now reads
+// from the cache levels it has just written through.  No other workgroup reads or writes these rows.
+template <bool LBG, int NB, bool PEND = false>
 __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, MfmaWideBfTables tb) {
+    static_assert(!PEND || LBG, "a pending residual update belongs to the first pass of an LBG fit");
     constexpr int NBMAX = 8;
     __shared__ u32x4 lds_a[2][NBMAX * 128];  // 2 stages x 16 dimensions x 256 centroids x {high, low}: 2 x 16 KB
     __shared__ float lds_c2[NBMAX * 32];
@@ -837,7 +843,34 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
     }
     if (tb.shifted[s] != 0)
         for (int i = threadIdx.x; i < sd; i += 256) lds_mu[i] = tb.mu[(size_t)s * sd + i];
-    __syncthreads();
+    if constexpr (PEND) {
+        const int64_t row0 = (int64_t)blockIdx.x * 128;
+        const int nrows = a.n - row0 < 128 ? (int)(a.n - row0) : 128;
+        float *xw = const_cast<float *>(a.x) + row0 * a.ld;
+        const uint8_t *pc = a.pend_codes + row0;
+        const int per_row = sd / 4, total = nrows * per_row;  // 16-byte pieces
+        constexpr int B = 8;  // pieces of a thread in flight together
+        for (int i0 = threadIdx.x; i0 < total; i0 += 256 * B) {
+            float4 v[B], c[B];
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+                const int i = i0 + 256 * u < total ? i0 + 256 * u : i0;
+                const int rr = i / per_row, cc = i - rr * per_row;
+                v[u] = *reinterpret_cast<const float4 *>(xw + (int64_t)rr * a.ld + 4 * cc);
+                c[u] = *reinterpret_cast<const float4 *>(a.pend_cb + (size_t)pc[rr] * sd + 4 * cc);
+            }
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+                const int i = i0 + 256 * u;
+                if (i < total) {
+                    const int rr = i / per_row, cc = i - rr * per_row;
+                    *reinterpret_cast<float4 *>(xw + (int64_t)rr * a.ld + 4 * cc) =
+                        make_float4(v[u].x - c[u].x, v[u].y - c[u].y, v[u].z - c[u].z, v[u].w - c[u].w);
+                }
+            }
+        }
+    }
+    __syncthreads();  // (PEND: the updated rows are visible to every wave of the workgroup)
 
     const int64_t row = (int64_t)blockIdx.x * 128 + wave * 32 + r;
     const bool valid = row < a.n;

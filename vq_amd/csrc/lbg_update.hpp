@@ -86,6 +86,18 @@ static __global__ void k_gather_rows(const float *__restrict__ x, int64_t ld, in
     cb[i] = x[(int64_t)idx[sj] * ld + (int64_t)s * sd + t];
 }
 
+// The same from a residual whose update is still pending (one column block):
+// codebook[j][t] = x[idx[j]][t] - pend_cb[pend_codes[idx[j]]][t], the row as the update will leave it.
+static __global__ void k_gather_rows_pend(const float *__restrict__ x, int64_t ld, int k, int sd,
+                                          const uint32_t *__restrict__ idx, float *__restrict__ cb,
+                                          const float *__restrict__ pend_cb, const uint8_t *__restrict__ pend_codes) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)k * sd) return;
+    const int t = (int)(i % sd);
+    const uint32_t row = idx[i / sd];
+    cb[i] = x[(int64_t)row * ld + t] - pend_cb[(size_t)pend_codes[row] * sd + t];
+}
+
 // One wave per (part, column block): histogram of the codes of kPartRows rows.
 static __global__ void __launch_bounds__(64) k_lbg_hist(LbgState st, int64_t n) {
     side_chain_priority();

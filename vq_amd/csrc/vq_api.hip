@@ -279,8 +279,12 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     {
         ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
 #define WIDE(NB)                                                                                             \
-    hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG, NB>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0, \
-                       ctx->stream, a, tb)
+    if (LBG && a.pend_cb)                                                                                    \
+        hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG, NB, LBG>), dim3(cdiv(a.n, 128), (unsigned)a.m),     \
+                           dim3(256), 0, ctx->stream, a, tb);                                                \
+    else                                                                                                     \
+        hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG, NB>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0, \
+                           ctx->stream, a, tb)
         switch (nb) {
         case 1: WIDE(1); break;
         case 2: WIDE(2); break;
@@ -1029,10 +1033,14 @@ int32_t vq_copy_f32(vq_ctx *ctx, float *d_dst, const float *d_src, int64_t count
     return VQ_OK;
 }
 
-int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t m, int32_t sd,
-                   int32_t k, int32_t max_iters, const uint32_t *h_init_idx,
-                   const uint32_t *h_reseed_stream, int32_t n_reseed, float *d_codebooks,
-                   int32_t *h_iters_run, int32_t *h_reseeds_used) {
+// pend_cb / pend_codes: a residual update x[i] -= pend_cb[pend_codes[i]] that the fit applies to the
+// rows in place as its first assignment pass reads them (the caller has checked that this shape's
+// first pass is the kernel that can: lbg_pending_fusable).
+static int32_t lbg_fit_impl(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t m, int32_t sd,
+                            int32_t k, int32_t max_iters, const uint32_t *h_init_idx,
+                            const uint32_t *h_reseed_stream, int32_t n_reseed, float *d_codebooks,
+                            int32_t *h_iters_run, int32_t *h_reseeds_used, const float *pend_cb,
+                            const uint8_t *pend_codes) {
     if (!ctx) return VQ_ERR_INVALID_ARG;
     if (k == 0) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: k must be greater than 0");
     VQ_TRY(check_common(ctx, d_x, n, ld, m, sd, k, 65536));
@@ -1109,8 +1117,12 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
                                    sizeof(uint32_t) * (size_t)m * n_reseed, hipMemcpyHostToDevice, st));
     VQ_HIP(ctx, hipMemsetAsync(S.codes, 0, (size_t)m * n, st));  // assignments = vec![0; n], utils.rs:55
     hipLaunchKernelGGL(vq::k_lbg_init, dim3(cdiv(m, 64)), dim3(64), 0, st, S, m);
-    hipLaunchKernelGGL(vq::k_gather_rows, dim3(cdiv((int64_t)m * k * sd, 256)), dim3(256), 0, st, d_x,
-                       ld, m, k, sd, (const uint32_t *)ctx->idx.p, d_codebooks);
+    if (pend_cb)
+        hipLaunchKernelGGL(vq::k_gather_rows_pend, dim3(cdiv((int64_t)k * sd, 256)), dim3(256), 0, st, d_x, ld, k, sd,
+                           (const uint32_t *)ctx->idx.p, d_codebooks, pend_cb, pend_codes);
+    else
+        hipLaunchKernelGGL(vq::k_gather_rows, dim3(cdiv((int64_t)m * k * sd, 256)), dim3(256), 0, st, d_x,
+                           ld, m, k, sd, (const uint32_t *)ctx->idx.p, d_codebooks);
     VQ_HIP(ctx, hipGetLastError());
 
     vq::AssignArgs a;
@@ -1136,6 +1148,8 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
     hipEvent_t prev_done = nullptr;
     for (int it = 0; it < max_iters; ++it) {
         hipEvent_t started = nullptr, done = nullptr;
+        a.pend_cb = it == 0 ? pend_cb : nullptr;  // the first pass leaves the rows updated
+        a.pend_codes = it == 0 ? pend_codes : nullptr;
         {
             ProfSpan sp(ctx, fused_tail ? -1 : VQ_PROF_LBG_ASSIGN);
             VQ_TRY(launch_assign<true>(ctx, VQ_SQEUCLIDEAN, a, sd, fused_tail && it > 0, &started, &done));
@@ -1217,6 +1231,44 @@ int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t
         return fail(ctx, VQ_ERR_RESEED_EXHAUSTED,
                     "re-seed stream exhausted: pass n_reseed = k*max_iters");
     return VQ_OK;
+}
+
+int32_t vq_lbg_fit(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld, int32_t m, int32_t sd,
+                   int32_t k, int32_t max_iters, const uint32_t *h_init_idx,
+                   const uint32_t *h_reseed_stream, int32_t n_reseed, float *d_codebooks,
+                   int32_t *h_iters_run, int32_t *h_reseeds_used) {
+    return lbg_fit_impl(ctx, d_x, n, ld, m, sd, k, max_iters, h_init_idx, h_reseed_stream, n_reseed, d_codebooks,
+                        h_iters_run, h_reseeds_used, nullptr, nullptr);
+}
+
+int32_t vq_lbg_fit_residual(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t dim, int32_t k,
+                            int32_t max_iters, const uint32_t *h_init_idx, const uint32_t *h_reseed_stream,
+                            int32_t n_reseed, float *d_codebook, const float *d_prev_codebook, int32_t k_prev,
+                            const uint8_t *d_prev_codes, int32_t *h_iters_run, int32_t *h_reseeds_used) {
+    if (!ctx) return VQ_ERR_INVALID_ARG;
+    if (!d_prev_codebook || !d_prev_codes || k_prev <= 0 || k_prev > 256)
+        return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: the previous stage's codebook and codes");
+    // The first assignment pass can apply the update as it reads the rows when it is the matrix-core
+    // pass over one wide column block and there is a first pass; the arguments the fused path does
+    // not check itself are checked by the two calls of the other path.
+    vq::AssignArgs a;
+    a.x = d_res;
+    a.n = n;
+    a.ld = ld;
+    a.m = 1;
+    a.k = k;
+    a.cb = d_codebook;
+    const bool fusable = d_res && d_codebook && n >= k && k >= 1 && k <= vq::kMaxK && dim >= 16 && ld >= dim &&
+                         max_iters >= 1 && (reinterpret_cast<uintptr_t>(d_prev_codebook) & 15) == 0 &&
+                         mfma_wide_applicable<vq::M_SQ, true>(ctx, a, dim) &&
+                         !mfma_applicable<vq::M_SQ, true>(ctx, a, dim);
+    if (!fusable) {
+        VQ_TRY(vq_residual_sub(ctx, d_res, n, ld, dim, k_prev, d_prev_codebook, d_prev_codes));
+        return lbg_fit_impl(ctx, d_res, n, ld, 1, dim, k, max_iters, h_init_idx, h_reseed_stream, n_reseed,
+                            d_codebook, h_iters_run, h_reseeds_used, nullptr, nullptr);
+    }
+    return lbg_fit_impl(ctx, d_res, n, ld, 1, dim, k, max_iters, h_init_idx, h_reseed_stream, n_reseed, d_codebook,
+                        h_iters_run, h_reseeds_used, d_prev_codebook, d_prev_codes);
 }
 
 int32_t vq_assign(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,

@@ -611,12 +611,21 @@ public:
         q.codebooks_ = DeviceBuffer<float>(dev, std::max<size_t>(stages * k * dim, 1));
         std::vector<uint8_t> zeros(n, 0);
         size_t produced = 0;
+        const float *pending_cb = nullptr;  // a residual update that rides on the next stage's fit
         for (size_t st = 0; st < stages; ++st) {
             float *cb = q.codebooks_.get() + st * k * dim;
-            dev->check(vq_lbg_fit(c, dres.get(), (int64_t)n, (int64_t)dim, 1, (int32_t)dim, (int32_t)k,
-                                  (int32_t)max_iters, streams->init.data() + st * k,
-                                  streams->reseed.data() + st * (size_t)streams->n_reseed, streams->n_reseed, cb,
-                                  nullptr, nullptr));  // rvq.rs:107
+            if (pending_cb)  // rvq.rs:127 of the stage before, then rvq.rs:107
+                dev->check(vq_lbg_fit_residual(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)k,
+                                               (int32_t)max_iters, streams->init.data() + st * k,
+                                               streams->reseed.data() + st * (size_t)streams->n_reseed,
+                                               streams->n_reseed, cb, pending_cb, (int32_t)k, dcodes.p8(), nullptr,
+                                               nullptr));
+            else
+                dev->check(vq_lbg_fit(c, dres.get(), (int64_t)n, (int64_t)dim, 1, (int32_t)dim, (int32_t)k,
+                                      (int32_t)max_iters, streams->init.data() + st * k,
+                                      streams->reseed.data() + st * (size_t)streams->n_reseed, streams->n_reseed, cb,
+                                      nullptr, nullptr));  // rvq.rs:107
+            pending_cb = nullptr;
             ++produced;
             // The residuals are a local of the reference's fit (rvq.rs:103) and nothing follows the
             // last stage: its residual update and norm test (111-141) cannot be observed and are left out.
@@ -625,6 +634,12 @@ public:
                 dcodes.narrow().upload(zeros.data(), n);
             else
                 dev->check(abi_assign(c, metric, dres.get(), n, dim, 1, dim, k, cb, dcodes));  // rvq.rs:116-125
+            if (!dcodes.wide() && !(epsilon > 0.f)) {
+                // nothing looks at the residual before the next stage trains on it: the update is
+                // handed to that fit, whose first pass over the rows applies it
+                pending_cb = cb;
+                continue;
+            }
             dev->check(dcodes.wide()
                            ? vq_residual_sub_u16(c, dres.get(), (int64_t)n, (int64_t)dim, (int32_t)dim, (int32_t)k, cb,
                                                  dcodes.p16())
