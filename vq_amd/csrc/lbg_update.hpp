@@ -335,18 +335,21 @@ static __global__ void __launch_bounds__(64) k_lbg_scatter(LbgState st, int64_t 
     }
 }
 
-// The same scatter by a workgroup of four waves per (part, column block), for the shapes whose
-// every row is listed (no streaming sums): wave w ranks the rows [1024 w, 1024 w + 1024) of the
-// part.  A first sweep counts the codes of each quarter, so that a wave's first position inside
-// cluster j is the part's position plus the members in the quarters before its own; the order of
-// the rows inside a cluster stays the row order.  One wave per part is a chain of 64 dependent
-// LDS round trips per part and a handful of waves on the whole GPU when there is one column block.
+// The same scatter by a workgroup of four waves per (part, column block): wave w ranks the rows
+// [1024 w, 1024 w + 1024) of the part.  A first sweep counts the listed codes of each quarter, so
+// that a wave's first position inside cluster j is the part's position plus the members in the
+// quarters before its own; the order of the rows inside a cluster stays the row order.  One wave
+// per part is a chain of 64 dependent LDS round trips per part (and a handful of waves on the whole
+// GPU when there is one column block).
 static __global__ void __launch_bounds__(256) k_lbg_scatter_wg(LbgState st, int64_t n) {
+    side_chain_priority();
     const int s = blockIdx.y, b = blockIdx.x;
     if (st.done[s]) return;
+    if (st.stream && st.nsmall[s] == 0) return;
     constexpr int kQuarter = kPartRows / 4;
     __shared__ uint32_t cntq[4][kMaxK];
     __shared__ uint32_t base[4][kMaxK];
+    __shared__ uint8_t listed[kMaxK];
     __shared__ __attribute__((aligned(16))) uint8_t pcodes[kPartRows];
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const uint8_t *codes = st.codes + (size_t)s * n;
@@ -355,6 +358,7 @@ static __global__ void __launch_bounds__(256) k_lbg_scatter_wg(LbgState st, int6
     const int64_t hi = lo + kPartRows < n ? lo + kPartRows : n;
     const int rows = (int)(hi - lo);
     for (int j = threadIdx.x; j < 4 * kMaxK; j += 256) (&cntq[0][0])[j] = 0u;
+    listed[threadIdx.x] = (!st.stream || st.count[(size_t)s * kMaxK + threadIdx.x] <= (uint32_t)kSeqMax) ? 1 : 0;
     // the part's codes into LDS, 16 per thread
     {
         const int64_t r0 = lo + 16 * (int64_t)threadIdx.x;
@@ -371,7 +375,10 @@ static __global__ void __launch_bounds__(256) k_lbg_scatter_wg(LbgState st, int6
     }
     __syncthreads();
     const int q0 = w * kQuarter, q1 = q0 + kQuarter < rows ? q0 + kQuarter : rows;
-    for (int i = q0 + lane; i < q1; i += 64) atomicAdd(&cntq[w][pcodes[i]], 1u);
+    for (int i = q0 + lane; i < q1; i += 64) {
+        const uint32_t c = pcodes[i];
+        if (listed[c]) atomicAdd(&cntq[w][c], 1u);
+    }
     __syncthreads();
     {
         const uint32_t *h = st.hist + ((size_t)s * st.nparts + b) * kMaxK;
@@ -389,9 +396,11 @@ static __global__ void __launch_bounds__(256) k_lbg_scatter_wg(LbgState st, int6
     const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     for (int i0 = q0; i0 < q1; i0 += 64) {
         const int i = i0 + lane;
-        const bool valid = i < q1;
+        bool valid = i < q1;
         const uint32_t c = valid ? pcodes[i] : 0u;
+        valid = valid && listed[c];
         uint64_t mask = __ballot(valid);
+        if (mask == 0) continue;  // uniform
 #pragma unroll
         for (int bit = 0; bit < 8; ++bit) {
             const bool set = (c >> bit) & 1u;

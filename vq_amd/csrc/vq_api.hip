@@ -1180,7 +1180,7 @@ static int32_t lbg_fit_impl(vq_ctx *ctx, const float *d_x, int64_t n, int64_t ld
         hipLaunchKernelGGL(vq::k_lbg_scan_seg, dim3(nseg, m), dim3(256), 0, gs, S);
         hipLaunchKernelGGL(vq::k_lbg_plan, dim3(m), dim3(256), 0, gs, S, k);
         hipLaunchKernelGGL(vq::k_lbg_scan_blocks, dim3(nseg, m), dim3(256), 0, gs, S);
-        if (stream)
+        if (stream)  // beside the streaming kernel: one wave per part (four waves per part take its resources: 40 us, and 15 us more for the streaming kernel)
             hipLaunchKernelGGL(vq::k_lbg_scatter, dim3(nparts, m), dim3(64), 0, gs, S, n);
         else  // every row is listed: four waves per part
             hipLaunchKernelGGL(vq::k_lbg_scatter_wg, dim3(nparts, m), dim3(256), 0, gs, S, n);
