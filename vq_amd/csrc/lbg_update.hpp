@@ -234,16 +234,15 @@ static __global__ void __launch_bounds__(256) k_lbg_scan_blocks(LbgState st) {
     const bool leaves = !st.stream && st.count[sj] > (uint32_t)kSeqMax;
     const uint32_t first = st.start[sj];
     uint2 *desc = st.leaf_desc + (size_t)s * st.leaf_cap + st.leaf_start[sj] + b0;
-    for (int c0 = 0; c0 < b1 - b0; c0 += 8) {
-        uint32_t v[8];
+    // the segment's entries in one memory round trip (unconditional loads, clamped to the last part)
+    uint32_t v[kScanSeg];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = (b0 + c0 + u < b1) ? h[(size_t)(c0 + u) * kMaxK] : 0u;
+    for (int u = 0; u < kScanSeg; ++u) v[u] = h[(size_t)(b0 + u < b1 ? u : b1 - 1 - b0) * kMaxK];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            if (b0 + c0 + u < b1) {
-                h[(size_t)(c0 + u) * kMaxK] = run;
-                if (leaves) desc[c0 + u] = make_uint2(first + run, first + run + v[u]);
-            }
+    for (int u = 0; u < kScanSeg; ++u) {
+        if (b0 + u < b1) {
+            h[(size_t)u * kMaxK] = run;
+            if (leaves) desc[u] = make_uint2(first + run, first + run + v[u]);
             run += v[u];
         }
     }
