@@ -158,6 +158,53 @@ def test_rvq_quantize_epsilon_stops_rows_individually(ctx):
     assert np.array_equal(drec.download(), wrec)
 
 
+@pytest.mark.parametrize("n,dim,ld,stages,k,eps,metric", [
+    (3000, 256, 256, 1, 256, 0.0, O.EUCLIDEAN),    # one stage: no residual at all
+    (3000, 256, 256, 4, 256, 0.0, O.EUCLIDEAN),    # the stage shape of the wide pass
+    (1500, 64, 80, 3, 16, 0.0, O.SQEUCLIDEAN),     # rows inside a wider buffer, read where they lie
+    (1500, 64, 70, 3, 16, 0.0, O.COSINE),          # a row stride that is no multiple of 4: copied first
+    (1500, 64, 70, 3, 16, 0.0, O.SQEUCLIDEAN),     # ... and the updates ride on the next stage's pass, in place
+    (2100, 40, 44, 5, 7, 0.0, O.EUCLIDEAN),        # five stages of an odd multiple of 8 floats
+    (130, 16, 16, 2, 2, 0.0, O.SQEUCLIDEAN),
+    (5000, 24, 24, 3, 256, float("nan"), O.EUCLIDEAN),  # a threshold that no norm is below
+    (901, 30, 33, 2, 5, 0.0, O.MANHATTAN),         # a width that is no multiple of 4
+    (901, 30, 33, 1, 5, 0.0, O.MANHATTAN),
+    (2000, 32, 48, 4, 8, 4.5, O.EUCLIDEAN),        # rows stop at different stages
+    (2000, 32, 32, 1, 8, 100.0, O.EUCLIDEAN),      # every row stops after the one stage
+    (700, 16, 16, 3, 1, 0.0, O.EUCLIDEAN),         # one centroid per stage
+    (1200, 128, 128, 2, 300, 0.0, O.EUCLIDEAN),    # 16-bit codes
+    (1200, 128, 132, 1, 300, 0.0, O.SQEUCLIDEAN),
+])
+def test_rvq_encode_first_and_last_stage_paths(ctx, n, dim, ld, stages, k, eps, metric):
+    """vq_rvq_encode against the oracle where the first stage reads the caller's rows in place (or cannot)
+    and the last stage only records its codes; the caller's buffer stays as it was."""
+    rng = np.random.default_rng(n + dim + ld + stages)
+    buf = rng.standard_normal((n, ld)).astype(F)
+    cb = (rng.standard_normal((stages, k, dim)) * np.array([1.0, 0.6, 0.4, 0.3, 0.2])[:stages, None, None]).astype(F)
+    if eps > 0:  # rows at different distances from a first-stage centroid
+        buf[:, :dim] = cb[0][rng.integers(0, k, n)] + buf[:, :dim] * rng.uniform(0.3, 1.5, (n, 1)).astype(F)
+    x = np.ascontiguousarray(buf[:, :dim])
+    wcodes, wrec = O.rvq_quantize(metric, x, cb, eps)
+    dx, dcb = ctx.to_device(buf), ctx.to_device(cb)
+    wide = k > 256
+    dcodes = ctx.empty((n, stages), np.uint16 if wide else np.uint8)
+    dused = ctx.empty(n, np.uint8)
+    drec = ctx.empty((n, dim), np.uint16)
+    (ctx.rvq_encode_u16 if wide else ctx.rvq_encode)(metric, dx, n, ld, dim, stages, k, dcb, eps, dcodes, dused, drec)
+    used = dused.download()
+    reached = wcodes != 0xFFFFFFFF
+    assert np.array_equal(used, reached.sum(1))
+    if eps == 4.5:
+        assert used.min() < used.max()
+    got = dcodes.download()
+    assert np.array_equal(got[reached], wcodes[reached].astype(got.dtype))
+    assert np.all(got[~reached] == 0)
+    assert np.array_equal(drec.download(), wrec)
+    assert np.array_equal(dx.download().view(np.uint32), buf.view(np.uint32))
+    for b in (dx, dcb, dcodes, dused, drec):
+        b.free()
+
+
 def test_rvq_k1_and_early_training_stop(ctx):
     x = np.tile(np.array([[1, 2, 3, 4]], F), (20, 1))
     init = np.array([[0, 1], [0, 1], [0, 1]], np.uint32)

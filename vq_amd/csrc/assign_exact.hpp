@@ -28,11 +28,14 @@ struct AssignArgs {
     int *changed;         // LBG mode: changed[s] set to 1 when any code of block s differs
     const int *done;      // LBG mode: blocks with done[s] != 0 are skipped
     float *dist = nullptr;  // encode mode, k_assign_mfma_bf only: [n][m] distance of the chosen centroid, or null
-    // A residual update that the pass applies as it reads the rows (single wide column block, LBG
-    // mode, k_assign_mfma_wide_bf only): x[i] -= pend_cb[pend_codes[i]] is computed on the values a
-    // lane has just loaded, used, and written back in place.  Null: the rows are read as they are.
+    // A residual update that the pass applies before it scores the rows (single wide column block,
+    // k_assign_mfma_wide_bf only): x[i] = src[i] - pend_cb[pend_codes[i]], where src is the rows
+    // themselves (an update in place) or, pend_src != null, other rows of stride pend_src_ld that
+    // stay as they are.  pend_cb null: the rows are read as they are.
     const float *pend_cb = nullptr;
     const uint8_t *pend_codes = nullptr;
+    const float *pend_src = nullptr;
+    int64_t pend_src_ld = 0;
 };
 
 // Called by the lanes of a wave that changed a code.  Every store to one address is serialised

@@ -810,14 +810,14 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // grid (ceil(n/128), m); 256 threads = 4 waves, one tile of 32 rows each against every centroid.
 // NB = tiles of 32 centroids (tb.nb), a template parameter so that the chains of matrix
 // instructions are straight-line code.
-// PEND (LBG mode, one column block): the rows are a residual whose update by the previous stage's
-// codebook is still pending, x[i] -= pend_cb[pend_codes[i]] (src/rvq.rs:124-129).  A workgroup first
-// updates its own 128 rows in place — whole rows per wave instruction, one f32 subtraction per
-// element, as the separate pass would — and then scores them as any other rows, which it now reads
-// from the cache levels it has just written through.  No other workgroup reads or writes these rows.
+// PEND (one column block): the rows are a residual whose update by the previous stage's codebook is
+// still pending, x[i] -= pend_cb[pend_codes[i]] (src/rvq.rs:124-129 in a fit, 200-202 in an encode).
+// A workgroup first updates its own 128 rows — whole rows per wave instruction, one f32 subtraction
+// per element, as the separate pass would; in place, or from the rows of a.pend_src into a.x — and
+// then scores them as any other rows, which it now reads from the cache levels it has just written
+// through.  No other workgroup reads or writes these rows.
 template <bool LBG, int NB, bool PEND = false>
 __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, MfmaWideBfTables tb) {
-    static_assert(!PEND || LBG, "a pending residual update belongs to the first pass of an LBG fit");
     constexpr int NBMAX = 8;
     __shared__ u32x4 lds_a[2][NBMAX * 128];  // 2 stages x 16 dimensions x 256 centroids x {high, low}: 2 x 16 KB
     __shared__ float lds_c2[NBMAX * 32];
@@ -847,6 +847,8 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
         const int64_t row0 = (int64_t)blockIdx.x * 128;
         const int nrows = a.n - row0 < 128 ? (int)(a.n - row0) : 128;
         float *xw = const_cast<float *>(a.x) + row0 * a.ld;
+        const float *xr = a.pend_src ? a.pend_src + row0 * a.pend_src_ld : xw;
+        const int64_t xr_ld = a.pend_src ? a.pend_src_ld : a.ld;
         const uint8_t *pc = a.pend_codes + row0;
         const int per_row = sd / 4, total = nrows * per_row;  // 16-byte pieces
         constexpr int B = 8;  // pieces of a thread in flight together
@@ -856,7 +858,7 @@ __global__ void __launch_bounds__(256, 2) k_assign_mfma_wide_bf(AssignArgs a, Mf
             for (int u = 0; u < B; ++u) {
                 const int i = i0 + 256 * u < total ? i0 + 256 * u : i0;
                 const int rr = i / per_row, cc = i - rr * per_row;
-                v[u] = *reinterpret_cast<const float4 *>(xw + (int64_t)rr * a.ld + 4 * cc);
+                v[u] = *reinterpret_cast<const float4 *>(xr + (int64_t)rr * xr_ld + 4 * cc);
                 c[u] = *reinterpret_cast<const float4 *>(a.pend_cb + (size_t)pc[rr] * sd + 4 * cc);
             }
 #pragma unroll

@@ -176,9 +176,23 @@ int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t 
 // Launchers defined in vq_api.hip, used by the RVQ / OPQ entry points.
 // d_dist (optional, n x m floats): receives the chosen centroids' distances where the kernel that runs
 // computes them anyway; *dist_written says whether it did.
+// pend (optional; one column block, and only where assign_pending_fusable says so): a residual
+// update that the pass applies to the rows before it scores them, d_x[i] = src[i] - cb[codes[i]]
+// with src = the rows of d_x themselves (src null: d_x is updated in place) or other rows of stride
+// src_ld that stay as they are.
+struct PendingUpdate {
+    const float *cb;
+    const uint8_t *codes;
+    const float *src;
+    int64_t src_ld;
+};
 int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                      int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes, float *d_dist = nullptr,
-                     bool *dist_written = nullptr);
+                     bool *dist_written = nullptr, const PendingUpdate *pend = nullptr);
+// Whether the assignment of these rows (one column block of sd floats) runs on the pass that can
+// take a pending update along.
+bool assign_pending_fusable(const vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t sd,
+                            int32_t k, const float *d_codebook);
 
 // Defined in vq_api_bigk.hip: the same for any k up to 65536 with 16-bit codes, and the LBG above
 // 256 centroids (arguments as vq_lbg_fit, already validated).

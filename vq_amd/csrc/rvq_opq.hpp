@@ -24,14 +24,17 @@ static __global__ void __launch_bounds__(256) k_residual_sub(float *__restrict__
 // The same, four components per lane (dim and ld multiples of 4, 16-byte aligned pointers); a
 // workgroup covers 1024 consecutive float4 of the n x dim/4 grid.  active == nullptr: every row.
 // codes_out / used (both or neither): RVQ encode bookkeeping of the stage, written by the lane
-// that holds a row's first components (src/rvq.rs:196-202).
+// that holds a row's first components (src/rvq.rs:196-202).  The rows are read from src (row
+// stride src_ld floats) and written to res: the same buffer for an update in place, or the
+// caller's rows for the first stage of an encode, whose inactive rows do not occur.
 template <typename CodeT>
-static __global__ void __launch_bounds__(256) k_residual_sub4(float *__restrict__ res, int64_t n, int64_t ld,
-                                                       int dim4, const float *__restrict__ cb,
+static __global__ void __launch_bounds__(256) k_residual_sub4(float *res, int64_t n, int64_t ld, int dim4,
+                                                       const float *__restrict__ cb,
                                                        const CodeT *__restrict__ codes,
                                                        const uint8_t *__restrict__ active,
                                                        CodeT *__restrict__ codes_out, int stages, int stage,
-                                                       uint8_t *__restrict__ used) {
+                                                       uint8_t *__restrict__ used, const float *src,
+                                                       int64_t src_ld) {
     const int64_t first = (int64_t)blockIdx.x * 1024;
     const int64_t row0 = first / dim4;            // uniform
     const uint32_t rem0 = (uint32_t)(first % dim4);
@@ -50,13 +53,27 @@ static __global__ void __launch_bounds__(256) k_residual_sub4(float *__restrict_
         if (!on) continue;
         float4 *p = reinterpret_cast<float4 *>(res + row * ld) + t4;
         const float4 c = reinterpret_cast<const float4 *>(cb + (size_t)code * dim4 * 4)[t4];
-        float4 v = *p;
+        float4 v = reinterpret_cast<const float4 *>(src + row * src_ld)[t4];
         v.x = v.x - c.x;
         v.y = v.y - c.y;
         v.z = v.z - c.z;
         v.w = v.w - c.w;
         *p = v;
     }
+}
+
+// The bookkeeping of an encode's last stage alone: nothing reads the residual after it
+// (src/rvq.rs:200-206: the norm test of the last stage only ends a loop that is over).
+template <typename CodeT>
+static __global__ void __launch_bounds__(256) k_rvq_stage_record(int64_t n, const CodeT *__restrict__ stage_codes,
+                                                          const uint8_t *__restrict__ active,
+                                                          CodeT *__restrict__ codes_out, int stages, int stage,
+                                                          uint8_t *__restrict__ used) {
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= n) return;
+    const bool on = active[row] != 0;
+    codes_out[row * stages + stage] = on ? stage_codes[row] : (CodeT)0;
+    if (on) used[row] = (uint8_t)(stage + 1);
 }
 
 // norms[i] = sqrt(sum_t x[i][t]^2), sequential f32 order (src/rvq.rs:134-135).

@@ -279,8 +279,8 @@ int32_t launch_mfma_wide(vq_ctx *ctx, const vq::AssignArgs &a, int sd) {
     {
         ProfSpan sp(ctx, VQ_PROF_ASSIGN_KERNEL);
 #define WIDE(NB)                                                                                             \
-    if (LBG && a.pend_cb)                                                                                    \
-        hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG, NB, LBG>), dim3(cdiv(a.n, 128), (unsigned)a.m),     \
+    if (a.pend_cb)                                                                                           \
+        hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG, NB, true>), dim3(cdiv(a.n, 128), (unsigned)a.m),    \
                            dim3(256), 0, ctx->stream, a, tb);                                                \
     else                                                                                                     \
         hipLaunchKernelGGL((vq::k_assign_mfma_wide_bf<LBG, NB>), dim3(cdiv(a.n, 128), (unsigned)a.m), dim3(256), 0, \
@@ -537,9 +537,23 @@ int32_t check_common(vq_ctx *ctx, const void *x, int64_t n, int64_t ld, int32_t 
 }
 
 
+bool assign_pending_fusable(const vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t sd,
+                            int32_t k, const float *d_codebook) {
+    vq::AssignArgs a;
+    a.x = d_x;
+    a.n = n;
+    a.ld = ld;
+    a.m = 1;
+    a.k = k;
+    a.cb = d_codebook;
+    if (k < 1 || sd % 4 != 0) return false;
+    return (metric == VQ_SQEUCLIDEAN && mfma_wide_applicable<vq::M_SQ, false>(ctx, a, sd)) ||
+           (metric == VQ_EUCLIDEAN && mfma_wide_applicable<vq::M_EUCLID, false>(ctx, a, sd));
+}
+
 int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int64_t ld, int32_t m,
                   int32_t sd, int32_t k, const float *d_codebooks, uint8_t *d_codes, float *d_dist,
-                  bool *dist_written) {
+                  bool *dist_written, const PendingUpdate *pend) {
     if (dist_written) *dist_written = false;
     VQ_TRY(check_common(ctx, d_x, n, ld, m, sd, k));
     if (!d_codebooks || !d_codes) return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: null pointer");
@@ -558,6 +572,16 @@ int32_t assign_codes(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, i
     a.codes = d_codes;
     a.changed = nullptr;
     a.done = nullptr;
+    if (pend) {
+        if (m != 1 || !assign_pending_fusable(ctx, metric, d_x, n, ld, sd, k, d_codebooks) || !pend->cb ||
+            !pend->codes || (reinterpret_cast<uintptr_t>(pend->cb) & 15) != 0 ||
+            (pend->src && (pend->src_ld % 4 != 0 || (reinterpret_cast<uintptr_t>(pend->src) & 15) != 0)))
+            return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter: no pass that takes a pending update");
+        a.pend_cb = pend->cb;
+        a.pend_codes = pend->codes;
+        a.pend_src = pend->src;
+        a.pend_src_ld = pend->src_ld;
+    }
     if (metric == VQ_COSINE) {
         float *cnorm = (float *)(ctx->static_scratch + kNoAllocNormOff);
         if (!ctx->no_alloc) {

@@ -29,7 +29,7 @@ int32_t residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t d
         ((reinterpret_cast<uintptr_t>(d_res) | reinterpret_cast<uintptr_t>(d_codebook)) & 15) == 0)
         hipLaunchKernelGGL(vq::k_residual_sub4<CodeT>, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, ctx->stream,
                            d_res, n, ld, dim / 4, d_codebook, d_codes, (const uint8_t *)nullptr, (CodeT *)nullptr, 0, 0,
-                           (uint8_t *)nullptr);
+                           (uint8_t *)nullptr, (const float *)d_res, ld);
     else
         hipLaunchKernelGGL(vq::k_residual_sub<CodeT>, dim3(cdiv(n * dim, 256)), dim3(256), 0, ctx->stream, d_res, n,
                            ld, dim, d_codebook, d_codes, 1);
@@ -37,13 +37,13 @@ int32_t residual_sub(vq_ctx *ctx, float *d_res, int64_t n, int64_t ld, int32_t d
     return VQ_OK;
 }
 
-inline int32_t assign_any(vq_ctx *ctx, int32_t metric, const float *x, int64_t n, int32_t dim, int32_t k,
-                          const float *cb, uint8_t *codes) {
-    return assign_codes(ctx, metric, x, n, dim, 1, dim, k, cb, codes);
+inline int32_t assign_any(vq_ctx *ctx, int32_t metric, const float *x, int64_t n, int64_t ld, int32_t dim,
+                          int32_t k, const float *cb, uint8_t *codes) {
+    return assign_codes(ctx, metric, x, n, ld, 1, dim, k, cb, codes);
 }
-inline int32_t assign_any(vq_ctx *ctx, int32_t metric, const float *x, int64_t n, int32_t dim, int32_t k,
-                          const float *cb, uint16_t *codes) {
-    return assign_codes_u16(ctx, metric, x, n, dim, 1, dim, k, cb, codes);
+inline int32_t assign_any(vq_ctx *ctx, int32_t metric, const float *x, int64_t n, int64_t ld, int32_t dim,
+                          int32_t k, const float *cb, uint16_t *codes) {
+    return assign_codes_u16(ctx, metric, x, n, ld, 1, dim, k, cb, codes);
 }
 
 template <typename CodeT>
@@ -57,32 +57,68 @@ int32_t rvq_encode(vq_ctx *ctx, int32_t metric, const float *d_x, int64_t n, int
         return fail(ctx, VQ_ERR_INVALID_ARG, "Invalid parameter");
     VQ_HIP(ctx, hipSetDevice(ctx->device));
     hipStream_t st = ctx->stream;
-    VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(float) * (size_t)n * dim));   // residual
-    VQ_TRY(ensure(ctx, ctx->tmp_e, (size_t)n * (2 + sizeof(CodeT)) + 16));  // stage codes, active, used
+    const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(d_codebooks) & 15) == 0;
+    // The first stage reads the caller's rows where they lie and writes the first residual; the last
+    // stage leaves the residual alone.  One stage then needs no residual buffer at all.
+    const bool direct = vec4 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(d_x) & 15) == 0;
+    const bool need_res = stages > 1 || (stages == 1 && !direct);
+    if (need_res) VQ_TRY(ensure(ctx, ctx->tmp_c, sizeof(float) * (size_t)n * dim));   // residual
+    const size_t codes_bytes = ((size_t)n * sizeof(CodeT) + 3) & ~(size_t)3;
+    VQ_TRY(ensure(ctx, ctx->tmp_e, 2 * codes_bytes + 2 * (size_t)n + 16));  // stage codes (two), active, used
     VQ_TRY(ensure(ctx, ctx->tmp_a, sizeof(float) * (size_t)n));         // row norms
     float *norms = (float *)ctx->tmp_a.p;
     float *res = (float *)ctx->tmp_c.p;
-    CodeT *stage_codes = (CodeT *)ctx->tmp_e.p;
-    uint8_t *active = (uint8_t *)ctx->tmp_e.p + (((size_t)n * sizeof(CodeT) + 3) & ~(size_t)3);
+    CodeT *stage_codes[2] = {(CodeT *)ctx->tmp_e.p, (CodeT *)((uint8_t *)ctx->tmp_e.p + codes_bytes)};
+    uint8_t *active = (uint8_t *)ctx->tmp_e.p + 2 * codes_bytes;
     uint8_t *used = active + n;
-    VQ_HIP(ctx, hipMemcpy2DAsync(res, sizeof(float) * dim, d_x, sizeof(float) * ld, sizeof(float) * dim,
-                                 (size_t)n, hipMemcpyDeviceToDevice, st));
-    const bool vec4 = dim % 4 == 0 && (reinterpret_cast<uintptr_t>(d_codebooks) & 15) == 0;
+    // With no norm test between the stages (epsilon <= 0: every row uses every stage) the update of
+    // the residual by a stage's centroids waits for the next stage's assignment, where that pass can
+    // take it along: one pass over the rows per stage instead of two.
+    bool defer = false;
+    if constexpr (sizeof(CodeT) == 1)
+        defer = !(epsilon > 0.0f) && stages > 1 && k >= 2 && vec4 &&
+                assign_pending_fusable(ctx, metric, res, n, dim, dim, k, d_codebooks);
+    if (need_res && !direct)
+        VQ_HIP(ctx, hipMemcpy2DAsync(res, sizeof(float) * dim, d_x, sizeof(float) * ld, sizeof(float) * dim,
+                                     (size_t)n, hipMemcpyDeviceToDevice, st));
     hipLaunchKernelGGL(vq::k_fill<uint8_t>, dim3(cdiv(n, 256)), dim3(256), 0, st, active, n, (uint8_t)1);
     hipLaunchKernelGGL(vq::k_fill<uint8_t>, dim3(cdiv(n, 256)), dim3(256), 0, st, used, n, (uint8_t)0);
+    const float *pend_cb = nullptr;  // the stage whose update of the residual is still to come
+    const CodeT *pend_codes = nullptr;
+    bool pend_from_x = false;        // ... and reads the caller's rows
     for (int s = 0; s < stages; ++s) {
         const float *cb = d_codebooks + (size_t)s * k * dim;
-        if (k < 2)  // src/rvq.rs:186-187
-            hipLaunchKernelGGL(vq::k_fill<CodeT>, dim3(cdiv(n, 256)), dim3(256), 0, st, stage_codes, n, (CodeT)0);
-        else
-            VQ_TRY(assign_any(ctx, metric, res, n, dim, k, cb, stage_codes));
+        CodeT *cur = stage_codes[s & 1];
+        const bool from_x = direct && s == 0;
+        const float *rows = from_x ? d_x : res;
+        const int64_t rows_ld = from_x ? ld : (int64_t)dim;
+        if (k < 2) {  // src/rvq.rs:186-187
+            hipLaunchKernelGGL(vq::k_fill<CodeT>, dim3(cdiv(n, 256)), dim3(256), 0, st, cur, n, (CodeT)0);
+        } else if (pend_cb) {
+            if constexpr (sizeof(CodeT) == 1) {
+                const PendingUpdate pu{pend_cb, pend_codes, pend_from_x ? d_x : nullptr, pend_from_x ? ld : 0};
+                VQ_TRY(assign_codes(ctx, metric, res, n, dim, 1, dim, k, cb, cur, nullptr, nullptr, &pu));
+            }
+            pend_cb = nullptr;
+        } else {
+            VQ_TRY(assign_any(ctx, metric, rows, n, rows_ld, dim, k, cb, cur));
+        }
+        if (s == stages - 1 || defer) {
+            hipLaunchKernelGGL(vq::k_rvq_stage_record<CodeT>, dim3(cdiv(n, 256)), dim3(256), 0, st, n,
+                               (const CodeT *)cur, (const uint8_t *)active, d_codes, stages, s, used);
+            if (s == stages - 1) break;
+            pend_cb = cb;
+            pend_codes = cur;
+            pend_from_x = from_x;
+            continue;
+        }
         if (vec4)
             hipLaunchKernelGGL(vq::k_residual_sub4<CodeT>, dim3(cdiv(n * (dim / 4), 1024)), dim3(256), 0, st, res, n,
-                               (int64_t)dim, dim / 4, cb, (const CodeT *)stage_codes, (const uint8_t *)active, d_codes,
-                               stages, s, used);
+                               (int64_t)dim, dim / 4, cb, (const CodeT *)cur, (const uint8_t *)active, d_codes,
+                               stages, s, used, rows, rows_ld);
         else
             hipLaunchKernelGGL(vq::k_rvq_stage_apply<CodeT>, dim3(cdiv(n * dim, 256)), dim3(256), 0, st, res, n, dim,
-                               cb, (const CodeT *)stage_codes, d_codes, stages, s, (const uint8_t *)active, used);
+                               cb, (const CodeT *)cur, d_codes, stages, s, (const uint8_t *)active, used);
         if (epsilon > 0.0f) {  // a norm is never below a non-positive threshold
             hipLaunchKernelGGL(vq::k_row_norms, dim3(cdiv(n, 64)), dim3(64), 0, st, res, n, (int64_t)dim, dim,
                                norms);
