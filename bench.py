@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0
 PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X published dense bf16 matrix peak
 # rocprofv3 FETCH_SIZE / WRITE_SIZE of one LBG launch of k_assign_mfma_bf (KiB per dispatch), scaled by
 # the plain copy kernel (FETCH x 2.000, WRITE x 1.000): profiles/pq_fit_encode_1Mx128.md
-MEASURED_ASSIGN_TRAFFIC_BYTES = int((273015.0 * 2.000 + 12678.0 * 1.000) * 1024)
+MEASURED_ASSIGN_TRAFFIC_BYTES = int((273044.0 * 2.000 + 12678.0 * 1.000) * 1024)
 
 
 def log(*a):
