@@ -95,12 +95,21 @@ def test_random_rvq_encode(ctx, case):
     x = gen(rng, n, dim, kind)
     cb = (gen(rng, stages * k, dim, kind).reshape(stages, k, dim) * F(0.5)).astype(F)
     eps = float(rng.choice([0.0, 0.0, 0.5, 3.0]))
-    dx, dcb = ctx.to_device(x), ctx.to_device(cb)
+    ld = dim + int(rng.choice([0, 0, 1, 4, 8]))  # the rows inside a wider buffer, aligned or not
+    buf = np.full((n, ld), 7.0, F)
+    buf[:, :dim] = x
+    dx, dcb = ctx.to_device(buf), ctx.to_device(cb)
     dall = ctx.empty((n, stages), np.uint8)
     drec = ctx.empty((n, dim), np.uint16)
     dused = ctx.empty(n, np.uint8)
     for metric in (vq_amd.SQEUCLIDEAN, vq_amd.EUCLIDEAN, vq_amd.COSINE, vq_amd.MANHATTAN):
         with np.errstate(all="ignore"):
             wc, wr = O.rvq_quantize(metric, x, cb, eps)
-        ctx.rvq_encode(metric, dx, n, dim, dim, stages, k, dcb, eps, dall, dused, drec)
-        assert np.array_equal(drec.download(), wr), (metric, n, dim, stages, k, eps, kind)
+        ctx.rvq_encode(metric, dx, n, ld, dim, stages, k, dcb, eps, dall, dused, drec)
+        reached = wc != 0xFFFFFFFF
+        got = dall.download()
+        assert np.array_equal(dused.download(), reached.sum(1)), (metric, n, dim, ld, stages, k, eps, kind)
+        assert np.array_equal(got[reached], wc[reached].astype(np.uint8)), (metric, n, dim, ld, stages, k, eps, kind)
+        assert np.all(got[~reached] == 0)
+        assert np.array_equal(drec.download(), wr), (metric, n, dim, ld, stages, k, eps, kind)
+    assert np.array_equal(dx.download().view(np.uint32), buf.view(np.uint32))  # the caller's rows stay as they were
